@@ -1,0 +1,136 @@
+"""TEST INFRASTRUCTURE -- ctypes binding of the scalar C oracle (q4_oracle.c).
+
+A checker, not a product path: only tests/, the smoke check and the cpu_baseline
+leg of bench.py import this module.  See the header of q4_oracle.c for what each
+function restates (reference file:line) and for its pinning status.
+
+All tensors are numpy arrays (or anything exposing the buffer protocol through
+``numpy.asarray``) that are updated IN PLACE, like the reference's kernels update
+their torch tensors in place (optim/cuda_fused_interface.cc:19-39).
+bf16 data is passed as uint16 bit patterns.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libq4oracle.so")
+
+BLOCK = 128
+FP32, BF16 = 0, 1
+
+
+def build(force=False):
+    """Compile q4_oracle.c with gcc (seconds)."""
+    if force or not os.path.exists(_SO) or (
+        os.path.getmtime(_SO) < os.path.getmtime(os.path.join(_HERE, "q4_oracle.c"))
+    ):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libq4oracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_SO)
+        f, i64, vp, ci = ctypes.c_float, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+        L.q4o_tables.argtypes = [ci, vp, vp]
+        L.q4o_quantize_search.argtypes = [ci, f]
+        L.q4o_quantize_search.restype = ci
+        L.q4o_quantize_count.argtypes = [ci, f]
+        L.q4o_quantize_count.restype = ci
+        L.q4o_derive_scalars.argtypes = [f, f, f, f, f, vp]
+        L.q4o_step_quant.argtypes = [vp, vp, vp, vp, vp, vp, i64, ci, ci, f, f, f, f, f, f]
+        L.q4o_step_unquant.argtypes = [vp, vp, vp, vp, i64, ci, ci, f, f, f, f, f, f]
+        L.q4o_dequant.argtypes = [vp, vp, i64, ci, vp]
+        L.q4o_quant.argtypes = [vp, i64, ci, vp, vp]
+        _lib = L
+    return _lib
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _dtype_tag(a):
+    if a.dtype == np.float32:
+        return FP32
+    if a.dtype == np.uint16:
+        return BF16
+    raise TypeError(f"expected float32 or uint16 (bf16 bits), got {a.dtype}")
+
+
+def tables(which):
+    """(qmap[16], qmid[15]) as float32 arrays; which 0 = first moment, 1 = second."""
+    qmap = np.empty(16, np.float32)
+    qmid = np.empty(15, np.float32)
+    lib().q4o_tables(which, _ptr(qmap), _ptr(qmid))
+    return qmap, qmid
+
+
+def quantize_search(which, x):
+    return lib().q4o_quantize_search(which, float(np.float32(x)))
+
+
+def quantize_count(which, x):
+    return lib().q4o_quantize_count(which, float(np.float32(x)))
+
+
+def derive_scalars(beta1, beta2, lr, weight_decay, step):
+    """fp32 {correction1, correction2_sqrt, step_size, weight_decay_update,
+    resid_beta1, resid_beta2} exactly as the reference launcher derives them."""
+    out = np.empty(6, np.float32)
+    lib().q4o_derive_scalars(beta1, beta2, lr, weight_decay, float(step), _ptr(out))
+    return out
+
+
+def state_sizes(numel):
+    """(code bytes per state, scales per state) for a tensor of numel elements."""
+    return (numel + 1) // 2, (numel + BLOCK - 1) // BLOCK
+
+
+def step_quant(p, g, m_codes, v_codes, m_scale, v_scale, *, beta1, beta2, lr,
+               weight_decay, eps, step):
+    n = p.size
+    nbytes, nblk = state_sizes(n)
+    assert g.size == n and m_codes.size == nbytes and v_codes.size == nbytes
+    assert m_scale.size == nblk and v_scale.size == nblk
+    assert m_codes.dtype == np.uint8 and v_codes.dtype == np.uint8
+    assert m_scale.dtype == np.float32 and v_scale.dtype == np.float32
+    for a in (p, g, m_codes, v_codes, m_scale, v_scale):
+        assert a.flags.c_contiguous
+    lib().q4o_step_quant(_ptr(p), _ptr(g), _ptr(m_codes), _ptr(v_codes), _ptr(m_scale),
+                         _ptr(v_scale), n, _dtype_tag(p), _dtype_tag(g), beta1, beta2, lr,
+                         weight_decay, eps, float(step))
+
+
+def step_unquant(p, g, m, v, *, beta1, beta2, lr, weight_decay, eps, step):
+    n = p.size
+    assert g.size == n and m.size == n and v.size == n
+    assert m.dtype == np.float32 and v.dtype == np.float32
+    for a in (p, g, m, v):
+        assert a.flags.c_contiguous
+    lib().q4o_step_unquant(_ptr(p), _ptr(g), _ptr(m), _ptr(v), n, _dtype_tag(p),
+                           _dtype_tag(g), beta1, beta2, lr, weight_decay, eps, float(step))
+
+
+def dequant(codes, scale, numel, which):
+    out = np.empty(numel, np.float32)
+    lib().q4o_dequant(_ptr(codes), _ptr(scale), numel, which, _ptr(out))
+    return out
+
+
+def quant(x, which):
+    x = np.ascontiguousarray(x, np.float32).ravel()
+    nbytes, nblk = state_sizes(x.size)
+    codes = np.zeros(nbytes, np.uint8)
+    scale = np.zeros(nblk, np.float32)
+    lib().q4o_quant(_ptr(x), x.size, which, _ptr(codes), _ptr(scale))
+    return codes, scale

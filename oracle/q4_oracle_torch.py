@@ -1,0 +1,136 @@
+"""TEST INFRASTRUCTURE -- vectorised torch-CPU restatement of the reference's
+PyTorch path for the 4-bit AdamW step.
+
+A checker and the timed CPU baseline, not a product path: only tests/, the smoke
+check and the cpu_baseline leg of bench.py import this module.
+
+It keeps the three-pass structure of the reference's pure-PyTorch draft
+(optim/adamw_fourbit_triton.py:385-495): (1) unpack + dequantize the moments into
+materialised fp32 tensors, (2) AdamW update with separate torch ops, (3) per-128
+abs-max, divide, quantize, pack (optim/adamw_fourbit_triton.py:618-630,
+:1020-1047).  Operation order and fp32 derived scalars follow the fused CUDA path
+(optim/cuda_adamw_kernels.cu:334-351, :435-440) so that this file and the scalar
+C oracle (q4_oracle.c) are two independent statements of one arithmetic and must
+agree bit for bit.  The reference's per-element Python binary search
+(adamw_fourbit_triton.py:1002-1009) is replaced by torch.bucketize over the
+midpoint table, which returns the same code for every non-NaN input.
+
+Every torch op below rounds once to fp32; none of them takes an ``alpha``/``value``
+multiplier, so no fused multiply-add hides in the update.
+"""
+import math
+
+import numpy as np
+import torch
+
+BLOCK = 128
+
+# optim/adamw_fourbit_triton.py:16-97 (same literals as cuda_adamw_kernels.cu:25-98)
+_QMAP_M = [-0.8875, -0.6625, -0.4375, -0.2125, -0.0775, -0.0325, -0.0055, 0.0,
+           0.0055, 0.0325, 0.0775, 0.2125, 0.4375, 0.6625, 0.8875, 1.0]
+_QMID_M = [-0.775, -0.55, -0.325, -0.145, -0.055, -0.019, -0.00275, 0.00275,
+           0.019, 0.055, 0.145, 0.325, 0.55, 0.775, 0.94375]
+_QMAP_V = [(k + 1) / 16 for k in range(16)]
+_QMID_V = [(2 * k + 1) / 32 for k in range(1, 16)]
+
+QMAP = (torch.tensor(_QMAP_M, dtype=torch.float32), torch.tensor(_QMAP_V, dtype=torch.float32))
+QMID = (torch.tensor(_QMID_M, dtype=torch.float32), torch.tensor(_QMID_V, dtype=torch.float32))
+
+
+def derive_scalars(beta1, beta2, lr, weight_decay, step):
+    """cuda_adamw_kernels.cu:435-440 in fp32 tensors (0-dim)."""
+    f = lambda x: torch.tensor(x, dtype=torch.float32)
+    one = f(1.0)
+    b1, b2, lr_, wd, st = f(beta1), f(beta2), f(lr), f(weight_decay), f(float(step))
+    # powf as a double-precision pow rounded once to fp32 (torch.pow on fp32 tensors
+    # is a vectorised approximation that differs from libm's powf in the last bit)
+    pw1 = f(math.pow(b1.item(), float(step)))
+    pw2 = f(math.pow(b2.item(), float(step)))
+    c1 = one - pw1
+    c2s = f(math.sqrt((one - pw2).item()))
+    return dict(c1=c1, c2s=c2s, ss=lr_ / c1, wdu=one - lr_ * wd, r1=one - b1, r2=one - b2,
+                b1=b1, b2=b2)
+
+
+def unpack(codes, numel):
+    """byte i -> elements 2i (low nibble) and 2i+1 (high nibble)."""
+    lo = codes & 15
+    hi = codes >> 4
+    return torch.stack((lo, hi), dim=1).reshape(-1)[:numel].to(torch.int64)
+
+
+def pack(q, numel):
+    if numel % 2:
+        q = torch.cat((q, q.new_zeros(1)))
+    q = q.reshape(-1, 2).to(torch.uint8)
+    return q[:, 0] | (q[:, 1] << 4)
+
+
+def dequantize(codes, scale, numel, which):
+    """pass 1: materialise an fp32 moment (adamw_fourbit_triton.py:423-450)."""
+    idx = unpack(codes, numel)
+    vals = QMAP[which][idx]
+    s = scale.repeat_interleave(BLOCK)[:numel]
+    return vals * s
+
+
+def quantize(x, which):
+    """pass 3: group abs-max, divide, nearest code, pack."""
+    numel = x.numel()
+    nblk = (numel + BLOCK - 1) // BLOCK
+    padded = torch.zeros(nblk * BLOCK, dtype=torch.float32)
+    padded[:numel] = x
+    grouped = padded.view(nblk, BLOCK)
+    max1 = grouped.abs().amax(dim=1, keepdim=True)          # :623-624, :1078-1087
+    qx = grouped.div(max1)                                   # :625 (0/0 -> NaN)
+    # number of midpoints strictly below x; NaN must land on 0
+    q = torch.bucketize(torch.nan_to_num(qx, nan=-2.0), QMID[which], right=False)
+    return pack(q.reshape(-1)[:numel], numel), max1.reshape(-1)
+
+
+def adamw_update(p, g, m, v, sc, eps):
+    """pass 2: cuda_adamw_kernels.cu:334-351 with separate, individually rounded ops."""
+    m_new = sc["b1"] * m + sc["r1"] * g
+    v_new = sc["b2"] * v + sc["r2"] * (g * g)
+    # torch.sqrt on CPU fp32 is not correctly rounded in every lane; numpy's is
+    root = torch.from_numpy(np.sqrt(v_new.numpy()))
+    denom = root / sc["c2s"] + torch.tensor(eps, dtype=torch.float32)
+    p_new = p * sc["wdu"] - sc["ss"] * (m_new / denom)
+    return p_new, m_new, v_new
+
+
+def step_quant(p, g, m_codes, v_codes, m_scale, v_scale, *, beta1, beta2, lr,
+               weight_decay, eps, step):
+    """Returns new (p, m_codes, v_codes, m_scale, v_scale); p keeps its dtype."""
+    numel = p.numel()
+    sc = derive_scalars(beta1, beta2, lr, weight_decay, step)
+    m = dequantize(m_codes, m_scale, numel, 0)
+    v = dequantize(v_codes, v_scale, numel, 1)
+    p_new, m_new, v_new = adamw_update(p.reshape(-1).float(), g.reshape(-1).float(), m, v, sc, eps)
+    mc, ms = quantize(m_new, 0)
+    vc, vs = quantize(v_new, 1)
+    return p_new.to(p.dtype).view_as(p), mc, vc, ms, vs
+
+
+def step_unquant(p, g, m, v, *, beta1, beta2, lr, weight_decay, eps, step):
+    sc = derive_scalars(beta1, beta2, lr, weight_decay, step)
+    p_new, m_new, v_new = adamw_update(p.reshape(-1).float(), g.reshape(-1).float(),
+                                       m.reshape(-1), v.reshape(-1), sc, eps)
+    return p_new.to(p.dtype).view_as(p), m_new, v_new
+
+
+def closed_form_tables():
+    """Independent constructions of the four tables (double precision, then fp32):
+    second moment k/16 and (2k+1)/32 (quant_opt_base.py:88-102); first moment from
+    the dynamic-exponent construction (quant_opt_base.py:55-86): for exponent level
+    i = 0..2 the 2**i means of adjacent points of linspace(0.1, 1, 2**i + 1), scaled
+    by 10**(i - 2), mirrored, plus 0 and 1.0."""
+    pos = []
+    for i in range(3):
+        n = 2 ** i + 1
+        pts = [0.1 + (1.0 - 0.1) * k / (n - 1) for k in range(n)]
+        means = [(pts[k] + pts[k + 1]) / 2 for k in range(n - 1)]
+        pos += [10.0 ** (i - 2) * x for x in means]
+    qm = sorted([-x for x in pos] + [0.0] + pos + [1.0])
+    mid_m = [(qm[j] + qm[j + 1]) / 2 for j in range(15)]
+    return qm, mid_m, _QMAP_V, _QMID_V
