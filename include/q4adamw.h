@@ -1,0 +1,142 @@
+/*
+ * q4adamw -- C ABI of the MI355X (gfx950) fused 4-bit AdamW step.
+ *
+ * One shared library, plain pointers and sizes, no torch or pybind11 types.  The
+ * entry points stand where the reference's pybind11 module `quantfour_cuda`
+ * stands (optim/cuda_fused_interface.cc:66-69): same argument roles, same order
+ * (param, grad, first moment, second moment, first-moment scales, second-moment
+ * scales, beta1, beta2, lr, weight_decay, eps, step), every hyper-parameter an
+ * fp32 value as pybind11 narrows them there.  Differences that a C ABI forces:
+ * element count and dtypes are explicit, the HIP stream is explicit, and the
+ * status comes back as an int instead of a C++ exception.
+ *
+ * All device pointers are borrowed for the duration of the call; tensors are
+ * updated in place; nothing is retained except an internal descriptor cache that
+ * q4adamw_release() frees.  Calls are asynchronous with respect to the host: work
+ * is enqueued on `stream` (a hipStream_t; NULL is the default stream).
+ *
+ * Return value: 0 on success, negative for an argument error, positive for a
+ * hipError_t raised by the runtime.  q4adamw_last_error() describes the last
+ * failure on the calling thread.
+ */
+#ifndef Q4ADAMW_H
+#define Q4ADAMW_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define Q4ADAMW_FP32 0
+#define Q4ADAMW_BF16 1
+
+#define Q4ADAMW_BLOCK 128 /* elements per quantization block (one scale each) */
+
+#define Q4ADAMW_ERR_ARG (-1)       /* null pointer, negative size, bad dtype tag */
+#define Q4ADAMW_ERR_ALIGN (-2)     /* pointer not aligned for vector access      */
+#define Q4ADAMW_ERR_HYPER (-3)     /* hyper-parameter outside its domain         */
+#define Q4ADAMW_ERR_TOO_LARGE (-4) /* launch would exceed the grid limit         */
+
+/*
+ * One quantized tensor.  Field order follows the tensor arguments of
+ * fused_4bit (optim/cuda_fused_interface.cc:19-21).
+ *   p             numel elements, fp32 or bf16, 16-byte aligned
+ *   g             numel elements, fp32 or bf16, 16-byte aligned
+ *   exp_avg       (numel+1)/2 bytes; byte i = code(2i) | code(2i+1) << 4
+ *   exp_avg_sq    same layout
+ *   exp_avg_scale ceil(numel/128) fp32 block scales of exp_avg
+ *   exp_avg_sq_scale  same for exp_avg_sq
+ * Code buffers must be 4-byte aligned.
+ */
+typedef struct q4adamw_tensor {
+  void *p;
+  const void *g;
+  uint8_t *exp_avg;
+  uint8_t *exp_avg_sq;
+  float *exp_avg_scale;
+  float *exp_avg_sq_scale;
+  int64_t numel;
+} q4adamw_tensor;
+
+/*
+ * One non-quantized tensor (fp32 moments), fields in the order of the tensor
+ * arguments of fused_single_tensor (optim/cuda_fused_interface.cc:49-53).
+ */
+typedef struct q4adamw_small_tensor {
+  void *p;
+  const void *g;
+  float *exp_avg;
+  float *exp_avg_sq;
+  int64_t numel;
+} q4adamw_small_tensor;
+
+/*
+ * Fused 4-bit AdamW step on one tensor.
+ * Replaces fused_4bit (optim/cuda_fused_interface.cc:19-39) and its launcher
+ * cuda_fused_4bit (optim/cuda_adamw_kernels.cu:422-469).
+ */
+int q4adamw_fused_4bit(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_avg_sq,
+                       float *exp_avg_scale, float *exp_avg_sq_scale, int64_t numel,
+                       int p_dtype, int g_dtype, float beta1, float beta2, float lr,
+                       float weight_decay, float eps, float step, void *stream);
+
+/*
+ * The same step over many tensors in one launch.  All tensors share dtypes,
+ * hyper-parameters and step.  `tensors` is a host array.  Replaces the reference's
+ * per-parameter Python loop around fused_4bit (optim/fused_quantfour.py:171-292).
+ */
+int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dtype,
+                             int g_dtype, float beta1, float beta2, float lr,
+                             float weight_decay, float eps, float step, void *stream);
+
+/*
+ * Non-quantized AdamW step (fp32 moments) on one tensor.
+ * Replaces fused_single_tensor (optim/cuda_fused_interface.cc:49-64) and
+ * cuda_fused_single_tensor (optim/cuda_adamw_kernels.cu:136-164).
+ */
+int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *exp_avg_sq,
+                                int64_t numel, int p_dtype, int g_dtype, float beta1,
+                                float beta2, float lr, float weight_decay, float eps,
+                                float step, void *stream);
+
+/* Many non-quantized tensors in one launch (`tensors` is a host array). */
+int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int count,
+                                      int p_dtype, int g_dtype, float beta1, float beta2,
+                                      float lr, float weight_decay, float eps, float step,
+                                      void *stream);
+
+/*
+ * Host-only: the six fp32 scalars the launcher derives from the hyper-parameters
+ * (optim/cuda_adamw_kernels.cu:435-440), in that order: correction1,
+ * correction2_sqrt, step_size, weight_decay_update, resid_beta1, resid_beta2.
+ */
+void q4adamw_derive_scalars(float beta1, float beta2, float lr, float weight_decay,
+                            float step, float *out6);
+
+/*
+ * Host-only: code books and thresholds as the kernels hold them
+ * (optim/cuda_adamw_kernels.cu:25-98).  which: 0 first moment, 1 second moment.
+ */
+void q4adamw_tables(int which, float *qmap16, float *qmid15);
+
+/*
+ * Host-only: entry `index` (0..2047) of the first-moment bucket table the fused
+ * kernel builds in LDS; out2[0] = lower guard bound with the base code in its low
+ * nibble, out2[1] = upper guard bound (fp32 bit patterns).  For tests.
+ */
+int q4adamw_mtable_entry(uint32_t index, uint32_t *out2);
+
+/* Frees the cached descriptor buffers of every device.  Safe to call twice. */
+int q4adamw_release(void);
+
+/* Message for the last non-zero status returned on this thread ("" if none). */
+const char *q4adamw_last_error(void);
+
+/* ABI version: major * 1000 + minor. */
+int q4adamw_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* Q4ADAMW_H */

@@ -1,0 +1,97 @@
+"""ctypes binding of libq4adamw.so (declarations: include/q4adamw.h).
+
+There is no fallback: if the library is missing, loading raises, and every
+optimizer step raises with it.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libq4adamw.so")
+
+FP32, BF16 = 0, 1
+BLOCK = 128
+
+
+class Q4Tensor(ctypes.Structure):
+    """struct q4adamw_tensor"""
+    _fields_ = [
+        ("p", ctypes.c_void_p),
+        ("g", ctypes.c_void_p),
+        ("exp_avg", ctypes.c_void_p),
+        ("exp_avg_sq", ctypes.c_void_p),
+        ("exp_avg_scale", ctypes.c_void_p),
+        ("exp_avg_sq_scale", ctypes.c_void_p),
+        ("numel", ctypes.c_int64),
+    ]
+
+
+class Q4SmallTensor(ctypes.Structure):
+    """struct q4adamw_small_tensor"""
+    _fields_ = [
+        ("p", ctypes.c_void_p),
+        ("g", ctypes.c_void_p),
+        ("exp_avg", ctypes.c_void_p),
+        ("exp_avg_sq", ctypes.c_void_p),
+        ("numel", ctypes.c_int64),
+    ]
+
+
+EXPORTS = (
+    "q4adamw_fused_4bit",
+    "q4adamw_fused_4bit_multi",
+    "q4adamw_fused_single_tensor",
+    "q4adamw_fused_single_tensor_multi",
+    "q4adamw_derive_scalars",
+    "q4adamw_tables",
+    "q4adamw_mtable_entry",
+    "q4adamw_release",
+    "q4adamw_last_error",
+    "q4adamw_version",
+)
+
+_lib = None
+
+
+def load():
+    """Returns the loaded library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m quantfour_adamw_cuda_amd.build` "
+            "(needs hipcc); the 4-bit AdamW step has no other implementation")
+    L = ctypes.CDLL(LIB_PATH)
+    f, i, i64, vp = ctypes.c_float, ctypes.c_int, ctypes.c_int64, ctypes.c_void_p
+    hyper = [f, f, f, f, f, f]  # beta1, beta2, lr, weight_decay, eps, step
+    L.q4adamw_fused_4bit.argtypes = [vp, vp, vp, vp, vp, vp, i64, i, i] + hyper + [vp]
+    L.q4adamw_fused_4bit.restype = i
+    L.q4adamw_fused_4bit_multi.argtypes = [ctypes.POINTER(Q4Tensor), i, i, i] + hyper + [vp]
+    L.q4adamw_fused_4bit_multi.restype = i
+    L.q4adamw_fused_single_tensor.argtypes = [vp, vp, vp, vp, i64, i, i] + hyper + [vp]
+    L.q4adamw_fused_single_tensor.restype = i
+    L.q4adamw_fused_single_tensor_multi.argtypes = [ctypes.POINTER(Q4SmallTensor), i, i, i] + hyper + [vp]
+    L.q4adamw_fused_single_tensor_multi.restype = i
+    L.q4adamw_derive_scalars.argtypes = [f, f, f, f, f, ctypes.POINTER(f)]
+    L.q4adamw_derive_scalars.restype = None
+    L.q4adamw_tables.argtypes = [i, ctypes.POINTER(f), ctypes.POINTER(f)]
+    L.q4adamw_tables.restype = None
+    L.q4adamw_mtable_entry.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
+    L.q4adamw_mtable_entry.restype = i
+    L.q4adamw_release.argtypes = []
+    L.q4adamw_release.restype = i
+    L.q4adamw_last_error.argtypes = []
+    L.q4adamw_last_error.restype = ctypes.c_char_p
+    L.q4adamw_version.argtypes = []
+    L.q4adamw_version.restype = i
+    _lib = L
+    return L
+
+
+def check(status, what):
+    """Turns a non-zero status into the RuntimeError the reference's bindings raise
+    from AT_CUDA_CHECK / AT_ASSERTM (optim/cuda_adamw_kernels.cu:140, :163, :468)."""
+    if status != 0:
+        msg = load().q4adamw_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed with status {status}: {msg}")

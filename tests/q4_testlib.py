@@ -1,0 +1,135 @@
+"""Shared helpers of the parity tests: seeded inputs for the benchmark
+configurations and the comparison of a device step with the CPU oracle."""
+import numpy as np
+import torch
+
+from oracle import q4_oracle as oc
+
+HP = dict(beta1=0.9, beta2=0.999, lr=1e-3, weight_decay=0.01, eps=1e-8)
+HP_DRIVER = dict(beta1=0.8, beta2=0.88, lr=5e-3, weight_decay=0.03, eps=1e-8)  # tests/driver.py:28-31
+
+
+def bits(a):
+    """uint32 view of an fp32 numpy array (for bit-exact comparison incl. -0.0, NaN)."""
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def bf16_bits(t):
+    """torch bf16 tensor -> numpy uint16 bit patterns."""
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16).copy()
+
+
+def to_np(t):
+    if t.dtype == torch.bfloat16:
+        return bf16_bits(t).reshape(-1)
+    return t.detach().cpu().contiguous().numpy().reshape(-1).copy()
+
+
+def grads_config1(gen, n):
+    """N(0, 1e-3^2) with 0.1 % of the entries replaced by +-1e-1 outliers."""
+    g = torch.randn(n, generator=gen) * 1e-3
+    mask = torch.rand(n, generator=gen) < 1e-3
+    sign = torch.where(torch.rand(n, generator=gen) < 0.5, -1.0, 1.0)
+    return torch.where(mask, sign * 1e-1, g)
+
+
+def grads_config3(gen, n):
+    """20 % exact zeros, 1 % fp32 denormals, 0.01 % +-1e3 outliers, rest N(0, 1e-3^2)."""
+    g = torch.randn(n, generator=gen) * 1e-3
+    u = torch.rand(n, generator=gen)
+    sign = torch.where(torch.rand(n, generator=gen) < 0.5, -1.0, 1.0)
+    den_bits = torch.randint(1, 1 << 23, (n,), generator=gen, dtype=torch.int32)
+    den = den_bits.view(torch.float32) * sign
+    g = torch.where(u < 0.20, torch.zeros(()), g)
+    g = torch.where((u >= 0.20) & (u < 0.21), den, g)
+    g = torch.where((u >= 0.21) & (u < 0.2101), sign * 1e3, g)
+    return g
+
+
+def grads_student_t(gen, n, scale=1e-4):
+    """Student-t with 3 degrees of freedom, scaled."""
+    z = torch.randn(n, generator=gen)
+    c = torch.randn(3, n, generator=gen).square().sum(0) / 3.0
+    return z / c.sqrt() * scale
+
+
+class OracleTensor:
+    """CPU-side twin of one quantized tensor, stepped by the C oracle."""
+
+    def __init__(self, p):
+        self.p = to_np(p)
+        n = self.p.size
+        nbytes, nblk = oc.state_sizes(n)
+        self.m = np.zeros(nbytes, np.uint8)
+        self.v = np.zeros(nbytes, np.uint8)
+        self.sm = np.zeros(nblk, np.float32)
+        self.sv = np.zeros(nblk, np.float32)
+
+    def step(self, g, step, hp=HP):
+        """Returns the parameters the step started from."""
+        prev = self.p.copy()
+        oc.step_quant(self.p, to_np(g), self.m, self.v, self.sm, self.sv, step=step, **hp)
+        return prev
+
+    def resync(self, p_dev):
+        """Continue from the device's parameters, so that the parameter bound stays a
+        per-step bound (the moments never depend on the parameters)."""
+        self.p[:] = to_np(p_dev)
+
+
+class DeviceTensor:
+    """Device-side state of one quantized tensor for the functional entry points."""
+
+    def __init__(self, p, device):
+        self.p = p.detach().clone().to(device).reshape(-1).contiguous()
+        n = self.p.numel()
+        nbytes, nblk = oc.state_sizes(n)
+        self.m = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        self.v = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        self.sm = torch.zeros(nblk, dtype=torch.float32, device=device)
+        self.sv = torch.zeros(nblk, dtype=torch.float32, device=device)
+
+
+def p_close(p_dev, p_ref, p_prev, bf16=False):
+    """Parameter tolerance for ONE step from identical inputs.
+    fp32: |dev - ref| <= 1e-6 * max(|ref|, |ref - prev|): 1e-6 relative to the parameter
+    or, for parameters near zero (where a relative bound on the parameter alone cannot
+    hold for anything but bit-identical arithmetic), relative to the step it took.
+    bf16 parameters: at most one bf16 ulp, measured on the same scale.
+    Returns (ok, worst ratio or ulps)."""
+    if bf16:
+        # one bf16 ulp of the larger of the parameter and the step it took (a parameter
+        # that cancels against its update lands near zero, where its own ulp is tiny)
+        f = lambda u: (u.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        dev, ref, prev = f(p_dev), f(p_ref), f(p_prev)
+        scale = np.maximum(np.maximum(np.abs(ref), np.abs(ref - prev)), np.finfo(np.float32).tiny)
+        ulp = 2.0 ** (np.floor(np.log2(scale)) - 7)
+        worst = float((np.abs(dev - ref) / ulp).max())
+        return worst <= 1.0, worst
+    ref = p_ref.astype(np.float64)
+    diff = np.abs(p_dev.astype(np.float64) - ref)
+    scale = np.maximum(np.abs(ref), np.abs(ref - p_prev.astype(np.float64)))
+    scale = np.maximum(scale, np.finfo(np.float32).tiny)
+    worst = float((diff / scale).max())
+    return worst <= 1e-6, worst
+
+
+def assert_state_equal(dev, ref, p_prev, what=""):
+    """codes and scales bit-exact, parameters within tolerance; p_prev holds the
+    parameters both sides started the step from."""
+    m = dev.m.cpu().numpy()
+    v = dev.v.cpu().numpy()
+    sm = dev.sm.cpu().numpy()
+    sv = dev.sv.cpu().numpy()
+    bad = np.flatnonzero(bits(sm) != bits(ref.sm))
+    assert bad.size == 0, f"{what}: first-moment scales differ at blocks {bad[:5]}: {sm[bad[:5]]} vs {ref.sm[bad[:5]]}"
+    bad = np.flatnonzero(bits(sv) != bits(ref.sv))
+    assert bad.size == 0, f"{what}: second-moment scales differ at blocks {bad[:5]}: {sv[bad[:5]]} vs {ref.sv[bad[:5]]}"
+    bad = np.flatnonzero(m != ref.m)
+    assert bad.size == 0, f"{what}: first-moment codes differ at bytes {bad[:5]}: {m[bad[:5]]} vs {ref.m[bad[:5]]} ({bad.size} bytes)"
+    bad = np.flatnonzero(v != ref.v)
+    assert bad.size == 0, f"{what}: second-moment codes differ at bytes {bad[:5]}: {v[bad[:5]]} vs {ref.v[bad[:5]]} ({bad.size} bytes)"
+    is_bf16 = dev.p.dtype == torch.bfloat16
+    ok, worst = p_close(to_np(dev.p), ref.p, p_prev, bf16=is_bf16)
+    assert ok, f"{what}: parameters out of tolerance (worst {worst})"
+    return worst

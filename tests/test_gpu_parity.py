@@ -1,0 +1,243 @@
+"""GPU parity tests: the HIP step, called through the C ABI, against the CPU oracle
+on identical seeded inputs.  Packed codes and block scales must be bit-exact;
+parameters within 1e-6 relative (fp32) or one bf16 ulp (bf16 parameters)."""
+import numpy as np
+import pytest
+import torch
+
+import quantfour_adamw_cuda_amd as q4
+from oracle import q4_oracle as oc
+from tests.q4_testlib import (HP, HP_DRIVER, DeviceTensor, OracleTensor, assert_state_equal, bits,
+                              grads_config1, grads_config3, grads_student_t, p_close, to_np)
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def run_steps(p0, grad_fn, steps, device, hp=HP, g_dtype=torch.float32, what=""):
+    """Steps one tensor on the device and in the oracle; checks after every step."""
+    dev = DeviceTensor(p0, device)
+    ref = OracleTensor(p0)
+    worst = 0.0
+    for t in range(1, steps + 1):
+        g = grad_fn(t).to(g_dtype)
+        say(f"[{what}] step {t} numel {p0.numel()} p {p0.dtype} g {g_dtype}")
+        q4.fused_4bit(dev.p, g.to(device).reshape(-1), dev.m, dev.v, dev.sm, dev.sv,
+                      hp["beta1"], hp["beta2"], hp["lr"], hp["weight_decay"], hp["eps"], t)
+        torch.cuda.synchronize()
+        prev = ref.step(g, t, hp)
+        worst = max(worst, assert_state_equal(dev, ref, prev, f"{what} step {t}"))
+        ref.resync(dev.p)
+    return worst
+
+
+def test_config1_single_tensor(cuda):
+    """4096x4096 fp32, seed 0, outlier-laden grads, 10 steps."""
+    gen = torch.Generator().manual_seed(0)
+    n = 4096 * 4096
+    p0 = torch.randn(n, generator=gen) * 0.02
+    worst = run_steps(p0, lambda t: grads_config1(gen, n), 10, cuda, what="config1")
+    say(f"config1 worst relative parameter error {worst:.3e}")
+
+
+@pytest.mark.parametrize("n", [1, 2, 127, 128, 129, 511, 512, 513, 4095, 4097, 1000003, 3 * 1000003])
+def test_ragged_lengths(cuda, n):
+    """Tail blocks, odd lengths (half-filled last byte), zeros and denormals in the grads."""
+    gen = torch.Generator().manual_seed(1000 + n % 997)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    run_steps(p0, lambda t: grads_config3(gen, n), 3, cuda, what=f"ragged n={n}")
+
+
+def test_all_zero_blocks_and_guard_bytes(cuda):
+    """Blocks whose grads stay zero keep zero codes and zero scales; bytes past the
+    packed length and scales past the last block are never written."""
+    n = 128 * 9 + 37
+    gen = torch.Generator().manual_seed(7)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    g = torch.randn(n, generator=gen) * 1e-3
+    g[128:384] = 0.0          # two all-zero blocks
+    g[640:768] = 0.0
+    nbytes, nblk = oc.state_sizes(n)
+    pad = 64
+    dev = DeviceTensor(p0, cuda)
+    m_big = torch.full((nbytes + pad,), 0xA5, dtype=torch.uint8, device=cuda)
+    v_big = torch.full((nbytes + pad,), 0x5A, dtype=torch.uint8, device=cuda)
+    sm_big = torch.full((nblk + pad,), 123.0, device=cuda)
+    sv_big = torch.full((nblk + pad,), 321.0, device=cuda)
+    p_big = torch.full((n + pad,), 9.0, device=cuda)
+    m_big[:nbytes] = 0
+    v_big[:nbytes] = 0
+    sm_big[:nblk] = 0
+    sv_big[:nblk] = 0
+    p_big[:n] = p0.to(cuda)
+    ref = OracleTensor(p0)
+    for t in range(1, 4):
+        say(f"[zero blocks] step {t}")
+        q4.fused_4bit(p_big[:n], g.to(cuda), m_big[:nbytes], v_big[:nbytes], sm_big[:nblk],
+                      sv_big[:nblk], HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"],
+                      HP["eps"], t)
+        torch.cuda.synchronize()
+        prev = ref.step(g, t)
+        dev.p, dev.m, dev.v, dev.sm, dev.sv = p_big[:n], m_big[:nbytes], v_big[:nbytes], sm_big[:nblk], sv_big[:nblk]
+        assert_state_equal(dev, ref, prev, f"zero blocks step {t}")
+        ref.resync(dev.p)
+        for b in (1, 2, 5):
+            assert ref.sm[b] == 0 and ref.sv[b] == 0
+            assert not ref.m[b * 64:(b + 1) * 64].any() and not ref.v[b * 64:(b + 1) * 64].any()
+    assert (m_big[nbytes:] == 0xA5).all() and (v_big[nbytes:] == 0x5A).all()
+    assert (sm_big[nblk:] == 123.0).all() and (sv_big[nblk:] == 321.0).all()
+    assert (p_big[n:] == 9.0).all()
+
+
+def _nudge(x, d):
+    """x moved by d ulps away from (d > 0) or towards (d < 0) zero."""
+    u = np.float32(x).view(np.uint32)
+    return np.uint32(int(u) + d).view(np.float32)
+
+
+def _threshold_probe_grads(n_blocks, rng):
+    """Gradients that, from zero state, put the normalised moments exactly on and
+    within a few ulps of every quantization threshold.  From zero state
+    m' = r1*g and v' = r2*g*g, so the block's largest |g| fixes the scale and the
+    others are chosen as threshold * largest, nudged by -3..+3 ulps."""
+    qm_mid = oc.tables(0)[1]
+    qv_mid = oc.tables(1)[1]
+    g = np.zeros((n_blocks, 128), np.float32)
+    for b in range(n_blocks):
+        big = np.float32(10.0 ** rng.uniform(-6, 0))
+        row = []
+        for mid in qm_mid:
+            base = np.float32(np.float32(mid) * big)
+            row += [_nudge(base, d) for d in range(-3, 4)]
+        for mid in qv_mid:
+            base = np.float32(np.sqrt(np.float64(mid)) * big)
+            row += [_nudge(base, d) for d in (-1, 0, 1)]
+        row = np.array(row, np.float32)
+        rng.shuffle(row)
+        row = row[:127]
+        g[b, 0] = big
+        g[b, 1:1 + row.size] = row
+    return g.reshape(-1)
+
+
+def test_threshold_neighbourhoods(cuda):
+    """Binary-search boundary ties: values on and next to every threshold."""
+    rng = np.random.default_rng(3)
+    n_blocks = 4096
+    g_np = _threshold_probe_grads(n_blocks, rng)
+    n = g_np.size
+    gen = torch.Generator().manual_seed(3)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    g = torch.from_numpy(g_np)
+    run_steps(p0, lambda t: g if t == 1 else g * float(1 + 0.37 * t), 3, cuda, what="thresholds")
+
+
+def test_dense_threshold_sweep(cuda):
+    """Every block holds one element of magnitude 1 and 127 elements spread over a
+    narrow band around one threshold, so that many quotients fall inside the
+    kernel's guard bands and take its exact path."""
+    qm_mid, qv_mid = oc.tables(0)[1], oc.tables(1)[1]
+    rng = np.random.default_rng(11)
+    rows = []
+    for mid in list(qm_mid) + [float(np.sqrt(x)) for x in qv_mid]:
+        for _ in range(64):
+            big = np.float32(10.0 ** rng.uniform(-5, -1))
+            band = np.float32(mid) * big * (1.0 + rng.uniform(-4e-6, 4e-6, 127))
+            rows.append(np.concatenate(([big], band)).astype(np.float32))
+    g_np = np.concatenate(rows)
+    n = g_np.size
+    gen = torch.Generator().manual_seed(5)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    g = torch.from_numpy(g_np)
+    run_steps(p0, lambda t: g, 2, cuda, what="dense thresholds")
+
+
+def test_extreme_scales(cuda):
+    """Blocks whose abs-max is denormal, tiny, huge: the kernel's reciprocal path does
+    not apply there and the exact path must take over."""
+    rng = np.random.default_rng(5)
+    rows = []
+    for e in (-44, -40, -38, -36, -34, -30, -20, -10, 0, 10, 15, 17):
+        for _ in range(8):
+            rows.append((rng.standard_normal(128) * 10.0 ** e).astype(np.float32))
+    g_np = np.concatenate(rows)
+    n = g_np.size
+    gen = torch.Generator().manual_seed(9)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    g = torch.from_numpy(g_np)
+    run_steps(p0, lambda t: g * float(t), 3, cuda, what="extreme scales")
+
+
+@pytest.mark.parametrize("p_dtype,g_dtype", [(torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32)])
+def test_bf16_io(cuda, p_dtype, g_dtype):
+    """bf16 gradient and bf16 parameter variants (Llama-shaped distributions)."""
+    gen = torch.Generator().manual_seed(21)
+    n = 1024 * 4096 + 777
+    p0 = (torch.randn(n, generator=gen) * 0.02).to(p_dtype)
+    run_steps(p0, lambda t: grads_student_t(gen, n), 3, cuda, g_dtype=g_dtype,
+              what=f"bf16 io p={p_dtype} g={g_dtype}")
+
+
+def test_driver_hyperparameters(cuda):
+    """The reference test's non-default hyper-parameters (tests/driver.py:28-31)."""
+    gen = torch.Generator().manual_seed(2020)
+    n = 300000
+    p0 = torch.randn(n, generator=gen) * 0.1
+    run_steps(p0, lambda t: torch.randn(n, generator=gen) * 1e-2, 10, cuda, hp=HP_DRIVER,
+              what="driver hp")
+
+
+def test_multi_tensor_matches_single(cuda):
+    """One multi-tensor launch equals per-tensor launches bit for bit (params too)."""
+    gen = torch.Generator().manual_seed(31)
+    sizes = [5000, 4097, 128 * 300, 1000003, 9, 70001, 512 * 64, 512 * 64 + 1]
+    ps = [torch.randn(n, generator=gen) * 0.02 for n in sizes]
+    a = [DeviceTensor(p, cuda) for p in ps]
+    b = [DeviceTensor(p, cuda) for p in ps]
+    for t in range(1, 4):
+        gs = [grads_config3(gen, n).to(cuda) for n in sizes]
+        say(f"[multi] step {t}")
+        q4.fused_4bit_multi([x.p for x in a], gs, [x.m for x in a], [x.v for x in a],
+                            [x.sm for x in a], [x.sv for x in a], HP["beta1"], HP["beta2"],
+                            HP["lr"], HP["weight_decay"], HP["eps"], t)
+        for x, g in zip(b, gs):
+            q4.fused_4bit(x.p, g, x.m, x.v, x.sm, x.sv, HP["beta1"], HP["beta2"], HP["lr"],
+                          HP["weight_decay"], HP["eps"], t)
+        torch.cuda.synchronize()
+        for x, y in zip(a, b):
+            assert torch.equal(x.m, y.m) and torch.equal(x.v, y.v)
+            assert torch.equal(x.sm.view(torch.int32), y.sm.view(torch.int32))
+            assert torch.equal(x.sv.view(torch.int32), y.sv.view(torch.int32))
+            assert torch.equal(x.p.view(torch.int32), y.p.view(torch.int32))
+
+
+def test_unquantized_step_vs_oracle(cuda):
+    """Small-tensor path: fp32 moments bit-exact, params within tolerance."""
+    gen = torch.Generator().manual_seed(41)
+    sizes = [1, 768, 2304, 3072, 4096, 10000]
+    ps = [torch.randn(n, generator=gen) * 0.02 for n in sizes]
+    dp = [p.clone().to(cuda) for p in ps]
+    dm = [torch.zeros(n, device=cuda) for n in sizes]
+    dv = [torch.zeros(n, device=cuda) for n in sizes]
+    rp = [p.numpy().copy() for p in ps]
+    rm = [np.zeros(n, np.float32) for n in sizes]
+    rv = [np.zeros(n, np.float32) for n in sizes]
+    for t in range(1, 6):
+        gs = [grads_config3(gen, n) for n in sizes]
+        say(f"[unquant] step {t}")
+        q4.fused_single_tensor_multi(dp, [g.to(cuda) for g in gs], dm, dv, HP["beta1"], HP["beta2"],
+                                     HP["lr"], HP["weight_decay"], HP["eps"], t)
+        torch.cuda.synchronize()
+        for i, g in enumerate(gs):
+            prev = rp[i].copy()
+            oc.step_unquant(rp[i], g.numpy(), rm[i], rv[i], step=t, **HP)
+            assert np.array_equal(bits(dm[i].cpu().numpy()), bits(rm[i]))
+            assert np.array_equal(bits(dv[i].cpu().numpy()), bits(rv[i]))
+            ok, worst = p_close(dp[i].cpu().numpy(), rp[i], prev)
+            assert ok, f"unquant params worst {worst}"
+            rp[i][:] = dp[i].cpu().numpy()
