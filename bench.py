@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused 4-bit AdamW step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b]
+
+One "step" is one `optimizer.step()` over the whole synthetic parameter set: one
+multi-tensor launch of the fused 4-bit kernel plus one launch of the non-quantized
+kernel for the tensors of at most 4096 elements.  Inputs are resident in HBM before
+the timed region starts.  Prints ONE JSON line:
+
+  value         parameters updated per second over the timed region (wall clock
+                around K steps, synchronised on both sides)
+  roofline      the fused kernel against HBM: algorithmic bytes per launch divided
+                by its average duration, measured with events on the launch stream
+                inside the same timed region
+  cpu_baseline  the CPU oracle (vectorised torch restatement of the reference's
+                PyTorch path) timed on this machine's host cores on a bounded
+                sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+HP = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+
+
+def llama3_8b_shapes():
+    shapes = [("embed_tokens", (128256, 4096)), ("lm_head", (128256, 4096))]
+    for i in range(32):
+        shapes += [
+            (f"layers.{i}.q_proj", (4096, 4096)),
+            (f"layers.{i}.k_proj", (1024, 4096)),
+            (f"layers.{i}.v_proj", (1024, 4096)),
+            (f"layers.{i}.o_proj", (4096, 4096)),
+            (f"layers.{i}.gate_proj", (14336, 4096)),
+            (f"layers.{i}.up_proj", (14336, 4096)),
+            (f"layers.{i}.down_proj", (4096, 14336)),
+            (f"layers.{i}.input_layernorm", (4096,)),
+            (f"layers.{i}.post_attention_layernorm", (4096,)),
+        ]
+    shapes.append(("norm", (4096,)))
+    return shapes
+
+
+def llama2_13b_shapes():
+    shapes = [("embed_tokens", (32000, 5120)), ("lm_head", (32000, 5120))]
+    for i in range(40):
+        shapes += [(f"layers.{i}.{n}_proj", (5120, 5120)) for n in "qkvo"]
+        shapes += [
+            (f"layers.{i}.gate_proj", (13824, 5120)),
+            (f"layers.{i}.up_proj", (13824, 5120)),
+            (f"layers.{i}.down_proj", (5120, 13824)),
+            (f"layers.{i}.input_layernorm", (5120,)),
+            (f"layers.{i}.post_attention_layernorm", (5120,)),
+        ]
+    return shapes
+
+
+def gpt2_small_shapes():
+    shapes = [("wte", (50257, 768)), ("wpe", (1024, 768))]
+    for i in range(12):
+        shapes += [
+            (f"h.{i}.ln_1.weight", (768,)), (f"h.{i}.ln_1.bias", (768,)),
+            (f"h.{i}.attn.c_attn.weight", (768, 2304)), (f"h.{i}.attn.c_attn.bias", (2304,)),
+            (f"h.{i}.attn.c_proj.weight", (768, 768)), (f"h.{i}.attn.c_proj.bias", (768,)),
+            (f"h.{i}.ln_2.weight", (768,)), (f"h.{i}.ln_2.bias", (768,)),
+            (f"h.{i}.mlp.c_fc.weight", (768, 3072)), (f"h.{i}.mlp.c_fc.bias", (3072,)),
+            (f"h.{i}.mlp.c_proj.weight", (3072, 768)), (f"h.{i}.mlp.c_proj.bias", (768,)),
+        ]
+    shapes += [("ln_f.weight", (768,)), ("ln_f.bias", (768,))]
+    return shapes
+
+
+WORKLOADS = {
+    # name: (shapes, param dtype, grad dtype, grad distribution, description)
+    "llama3-8b": (llama3_8b_shapes, "float32", "bfloat16", "student_t",
+                  "Llama-3-8B parameter set (BASELINE configs[3]): 291 tensors, fp32 master "
+                  "params, bf16 grads, 4-bit m/v, block 128"),
+    "llama2-13b": (llama2_13b_shapes, "bfloat16", "bfloat16", "student_t",
+                   "Llama-2-13B-shaped parameter set (BASELINE configs[4]): 362 tensors, bf16 "
+                   "params, bf16 grads, 4-bit m/v, block 128"),
+    "gpt2-small": (gpt2_small_shapes, "float32", "float32", "normal_outliers",
+                   "GPT-2-small parameter set (BASELINE configs[1]): 148 tensors, fp32 params and "
+                   "grads, 4-bit m/v, block 128"),
+    "single-4096": (lambda: [("w", (4096, 4096))], "float32", "float32", "normal_outliers",
+                    "single fp32 4096x4096 tensor (BASELINE configs[0])"),
+}
+
+
+def make_grad(torch, shape, dist, gen, device, dtype):
+    n = 1
+    for s in shape:
+        n *= s
+    if dist == "student_t":
+        z = torch.randn(n, generator=gen, device=device)
+        c = torch.zeros(n, device=device)
+        for _ in range(3):
+            c += torch.randn(n, generator=gen, device=device).square_()
+        g = z * torch.rsqrt(c / 3.0) * 1e-4
+    else:
+        g = torch.randn(n, generator=gen, device=device) * 1e-3
+        mask = torch.rand(n, generator=gen, device=device) < 1e-3
+        sign = torch.where(torch.rand(n, generator=gen, device=device) < 0.5, -1.0, 1.0)
+        g = torch.where(mask, sign * 1e-1, g)
+    return g.to(dtype).view(shape)
+
+
+def bytes_per_param(p_dtype, g_dtype):
+    """Algorithmic HBM bytes per parameter of the fused kernel: p read + write, g read,
+    one nibble of each moment read + write, two fp32 scales per 128 read + write."""
+    pb = 4 if p_dtype == "float32" else 2
+    gb = 4 if g_dtype == "float32" else 2
+    return 2 * pb + gb + 2 * (0.5 + 0.5) + 2 * 2 * 4 / 128.0
+
+
+def cpu_baseline(torch, params, grads_set, hp, budget_s=20.0):
+    """Times the torch-CPU oracle on the first quantized tensors of the workload until
+    about budget_s seconds of CPU work have been spent."""
+    from oracle import q4_oracle_torch as ot
+    done_params, spent, used = 0, 0.0, []
+    for p, g in zip(params, grads_set):
+        if p.numel() <= 4096 or p.numel() > (1 << 26):
+            continue
+        pc = p.detach().float().cpu().reshape(-1)
+        gc = g.detach().cpu().reshape(-1)
+        n = pc.numel()
+        mc = torch.zeros((n + 1) // 2, dtype=torch.uint8)
+        vc = mc.clone()
+        ms = torch.zeros((n + 127) // 128)
+        vs = ms.clone()
+        ot.step_quant(pc[:4096], gc[:4096], mc[:2048], vc[:2048], ms[:32], vs[:32], step=1,
+                      beta1=hp["betas"][0], beta2=hp["betas"][1], lr=hp["lr"],
+                      weight_decay=hp["weight_decay"], eps=hp["eps"])  # warm caches
+        for step in (1, 2):
+            t0 = time.perf_counter()
+            pc, mc, vc, ms, vs = ot.step_quant(pc, gc, mc, vc, ms, vs, step=step,
+                                               beta1=hp["betas"][0], beta2=hp["betas"][1],
+                                               lr=hp["lr"], weight_decay=hp["weight_decay"],
+                                               eps=hp["eps"])
+            spent += time.perf_counter() - t0
+            done_params += n
+        used.append(f"{tuple(p.shape)}x2 steps")
+        if spent >= budget_s:
+            break
+    return {
+        "value": done_params / spent if spent else None,
+        "unit": "params/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "torch-CPU 3-pass oracle on tensors " + ", ".join(used) + f" ({spent:.1f} s)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama3-8b", choices=sorted(WORKLOADS))
+    ap.add_argument("--grad-sets", type=int, default=2,
+                    help="distinct pre-generated gradient sets rotated over the steps")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures the optimizer step on ONE GPU; the step needs "
+                 "no collectives and every rank of a sharded job would run this same kernel "
+                 "on its own shard. Run with --gpus 1.")
+
+    import torch
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    shapes_fn, p_dtype_s, g_dtype_s, dist, desc = WORKLOADS[args.workload]
+    p_dtype, g_dtype = getattr(torch, p_dtype_s), getattr(torch, g_dtype_s)
+    shapes = shapes_fn()
+
+    gen = torch.Generator(device=device).manual_seed(0)
+    params = []
+    for _, shape in shapes:
+        p = (torch.randn(shape, generator=gen, device=device) * 0.02).to(p_dtype)
+        p = torch.nn.Parameter(p, requires_grad=True)
+        if g_dtype != p_dtype:
+            p.grad_dtype = g_dtype  # fp32 master parameter with a bf16 gradient
+        params.append(p)
+    grad_sets = [[make_grad(torch, shape, dist, gen, device, g_dtype) for _, shape in shapes]
+                 for _ in range(max(1, args.grad_sets))]
+    total_params = sum(p.numel() for p in params)
+    quant_params = sum(p.numel() for p in params if p.numel() > 4096)
+
+    opt = AdamWFused_QuantFour(params, **HP)
+    opt.kernel_timing = []  # (kind, start event, end event) per launch
+
+    def one_step(i):
+        gs = grad_sets[i % len(grad_sets)]
+        for p, g in zip(params, gs):
+            p.grad = g
+        opt.step()
+
+    for i in range(args.warmup):
+        one_step(i)
+    torch.cuda.synchronize()
+    opt.kernel_timing.clear()
+
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        one_step(args.warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    fused_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "fused_4bit"]
+    avg_kernel_s = sum(fused_ms) / len(fused_ms) / 1e3
+    algo_bytes = quant_params * bytes_per_param(p_dtype_s, g_dtype_s)
+    achieved = algo_bytes / avg_kernel_s / 1e9
+
+    out = {
+        "metric": "params_updated_per_sec_fused_4bit_adamw_step",
+        "value": total_params * args.steps / elapsed,
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": desc,
+            "tensors": len(params),
+            "params": total_params,
+            "params_quantized": quant_params,
+            "param_dtype": p_dtype_s,
+            "grad_dtype": g_dtype_s,
+            "grad_sets": len(grad_sets),
+            "hyper": {"lr": HP["lr"], "betas": list(HP["betas"]), "eps": HP["eps"],
+                      "weight_decay": HP["weight_decay"]},
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "fused_4bit_kernel",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": algo_bytes,
+            "avg_launch_ms": avg_kernel_s * 1e3,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, params, grad_sets[0], HP)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -5,15 +5,18 @@
 // (-ffp-contract=off matters: the moment updates must be individually rounded
 // fp32 multiplies and adds; fused multiply-adds appear only where written out).
 //
-// Work decomposition of the fused kernel
-//   tile      = 512 consecutive elements = 4 quantization blocks, handled by one
-//               wave64 in one pass: lane l owns elements [8l, 8l+8), so a block is
-//               exactly one 16-lane DPP row and its abs-max needs four DPP steps,
-//               no LDS and no barrier.
-//   chunk     = 8 * tiles_per_wave consecutive tiles of ONE tensor, handled by one
-//               512-thread workgroup; wave w takes tiles w, w+8, w+16, ...
-//   launch    = all chunks of all tensors; a workgroup finds its tensor by binary
-//               search over the per-tensor first-chunk prefix (scalar loads).
+// Work decomposition of the fused kernel (shaped by measurement: HBM on this part
+// streams best when every wave is short-lived, touches 1 KiB of the widest stream
+// with ONE 16-byte access per lane, and every access is marked non-temporal)
+//   tile    = 256 consecutive elements = 2 quantization blocks = one wave64, one
+//             pass: lane l owns elements [4l, 4l+4).  A block is 32 lanes: its
+//             abs-max is one v_permlane16_swap plus four DPP row steps, no LDS
+//             traffic and no barrier.
+//   chunk   = 4 tiles (1024 elements) of ONE tensor = one 256-thread workgroup.
+//   launch  = all chunks of up to kMaxTensors tensors.  The tensor descriptors and
+//             the per-tensor first-chunk prefix travel in the kernel arguments, so
+//             a workgroup finds its tensor with two scalar loads from the kernarg
+//             segment and nothing is staged in device memory.
 // Per element the kernel reads p, g and one nibble of each moment, and writes p
 // and one nibble of each moment; per block it reads and writes two fp32 scales.
 #include <hip/hip_runtime.h>
@@ -21,41 +24,20 @@
 #include <stdint.h>
 #include <string.h>
 
-#include <algorithm>
-#include <mutex>
 #include <string>
-#include <vector>
 
 #include "../../include/q4adamw.h"
 #include "q4adamw_tables.h"
 
 namespace q4 {
 
-constexpr int kTile = 512;
-constexpr int kWaves = 8;
+constexpr int kTile = 256;                 // elements per wave
+constexpr int kWaves = 4;                  // waves per workgroup
 constexpr int kThreads = kWaves * 64;
-constexpr int kSmallThreads = 256;
-constexpr int kSmallChunk = 4096;
-
-struct TensorDesc {  // 64 bytes, device-visible
-  void *p;
-  const void *g;
-  uint32_t *m;
-  uint32_t *v;
-  float *sm;
-  float *sv;
-  int64_t numel;
-  int64_t chunk0;  // index of this tensor's first chunk in the launch
-};
-
-struct SmallDesc {  // 48 bytes
-  void *p;
-  const void *g;
-  float *m;
-  float *v;
-  int64_t numel;
-  int64_t chunk0;
-};
+constexpr int kChunk = kTile * kWaves;     // elements per workgroup
+constexpr int kMaxTensors = 48;            // tensors per fused launch
+constexpr int kSmallChunk = 1024;          // elements per workgroup, non-quantized kernel
+constexpr int kMaxSmallTensors = 64;
 
 // derived on the host exactly as optim/cuda_adamw_kernels.cu:435-440
 struct StepConsts {
@@ -65,6 +47,50 @@ struct StepConsts {
   float eps;
 };
 
+struct TensorDesc {  // 56 bytes
+  void *p;
+  const void *g;
+  uint8_t *m;
+  uint8_t *v;
+  float *sm;
+  float *sv;
+  int64_t numel;
+};
+
+// Kernel arguments of one fused launch (about 3 KiB, passed by value).
+// first_chunk[i] = index of tensor i's first chunk; entries past ntensors hold
+// 0xffffffff.  pivot[k] = first_chunk[8k] lets a workgroup find its tensor with two
+// 8-wide scalar loads.
+struct FusedArgs {
+  StepConsts sc;
+  int ntensors;
+  uint32_t pivot[8];
+  uint32_t first_chunk[kMaxTensors + 8];
+  TensorDesc desc[kMaxTensors];
+};
+
+struct SmallDesc {  // 40 bytes
+  void *p;
+  const void *g;
+  float *m;
+  float *v;
+  int64_t numel;
+};
+
+struct SmallArgs {
+  StepConsts sc;
+  int ntensors;
+  uint32_t pivot[8];
+  uint32_t first_chunk[kMaxSmallTensors + 8];
+  SmallDesc desc[kMaxSmallTensors];
+};
+
+static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+
+// bucket table entries that hold a threshold and the two code books (see
+// q4adamw_tables.h), read by every workgroup at start-up
+__device__ const WorkgroupTables kWorkgroupTables = make_workgroup_tables();
+
 // ---------------------------------------------------------------------------
 // device helpers
 // ---------------------------------------------------------------------------
@@ -73,11 +99,22 @@ struct StepConsts {
 template <typename T>
 using gptr = __attribute__((address_space(1))) T *;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
 __device__ __forceinline__ gptr<T> as_global(const void *p) {
   return (gptr<T>)(uintptr_t)p;
+}
+
+// Every byte is touched once per step: stream past the caches.
+template <typename T>
+__device__ __forceinline__ T stream_load(gptr<const T> p) {
+  return __builtin_nontemporal_load(p);
+}
+template <typename T>
+__device__ __forceinline__ void stream_store(gptr<T> p, T v) {
+  __builtin_nontemporal_store(v, p);
 }
 
 template <int CTRL>
@@ -86,11 +123,14 @@ __device__ __forceinline__ uint32_t dpp_umax(uint32_t x) {
   return x > y ? x : y;
 }
 
-// Max over the 16 lanes of a DPP row, result in every lane of the row.  The input
-// is a non-negative float (an abs-max), so its bit pattern orders like an unsigned
-// integer and the reduction is four v_max_u32 with a DPP operand.
-__device__ __forceinline__ float row_max16(float x) {
+// Max over the 32 lanes of a quantization block (lanes 0-31 or 32-63), result in
+// every lane of the block.  The input is a non-negative float (an abs-max), so its
+// bit pattern orders like an unsigned integer.
+__device__ __forceinline__ float block_max32(float x) {
   uint32_t u = f2bits(x);
+  // rows 0<->1 and 2<->3 exchanged: lane i of a row meets lane i of its partner row
+  const auto sw = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  u = sw[0] > sw[1] ? sw[0] : sw[1];
   u = dpp_umax<0xB1>(u);   // quad_perm [1,0,3,2]
   u = dpp_umax<0x4E>(u);   // quad_perm [2,3,0,1]
   u = dpp_umax<0x141>(u);  // row_half_mirror
@@ -104,25 +144,21 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nea
   return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
-// eight consecutive elements starting at element index e0 (a multiple of 8)
+// four consecutive elements starting at element index e0 (a multiple of 4)
 template <bool BF, bool FULL>
-__device__ __forceinline__ void load8(const void *base, int64_t e0, int nv, float (&x)[8]) {
+__device__ __forceinline__ void load4(const void *base, int64_t e0, int nv, float (&x)[4]) {
   if (FULL) {
     if (BF) {
-      const u32x4 w = *as_global<const u32x4>(static_cast<const uint16_t *>(base) + e0);
+      const u32x2 w = stream_load(as_global<const u32x2>(static_cast<const uint16_t *>(base) + e0));
       x[0] = bits2f(w.x << 16); x[1] = bits2f(w.x & 0xffff0000u);
       x[2] = bits2f(w.y << 16); x[3] = bits2f(w.y & 0xffff0000u);
-      x[4] = bits2f(w.z << 16); x[5] = bits2f(w.z & 0xffff0000u);
-      x[6] = bits2f(w.w << 16); x[7] = bits2f(w.w & 0xffff0000u);
     } else {
-      const gptr<const f32x4> q = as_global<const f32x4>(static_cast<const float *>(base) + e0);
-      const f32x4 a = q[0], b = q[1];
+      const f32x4 a = stream_load(as_global<const f32x4>(static_cast<const float *>(base) + e0));
       x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
-      x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < 4; ++j) {
       x[j] = 0.0f;
       if (j < nv) {
         x[j] = BF ? bf16_bits_to_f32(as_global<const uint16_t>(base)[e0 + j])
@@ -133,23 +169,19 @@ __device__ __forceinline__ void load8(const void *base, int64_t e0, int nv, floa
 }
 
 template <bool BF, bool FULL>
-__device__ __forceinline__ void store8(void *base, int64_t e0, int nv, const float (&x)[8]) {
+__device__ __forceinline__ void store4(void *base, int64_t e0, int nv, const float (&x)[4]) {
   if (FULL) {
     if (BF) {
-      u32x4 w;
+      u32x2 w;
       w.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
       w.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
-      w.z = f32_to_bf16_bits(x[4]) | (f32_to_bf16_bits(x[5]) << 16);
-      w.w = f32_to_bf16_bits(x[6]) | (f32_to_bf16_bits(x[7]) << 16);
-      *as_global<u32x4>(static_cast<uint16_t *>(base) + e0) = w;
+      stream_store(as_global<u32x2>(static_cast<uint16_t *>(base) + e0), w);
     } else {
-      const gptr<f32x4> q = as_global<f32x4>(static_cast<float *>(base) + e0);
-      q[0] = f32x4{x[0], x[1], x[2], x[3]};
-      q[1] = f32x4{x[4], x[5], x[6], x[7]};
+      stream_store(as_global<f32x4>(static_cast<float *>(base) + e0), f32x4{x[0], x[1], x[2], x[3]});
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < 4; ++j) {
       if (j < nv) {
         if (BF) as_global<uint16_t>(base)[e0 + j] = (uint16_t)f32_to_bf16_bits(x[j]);
         else as_global<float>(base)[e0 + j] = x[j];
@@ -158,18 +190,18 @@ __device__ __forceinline__ void store8(void *base, int64_t e0, int nv, const flo
   }
 }
 
-// Exact quantization of eight values of one state: IEEE division by the block
-// scale, then the number of thresholds strictly below the quotient
-// (cuda_adamw_kernels.cu:167-194 in closed form).  0/0 is NaN and gets code 0.
-struct F8 {
-  float x[8];
+struct F4 {
+  float x[4];
 };
 
+// Exact quantization of four values of one state: IEEE division by the block
+// scale, then the number of thresholds strictly below the quotient
+// (cuda_adamw_kernels.cu:167-194 in closed form).  0/0 is NaN and gets code 0.
 template <bool SECOND>
-__device__ __noinline__ uint32_t quantize8_exact(F8 v, float scale) {
+__device__ __noinline__ uint32_t quantize4_exact(F4 v, float scale) {
   uint32_t word = 0;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int j = 0; j < 4; ++j) {
     const float q = v.x[j] / scale;
     uint32_t c = 0;
 #pragma unroll
@@ -194,36 +226,92 @@ constexpr float kScaleLo = 7.888609052210118e-31f;   // 2^-100
 constexpr float kScaleHi = 1.2676506002282294e+30f;  // 2^100
 constexpr float kVGuard = 7.62939453125e-06f;        // 2^-17, in units of 16*q
 
+// Uniform search of the launch's tensor list: the last tensor whose first chunk is
+// <= chunk.  first_chunk[0] is 0, so the result is never negative.
+template <typename Args>
+__device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
+  int group = 0;
+#pragma unroll
+  for (int k = 1; k < 8; ++k) group += (a.pivot[k] <= chunk) ? 1 : 0;
+  int within = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) within += (a.first_chunk[group * 8 + k] <= chunk) ? 1 : 0;
+  return group * 8 + within - 1;
+}
+
+// LDS tables of a workgroup: the full-size bucket table, of which only the 76
+// entries that a clamped quotient can reach are written (the rest is never read),
+// and the two code books.
+struct LdsTables {
+  __attribute__((aligned(16))) char mtab[kMtabEntries * 8];
+  float qm[16];
+  float qv[16];
+};
+
+// This thread's slot of the workgroup tables, requested from memory as the very
+// first thing a wave does (only the first two waves hold slots).
+struct TableSlot {
+  uint32_t a, b;
+};
+
+__device__ __forceinline__ TableSlot request_table_slot(int tid) {
+  TableSlot s{0u, 0u};
+  if (tid < 128) {
+    s.a = kWorkgroupTables.a[tid];
+    s.b = kWorkgroupTables.b[tid];
+  }
+  return s;
+}
+
+// Writes the slot into LDS and waits for the whole workgroup.  Called by every wave
+// exactly once, after it has issued its global loads, so that the latencies
+// overlap.  The fences order LDS only: a full __syncthreads() would also drain the
+// outstanding global loads.
+__device__ __forceinline__ void setup_tables(LdsTables &lds, int tid, TableSlot s) {
+  if (tid < (int)(2 * kBucketsPerSign)) {
+    *reinterpret_cast<uint2 *>(lds.mtab + compact_slot_bucket((uint32_t)tid) * 8) = make_uint2(s.a, s.b);
+  } else if (tid >= 96 && tid < 112) {
+    lds.qm[tid - 96] = bits2f(s.a);
+  } else if (tid >= 112 && tid < 128) {
+    lds.qv[tid - 112] = bits2f(s.a);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---------------------------------------------------------------------------
-// one tile of one tensor
+// one tile (256 elements) of one tensor
 // ---------------------------------------------------------------------------
 template <bool PBF, bool GBF, bool FULL>
-__device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane,
-                                             const StepConsts &sc, const uint2 *mtab,
-                                             const float *lds_qm, const float *lds_qv) {
+__device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int tid,
+                                             const StepConsts &sc, LdsTables &lds, TableSlot slot) {
+  const char *lds_mtab = lds.mtab;
+  const float *lds_qm = lds.qm;
+  const float *lds_qv = lds.qv;
   const int64_t numel = T.numel;
-  const int64_t e0 = tile * kTile + (int64_t)lane * 8;
-  int nv = 8;
+  const int64_t e0 = tile * kTile + (int64_t)lane * 4;
+  int nv = 4;
   if (!FULL) {
     const int64_t rem = numel - e0;
-    nv = rem >= 8 ? 8 : (rem > 0 ? (int)rem : 0);
+    nv = rem >= 4 ? 4 : (rem > 0 ? (int)rem : 0);
   }
-  const int64_t blk = e0 >> 7;
-  const bool row_ok = FULL || (blk << 7) < numel;
+  const int64_t blk = tile * 2 + (lane >> 5);
+  const bool blk_ok = FULL || (blk << 7) < numel;
 
-  float p[8], g[8];
-  load8<PBF, FULL>(T.p, e0, nv, p);
-  load8<GBF, FULL>(T.g, e0, nv, g);
+  float p[4], g[4];
+  load4<PBF, FULL>(T.p, e0, nv, p);
+  load4<GBF, FULL>(T.g, e0, nv, g);
   uint32_t mw = 0, vw = 0;
   if (FULL) {
-    mw = as_global<const uint32_t>(T.m)[e0 >> 3];
-    vw = as_global<const uint32_t>(T.v)[e0 >> 3];
+    mw = stream_load(as_global<const uint16_t>(T.m) + (e0 >> 2));
+    vw = stream_load(as_global<const uint16_t>(T.v) + (e0 >> 2));
   } else {
     const gptr<const uint8_t> mb = as_global<const uint8_t>(T.m) + (e0 >> 1);
     const gptr<const uint8_t> vb = as_global<const uint8_t>(T.v) + (e0 >> 1);
     const int nb = (nv + 1) >> 1;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < 2; ++k) {
       if (k < nb) {
         mw |= (uint32_t)mb[k] << (8 * k);
         vw |= (uint32_t)vb[k] << (8 * k);
@@ -231,16 +319,17 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     }
   }
   float sm_old = 0.0f, sv_old = 0.0f;
-  if (row_ok) {
-    sm_old = as_global<const float>(T.sm)[blk];
-    sv_old = as_global<const float>(T.sv)[blk];
+  if (blk_ok) {
+    sm_old = stream_load(as_global<const float>(T.sm) + blk);
+    sv_old = stream_load(as_global<const float>(T.sv) + blk);
   }
+  setup_tables(lds, tid, slot);
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
-  F8 mn, vn;
+  F4 mn, vn;
   float am = 0.0f, av = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int j = 0; j < 4; ++j) {
     const float m_old = lds_qm[(mw >> (4 * j)) & 15u] * sm_old;
     const float v_old = lds_qv[(vw >> (4 * j)) & 15u] * sv_old;
     const float gj = g[j];
@@ -256,14 +345,14 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
     av = __builtin_fmaxf(av, v);
   }
-  store8<PBF, FULL>(T.p, e0, nv, p);
+  store4<PBF, FULL>(T.p, e0, nv, p);
 
   // block scales (exact: max is order independent)
-  am = row_max16(am);
-  av = row_max16(av);
-  if (row_ok && (lane & 15) == 0) {
-    as_global<float>(T.sm)[blk] = am;
-    as_global<float>(T.sv)[blk] = av;
+  am = block_max32(am);
+  av = block_max32(av);
+  if (blk_ok && (lane & 31) == 0) {
+    stream_store(as_global<float>(T.sm) + blk, am);
+    stream_store(as_global<float>(T.sv) + blk, av);
   }
 
   // fast quantization: multiply by a refined reciprocal, decide every code whose
@@ -275,39 +364,44 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   uint32_t mword = 0, vword = 0;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int j = 0; j < 4; ++j) {
+    // first moment: bucket = top 11 bits of the quotient, clamped per sign to the
+    // lowest bucket the workgroup built
     const float qm = mn.x[j] * rm;
-    const uint2 ent = mtab[f2bits(qm) >> 21];
+    uint32_t a = (f2bits(qm) >> 18) & 0x3FF8u;
+    const uint32_t floor_a = (a & (kNegativeBuckets * 8u)) | (kBucketFloor * 8u);
+    a = a > floor_a ? a : floor_a;
+    const uint2 ent = *reinterpret_cast<const uint2 *>(lds_mtab + a);
     const bool above_hi = qm > bits2f(ent.y);
     const bool above_lo = qm > bits2f(ent.x);
     redo |= (above_hi != above_lo);
     mword |= ((ent.x & 15u) + (above_hi ? 1u : 0u)) << (4 * j);
 
     // second moment: thresholds at 16q = k + 0.5, k = 1..15
-    const float a = __builtin_fmaf(vn.x[j] * rv, 16.0f, kVGuard - 0.5f);
-    redo |= __builtin_amdgcn_fractf(a) < 2.0f * kVGuard;
-    vword |= (uint32_t)(int)a << (4 * j);  // a > -1, so truncation gives 0 for a < 0
+    const float t = __builtin_fmaf(vn.x[j] * rv, 16.0f, kVGuard - 0.5f);
+    redo |= __builtin_amdgcn_fractf(t) < 2.0f * kVGuard;
+    vword |= (uint32_t)(int)t << (4 * j);  // t > -1, so truncation gives 0 for t < 0
   }
   if (__builtin_expect(redo, 0)) {
-    mword = quantize8_exact<false>(mn, am);
-    vword = quantize8_exact<true>(vn, av);
+    mword = quantize4_exact<false>(mn, am);
+    vword = quantize4_exact<true>(vn, av);
   }
   if (am == 0.0f) mword = 0;  // 0/0: code 0 for the whole block
   if (!FULL) {
-    const uint32_t keep = nv >= 8 ? 0xffffffffu : ((1u << (4 * nv)) - 1u);
+    const uint32_t keep = nv >= 4 ? 0xffffu : ((1u << (4 * nv)) - 1u);
     mword &= keep;
     vword &= keep;
   }
 
   if (FULL) {
-    as_global<uint32_t>(T.m)[e0 >> 3] = mword;
-    as_global<uint32_t>(T.v)[e0 >> 3] = vword;
+    stream_store(as_global<uint16_t>(T.m) + (e0 >> 2), (uint16_t)mword);
+    stream_store(as_global<uint16_t>(T.v) + (e0 >> 2), (uint16_t)vword);
   } else {
     const gptr<uint8_t> mb = as_global<uint8_t>(T.m) + (e0 >> 1);
     const gptr<uint8_t> vb = as_global<uint8_t>(T.v) + (e0 >> 1);
     const int nb = (nv + 1) >> 1;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < 2; ++k) {
       if (k < nb) {
         mb[k] = (uint8_t)(mword >> (8 * k));
         vb[k] = (uint8_t)(vword >> (8 * k));
@@ -317,62 +411,35 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
 }
 
 template <bool PBF, bool GBF>
-__global__ __launch_bounds__(kThreads) void fused_4bit_kernel(
-    const TensorDesc *__restrict__ descs, int ntensors, TensorDesc one, int tiles_per_wave,
-    StepConsts sc) {
-  __shared__ uint2 mtab[kMtabEntries];
-  __shared__ float lds_qm[16];
-  __shared__ float lds_qv[16];
+__global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
+  __shared__ LdsTables lds;
   const int tid = threadIdx.x;
-  for (int i = tid; i < (int)kMtabEntries; i += kThreads) {
-    const MtabEntry e = mtab_entry((uint32_t)i);
-    mtab[i] = make_uint2(e.lo, e.hi);
-  }
-  if (tid < 16) {
-    lds_qm[tid] = bits2f(kQmapMBits[tid]);
-    lds_qv[tid] = qmap_v(tid);
-  }
-  __syncthreads();
-
-  const int64_t chunk = blockIdx.x;
-  TensorDesc T = one;
-  if (ntensors > 0) {
-    int lo = 0, hi = ntensors - 1;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (descs[mid].chunk0 <= chunk) lo = mid; else hi = mid - 1;
-    }
-    T = descs[lo];
-  }
+  const TableSlot slot = request_table_slot(tid);
+  const uint32_t chunk = blockIdx.x;
+  const int t = find_tensor(args, chunk);
+  const TensorDesc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int64_t ntiles = (T.numel + kTile - 1) / kTile;
-  const int64_t tile0 = (chunk - T.chunk0) * (int64_t)(kWaves * tiles_per_wave) + wave;
-  for (int k = 0; k < tiles_per_wave; ++k) {
-    const int64_t tile = tile0 + (int64_t)k * kWaves;
-    if (tile >= ntiles) break;
-    if ((tile + 1) * kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, sc, mtab, lds_qm, lds_qv);
-    else process_tile<PBF, GBF, false>(T, tile, lane, sc, mtab, lds_qm, lds_qv);
+  const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
+  const int64_t begin = tile * kTile;
+  if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
+    setup_tables(lds, tid, slot);
+    return;
   }
+  if (begin + kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, tid, args.sc, lds, slot);
+  else process_tile<PBF, GBF, false>(T, tile, lane, tid, args.sc, lds, slot);
 }
 
 // Non-quantized step for small tensors (cuda_adamw_kernels.cu:100-133): fp32
 // moments in place, same derived scalars and operation order as the fused path.
 template <bool PBF, bool GBF>
-__global__ __launch_bounds__(kSmallThreads) void single_tensor_kernel(
-    const SmallDesc *__restrict__ descs, int ntensors, SmallDesc one, StepConsts sc) {
-  const int64_t chunk = blockIdx.x;
-  SmallDesc T = one;
-  if (ntensors > 0) {
-    int lo = 0, hi = ntensors - 1;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (descs[mid].chunk0 <= chunk) lo = mid; else hi = mid - 1;
-    }
-    T = descs[lo];
-  }
-  const int64_t base = (chunk - T.chunk0) * kSmallChunk;
+__global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args) {
+  const uint32_t chunk = blockIdx.x;
+  const int t = find_tensor(args, chunk);
+  const SmallDesc &T = args.desc[t];
+  const StepConsts &sc = args.sc;
+  const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kSmallChunk;
   const int64_t end = base + kSmallChunk < T.numel ? base + kSmallChunk : T.numel;
-  for (int64_t i = base + threadIdx.x; i < end; i += kSmallThreads) {
+  for (int64_t i = base + threadIdx.x; i < end; i += 256) {
     const float gi = GBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.g)[i])
                          : as_global<const float>(T.g)[i];
     const float pi = PBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.p)[i])
@@ -432,173 +499,45 @@ static int make_consts(float beta1, float beta2, float lr, float wd, float eps, 
 
 static bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-// Device copies of descriptor tables.  A small ring per device: a table whose
-// bytes equal what a slot already holds is not uploaded again; a slot is only
-// overwritten after the last launch that read it has finished.
-struct Slot {
-  void *dev = nullptr;
-  void *host = nullptr;  // pinned staging
-  size_t cap = 0;
-  hipEvent_t done = nullptr;
-  bool pending = false;
-  std::vector<char> content;
-};
-struct DevCache {
-  int device = -1;
-  Slot slots[4];
-  int next = 0;
-};
-static std::mutex g_mu;
-static std::vector<DevCache *> g_caches;
-
-static DevCache *cache_for(int device) {
-  for (DevCache *c : g_caches)
-    if (c->device == device) return c;
-  DevCache *c = new DevCache();
-  c->device = device;
-  g_caches.push_back(c);
-  return c;
-}
-
-// returns the device address of a copy of blob; *slot_out is the slot to mark
-static int stage_table(const void *blob, size_t bytes, hipStream_t stream, void **dev_out,
-                       Slot **slot_out) {
-  int device = 0;
-  Q4_HIP(hipGetDevice(&device));
-  DevCache *c = cache_for(device);
-  for (Slot &s : c->slots) {
-    if (s.dev && s.content.size() == bytes && memcmp(s.content.data(), blob, bytes) == 0) {
-      *dev_out = s.dev;
-      *slot_out = &s;
-      return 0;
-    }
-  }
-  Slot &s = c->slots[c->next];
-  c->next = (c->next + 1) % 4;
-  if (s.pending) {
-    Q4_HIP(hipEventSynchronize(s.done));
-    s.pending = false;
-  }
-  if (s.cap < bytes) {
-    if (s.dev) Q4_HIP(hipFree(s.dev));
-    if (s.host) Q4_HIP(hipHostFree(s.host));
-    s.dev = s.host = nullptr;
-    s.cap = 0;
-    s.content.clear();
-    const size_t cap = std::max<size_t>(bytes * 2, 4096);
-    Q4_HIP(hipMalloc(&s.dev, cap));
-    Q4_HIP(hipHostMalloc(&s.host, cap, hipHostMallocDefault));
-    s.cap = cap;
-  }
-  if (!s.done) Q4_HIP(hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
-  memcpy(s.host, blob, bytes);
-  s.content.assign(static_cast<const char *>(blob), static_cast<const char *>(blob) + bytes);
-  Q4_HIP(hipMemcpyAsync(s.dev, s.host, bytes, hipMemcpyHostToDevice, stream));
-  *dev_out = s.dev;
-  *slot_out = &s;
-  return 0;
-}
-
-static int mark_slot(Slot *s, hipStream_t stream) {
-  Q4_HIP(hipEventRecord(s->done, stream));
-  s->pending = true;
-  return 0;
-}
-
-static int pick_tiles_per_wave(int64_t total_tiles) {
-  // keep at least ~16 workgroups per CU in the launch before lengthening chunks
-  int tpw = 8;
-  while (tpw > 1 && total_tiles / (kWaves * tpw) < 4096) tpw >>= 1;
-  return tpw;
-}
-
-template <typename K>
-static void launch_fused(K kernel, int64_t grid, hipStream_t stream, const TensorDesc *dev,
-                         int n, const TensorDesc &one, int tpw, const StepConsts &sc) {
-  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, stream, dev, n, one, tpw, sc);
-}
-
-static int run_fused(std::vector<TensorDesc> &descs, int p_dtype, int g_dtype,
-                     const StepConsts &sc, hipStream_t stream) {
-  int64_t total_tiles = 0;
-  for (const TensorDesc &d : descs) total_tiles += (d.numel + kTile - 1) / kTile;
-  if (total_tiles == 0) return 0;
-  const int tpw = pick_tiles_per_wave(total_tiles);
-  int64_t chunks = 0;
-  for (TensorDesc &d : descs) {
-    d.chunk0 = chunks;
-    const int64_t tiles = (d.numel + kTile - 1) / kTile;
-    chunks += (tiles + kWaves * tpw - 1) / (kWaves * tpw);
-  }
-  if (chunks > 0x7fffffffLL) return fail(Q4ADAMW_ERR_TOO_LARGE, "too many chunks for one launch");
-
-  const TensorDesc *dev = nullptr;
-  int n = 0;
-  Slot *slot = nullptr;
-  TensorDesc one = descs[0];
-  std::unique_lock<std::mutex> lock(g_mu, std::defer_lock);
-  if (descs.size() > 1) {
-    lock.lock();
-    void *d = nullptr;
-    const int rc = stage_table(descs.data(), descs.size() * sizeof(TensorDesc), stream, &d, &slot);
-    if (rc) return rc;
-    dev = static_cast<const TensorDesc *>(d);
-    n = (int)descs.size();
-  }
-  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  if (!pb && !gb) launch_fused(fused_4bit_kernel<false, false>, chunks, stream, dev, n, one, tpw, sc);
-  else if (!pb && gb) launch_fused(fused_4bit_kernel<false, true>, chunks, stream, dev, n, one, tpw, sc);
-  else if (pb && !gb) launch_fused(fused_4bit_kernel<true, false>, chunks, stream, dev, n, one, tpw, sc);
-  else launch_fused(fused_4bit_kernel<true, true>, chunks, stream, dev, n, one, tpw, sc);
-  Q4_HIP(hipGetLastError());
-  if (slot) return mark_slot(slot, stream);
-  return 0;
-}
-
-template <typename K>
-static void launch_small(K kernel, int64_t grid, hipStream_t stream, const SmallDesc *dev, int n,
-                         const SmallDesc &one, const StepConsts &sc) {
-  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kSmallThreads), 0, stream, dev, n, one, sc);
-}
-
-static int run_small(std::vector<SmallDesc> &descs, int p_dtype, int g_dtype, const StepConsts &sc,
-                     hipStream_t stream) {
-  int64_t chunks = 0;
-  for (SmallDesc &d : descs) {
-    d.chunk0 = chunks;
-    chunks += (d.numel + kSmallChunk - 1) / kSmallChunk;
-  }
-  if (chunks == 0) return 0;
-  if (chunks > 0x7fffffffLL) return fail(Q4ADAMW_ERR_TOO_LARGE, "too many chunks for one launch");
-  const SmallDesc *dev = nullptr;
-  int n = 0;
-  Slot *slot = nullptr;
-  SmallDesc one = descs[0];
-  std::unique_lock<std::mutex> lock(g_mu, std::defer_lock);
-  if (descs.size() > 1) {
-    lock.lock();
-    void *d = nullptr;
-    const int rc = stage_table(descs.data(), descs.size() * sizeof(SmallDesc), stream, &d, &slot);
-    if (rc) return rc;
-    dev = static_cast<const SmallDesc *>(d);
-    n = (int)descs.size();
-  }
-  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  if (!pb && !gb) launch_small(single_tensor_kernel<false, false>, chunks, stream, dev, n, one, sc);
-  else if (!pb && gb) launch_small(single_tensor_kernel<false, true>, chunks, stream, dev, n, one, sc);
-  else if (pb && !gb) launch_small(single_tensor_kernel<true, false>, chunks, stream, dev, n, one, sc);
-  else launch_small(single_tensor_kernel<true, true>, chunks, stream, dev, n, one, sc);
-  Q4_HIP(hipGetLastError());
-  if (slot) return mark_slot(slot, stream);
-  return 0;
-}
-
 static int check_dtypes(int p_dtype, int g_dtype) {
   if ((p_dtype != Q4ADAMW_FP32 && p_dtype != Q4ADAMW_BF16) ||
       (g_dtype != Q4ADAMW_FP32 && g_dtype != Q4ADAMW_BF16))
     return fail(Q4ADAMW_ERR_ARG, "dtype tag must be Q4ADAMW_FP32 or Q4ADAMW_BF16");
   return 0;
 }
+
+// Completes prefix and pivots of a launch batch and launches it.  Args is FusedArgs
+// or SmallArgs; `chunks` is the batch's total chunk count.
+template <typename Args, typename Kernel>
+static int launch_batch(Args &a, int capacity, uint64_t chunks, Kernel kernel, int threads,
+                        hipStream_t stream) {
+  for (int i = a.ntensors; i < capacity + 8; ++i) a.first_chunk[i] = 0xffffffffu;
+  for (int k = 0; k < 8; ++k) a.pivot[k] = k * 8 < capacity + 8 ? a.first_chunk[k * 8] : 0xffffffffu;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)chunks), dim3(threads), 0, stream, a);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
+typedef void (*FusedKernel)(const FusedArgs);
+typedef void (*SmallKernel)(const SmallArgs);
+
+static FusedKernel pick_fused(int p_dtype, int g_dtype) {
+  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
+  if (!pb && !gb) return fused_4bit_kernel<false, false>;
+  if (!pb && gb) return fused_4bit_kernel<false, true>;
+  if (pb && !gb) return fused_4bit_kernel<true, false>;
+  return fused_4bit_kernel<true, true>;
+}
+
+static SmallKernel pick_small(int p_dtype, int g_dtype) {
+  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
+  if (!pb && !gb) return single_tensor_kernel<false, false>;
+  if (!pb && gb) return single_tensor_kernel<false, true>;
+  if (pb && !gb) return single_tensor_kernel<true, false>;
+  return single_tensor_kernel<true, true>;
+}
+
+constexpr uint64_t kMaxChunksPerLaunch = 0x7fffffffull;  // grid.x limit
 
 }  // namespace q4
 
@@ -640,34 +579,52 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
                              float step, void *stream) {
   if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
-  StepConsts sc;
-  if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &sc)) return rc;
-  std::vector<TensorDesc> descs;
-  descs.reserve(count);
+  FusedArgs a;
+  if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
+  const uintptr_t p_align = p_dtype == Q4ADAMW_BF16 ? 8 : 16, g_align = g_dtype == Q4ADAMW_BF16 ? 8 : 16;
+  // validate everything before the first launch
   for (int i = 0; i < count; ++i) {
     const q4adamw_tensor &t = tensors[i];
     if (t.numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
     if (t.numel == 0) continue;
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.exp_avg_sq_scale)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
-    if (!aligned(t.p, 16) || !aligned(t.g, 16))
-      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be 16-byte aligned");
-    if (!aligned(t.exp_avg, 4) || !aligned(t.exp_avg_sq, 4) || !aligned(t.exp_avg_scale, 4) ||
+    if (!aligned(t.p, p_align) || !aligned(t.g, g_align))
+      return fail(Q4ADAMW_ERR_ALIGN,
+                  "param and grad must be aligned to four elements (16 bytes fp32, 8 bytes bf16)");
+    if (!aligned(t.exp_avg, 2) || !aligned(t.exp_avg_sq, 2) || !aligned(t.exp_avg_scale, 4) ||
         !aligned(t.exp_avg_sq_scale, 4))
-      return fail(Q4ADAMW_ERR_ALIGN, "code and scale buffers must be 4-byte aligned");
-    TensorDesc d;
+      return fail(Q4ADAMW_ERR_ALIGN, "code buffers must be 2-byte aligned, scale buffers 4-byte aligned");
+    if ((uint64_t)(t.numel + kChunk - 1) / kChunk > kMaxChunksPerLaunch)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const FusedKernel kernel = pick_fused(p_dtype, g_dtype);
+  a.ntensors = 0;
+  uint64_t chunks = 0;
+  for (int i = 0; i < count; ++i) {
+    const q4adamw_tensor &t = tensors[i];
+    if (t.numel == 0) continue;
+    const uint64_t c = (uint64_t)(t.numel + kChunk - 1) / kChunk;
+    if (a.ntensors == kMaxTensors || chunks + c > kMaxChunksPerLaunch) {
+      if (int rc = launch_batch(a, kMaxTensors, chunks, kernel, kThreads, s)) return rc;
+      a.ntensors = 0;
+      chunks = 0;
+    }
+    TensorDesc &d = a.desc[a.ntensors];
     d.p = t.p;
     d.g = t.g;
-    d.m = reinterpret_cast<uint32_t *>(t.exp_avg);
-    d.v = reinterpret_cast<uint32_t *>(t.exp_avg_sq);
+    d.m = t.exp_avg;
+    d.v = t.exp_avg_sq;
     d.sm = t.exp_avg_scale;
     d.sv = t.exp_avg_sq_scale;
     d.numel = t.numel;
-    d.chunk0 = 0;
-    descs.push_back(d);
+    a.first_chunk[a.ntensors] = (uint32_t)chunks;
+    ++a.ntensors;
+    chunks += c;
   }
-  if (descs.empty()) return 0;
-  return run_fused(descs, p_dtype, g_dtype, sc, static_cast<hipStream_t>(stream));
+  if (a.ntensors > 0) return launch_batch(a, kMaxTensors, chunks, kernel, kThreads, s);
+  return 0;
 }
 
 int q4adamw_fused_4bit(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_avg_sq,
@@ -684,30 +641,45 @@ int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int c
                                       float weight_decay, float eps, float step, void *stream) {
   if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
-  StepConsts sc;
-  if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &sc)) return rc;
-  std::vector<SmallDesc> descs;
-  descs.reserve(count);
+  SmallArgs a;
+  if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
+  const uintptr_t pa = p_dtype == Q4ADAMW_BF16 ? 2 : 4, ga = g_dtype == Q4ADAMW_BF16 ? 2 : 4;
   for (int i = 0; i < count; ++i) {
     const q4adamw_small_tensor &t = tensors[i];
     if (t.numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
     if (t.numel == 0) continue;
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
-    const uintptr_t pa = p_dtype == Q4ADAMW_BF16 ? 2 : 4, ga = g_dtype == Q4ADAMW_BF16 ? 2 : 4;
     if (!aligned(t.p, pa) || !aligned(t.g, ga) || !aligned(t.exp_avg, 4) || !aligned(t.exp_avg_sq, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "tensor not aligned to its element size");
-    SmallDesc d;
+    if ((uint64_t)(t.numel + kSmallChunk - 1) / kSmallChunk > kMaxChunksPerLaunch)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const SmallKernel kernel = pick_small(p_dtype, g_dtype);
+  a.ntensors = 0;
+  uint64_t chunks = 0;
+  for (int i = 0; i < count; ++i) {
+    const q4adamw_small_tensor &t = tensors[i];
+    if (t.numel == 0) continue;
+    const uint64_t c = (uint64_t)(t.numel + kSmallChunk - 1) / kSmallChunk;
+    if (a.ntensors == kMaxSmallTensors || chunks + c > kMaxChunksPerLaunch) {
+      if (int rc = launch_batch(a, kMaxSmallTensors, chunks, kernel, 256, s)) return rc;
+      a.ntensors = 0;
+      chunks = 0;
+    }
+    SmallDesc &d = a.desc[a.ntensors];
     d.p = t.p;
     d.g = t.g;
     d.m = t.exp_avg;
     d.v = t.exp_avg_sq;
     d.numel = t.numel;
-    d.chunk0 = 0;
-    descs.push_back(d);
+    a.first_chunk[a.ntensors] = (uint32_t)chunks;
+    ++a.ntensors;
+    chunks += c;
   }
-  if (descs.empty()) return 0;
-  return run_small(descs, p_dtype, g_dtype, sc, static_cast<hipStream_t>(stream));
+  if (a.ntensors > 0) return launch_batch(a, kMaxSmallTensors, chunks, kernel, 256, s);
+  return 0;
 }
 
 int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *exp_avg_sq,
@@ -719,28 +691,10 @@ int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *e
                                            weight_decay, eps, step, stream);
 }
 
-int q4adamw_release(void) {
-  std::lock_guard<std::mutex> lock(g_mu);
-  int rc = 0;
-  int prev = 0;
-  const bool have_prev = hipGetDevice(&prev) == hipSuccess;
-  for (DevCache *c : g_caches) {
-    if (hipSetDevice(c->device) != hipSuccess) continue;
-    for (Slot &s : c->slots) {
-      if (s.pending && s.done) (void)hipEventSynchronize(s.done);
-      if (s.dev && hipFree(s.dev) != hipSuccess) rc = 1;
-      if (s.host && hipHostFree(s.host) != hipSuccess) rc = 1;
-      if (s.done) (void)hipEventDestroy(s.done);
-    }
-    delete c;
-  }
-  g_caches.clear();
-  if (have_prev) (void)hipSetDevice(prev);
-  return rc;
-}
+int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1000; }
+int q4adamw_version(void) { return 1001; }
 
 }  // extern "C"

@@ -64,7 +64,7 @@ struct MtabEntry {
   uint32_t hi;  // fp32 bits
 };
 
-Q4_HD inline MtabEntry mtab_entry(uint32_t idx) {
+Q4_HD constexpr MtabEntry mtab_entry(uint32_t idx) {
   const uint32_t sign = (idx >> 10) & 1u, mag = idx & 1023u, e = mag >> 2;
   uint32_t base = 0, thr = 0;
   bool has = false;
@@ -85,7 +85,7 @@ Q4_HD inline MtabEntry mtab_entry(uint32_t idx) {
       }
     }
   }
-  MtabEntry out;
+  MtabEntry out{};
   if (!has) {
     out.lo = kNoThr | base;
     out.hi = kNoThr;
@@ -106,6 +106,44 @@ Q4_HD inline MtabEntry mtab_entry(uint32_t idx) {
     out.hi = (m - kGuardUlps) | s;
   }
   return out;
+}
+
+// Only the buckets that can hold a threshold differ from "no threshold, base 7":
+// per sign, buckets kBucketFloor .. kBucketTop (|q| from 1.75 * 2^-10 to 1.25).
+// The kernel clamps smaller magnitudes up to the floor bucket and builds just these
+// entries in LDS, at their natural index, leaving the rest of the table untouched.
+constexpr uint32_t kBucketFloor = 471;                                  // exponent 117, mantissa 11b
+constexpr uint32_t kBucketTop = 508;                                    // exponent 127, mantissa 00b
+constexpr uint32_t kBucketsPerSign = kBucketTop - kBucketFloor + 1;     // 38
+constexpr uint32_t kNegativeBuckets = 1024;                             // index offset of the sign bit
+
+// What the first 128 threads of a workgroup copy into LDS, one slot each:
+// slots 0..75  : bucket entries (a = lo bound | base, b = hi bound)
+// slots 96..111: first-moment code book (a = fp32 bits)
+// slots 112..127: second-moment code book (a = fp32 bits)
+struct WorkgroupTables {
+  uint32_t a[128];
+  uint32_t b[128];
+};
+
+// slot j of the compact table <-> bucket index in the full table
+Q4_HD constexpr uint32_t compact_slot_bucket(uint32_t j) {
+  return j < kBucketsPerSign ? kBucketFloor + j
+                             : kNegativeBuckets + kBucketFloor + (j - kBucketsPerSign);
+}
+
+constexpr WorkgroupTables make_workgroup_tables() {
+  WorkgroupTables t{};
+  for (uint32_t j = 0; j < 2 * kBucketsPerSign; ++j) {
+    const MtabEntry e = mtab_entry(compact_slot_bucket(j));
+    t.a[j] = e.lo;
+    t.b[j] = e.hi;
+  }
+  for (uint32_t k = 0; k < 16; ++k) {
+    t.a[96 + k] = kQmapMBits[k];
+    t.a[112 + k] = f2bits(qmap_v((int)k));
+  }
+  return t;
 }
 
 }  // namespace q4

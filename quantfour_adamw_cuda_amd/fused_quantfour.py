@@ -77,6 +77,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         )
         super().__init__(params, defaults)
         self._launch_cache: Dict[Any, Any] = {}
+        # set to a list to collect ("fused_4bit" | "fused_single_tensor", start, end)
+        # event triples around every launch, recorded on the launch stream
+        self.kernel_timing = None
 
     # -- state ------------------------------------------------------------
     def init_qstate(self, p, state_name):
@@ -94,6 +97,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         """optim/fused_quantfour.py:73-84"""
         super().__setstate__(state)
         self._launch_cache = {}
+        self.__dict__.setdefault("kernel_timing", None)
         for group in self.param_groups:
             group.setdefault("fused", None)
         state_values = list(self.state.values())
@@ -250,6 +254,16 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                     self._launch_cache[cache_key] = cached
                 _, arr, (p_tag, g_tag) = cached
                 launch = _q.launch_table if quantized else _q.launch_small_table
-                launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step)
+                if self.kernel_timing is None:
+                    launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step)
+                else:
+                    with torch.cuda.device(device):
+                        start = torch.cuda.Event(enable_timing=True)
+                        end = torch.cuda.Event(enable_timing=True)
+                        start.record()
+                        launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step)
+                        end.record()
+                    kind = "fused_4bit" if quantized else "fused_single_tensor"
+                    self.kernel_timing.append((kind, start, end))
 
         return loss
