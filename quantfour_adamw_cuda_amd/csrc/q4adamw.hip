@@ -32,7 +32,10 @@
 namespace q4 {
 
 constexpr int kTile = 256;                 // elements per wave
-constexpr int kWaves = 4;                  // waves per workgroup
+#ifndef Q4_WAVES
+#define Q4_WAVES 4
+#endif
+constexpr int kWaves = Q4_WAVES;           // waves per workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kChunk = kTile * kWaves;     // elements per workgroup
 constexpr int kMaxTensors = 48;            // tensors per fused launch
@@ -107,14 +110,14 @@ __device__ __forceinline__ gptr<T> as_global(const void *p) {
   return (gptr<T>)(uintptr_t)p;
 }
 
-// Every byte is touched once per step: stream past the caches.
-template <typename T>
-__device__ __forceinline__ T stream_load(gptr<const T> p) {
-  return __builtin_nontemporal_load(p);
-}
-template <typename T>
-__device__ __forceinline__ void stream_store(gptr<T> p, T v) {
-  __builtin_nontemporal_store(v, p);
+// Full tiles go through buffer instructions: the tile's base address sits in a
+// scalar resource descriptor and each lane supplies a 32-bit byte offset, so no
+// vector ALU work goes into addresses.  aux = 2 is the non-temporal hint.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kNt = 2;
+
+__device__ __forceinline__ rsrc_t tile_rsrc(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
 }
 
 template <int CTRL>
@@ -123,19 +126,25 @@ __device__ __forceinline__ uint32_t dpp_umax(uint32_t x) {
   return x > y ? x : y;
 }
 
-// Max over the 32 lanes of a quantization block (lanes 0-31 or 32-63), result in
-// every lane of the block.  The input is a non-negative float (an abs-max), so its
-// bit pattern orders like an unsigned integer.
-__device__ __forceinline__ float block_max32(float x) {
-  uint32_t u = f2bits(x);
-  // rows 0<->1 and 2<->3 exchanged: lane i of a row meets lane i of its partner row
-  const auto sw = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  u = sw[0] > sw[1] ? sw[0] : sw[1];
+// Abs-max of both moments over the 32 lanes of a quantization block (lanes 0-31 or
+// 32-63), results in every lane of the block.  The inputs are non-negative floats,
+// so their bit patterns order like unsigned integers.  One v_permlane16_swap pairs
+// lane i of the block's first row with lane i of its second row and leaves the
+// first-moment partial max in the first row and the second-moment partial max in
+// the second row; four DPP steps then reduce both rows at once; a second swap
+// hands each row the other row's result.
+__device__ __forceinline__ void block_max32_pair(float &am, float &av) {
+  // after the swap: a = [am.r0, av.r0, am.r2, av.r2], b = [am.r1, av.r1, am.r3, av.r3]
+  const auto s1 = __builtin_amdgcn_permlane16_swap(f2bits(am), f2bits(av), false, false);
+  uint32_t u = s1[0] > s1[1] ? s1[0] : s1[1];
   u = dpp_umax<0xB1>(u);   // quad_perm [1,0,3,2]
   u = dpp_umax<0x4E>(u);   // quad_perm [2,3,0,1]
   u = dpp_umax<0x141>(u);  // row_half_mirror
   u = dpp_umax<0x140>(u);  // row_mirror
-  return bits2f(u);
+  // u = [max am, max av, max am, max av] per row; spread: a = rows (0,0,2,2), b = rows (1,1,3,3)
+  const auto s2 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  am = bits2f(s2[0]);
+  av = bits2f(s2[1]);
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return bits2f(h << 16); }
@@ -144,17 +153,17 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nea
   return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
-// four consecutive elements starting at element index e0 (a multiple of 4)
+// four consecutive elements starting at element e0 (a multiple of 4) of the tile at base
 template <bool BF, bool FULL>
-__device__ __forceinline__ void load4(const void *base, int64_t e0, int nv, float (&x)[4]) {
+__device__ __forceinline__ void load4(const void *base, uint32_t e0, int nv, float (&x)[4]) {
   if (FULL) {
     if (BF) {
-      const u32x2 w = stream_load(as_global<const u32x2>(static_cast<const uint16_t *>(base) + e0));
+      const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(tile_rsrc(base), e0 * 2, 0, kNt);
       x[0] = bits2f(w.x << 16); x[1] = bits2f(w.x & 0xffff0000u);
       x[2] = bits2f(w.y << 16); x[3] = bits2f(w.y & 0xffff0000u);
     } else {
-      const f32x4 a = stream_load(as_global<const f32x4>(static_cast<const float *>(base) + e0));
-      x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+      const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), e0 * 4, 0, kNt);
+      x[0] = bits2f(a.x); x[1] = bits2f(a.y); x[2] = bits2f(a.z); x[3] = bits2f(a.w);
     }
   } else {
 #pragma unroll
@@ -169,15 +178,16 @@ __device__ __forceinline__ void load4(const void *base, int64_t e0, int nv, floa
 }
 
 template <bool BF, bool FULL>
-__device__ __forceinline__ void store4(void *base, int64_t e0, int nv, const float (&x)[4]) {
+__device__ __forceinline__ void store4(void *base, uint32_t e0, int nv, const float (&x)[4]) {
   if (FULL) {
     if (BF) {
       u32x2 w;
       w.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
       w.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
-      stream_store(as_global<u32x2>(static_cast<uint16_t *>(base) + e0), w);
+      __builtin_amdgcn_raw_buffer_store_b64(w, tile_rsrc(base), e0 * 2, 0, kNt);
     } else {
-      stream_store(as_global<f32x4>(static_cast<float *>(base) + e0), f32x4{x[0], x[1], x[2], x[3]});
+      const u32x4 w = {f2bits(x[0]), f2bits(x[1]), f2bits(x[2]), f2bits(x[3])};
+      __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), e0 * 4, 0, kNt);
     }
   } else {
 #pragma unroll
@@ -198,7 +208,7 @@ struct F4 {
 // scale, then the number of thresholds strictly below the quotient
 // (cuda_adamw_kernels.cu:167-194 in closed form).  0/0 is NaN and gets code 0.
 template <bool SECOND>
-__device__ __noinline__ uint32_t quantize4_exact(F4 v, float scale) {
+__device__ __forceinline__ uint32_t quantize4_exact(const F4 &v, float scale) {
   uint32_t word = 0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -212,6 +222,16 @@ __device__ __noinline__ uint32_t quantize4_exact(F4 v, float scale) {
     word |= c << (4 * j);
   }
   return word;
+}
+
+// Per-sign lower clamp of a bucket byte offset: max(a, (a & sign bit) | floor).
+// Written as v_and_or_b32 because the compiler splits the and/or when both masks
+// are literals (a VOP3 encoding cannot hold two).
+__device__ __forceinline__ uint32_t clamp_bucket(uint32_t a) {
+  uint32_t floor_a;
+  const uint32_t sign_mask = kNegativeBuckets * 8u, floor_pos = kBucketFloor * 8u;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(floor_a) : "v"(a), "s"(sign_mask), "v"(floor_pos));
+  return a > floor_a ? a : floor_a;
 }
 
 // 1/s to within half an ulp for s in [2^-100, 2^100]: hardware estimate plus one
@@ -239,44 +259,55 @@ __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
   return group * 8 + within - 1;
 }
 
-// LDS tables of a workgroup: the full-size bucket table, of which only the 76
-// entries that a clamped quotient can reach are written (the rest is never read),
-// and the two code books.
-struct LdsTables {
-  __attribute__((aligned(16))) char mtab[kMtabEntries * 8];
-  float qm[16];
-  float qv[16];
-};
+// LDS tables of a workgroup, one array of 8-byte entries:
+//   [0, 2048)     bucket table of the first-moment quantizer; only the 76 entries
+//                 that a clamped quotient can reach are written, the rest is never read
+//   [2048, 2064)  first-moment code book  (value in .x)
+//   [2064, 2080)  second-moment code book (value in .x)
+constexpr uint32_t kLdsQm = kMtabEntries;
+constexpr uint32_t kLdsQv = kMtabEntries + 16;
+constexpr uint32_t kLdsEntries = kMtabEntries + 32;
 
-// This thread's slot of the workgroup tables, requested from memory as the very
-// first thing a wave does (only the first two waves hold slots).
+// The slots of the workgroup tables that this thread copies into LDS, requested
+// from memory as the very first thing a wave does.
+constexpr int kSlotsPerThread = (128 + kThreads - 1) / kThreads;
 struct TableSlot {
-  uint32_t a, b;
+  uint32_t a[kSlotsPerThread], b[kSlotsPerThread];
 };
 
 __device__ __forceinline__ TableSlot request_table_slot(int tid) {
-  TableSlot s{0u, 0u};
-  if (tid < 128) {
-    s.a = kWorkgroupTables.a[tid];
-    s.b = kWorkgroupTables.b[tid];
+  TableSlot s;
+#pragma unroll
+  for (int i = 0; i < kSlotsPerThread; ++i) {
+    const int slot = tid + i * kThreads;
+    s.a[i] = s.b[i] = 0u;
+    if (slot < 128) {
+      s.a[i] = kWorkgroupTables.a[slot];
+      s.b[i] = kWorkgroupTables.b[slot];
+    }
   }
   return s;
 }
 
-// Writes the slot into LDS and waits for the whole workgroup.  Called by every wave
-// exactly once, after it has issued its global loads, so that the latencies
-// overlap.  The fences order LDS only: a full __syncthreads() would also drain the
-// outstanding global loads.
-__device__ __forceinline__ void setup_tables(LdsTables &lds, int tid, TableSlot s) {
-  if (tid < (int)(2 * kBucketsPerSign)) {
-    *reinterpret_cast<uint2 *>(lds.mtab + compact_slot_bucket((uint32_t)tid) * 8) = make_uint2(s.a, s.b);
-  } else if (tid >= 96 && tid < 112) {
-    lds.qm[tid - 96] = bits2f(s.a);
-  } else if (tid >= 112 && tid < 128) {
-    lds.qv[tid - 112] = bits2f(s.a);
+// Writes the slots into LDS and waits for the whole workgroup.  Called by every
+// wave exactly once.  The fences order LDS only: a full __syncthreads() would also
+// drain outstanding global loads.
+__device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
+#pragma unroll
+  for (int i = 0; i < kSlotsPerThread; ++i) {
+    const int slot = tid + i * kThreads;
+    if (slot < 128) {
+      // slots 0..37 -> positive buckets, 38..75 -> negative buckets, 76..95 -> unused
+      // entries 0..19 (below every bucket that is read), 96..127 -> the code books
+      const int entry = slot + (slot < (int)kBucketsPerSign       ? (int)kBucketFloor
+                                : slot < (int)(2 * kBucketsPerSign) ? (int)(kNegativeBuckets + kBucketFloor - kBucketsPerSign)
+                                : slot < 96                          ? -76
+                                                                     : (int)kLdsQm - 96);
+      lds[entry] = make_uint2(s.a[i], s.b[i]);
+    }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
+  if (kWaves > 1) __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
@@ -285,30 +316,37 @@ __device__ __forceinline__ void setup_tables(LdsTables &lds, int tid, TableSlot 
 // ---------------------------------------------------------------------------
 template <bool PBF, bool GBF, bool FULL>
 __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int tid,
-                                             const StepConsts &sc, LdsTables &lds, TableSlot slot) {
-  const char *lds_mtab = lds.mtab;
-  const float *lds_qm = lds.qm;
-  const float *lds_qv = lds.qv;
+                                             const StepConsts &sc, uint2 *lds, const TableSlot &slot) {
+  // Uniform (scalar) part of every address: the tile's first element, byte and
+  // block; the per-lane part is a small 32-bit offset.
   const int64_t numel = T.numel;
-  const int64_t e0 = tile * kTile + (int64_t)lane * 4;
+  const int64_t tb = tile * kTile;
+  const void *p_tile = static_cast<const char *>(T.p) + tb * (PBF ? 2 : 4);
+  const void *g_tile = static_cast<const char *>(T.g) + tb * (GBF ? 2 : 4);
+  const uint8_t *m_tile = T.m + (tb >> 1);
+  const uint8_t *v_tile = T.v + (tb >> 1);
+  const float *sm_tile = T.sm + tile * 2;
+  const float *sv_tile = T.sv + tile * 2;
+  const uint32_t e0 = (uint32_t)lane * 4u;   // first element of this lane within the tile
+  const uint32_t half = (uint32_t)lane >> 5;  // which of the tile's two blocks
   int nv = 4;
+  bool blk_ok = true;
   if (!FULL) {
-    const int64_t rem = numel - e0;
+    const int64_t rem = numel - tb - (int64_t)e0;
     nv = rem >= 4 ? 4 : (rem > 0 ? (int)rem : 0);
+    blk_ok = tb + (int64_t)half * 128 < numel;
   }
-  const int64_t blk = tile * 2 + (lane >> 5);
-  const bool blk_ok = FULL || (blk << 7) < numel;
 
   float p[4], g[4];
-  load4<PBF, FULL>(T.p, e0, nv, p);
-  load4<GBF, FULL>(T.g, e0, nv, g);
+  load4<PBF, FULL>(p_tile, e0, nv, p);
+  load4<GBF, FULL>(g_tile, e0, nv, g);
   uint32_t mw = 0, vw = 0;
   if (FULL) {
-    mw = stream_load(as_global<const uint16_t>(T.m) + (e0 >> 2));
-    vw = stream_load(as_global<const uint16_t>(T.v) + (e0 >> 2));
+    mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), (uint32_t)lane * 2u, 0, kNt);
+    vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), (uint32_t)lane * 2u, 0, kNt);
   } else {
-    const gptr<const uint8_t> mb = as_global<const uint8_t>(T.m) + (e0 >> 1);
-    const gptr<const uint8_t> vb = as_global<const uint8_t>(T.v) + (e0 >> 1);
+    const gptr<const uint8_t> mb = as_global<const uint8_t>(m_tile) + (e0 >> 1);
+    const gptr<const uint8_t> vb = as_global<const uint8_t>(v_tile) + (e0 >> 1);
     const int nb = (nv + 1) >> 1;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -319,19 +357,28 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     }
   }
   float sm_old = 0.0f, sv_old = 0.0f;
-  if (blk_ok) {
-    sm_old = stream_load(as_global<const float>(T.sm) + blk);
-    sv_old = stream_load(as_global<const float>(T.sv) + blk);
+  if (FULL) {
+    sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), half * 4u, 0, kNt));
+    sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), half * 4u, 0, kNt));
+  } else if (blk_ok) {
+    sm_old = as_global<const float>(sm_tile)[half];
+    sv_old = as_global<const float>(sv_tile)[half];
   }
+#ifndef Q4_EARLY_BARRIER
   setup_tables(lds, tid, slot);
+#endif
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
   F4 mn, vn;
   float am = 0.0f, av = 0.0f;
+  const char *lds_bytes = reinterpret_cast<const char *>(lds);
+  const uint32_t mw8 = mw << 3, vw8 = vw << 3;  // nibble j * 8 = byte offset of its code-book entry
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const float m_old = lds_qm[(mw >> (4 * j)) & 15u] * sm_old;
-    const float v_old = lds_qv[(vw >> (4 * j)) & 15u] * sv_old;
+    const float m_old =
+        *reinterpret_cast<const float *>(lds_bytes + kLdsQm * 8 + ((mw8 >> (4 * j)) & 0x78u)) * sm_old;
+    const float v_old =
+        *reinterpret_cast<const float *>(lds_bytes + kLdsQv * 8 + ((vw8 >> (4 * j)) & 0x78u)) * sv_old;
     const float gj = g[j];
     float m = sc.b1 * m_old + sc.r1 * gj;
     float v = sc.b2 * v_old + sc.r2 * (gj * gj);
@@ -345,14 +392,18 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
     av = __builtin_fmaxf(av, v);
   }
-  store4<PBF, FULL>(T.p, e0, nv, p);
+  store4<PBF, FULL>(const_cast<void *>(p_tile), e0, nv, p);
 
   // block scales (exact: max is order independent)
-  am = block_max32(am);
-  av = block_max32(av);
+  block_max32_pair(am, av);
   if (blk_ok && (lane & 31) == 0) {
-    stream_store(as_global<float>(T.sm) + blk, am);
-    stream_store(as_global<float>(T.sv) + blk, av);
+    if (FULL) {
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), half * 4u, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), half * 4u, 0, kNt);
+    } else {
+      as_global<float>(sm_tile)[half] = am;
+      as_global<float>(sv_tile)[half] = av;
+    }
   }
 
   // fast quantization: multiply by a refined reciprocal, decide every code whose
@@ -360,7 +411,7 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   const bool safe_m = am >= kScaleLo && am <= kScaleHi;
   const bool safe_v = av >= kScaleLo && av <= kScaleHi;
   const float rm = safe_m ? refined_rcp(am) : 0.0f;
-  const float rv = safe_v ? refined_rcp(av) : 0.0f;
+  const float rv16 = safe_v ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   uint32_t mword = 0, vword = 0;
 #pragma unroll
@@ -369,16 +420,15 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     // lowest bucket the workgroup built
     const float qm = mn.x[j] * rm;
     uint32_t a = (f2bits(qm) >> 18) & 0x3FF8u;
-    const uint32_t floor_a = (a & (kNegativeBuckets * 8u)) | (kBucketFloor * 8u);
-    a = a > floor_a ? a : floor_a;
-    const uint2 ent = *reinterpret_cast<const uint2 *>(lds_mtab + a);
+    a = clamp_bucket(a);
+    const uint2 ent = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(lds) + a);
     const bool above_hi = qm > bits2f(ent.y);
     const bool above_lo = qm > bits2f(ent.x);
     redo |= (above_hi != above_lo);
     mword |= ((ent.x & 15u) + (above_hi ? 1u : 0u)) << (4 * j);
 
     // second moment: thresholds at 16q = k + 0.5, k = 1..15
-    const float t = __builtin_fmaf(vn.x[j] * rv, 16.0f, kVGuard - 0.5f);
+    const float t = __builtin_fmaf(vn.x[j], rv16, kVGuard - 0.5f);
     redo |= __builtin_amdgcn_fractf(t) < 2.0f * kVGuard;
     vword |= (uint32_t)(int)t << (4 * j);  // t > -1, so truncation gives 0 for t < 0
   }
@@ -394,11 +444,11 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   }
 
   if (FULL) {
-    stream_store(as_global<uint16_t>(T.m) + (e0 >> 2), (uint16_t)mword);
-    stream_store(as_global<uint16_t>(T.v) + (e0 >> 2), (uint16_t)vword);
+    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)mword, tile_rsrc(m_tile), (uint32_t)lane * 2u, 0, kNt);
+    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)vword, tile_rsrc(v_tile), (uint32_t)lane * 2u, 0, kNt);
   } else {
-    const gptr<uint8_t> mb = as_global<uint8_t>(T.m) + (e0 >> 1);
-    const gptr<uint8_t> vb = as_global<uint8_t>(T.v) + (e0 >> 1);
+    const gptr<uint8_t> mb = as_global<uint8_t>(m_tile) + (e0 >> 1);
+    const gptr<uint8_t> vb = as_global<uint8_t>(v_tile) + (e0 >> 1);
     const int nb = (nv + 1) >> 1;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -412,7 +462,7 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
 
 template <bool PBF, bool GBF>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
-  __shared__ LdsTables lds;
+  __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot(tid);
   const uint32_t chunk = blockIdx.x;
@@ -421,10 +471,15 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
   const int64_t begin = tile * kTile;
+#ifdef Q4_EARLY_BARRIER
+  setup_tables(lds, tid, slot);
+  if (begin >= T.numel) return;
+#else
   if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
     setup_tables(lds, tid, slot);
     return;
   }
+#endif
   if (begin + kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, tid, args.sc, lds, slot);
   else process_tile<PBF, GBF, false>(T, tile, lane, tid, args.sc, lds, slot);
 }
