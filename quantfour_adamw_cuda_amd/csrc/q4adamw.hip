@@ -16,7 +16,10 @@
 //   launch  = all chunks of up to kMaxTensors tensors.  The tensor descriptors and
 //             the per-tensor first-chunk prefix travel in the kernel arguments, so
 //             a workgroup finds its tensor with two scalar loads from the kernarg
-//             segment and nothing is staged in device memory.
+//             segment and nothing is staged in device memory.  Workgroup ids are
+//             dealt round-robin to the 8 XCDs; the kernel maps id -> chunk so that
+//             each XCD walks one contiguous eighth of the chunk space, which keeps
+//             neighbouring blocks' scales (4 bytes per block) in one L2.
 // Per element the kernel reads p, g and one nibble of each moment, and writes p
 // and one nibble of each moment; per block it reads and writes two fp32 scales.
 #include <hip/hip_runtime.h>
@@ -67,6 +70,8 @@ struct TensorDesc {  // 56 bytes
 struct FusedArgs {
   StepConsts sc;
   int ntensors;
+  uint32_t nchunks;        // chunks in this launch
+  uint32_t chunks_per_xcd; // ceil(nchunks / 8); the grid has 8 * chunks_per_xcd workgroups
   uint32_t pivot[8];
   uint32_t first_chunk[kMaxTensors + 8];
   TensorDesc desc[kMaxTensors];
@@ -358,8 +363,9 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   }
   float sm_old = 0.0f, sv_old = 0.0f;
   if (FULL) {
-    sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), half * 4u, 0, kNt));
-    sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), half * 4u, 0, kNt));
+    // scales are 4 bytes per block: cached, so that neighbouring blocks share lines
+    sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), half * 4u, 0, 0));
+    sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), half * 4u, 0, 0));
   } else if (blk_ok) {
     sm_old = as_global<const float>(sm_tile)[half];
     sv_old = as_global<const float>(sv_tile)[half];
@@ -398,8 +404,8 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   block_max32_pair(am, av);
   if (blk_ok && (lane & 31) == 0) {
     if (FULL) {
-      __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), half * 4u, 0, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), half * 4u, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), half * 4u, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), half * 4u, 0, 0);
     } else {
       as_global<float>(sm_tile)[half] = am;
       as_global<float>(sv_tile)[half] = av;
@@ -465,7 +471,8 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot(tid);
-  const uint32_t chunk = blockIdx.x;
+  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  if (chunk >= args.nchunks) return;  // whole workgroup: the grid is padded to a multiple of 8
   const int t = find_tensor(args, chunk);
   const TensorDesc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -563,11 +570,26 @@ static int check_dtypes(int p_dtype, int g_dtype) {
 
 // Completes prefix and pivots of a launch batch and launches it.  Args is FusedArgs
 // or SmallArgs; `chunks` is the batch's total chunk count.
+template <typename Args>
+static void finish_prefix(Args &a, int capacity) {
+  for (int i = a.ntensors; i < capacity + 8; ++i) a.first_chunk[i] = 0xffffffffu;
+  for (int k = 0; k < 8; ++k) a.pivot[k] = k * 8 < capacity + 8 ? a.first_chunk[k * 8] : 0xffffffffu;
+}
+
+static int launch_fused_batch(FusedArgs &a, uint64_t chunks, void (*kernel)(const FusedArgs),
+                              hipStream_t stream) {
+  finish_prefix(a, kMaxTensors);
+  a.nchunks = (uint32_t)chunks;
+  a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
+  hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, stream, a);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 template <typename Args, typename Kernel>
 static int launch_batch(Args &a, int capacity, uint64_t chunks, Kernel kernel, int threads,
                         hipStream_t stream) {
-  for (int i = a.ntensors; i < capacity + 8; ++i) a.first_chunk[i] = 0xffffffffu;
-  for (int k = 0; k < 8; ++k) a.pivot[k] = k * 8 < capacity + 8 ? a.first_chunk[k * 8] : 0xffffffffu;
+  finish_prefix(a, capacity);
   hipLaunchKernelGGL(kernel, dim3((unsigned)chunks), dim3(threads), 0, stream, a);
   Q4_HIP(hipGetLastError());
   return 0;
@@ -592,7 +614,7 @@ static SmallKernel pick_small(int p_dtype, int g_dtype) {
   return single_tensor_kernel<true, true>;
 }
 
-constexpr uint64_t kMaxChunksPerLaunch = 0x7fffffffull;  // grid.x limit
+constexpr uint64_t kMaxChunksPerLaunch = 0x7ffffff0ull;  // grid.x limit, with room for padding to 8
 
 }  // namespace q4
 
@@ -662,7 +684,7 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
     if (t.numel == 0) continue;
     const uint64_t c = (uint64_t)(t.numel + kChunk - 1) / kChunk;
     if (a.ntensors == kMaxTensors || chunks + c > kMaxChunksPerLaunch) {
-      if (int rc = launch_batch(a, kMaxTensors, chunks, kernel, kThreads, s)) return rc;
+      if (int rc = launch_fused_batch(a, chunks, kernel, s)) return rc;
       a.ntensors = 0;
       chunks = 0;
     }
@@ -678,7 +700,7 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
     ++a.ntensors;
     chunks += c;
   }
-  if (a.ntensors > 0) return launch_batch(a, kMaxTensors, chunks, kernel, kThreads, s);
+  if (a.ntensors > 0) return launch_fused_batch(a, chunks, kernel, s);
   return 0;
 }
 
