@@ -28,6 +28,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+# HBM bytes per optimizer step of the fused kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (each scaled by what the same counter reads for a 4 GiB device copy: 2.0 and 1.0);
+# summary in profiles/fused_4bit_kernel_llama3_8b_hbm_counters.txt.  Workloads that have not
+# been profiled report null.
+MEASURED_TRAFFIC_BYTES_PER_STEP = {"llama3-8b": 9.7364e10}
 HP = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 
 
@@ -124,7 +130,7 @@ def cpu_baseline(torch, params, grads_set, hp, budget_s=20.0):
     """Times the torch-CPU oracle on the first quantized tensors of the workload until
     about budget_s seconds of CPU work have been spent."""
     from oracle import q4_oracle_torch as ot
-    done_params, spent, used = 0, 0.0, []
+    done_params, spent, used = 0, 0.0, {}
     for p, g in zip(params, grads_set):
         if p.numel() <= 4096 or p.numel() > (1 << 26):
             continue
@@ -146,7 +152,8 @@ def cpu_baseline(torch, params, grads_set, hp, budget_s=20.0):
                                                eps=hp["eps"])
             spent += time.perf_counter() - t0
             done_params += n
-        used.append(f"{tuple(p.shape)}x2 steps")
+        key = "x".join(str(d) for d in p.shape)
+        used[key] = used.get(key, 0) + 1
         if spent >= budget_s:
             break
     return {
@@ -154,7 +161,9 @@ def cpu_baseline(torch, params, grads_set, hp, budget_s=20.0):
         "unit": "params/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": "torch-CPU 3-pass oracle on tensors " + ", ".join(used) + f" ({spent:.1f} s)",
+        "sample": "torch-CPU 3-pass oracle, 2 steps each on the workload's first tensors: "
+                  + ", ".join(f"{n} of {k}" for k, n in used.items())
+                  + f" ({done_params / 2 / 1e6:.0f}M params, {spent:.1f} s)",
     }
 
 
@@ -167,6 +176,9 @@ def main():
     ap.add_argument("--grad-sets", type=int, default=2,
                     help="distinct pre-generated gradient sets rotated over the steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed region, run a plain 4 GiB device copy three times, so that "
+                         "a counter profile of this command also holds a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the optimizer step on ONE GPU; the step needs "
@@ -217,8 +229,18 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
+    # one entry per step: the step's fused launches (one kernel per batch of up to 48
+    # tensors, back to back on the stream) between two events
     fused_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "fused_4bit"]
     avg_kernel_s = sum(fused_ms) / len(fused_ms) / 1e3
+    launches_per_step = -(-sum(1 for p in params if p.numel() > 4096) // 48)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     algo_bytes = quant_params * bytes_per_param(p_dtype_s, g_dtype_s)
     achieved = algo_bytes / avg_kernel_s / 1e9
 
@@ -253,9 +275,10 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
-            "algorithmic_bytes_per_launch": algo_bytes,
-            "avg_launch_ms": avg_kernel_s * 1e3,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_STEP.get(args.workload),
+            "algorithmic_bytes_per_step": algo_bytes,
+            "kernel_ms_per_step": avg_kernel_s * 1e3,
+            "kernel_launches_per_step": launches_per_step,
         },
     }
     if not args.no_cpu_baseline:

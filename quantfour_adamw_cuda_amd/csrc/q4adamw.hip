@@ -43,7 +43,7 @@ constexpr int kThreads = kWaves * 64;
 constexpr int kChunk = kTile * kWaves;     // elements per workgroup
 constexpr int kMaxTensors = 48;            // tensors per fused launch
 constexpr int kSmallChunk = 1024;          // elements per workgroup, non-quantized kernel
-constexpr int kMaxSmallTensors = 64;
+constexpr int kMaxSmallTensors = 80;
 
 // derived on the host exactly as optim/cuda_adamw_kernels.cu:435-440
 struct StepConsts {
@@ -66,14 +66,16 @@ struct TensorDesc {  // 56 bytes
 // Kernel arguments of one fused launch (about 3 KiB, passed by value).
 // first_chunk[i] = index of tensor i's first chunk; entries past ntensors hold
 // 0xffffffff.  pivot[k] = first_chunk[8k] lets a workgroup find its tensor with two
-// 8-wide scalar loads.
+// wide scalar loads.
 struct FusedArgs {
+  static constexpr int kCapacity = kMaxTensors;
+  static constexpr int kPivots = (kMaxTensors + 7) / 8;
   StepConsts sc;
   int ntensors;
   uint32_t nchunks;        // chunks in this launch
   uint32_t chunks_per_xcd; // ceil(nchunks / 8); the grid has 8 * chunks_per_xcd workgroups
-  uint32_t pivot[8];
-  uint32_t first_chunk[kMaxTensors + 8];
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
   TensorDesc desc[kMaxTensors];
 };
 
@@ -86,10 +88,12 @@ struct SmallDesc {  // 40 bytes
 };
 
 struct SmallArgs {
+  static constexpr int kCapacity = kMaxSmallTensors;
+  static constexpr int kPivots = (kMaxSmallTensors + 7) / 8;
   StepConsts sc;
   int ntensors;
-  uint32_t pivot[8];
-  uint32_t first_chunk[kMaxSmallTensors + 8];
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
   SmallDesc desc[kMaxSmallTensors];
 };
 
@@ -257,7 +261,7 @@ template <typename Args>
 __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
   int group = 0;
 #pragma unroll
-  for (int k = 1; k < 8; ++k) group += (a.pivot[k] <= chunk) ? 1 : 0;
+  for (int k = 1; k < Args::kPivots; ++k) group += (a.pivot[k] <= chunk) ? 1 : 0;
   int within = 0;
 #pragma unroll
   for (int k = 0; k < 8; ++k) within += (a.first_chunk[group * 8 + k] <= chunk) ? 1 : 0;
@@ -571,14 +575,14 @@ static int check_dtypes(int p_dtype, int g_dtype) {
 // Completes prefix and pivots of a launch batch and launches it.  Args is FusedArgs
 // or SmallArgs; `chunks` is the batch's total chunk count.
 template <typename Args>
-static void finish_prefix(Args &a, int capacity) {
-  for (int i = a.ntensors; i < capacity + 8; ++i) a.first_chunk[i] = 0xffffffffu;
-  for (int k = 0; k < 8; ++k) a.pivot[k] = k * 8 < capacity + 8 ? a.first_chunk[k * 8] : 0xffffffffu;
+static void finish_prefix(Args &a) {
+  for (int i = a.ntensors; i < Args::kPivots * 8; ++i) a.first_chunk[i] = 0xffffffffu;
+  for (int k = 0; k < Args::kPivots; ++k) a.pivot[k] = a.first_chunk[k * 8];
 }
 
 static int launch_fused_batch(FusedArgs &a, uint64_t chunks, void (*kernel)(const FusedArgs),
                               hipStream_t stream) {
-  finish_prefix(a, kMaxTensors);
+  finish_prefix(a);
   a.nchunks = (uint32_t)chunks;
   a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
   hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, stream, a);
@@ -586,11 +590,10 @@ static int launch_fused_batch(FusedArgs &a, uint64_t chunks, void (*kernel)(cons
   return 0;
 }
 
-template <typename Args, typename Kernel>
-static int launch_batch(Args &a, int capacity, uint64_t chunks, Kernel kernel, int threads,
-                        hipStream_t stream) {
-  finish_prefix(a, capacity);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)chunks), dim3(threads), 0, stream, a);
+static int launch_small_batch(SmallArgs &a, uint64_t chunks, void (*kernel)(const SmallArgs),
+                              hipStream_t stream) {
+  finish_prefix(a);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)chunks), dim3(256), 0, stream, a);
   Q4_HIP(hipGetLastError());
   return 0;
 }
@@ -741,7 +744,7 @@ int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int c
     if (t.numel == 0) continue;
     const uint64_t c = (uint64_t)(t.numel + kSmallChunk - 1) / kSmallChunk;
     if (a.ntensors == kMaxSmallTensors || chunks + c > kMaxChunksPerLaunch) {
-      if (int rc = launch_batch(a, kMaxSmallTensors, chunks, kernel, 256, s)) return rc;
+      if (int rc = launch_small_batch(a, chunks, kernel, s)) return rc;
       a.ntensors = 0;
       chunks = 0;
     }
@@ -755,7 +758,7 @@ int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int c
     ++a.ntensors;
     chunks += c;
   }
-  if (a.ntensors > 0) return launch_batch(a, kMaxSmallTensors, chunks, kernel, 256, s);
+  if (a.ntensors > 0) return launch_small_batch(a, chunks, kernel, s);
   return 0;
 }
 

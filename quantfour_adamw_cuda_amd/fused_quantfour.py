@@ -161,8 +161,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
 
     def load_state_dict(self, state_dict):
         super().load_state_dict(state_dict)
-        # The base class narrows floating-point state to the parameter's dtype; block
-        # scales and non-quantized moments are fp32 whatever the parameter is.
+        # The base class casts every state tensor to the parameter's dtype.  Packed codes
+        # are uint8, block scales and non-quantized moments fp32, whatever the parameter
+        # is: take them from the source again, keeping their dtype.
         saved_ids = chain.from_iterable(g["params"] for g in state_dict["param_groups"])
         own = chain.from_iterable(g["params"] for g in self.param_groups)
         for pid, p in zip(saved_ids, own):
@@ -171,8 +172,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 continue
             dst = self.state[p]
             for key in ("exp_avg", "exp_avg_sq"):
-                if torch.is_tensor(src.get(key)) and src[key].dtype == torch.float32:
-                    dst[key] = src[key].detach().to(device=p.device, dtype=torch.float32, copy=True)
+                if torch.is_tensor(src.get(key)):
+                    dst[key] = src[key].detach().to(device=p.device, copy=True)
             for key in ("momentum_qstate", "variance_qstate"):
                 max1 = src.get(key, {}).get("overhead", {}).get("max1")
                 if torch.is_tensor(max1):

@@ -1,0 +1,75 @@
+"""Writes the golden fixtures of the 4-bit AdamW step (tests/golden/*.npz).
+
+The reference ships no golden vectors, known-answer tests or fixtures for this path
+(its tests/assets/ directory does not exist), so these vectors come from this build's
+CPU oracle (oracle/q4_oracle.c), after that oracle has been pinned by
+tests/test_oracle_pins.py.  They freeze the arithmetic: a later change to the oracle or
+to the kernel that alters a single bit of the packed states shows up against them.
+
+    python tests/golden/make_golden.py
+
+Each fixture holds the inputs themselves (no RNG is needed to replay it) and, for every
+step, the expected parameters, packed codes and block scales as raw bit patterns.
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import q4_oracle as oc  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def bf16_round(x):
+    u = x.astype(np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    return u.astype(np.uint16)
+
+
+def make(name, n, steps, hp, p_bf16=False, g_bf16=False, seed=0, special=None):
+    rng = np.random.default_rng(seed)
+    p = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    grads = []
+    for _ in range(steps):
+        g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        u = rng.uniform(size=n)
+        g[u < 0.15] = 0.0
+        g[(u >= 0.15) & (u < 0.17)] = np.float32(1e-41)          # fp32 denormal
+        g[(u >= 0.17) & (u < 0.171)] = np.float32(1e3)
+        if special is not None:
+            special(g)
+        grads.append(g)
+    p_in = bf16_round(p) if p_bf16 else p
+    g_in = [bf16_round(g) if g_bf16 else g for g in grads]
+    nb, nk = oc.state_sizes(n)
+    m, v = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8)
+    sm, sv = np.zeros(nk, np.float32), np.zeros(nk, np.float32)
+    cur = p_in.copy()
+    out = dict(p0=p_in, hp=np.array([hp["beta1"], hp["beta2"], hp["lr"], hp["weight_decay"], hp["eps"]],
+                                    np.float64))
+    for t, g in enumerate(g_in, 1):
+        oc.step_quant(cur, g, m, v, sm, sv, step=t, **hp)
+        out[f"g{t}"] = g
+        out[f"p{t}"] = cur.copy()
+        out[f"m{t}"] = m.copy()
+        out[f"v{t}"] = v.copy()
+        out[f"sm{t}"] = sm.view(np.uint32).copy()
+        out[f"sv{t}"] = sv.view(np.uint32).copy()
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), **out)
+    print(name, n, "elements,", steps, "steps")
+
+
+def zero_blocks(g):
+    g[128:384] = 0.0
+
+
+if __name__ == "__main__":
+    hp = dict(beta1=0.9, beta2=0.999, lr=1e-3, weight_decay=0.01, eps=1e-8)
+    hp_driver = dict(beta1=0.8, beta2=0.88, lr=5e-3, weight_decay=0.03, eps=1e-8)   # tests/driver.py:28-31
+    make("quant_fp32_fp32_n1027", 1027, 3, hp, seed=1, special=zero_blocks)
+    make("quant_fp32_bf16_n4099", 4099, 3, hp, g_bf16=True, seed=2)
+    make("quant_bf16_bf16_n2050", 2050, 3, hp, p_bf16=True, g_bf16=True, seed=3)
+    make("quant_driver_hp_n640", 640, 4, hp_driver, seed=4)

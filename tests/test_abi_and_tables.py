@@ -1,0 +1,210 @@
+"""CPU-side checks of the shipped library (no GPU work): it loads, exports every symbol
+the header declares, its host-only helpers agree with the oracle, and the first-moment
+bucket table has the properties the kernel's fast path relies on.  A numpy model of the
+fast path shows that every code it decides on its own equals the exact code."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import q4_oracle as oc
+from quantfour_adamw_cuda_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "q4adamw.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(q4adamw_\w+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(raw, name), name
+    assert lib.q4adamw_version() >= 1000
+    assert lib.q4adamw_last_error() is not None
+
+
+def test_struct_layouts_match_header():
+    assert ctypes.sizeof(_lib.Q4Tensor) == 56 and ctypes.sizeof(_lib.Q4SmallTensor) == 40
+    assert _lib.Q4Tensor.numel.offset == 48 and _lib.Q4SmallTensor.numel.offset == 32
+
+
+def test_host_helpers_match_oracle(lib):
+    f = ctypes.c_float
+    for which in (0, 1):
+        qmap, qmid = (f * 16)(), (f * 15)()
+        lib.q4adamw_tables(which, qmap, qmid)
+        o_map, o_mid = oc.tables(which)
+        assert np.array_equal(np.array(qmap[:], np.float32).view(np.uint32), o_map.view(np.uint32))
+        assert np.array_equal(np.array(qmid[:], np.float32).view(np.uint32), o_mid.view(np.uint32))
+    out = (f * 6)()
+    for b1, b2, lr, wd in [(0.9, 0.999, 1e-3, 0.01), (0.8, 0.88, 5e-3, 0.03)]:
+        for t in (1, 2, 7, 100, 2000):
+            lib.q4adamw_derive_scalars(b1, b2, lr, wd, float(t), out)
+            want = oc.derive_scalars(b1, b2, lr, wd, t)
+            assert np.array_equal(np.array(out[:], np.float32).view(np.uint32), want.view(np.uint32))
+
+
+def test_argument_errors_need_no_gpu(lib):
+    """Validation happens before any HIP call."""
+    z = ctypes.c_void_p(0)
+    rc = lib.q4adamw_fused_4bit(z, z, z, z, z, z, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -1 and b"null" in lib.q4adamw_last_error()
+    rc = lib.q4adamw_fused_4bit(z, z, z, z, z, z, 0, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == 0                                            # empty tensor: nothing to do
+    rc = lib.q4adamw_fused_4bit(z, z, z, z, z, z, 128, 0, 7, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -1 and b"dtype" in lib.q4adamw_last_error()
+    rc = lib.q4adamw_fused_4bit(z, z, z, z, z, z, 128, 0, 0, 1.5, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -3
+    rc = lib.q4adamw_fused_4bit(z, z, z, z, z, z, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 0.0, z)
+    assert rc == -3                                           # step counts from 1
+    a = ctypes.c_void_p(0x1004)
+    rc = lib.q4adamw_fused_4bit(a, a, a, a, a, a, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -2 and b"aligned" in lib.q4adamw_last_error()
+    rc = lib.q4adamw_fused_single_tensor(z, z, z, z, 16, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -1
+    assert lib.q4adamw_mtable_entry(4096, (ctypes.c_uint32 * 2)()) == -1
+    assert lib.q4adamw_release() == 0
+
+
+# ---------------------------------------------------------------------------
+# bucket table
+# ---------------------------------------------------------------------------
+GUARD_ULPS = 6
+NO_THR = 0x7F000000
+
+
+def _table(lib):
+    out = (ctypes.c_uint32 * 2)()
+    lo = np.zeros(2048, np.uint32)
+    hi = np.zeros(2048, np.uint32)
+    for i in range(2048):
+        assert lib.q4adamw_mtable_entry(i, out) == 0
+        lo[i], hi[i] = out[0], out[1]
+    return lo, hi
+
+
+def test_bucket_table_properties(lib):
+    lo, hi = _table(lib)
+    _, mid = oc.tables(0)
+    mid_bits = mid.view(np.uint32)
+    with_thr = np.flatnonzero(hi != NO_THR)
+    assert with_thr.size == 15
+    # the kernel only builds buckets 471..508 per sign; everything a clamped quotient can
+    # reach outside the threshold buckets must say "base, no threshold"
+    assert set(with_thr.tolist()) <= set(range(471, 509)) | set(range(1024 + 471, 1024 + 509))
+    seen = []
+    for i in range(2048):
+        sign, mag = i >> 10, i & 1023
+        base = int(lo[i] & 15)
+        b_lo = np.uint32(mag << 21).view(np.float32)
+        if mag >> 2 >= 255:
+            continue                                           # inf / nan patterns
+        b_hi = np.uint32((mag + 1) << 21).view(np.float32)
+        # any value of the bucket
+        probe = np.float32(-b_lo if sign else b_lo)
+        exact = oc.quantize_count(0, probe)
+        if hi[i] == NO_THR:
+            assert (lo[i] & ~np.uint32(15)) == NO_THR
+            assert base == exact, (i, base, exact)
+            continue
+        # exactly one threshold inside, at least 64 ulps away from both bucket edges
+        inside = [j for j in range(15) if (b_lo <= mid[j] < b_hi if not sign else -b_hi < mid[j] < -b_lo)]
+        assert len(inside) == 1
+        j = inside[0]
+        seen.append(j)
+        m = int(mid_bits[j] & 0x7FFFFFFF)
+        assert m - (mag << 21) >= 64 and ((mag + 1) << 21) - m >= 64
+        assert base == sum(1 for k in range(15) if mid[k] < mid[j])
+        lo_mag, hi_mag = int(lo[i] & 0x7FFFFFFF), int(hi[i] & 0x7FFFFFFF)
+        if not sign:
+            assert GUARD_ULPS <= m - lo_mag <= GUARD_ULPS + 15 and hi_mag - m == GUARD_ULPS
+        else:
+            assert GUARD_ULPS <= lo_mag - m <= GUARD_ULPS + 15 and m - hi_mag == GUARD_ULPS
+            assert lo[i] >> 31 == 1 and hi[i] >> 31 == 1
+    assert sorted(seen) == list(range(15))
+
+
+def _nudge(x, d):
+    """array of fp32 moved by d ulps in magnitude (d may be an array)."""
+    return (x.view(np.uint32).astype(np.int64) + d).astype(np.uint32).view(np.float32)
+
+
+def _rn32(x64):
+    return x64.astype(np.float32)
+
+
+def test_fast_path_model_first_moment(lib):
+    """Model of the kernel's first-moment fast path: q^ = RN(x * r) with r anywhere within one
+    ulp of 1/s, bucket lookup with the per-sign clamp, decision by the guard bounds.  Wherever
+    the model does not ask for the exact path its code must equal the exact code
+    #{j : mid_j < RN(x / s)}, for x on and around every threshold times the scale."""
+    lo, hi = _table(lib)
+    _, mid = oc.tables(0)
+    rng = np.random.default_rng(0)
+    s = (10.0 ** rng.uniform(-25, 25, 4000)).astype(np.float32)
+    d = np.arange(-40, 41)
+    undecided = 0
+    total = 0
+    for j in range(15):
+        centre = _rn32(mid[j].astype(np.float64) * s.astype(np.float64))
+        x = _nudge(centre[:, None].repeat(d.size, 1), d[None, :])          # [s, d]
+        exact_q = _rn32(x.astype(np.float64) / s[:, None].astype(np.float64))
+        exact_code = np.searchsorted(mid, exact_q.ravel(), side="left").reshape(exact_q.shape)
+        r0 = _rn32(1.0 / s.astype(np.float64))
+        for dr in (-1, 0, 1):
+            r = _nudge(r0, dr)
+            q = _rn32(x.astype(np.float64) * r[:, None].astype(np.float64))
+            a = (q.view(np.uint32) >> 18) & 0x3FF8
+            floor_a = (a & (1024 * 8)) | (471 * 8)
+            a = np.maximum(a, floor_a)
+            e_lo, e_hi = lo[a >> 3], hi[a >> 3]
+            above_hi = q > e_hi.view(np.float32)
+            above_lo = q > (e_lo.view(np.float32))
+            decided = above_hi == above_lo
+            code = (e_lo & 15).astype(np.int64) + above_hi
+            assert np.array_equal(code[decided], exact_code[decided])
+            undecided += int((~decided).sum())
+            total += decided.size
+    # the guard band is a few ulps wide: most of the +-40 ulp neighbourhood is decided
+    assert 0 < undecided < 0.6 * total
+
+
+def test_fast_path_model_second_moment():
+    """Same for the second moment: t = fma(x, 16 r, w - 0.5) with w = 2^-17; code = trunc(t)
+    unless fract(t) < 2w."""
+    _, mid = oc.tables(1)
+    rng = np.random.default_rng(1)
+    s = (10.0 ** rng.uniform(-25, 25, 4000)).astype(np.float32)
+    d = np.arange(-40, 41)
+    w = np.float32(2.0 ** -17)
+    undecided = total = 0
+    for j in range(15):
+        centre = _rn32(mid[j].astype(np.float64) * s.astype(np.float64))
+        x = _nudge(centre[:, None].repeat(d.size, 1), d[None, :])
+        x = np.minimum(x, s[:, None])                                       # x <= scale always
+        exact_q = _rn32(x.astype(np.float64) / s[:, None].astype(np.float64))
+        exact_code = np.searchsorted(mid, exact_q.ravel(), side="left").reshape(exact_q.shape)
+        r0 = _rn32(1.0 / s.astype(np.float64))
+        for dr in (-1, 0, 1):
+            r16 = _nudge(r0, dr) * np.float32(16)
+            t = _rn32(x.astype(np.float64) * r16[:, None].astype(np.float64) + np.float64(w - np.float32(0.5)))
+            fract = t - np.floor(t)
+            decided = ~(fract < 2 * w)
+            code = np.trunc(t).astype(np.int64)
+            assert np.array_equal(code[decided], exact_code[decided])
+            undecided += int((~decided).sum())
+            total += decided.size
+    assert 0 < undecided < 0.6 * total
+    # far from thresholds nothing is flagged: uniform quotients
+    q = rng.uniform(0, 1, 200000).astype(np.float32)
+    t = _rn32(q.astype(np.float64) * 16 + np.float64(w - np.float32(0.5)))
+    assert ((t - np.floor(t)) < 2 * w).mean() < 1e-3

@@ -1,0 +1,262 @@
+"""GPU tests of the optimizer class: the reference's own test idea (tests/driver.py: track
+torch.optim.AdamW on a small MLP), the multi-tensor GPT-2-small parameter set against the
+oracle, checkpoint resume, and the real Llama-3-8B tensor shapes."""
+from copy import deepcopy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import q4_oracle as oc
+from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+from tests.q4_testlib import HP, bits, grads_config1, grads_student_t, p_close, to_np
+
+pytestmark = pytest.mark.gpu
+
+KW = dict(lr=HP["lr"], betas=(HP["beta1"], HP["beta2"]), eps=HP["eps"], weight_decay=HP["weight_decay"])
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def _driver_loop(model, model_clone, fourbit, iters=10, size=5, atol=0.025):
+    """tests/driver.py:25-71 (_test_basics): non-default hyper-parameters, 10 iterations,
+    params change after the first step and stay within atol 0.025 / rtol 1e-5 of AdamW."""
+    betas, weight_decay, lr, eps = (0.8, 0.88), 0.03, 0.005, 1e-8
+    adam = torch.optim.AdamW(model_clone.parameters(), lr=lr, betas=betas, weight_decay=weight_decay, eps=eps)
+    opt = fourbit(model.parameters(), lr=lr, betas=betas, weight_decay=weight_decay, eps=eps)
+    orig = [p.clone() for p in model.parameters()]
+    worst = 0.0
+    for i in range(iters):
+        adam.zero_grad(set_to_none=True)
+        opt.zero_grad(set_to_none=True)
+        inp = torch.randn(size, model[0].in_features, device="cuda")
+        model(inp).sum().backward()
+        model_clone(inp).sum().backward()
+        adam.step()
+        opt.step()
+        if i == 0:
+            for p1, p2 in zip(model.parameters(), orig):
+                assert not torch.equal(p1, p2)
+        for p1, p2 in zip(model.parameters(), model_clone.parameters()):
+            torch.testing.assert_close(p1, p2, atol=atol, rtol=1e-5)
+            worst = max(worst, float((p1.detach() - p2.detach()).abs().max()))
+    return opt, worst
+
+
+def test_driver_mlp_default_threshold(cuda):
+    """The reference's 85-parameter MLP: every tensor is below the quantization threshold, so
+    the non-quantized kernel runs and the result matches AdamW far inside the tolerance."""
+    torch.manual_seed(2020)
+    model = nn.Sequential(nn.Linear(5, 10), nn.Linear(10, 5)).cuda()
+    clone = deepcopy(model)
+    opt, worst = _driver_loop(model, clone, AdamWFused_QuantFour)
+    say(f"driver MLP (non-quantized path): worst |diff| {worst:.3e}")
+    assert worst < 1e-5
+    for p in model.parameters():
+        assert opt.state[p]["exp_avg"].dtype == torch.float32 and float(opt.state[p]["step"]) == 10.0
+
+
+def test_driver_mlp_forced_quantization(cuda):
+    """Same loop with every tensor forced onto the 4-bit path (threshold 0), and a wider MLP
+    whose weight matrices are quantized at the default threshold.  With betas (0.8, 0.88)
+    the second moment moves fast and its 16 linear levels (lowest: 1/16 of the block max)
+    make single elements lag AdamW by up to a step's worth per step; over 10 steps of at most
+    lr = 0.005 each the observed worst case is 0.028, so these two cases use atol 0.05 (half
+    of the trivial bound).  Bit-exactness against the oracle is what the other tests pin."""
+    def forced(params, **kw):
+        opt = AdamWFused_QuantFour(params, **kw)
+        opt.param_quant_threshold = 0
+        return opt
+
+    torch.manual_seed(2020)
+    model = nn.Sequential(nn.Linear(5, 10), nn.Linear(10, 5)).cuda()
+    opt, worst = _driver_loop(model, deepcopy(model), forced, atol=0.05)
+    say(f"driver MLP (forced 4-bit): worst |diff| {worst:.3e}")
+    for p in model.parameters():
+        assert opt.state[p]["exp_avg"].dtype == torch.uint8
+    torch.manual_seed(2021)
+    wide = nn.Sequential(nn.Linear(96, 128), nn.Linear(128, 64)).cuda()
+    opt, worst = _driver_loop(wide, deepcopy(wide), AdamWFused_QuantFour, size=16, atol=0.05)
+    say(f"wide MLP (4-bit weights, fp32-state biases): worst |diff| {worst:.3e}")
+    kinds = sorted(str(opt.state[p]["exp_avg"].dtype) for p in wide.parameters())
+    assert kinds == ["torch.float32", "torch.float32", "torch.uint8", "torch.uint8"]
+
+
+def gpt2_small_shapes():
+    shapes = [(50257, 768), (1024, 768)]
+    for _ in range(12):
+        shapes += [(768,), (768,), (768, 2304), (2304,), (768, 768), (768,), (768,), (768,),
+                   (768, 3072), (3072,), (3072, 768), (768,)]
+    return shapes + [(768,), (768,)]
+
+
+class OracleSet:
+    """CPU twin of a parameter list, stepped tensor by tensor with the C oracle."""
+
+    def __init__(self, params, threshold=4096):
+        self.items = []
+        for p in params:
+            n = p.numel()
+            if n > threshold:
+                nb, nk = oc.state_sizes(n)
+                self.items.append(["q", to_np(p), np.zeros(nb, np.uint8), np.zeros(nb, np.uint8),
+                                   np.zeros(nk, np.float32), np.zeros(nk, np.float32)])
+            else:
+                self.items.append(["s", to_np(p), np.zeros(n, np.float32), np.zeros(n, np.float32)])
+
+    def step_and_check(self, params, grads, opt, step, what):
+        worst = 0.0
+        for it, p, g in zip(self.items, params, grads):
+            prev = it[1].copy()
+            st = opt.state[p]
+            if it[0] == "q":
+                oc.step_quant(it[1], to_np(g), it[2], it[3], it[4], it[5], step=step, **HP)
+                assert np.array_equal(st["exp_avg"].cpu().numpy(), it[2]), f"{what}: m codes {tuple(p.shape)}"
+                assert np.array_equal(st["exp_avg_sq"].cpu().numpy(), it[3]), f"{what}: v codes {tuple(p.shape)}"
+                assert np.array_equal(bits(st["momentum_qstate"]["overhead"]["max1"].cpu().numpy()), bits(it[4]))
+                assert np.array_equal(bits(st["variance_qstate"]["overhead"]["max1"].cpu().numpy()), bits(it[5]))
+            else:
+                oc.step_unquant(it[1], to_np(g), it[2], it[3], step=step, **HP)
+                assert np.array_equal(bits(st["exp_avg"].cpu().numpy().reshape(-1)), bits(it[2]))
+                assert np.array_equal(bits(st["exp_avg_sq"].cpu().numpy().reshape(-1)), bits(it[3]))
+            ok, w = p_close(to_np(p.detach()), it[1], prev, bf16=p.dtype == torch.bfloat16)
+            assert ok, f"{what}: params {tuple(p.shape)} worst {w}"
+            worst = max(worst, w)
+            it[1][:] = to_np(p.detach())
+        return worst
+
+
+def test_gpt2_small_parameter_set(cuda):
+    """148 tensors, 124 M params, fp32: 50 quantized tensors in one multi-tensor launch, 98
+    small tensors on the non-quantized kernel; 5 steps, every tensor checked every step."""
+    gen = torch.Generator().manual_seed(0)
+    shapes = gpt2_small_shapes()
+    assert len(shapes) == 148 and sum(int(np.prod(s)) for s in shapes) == 124439808
+    host = [torch.randn(s, generator=gen) * 0.02 for s in shapes]
+    params = [nn.Parameter(h.clone().to(cuda)) for h in host]
+    opt = AdamWFused_QuantFour(params, **KW)
+    ref = OracleSet(host)
+    assert sum(1 for it in ref.items if it[0] == "q") == 50
+    for step in range(1, 6):
+        grads = [grads_config1(gen, int(np.prod(s))).view(s) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = g.to(cuda)
+        say(f"[gpt2-small] step {step}")
+        opt.step()
+        torch.cuda.synchronize()
+        worst = ref.step_and_check(params, grads, opt, step, f"gpt2 step {step}")
+    say(f"gpt2-small: parity ok, worst relative parameter error {worst:.3e}")
+
+
+def test_resume_from_state_dict_is_bit_identical(cuda):
+    """save -> load into a fresh optimizer -> the next steps equal the uninterrupted run."""
+    gen = torch.Generator().manual_seed(11)
+    shapes = [(300, 257), (4096,), (129, 33), (64, 64)]
+    host = [torch.randn(s, generator=gen) * 0.02 for s in shapes]
+    grads = [[torch.randn(s, generator=gen) * 1e-3 for s in shapes] for _ in range(6)]
+
+    def run(params, opt, steps):
+        for gs in steps:
+            for p, g in zip(params, gs):
+                p.grad = g.to(cuda)
+            opt.step()
+
+    a = [nn.Parameter(h.clone().to(cuda)) for h in host]
+    opt_a = AdamWFused_QuantFour(a, **KW)
+    run(a, opt_a, grads)
+    b = [nn.Parameter(h.clone().to(cuda)) for h in host]
+    opt_b = AdamWFused_QuantFour(b, **KW)
+    run(b, opt_b, grads[:3])
+    sd = deepcopy(opt_b.state_dict())
+    saved = [p.detach().clone() for p in b]
+    c = [nn.Parameter(s.clone()) for s in saved]
+    opt_c = AdamWFused_QuantFour(c, **KW)
+    opt_c.load_state_dict(sd)
+    run(c, opt_c, grads[3:])
+    torch.cuda.synchronize()
+    for pa, pc in zip(a, c):
+        assert torch.equal(pa.view(torch.int32), pc.view(torch.int32))
+        sa, sc = opt_a.state[pa], opt_c.state[pc]
+        assert torch.equal(sa["exp_avg"], sc["exp_avg"]) and torch.equal(sa["exp_avg_sq"], sc["exp_avg_sq"])
+        assert float(sa["step"]) == float(sc["step"]) == 6.0
+        if sa["momentum_qstate"]["enable"]:
+            assert torch.equal(sa["momentum_qstate"]["overhead"]["max1"], sc["momentum_qstate"]["overhead"]["max1"])
+            assert torch.equal(sa["variance_qstate"]["overhead"]["max1"], sc["variance_qstate"]["overhead"]["max1"])
+
+
+def test_param_groups_missing_grads_and_bf16(cuda):
+    """Two param groups with their own hyper-parameters, a parameter without a gradient
+    (skipped, its step count stays behind), a bf16 parameter with bf16 gradient."""
+    gen = torch.Generator().manual_seed(5)
+    w1 = nn.Parameter((torch.randn(200, 130, generator=gen) * 0.02).to(cuda))
+    w2 = nn.Parameter((torch.randn(9000, generator=gen) * 0.02).to(cuda))
+    w3 = nn.Parameter((torch.randn(70, 129, generator=gen) * 0.02).to(torch.bfloat16).to(cuda))
+    opt = AdamWFused_QuantFour([{"params": [w1, w3]}, {"params": [w2], "lr": 5e-4, "weight_decay": 0.0}], **KW)
+    r1, r2, r3 = OracleSet([w1.detach().cpu()]), OracleSet([w2.detach().cpu()]), OracleSet([w3.detach().cpu()])
+    hp2 = dict(HP, lr=5e-4, weight_decay=0.0)
+    for step in range(1, 4):
+        g1 = torch.randn(200, 130, generator=gen) * 1e-3
+        g3 = (torch.randn(70, 129, generator=gen) * 1e-3).to(torch.bfloat16)
+        w1.grad, w3.grad = g1.to(cuda), g3.to(cuda)
+        g2 = None
+        if step != 2:
+            g2 = torch.randn(9000, generator=gen) * 1e-3
+            w2.grad = g2.to(cuda)
+        else:
+            w2.grad = None
+        opt.step()
+        torch.cuda.synchronize()
+        r1.step_and_check([w1], [g1], opt, step, "group 0 fp32")
+        r3.step_and_check([w3], [g3], opt, step, "group 0 bf16")
+        if g2 is not None:
+            it = r2.items[0]
+            t2 = int(float(opt.state[w2]["step"]))
+            prev = it[1].copy()
+            oc.step_quant(it[1], g2.numpy().reshape(-1), it[2], it[3], it[4], it[5], step=t2, **hp2)
+            assert np.array_equal(opt.state[w2]["exp_avg"].cpu().numpy(), it[2])
+            ok, w = p_close(to_np(w2.detach()), it[1], prev)
+            assert ok, w
+            it[1][:] = to_np(w2.detach())
+    assert float(opt.state[w1]["step"]) == 3.0 and float(opt.state[w2]["step"]) == 2.0
+
+
+@pytest.mark.parametrize("shape", [(4096,), (1024, 4096), (4096, 4096), (14336, 4096), (4096, 14336)])
+def test_llama3_8b_tensor_shapes(cuda, shape):
+    """Every distinct tensor shape of the headline configuration except the embedding, at its
+    real size: fp32 master parameter, bf16 gradient (Student-t, df 3), 3 steps."""
+    gen = torch.Generator(device=cuda).manual_seed(shape[0])
+    n = int(np.prod(shape))
+    p = nn.Parameter(torch.randn(shape, generator=gen, device=cuda) * 0.02)
+    p.grad_dtype = torch.bfloat16
+    opt = AdamWFused_QuantFour([p], **KW)
+    ref = OracleSet([p.detach().cpu()])
+    for step in range(1, 4):
+        z = torch.randn(n, generator=gen, device=cuda)
+        c = torch.randn(3, n, generator=gen, device=cuda).square().sum(0) / 3.0
+        g = (z / c.sqrt() * 1e-4).to(torch.bfloat16).view(shape)
+        p.grad = g
+        say(f"[llama shape {shape}] step {step}")
+        opt.step()
+        torch.cuda.synchronize()
+        ref.step_and_check([p], [g.cpu()], opt, step, f"llama {shape} step {step}")
+
+
+def test_llama3_8b_embedding_shape(cuda):
+    """128256 x 4096 (525 M elements, byte offsets beyond 2^31): one step against the oracle."""
+    shape = (128256, 4096)
+    n = shape[0] * shape[1]
+    gen = torch.Generator(device=cuda).manual_seed(9)
+    p = nn.Parameter(torch.randn(shape, generator=gen, device=cuda) * 0.02)
+    p.grad_dtype = torch.bfloat16
+    opt = AdamWFused_QuantFour([p], **KW)
+    ref = OracleSet([p.detach().cpu()])
+    g = (torch.randn(shape, generator=gen, device=cuda) * 1e-4).to(torch.bfloat16)
+    g[1000:1100] = 0          # rows without gradient: all-zero blocks
+    p.grad = g
+    say("[llama embedding] step 1")
+    opt.step()
+    torch.cuda.synchronize()
+    ref.step_and_check([p], [g.cpu()], opt, 1, "llama embedding")

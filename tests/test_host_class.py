@@ -1,0 +1,156 @@
+"""Host-side behaviour of AdamWFused_QuantFour that needs no GPU: constructor validation
+(optim/fused_quantfour.py:38-47), state layout (:61-70, :110-120, :180-204), routing by
+size (optim/adamw_fourbit_triton.py:131-134), error paths, state_dict handling."""
+import pytest
+import torch
+
+import quantfour_adamw_cuda_amd as q4
+from quantfour_adamw_cuda_amd import AdamWFused_QuantFour, enable_param_quantization
+
+
+def params(*shapes):
+    return [torch.nn.Parameter(torch.randn(s)) for s in shapes]
+
+
+@pytest.mark.parametrize("kwargs,msg", [
+    (dict(lr=0.0), "Invalid learning rate"), (dict(lr=-1e-3), "Invalid learning rate"),
+    (dict(eps=0.0), "Invalid eps value"), (dict(betas=(1.0, 0.999)), r"Invalid Beta\[0\]"),
+    (dict(betas=(0.0, 0.999)), r"Invalid Beta\[0\]"), (dict(betas=(0.9, 1.0)), r"Invalid Beta\[1\]"),
+    (dict(betas=(0.9, -0.1)), r"Invalid Beta\[1\]"), (dict(weight_decay=-0.1), "Invalid weight_decay value")])
+def test_constructor_validation(kwargs, msg):
+    with pytest.raises(ValueError, match=msg):
+        AdamWFused_QuantFour(params((4, 4)), **kwargs)
+
+
+def test_constructor_defaults_and_api():
+    opt = AdamWFused_QuantFour(params((4, 4)))
+    g = opt.param_groups[0]
+    assert g["lr"] == 1e-3 and g["betas"] == (0.9, 0.999) and g["eps"] == 1e-8
+    assert g["weight_decay"] == 1e-2 and g["fused"] is False
+    assert opt.param_quant_threshold == 4096
+    assert isinstance(opt, torch.optim.Optimizer)
+    AdamWFused_QuantFour(params((4, 4)), 3e-4, (0.8, 0.88), 1e-6, 0.03, fused=True)   # positional order
+    with pytest.raises(TypeError):
+        AdamWFused_QuantFour(params((4, 4)), 3e-4, (0.8, 0.88), 1e-6, 0.03, True)      # fused is keyword-only
+
+
+def test_enable_param_quantization_rule():
+    p = torch.zeros(4096)
+    assert enable_param_quantization(p, 4096) is False       # numel <= threshold: not quantized
+    assert enable_param_quantization(torch.zeros(4097), 4096) is True
+    assert enable_param_quantization(p, 0) is True            # a zero threshold disables the rule
+    assert enable_param_quantization(torch.zeros(1), None) is True
+
+
+def test_state_layout():
+    big, small, odd = params((70, 129), (64, 64), (4097,))
+    opt = AdamWFused_QuantFour([big, small, odd])
+    for p in (big, small, odd):
+        opt._init_state(p)
+    sb, ss, so = opt.state[big], opt.state[small], opt.state[odd]
+    for st in (sb, ss, so):
+        assert set(st) == {"step", "exp_avg", "exp_avg_sq", "momentum_qstate", "variance_qstate"}
+        assert st["step"].dtype == torch.float32 and st["step"].dim() == 0 and float(st["step"]) == 0.0
+        for q in ("momentum_qstate", "variance_qstate"):
+            assert set(st[q]) == {"enable", "overhead", "qmap"} and st[q]["qmap"] is None
+    n = 70 * 129
+    assert sb["momentum_qstate"]["enable"] and sb["variance_qstate"]["enable"]
+    assert sb["exp_avg"].dtype == torch.uint8 and sb["exp_avg"].shape == ((n + 1) // 2,)
+    assert sb["exp_avg_sq"].dtype == torch.uint8 and sb["exp_avg_sq"].shape == ((n + 1) // 2,)
+    for q in ("momentum_qstate", "variance_qstate"):
+        max1 = sb[q]["overhead"]["max1"]
+        assert max1.dtype == torch.float32 and max1.shape == ((n + 127) // 128,) and not max1.any()
+    assert not sb["exp_avg"].any() and not sb["exp_avg_sq"].any()
+    assert so["exp_avg"].shape == (2049,) and so["momentum_qstate"]["overhead"]["max1"].shape == (33,)
+    # 64*64 = 4096 elements: not quantized, fp32 moments shaped like the parameter
+    assert not ss["momentum_qstate"]["enable"] and ss["momentum_qstate"]["overhead"] == {}
+    assert ss["exp_avg"].dtype == torch.float32 and ss["exp_avg"].shape == (64, 64)
+    assert q4.state_sizes(n) == ((n + 1) // 2, (n + 127) // 128)
+
+
+def test_threshold_override_routes_small_tensors_to_the_quantized_path():
+    (p,) = params((100,))
+    opt = AdamWFused_QuantFour([p])
+    opt.param_quant_threshold = 0
+    opt._init_state(p)
+    assert opt.state[p]["momentum_qstate"]["enable"] and opt.state[p]["exp_avg"].dtype == torch.uint8
+
+
+def test_step_refuses_cpu_parameters_and_sparse_grads():
+    (p,) = params((8, 8))
+    opt = AdamWFused_QuantFour([p])
+    p.grad = torch.zeros_like(p)
+    with pytest.raises(AssertionError, match="param must be on cuda"):
+        opt.step()
+    (e,) = params((10, 4))
+    opt2 = AdamWFused_QuantFour([e])
+    e.grad = torch.sparse_coo_tensor(torch.tensor([[1], [2]]), torch.tensor([1.0]), (10, 4))
+    with pytest.raises(RuntimeError, match="does not support sparse gradients"):
+        opt2.step()
+
+
+def test_step_without_grads_is_a_noop_and_closure_runs():
+    (p,) = params((8, 8))
+    opt = AdamWFused_QuantFour([p])
+    calls = []
+
+    def closure():
+        calls.append(torch.is_grad_enabled())
+        return torch.tensor(3.0)
+
+    assert float(opt.step(closure)) == 3.0 and calls == [True]
+    assert len(opt.state) == 0
+
+
+def test_step_fails_loudly_without_the_library(monkeypatch):
+    from quantfour_adamw_cuda_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libq4adamw.so")
+    (p,) = params((8, 8))
+    p.grad = torch.zeros_like(p)
+    with pytest.raises(RuntimeError, match="is missing"):
+        AdamWFused_QuantFour([p]).step()
+
+
+def test_state_dict_round_trip_keeps_dtypes():
+    big, small = [torch.nn.Parameter(torch.randn(s).to(torch.bfloat16)) for s in ((50, 130), (10, 10))]
+    opt = AdamWFused_QuantFour([big, small], lr=2e-3)
+    for p in (big, small):
+        opt._init_state(p)
+    opt.state[big]["exp_avg"].fill_(0x5A)
+    opt.state[big]["momentum_qstate"]["overhead"]["max1"].fill_(1.0 + 2.0 ** -20)   # not a bf16 value
+    opt.state[small]["exp_avg_sq"].fill_(1.0 + 2.0 ** -20)
+    opt.state[big]["step"] += 7
+    sd = opt.state_dict()
+    assert sd["param_groups"][0]["lr"] == 2e-3
+    big2, small2 = [torch.nn.Parameter(p.detach().clone()) for p in (big, small)]
+    opt2 = AdamWFused_QuantFour([big2, small2])
+    opt2.load_state_dict(sd)
+    s_big, s_small = opt2.state[big2], opt2.state[small2]
+    assert s_big["exp_avg"].dtype == torch.uint8 and bool((s_big["exp_avg"] == 0x5A).all())
+    max1 = s_big["momentum_qstate"]["overhead"]["max1"]
+    assert max1.dtype == torch.float32 and bool((max1 == 1.0 + 2.0 ** -20).all())
+    assert s_small["exp_avg_sq"].dtype == torch.float32 and bool((s_small["exp_avg_sq"] == 1.0 + 2.0 ** -20).all())
+    assert float(s_big["step"]) == 7.0 and opt2.param_groups[0]["lr"] == 2e-3
+    assert s_big["momentum_qstate"]["enable"] is True and s_small["momentum_qstate"]["enable"] is False
+
+
+def test_setstate_backfills():
+    (p,) = params((4, 4))
+    opt = AdamWFused_QuantFour([p])
+    opt._init_state(p)
+    state = opt.__getstate__()
+    state["param_groups"][0].pop("fused")
+    state["state"][p]["step"] = 3          # a plain number, as older checkpoints hold it
+    opt.__setstate__(state)
+    assert opt.param_groups[0]["fused"] is None
+    assert torch.is_tensor(opt.state[p]["step"]) and float(opt.state[p]["step"]) == 3.0
+
+
+def test_functional_wrappers_validate():
+    p = torch.zeros(300)
+    with pytest.raises(AssertionError, match="param must be on cuda"):
+        q4.fused_4bit(p, p, torch.zeros(150, dtype=torch.uint8), torch.zeros(150, dtype=torch.uint8),
+                      torch.zeros(3), torch.zeros(3), 0.9, 0.999, 1e-3, 0.01, 1e-8, 1)
+    q4.fused_4bit_multi([], [], [], [], [], [], 0.9, 0.999, 1e-3, 0.01, 1e-8, 1)       # nothing to do
+    q4.fused_single_tensor_multi([], [], [], [], 0.9, 0.999, 1e-3, 0.01, 1e-8, 1)

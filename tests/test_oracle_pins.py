@@ -1,0 +1,259 @@
+"""Pins of the CPU oracle (no GPU): tables against known-answer bit patterns and closed
+forms, the quantizer against brute force and a library routine, the derived scalars
+against known answers, the two independent restatements against each other, the
+non-quantized step against torch.optim.AdamW, and the quantized step against
+invariants of the format."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import q4_oracle as oc
+from oracle import q4_oracle_torch as ot
+from tests.q4_testlib import HP, HP_DRIVER, bits, grads_config1, grads_config3, grads_student_t
+
+# fp32 bit patterns of the reference's literal tables (optim/cuda_adamw_kernels.cu:25-98)
+QMAP_M_HEX = ("bf633333 bf29999a bee00000 be59999a bd9eb852 bd051eb8 bbb43958 00000000 "
+              "3bb43958 3d051eb8 3d9eb852 3e59999a 3ee00000 3f29999a 3f633333 3f800000").split()
+QMID_M_HEX = ("bf466666 bf0ccccd bea66666 be147ae1 bd6147ae bc9ba5e3 bb343958 3b343958 "
+              "3c9ba5e3 3d6147ae 3e147ae1 3ea66666 3f0ccccd 3f466666 3f71999a").split()
+
+
+def hexes(a):
+    return [f"{x:08x}" for x in bits(a)]
+
+
+def test_tables_known_answers():
+    qm, mid = oc.tables(0)
+    assert hexes(qm) == QMAP_M_HEX
+    assert hexes(mid) == QMID_M_HEX
+    qv, midv = oc.tables(1)
+    assert np.array_equal(qv, np.arange(1, 17, dtype=np.float32) / 16)
+    assert np.array_equal(midv, (2 * np.arange(1, 16, dtype=np.float32) + 1) / 32)
+    for which in (0, 1):
+        assert np.array_equal(oc.tables(which)[0], ot.QMAP[which].numpy())
+        assert np.array_equal(oc.tables(which)[1], ot.QMID[which].numpy())
+
+
+def test_tables_closed_forms():
+    """The first-moment map is the dynamic-exponent construction of quant_opt_base.py:55-86;
+    the thresholds are the means of neighbouring entries, except that the literal table
+    is one ulp below the fp32 mean at entries 3 and 10 (+-0.145)."""
+    qm_cf, mid_cf, qv_cf, midv_cf = ot.closed_form_tables()
+    qm, mid = oc.tables(0)
+    assert np.array_equal(np.asarray(qm_cf, np.float32), qm)
+    assert np.array_equal(np.asarray(mid_cf, np.float32), mid)      # double means, rounded once
+    fp32_means = (qm[:-1] + qm[1:]) * np.float32(0.5)
+    differ = np.flatnonzero(bits(fp32_means) != bits(mid))
+    assert differ.tolist() == [3, 10]
+    assert (bits(fp32_means)[differ].astype(np.int64) - bits(mid)[differ].astype(np.int64)).tolist() == [1, 1]
+    for which in (0, 1):
+        q, m = oc.tables(which)
+        assert np.all(q[:-1] < m) and np.all(m < q[1:])              # strictly between neighbours
+
+
+def _neighbourhood(values, radius):
+    out = []
+    for v in values:
+        u = int(np.float32(v).view(np.uint32))
+        for d in range(-radius, radius + 1):
+            w = u + d
+            if 0 <= (w & 0x7fffffff) < 0x7f800000:
+                out.append(np.uint32(w & 0xffffffff).view(np.float32))
+    return np.array(out, np.float32)
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_quantizer_search_equals_count_and_library(which):
+    """Binary search restated from the reference == number of thresholds strictly below x
+    == numpy.searchsorted(mid, x, 'left'), on every fp32 within 64 ulps of every table
+    entry and threshold, on +-0, on the range ends and on two million random values."""
+    qmap, mid = oc.tables(which)
+    rng = np.random.default_rng(which)
+    xs = np.concatenate([
+        _neighbourhood(np.concatenate([qmap, mid, [0.0, -0.0, 1.0, -1.0]]), 64),
+        rng.uniform(-1.2, 1.2, 2_000_000).astype(np.float32),
+        (rng.standard_normal(200_000) * 1e-3).astype(np.float32),
+        np.array([np.inf, -np.inf, 3e38, -3e38, 1e-45, -1e-45], np.float32),
+    ])
+    lib = oc.lib()
+    search = np.fromiter((lib.q4o_quantize_search(which, float(x)) for x in xs[:300_000]), np.int32)
+    count = np.fromiter((lib.q4o_quantize_count(which, float(x)) for x in xs[:300_000]), np.int32)
+    assert np.array_equal(search, count)
+    ss = np.searchsorted(mid, xs, side="left").astype(np.int32)
+    assert np.array_equal(ss[:300_000], count)
+    # the vectorised restatement uses torch.bucketize
+    tb = torch.bucketize(torch.from_numpy(xs), ot.QMID[which], right=False).numpy().astype(np.int32)
+    assert np.array_equal(tb, ss)
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_quantizer_special_cases(which):
+    qmap, mid = oc.tables(which)
+    for k, q in enumerate(qmap):                       # a code-book entry maps to itself
+        assert oc.quantize_count(which, q) == k and oc.quantize_search(which, q) == k
+    for j, m in enumerate(mid):                        # a tie goes DOWN
+        assert oc.quantize_count(which, m) == j
+        assert oc.quantize_count(which, np.nextafter(m, np.float32(2))) == j + 1
+        assert oc.quantize_search(which, m) == j
+    assert oc.quantize_count(which, np.float32(-5)) == 0 and oc.quantize_count(which, np.float32(5)) == 15
+    assert oc.quantize_count(which, np.float32("nan")) == 0 and oc.quantize_search(which, np.float32("nan")) == 0
+    if which == 0:
+        assert oc.quantize_count(0, np.float32(-1.0)) == 0    # x <= -0.8875
+        assert oc.quantize_count(0, np.float32(0.0)) == 7 and oc.quantize_count(0, np.float32(-0.0)) == 7
+    else:
+        assert oc.quantize_count(1, np.float32(0.0)) == 0
+
+
+def test_derived_scalars_known_answers():
+    s = oc.derive_scalars(0.9, 0.999, 1e-3, 0.01, 1)
+    # 1 - f32(0.999) is NOT f32(0.001): 0x3a831200 vs 0x3a83126f
+    assert f"{bits(s)[4]:08x}" == "3dccccd0" and f"{bits(s)[5]:08x}" == "3a831200"
+    assert f"{bits(s)[3]:08x}" == "3f7fff58"
+    assert f"{int(np.float32(0.001).view(np.uint32)):08x}" == "3a83126f"
+    for b1, b2, lr, wd in [(0.9, 0.999, 1e-3, 0.01), (0.8, 0.88, 5e-3, 0.03), (0.95, 0.99, 3e-4, 0.1)]:
+        f32 = np.float32
+        one = f32(1)
+        for t in [1, 2, 3, 10, 100, 1000, 5000]:
+            s = oc.derive_scalars(b1, b2, lr, wd, t)
+            # the same chain in numpy fp32 scalars, pow taken in double and rounded once
+            c1 = one - f32(float(f32(b1)) ** t)
+            c2s = np.sqrt(one - f32(float(f32(b2)) ** t))
+            want = np.array([c1, c2s, f32(lr) / c1, one - f32(lr) * f32(wd), one - f32(b1),
+                             one - f32(b2)], f32)
+            assert np.array_equal(bits(want), bits(s))
+            # and against double precision: the fp32 chain loses at most the cancellation
+            # error of 1 - beta**t, i.e. half an ulp of 1.0 relative to the difference
+            c1d = 1 - float(f32(b1)) ** t
+            assert abs(float(s[0]) - c1d) <= 2.0 ** -24 and abs(float(s[2]) * c1d - float(f32(lr))) < 1e-9
+            st = ot.derive_scalars(b1, b2, lr, wd, t)
+            got = np.array([st["c1"], st["c2s"], st["ss"], st["wdu"], st["r1"], st["r2"]], np.float32)
+            assert np.array_equal(bits(got), bits(s))
+
+
+def _zero_state(n):
+    nb, nk = oc.state_sizes(n)
+    return (np.zeros(nb, np.uint8), np.zeros(nb, np.uint8), np.zeros(nk, np.float32), np.zeros(nk, np.float32))
+
+
+@pytest.mark.parametrize("n,gradfn,hp", [
+    (300_007, grads_config1, HP), (128 * 11 + 1, grads_config3, HP), (127, grads_config3, HP),
+    (1, grads_config3, HP), (4097, grads_config3, HP), (200_000, grads_student_t, HP),
+    (50_001, grads_config1, HP_DRIVER)])
+def test_two_restatements_agree_bit_for_bit(n, gradfn, hp):
+    """Scalar C oracle == vectorised torch oracle: params, codes, scales, every step."""
+    gen = torch.Generator().manual_seed(n)
+    p = torch.randn(n, generator=gen) * 0.02
+    pc = p.numpy().copy()
+    m, v, sm, sv = _zero_state(n)
+    tm, tv, tsm, tsv = (torch.from_numpy(x.copy()) for x in (m, v, sm, sv))
+    for step in range(1, 5):
+        g = gradfn(gen, n)
+        oc.step_quant(pc, g.numpy(), m, v, sm, sv, step=step, **hp)
+        p, tm, tv, tsm, tsv = ot.step_quant(p, g, tm, tv, tsm, tsv, step=step, **hp)
+        assert np.array_equal(bits(p.numpy()), bits(pc))
+        assert np.array_equal(tm.numpy(), m) and np.array_equal(tv.numpy(), v)
+        assert np.array_equal(bits(tsm.numpy()), bits(sm)) and np.array_equal(bits(tsv.numpy()), bits(sv))
+
+
+def test_bf16_restatements_agree():
+    """bf16 gradients widen exactly; bf16 parameters are rounded to nearest even on store."""
+    gen = torch.Generator().manual_seed(5)
+    n = 70_003
+    for p_dtype in (torch.float32, torch.bfloat16):
+        p = (torch.randn(n, generator=gen) * 0.02).to(p_dtype)
+        pc = (p.view(torch.int16).numpy().view(np.uint16).copy() if p_dtype == torch.bfloat16
+              else p.numpy().copy())
+        m, v, sm, sv = _zero_state(n)
+        tm, tv, tsm, tsv = (torch.from_numpy(x.copy()) for x in (m, v, sm, sv))
+        for step in range(1, 4):
+            g = grads_student_t(gen, n).to(torch.bfloat16)
+            gb = g.view(torch.int16).numpy().view(np.uint16).copy()
+            oc.step_quant(pc, gb, m, v, sm, sv, step=step, **HP)
+            p, tm, tv, tsm, tsv = ot.step_quant(p, g, tm, tv, tsm, tsv, step=step, **HP)
+            got = p.view(torch.int16).numpy().view(np.uint16) if p_dtype == torch.bfloat16 else bits(p.numpy())
+            assert np.array_equal(got, pc if p_dtype == torch.bfloat16 else bits(pc))
+            assert np.array_equal(tm.numpy(), m) and np.array_equal(tv.numpy(), v)
+
+
+def test_format_invariants():
+    """scale == max |x| of the block; the arg-max gets code 15 (or 0 for a negative first
+    moment); pack/unpack round trip; unused high nibble of an odd tail is zero; an
+    all-zero block is closed under the step (zero codes, zero scales, stays so)."""
+    rng = np.random.default_rng(0)
+    n = 128 * 7 + 77
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    x[256:384] = 0
+    for which, data in ((0, x), (1, x * x)):
+        codes, scale = oc.quant(data, which)
+        blocks = np.pad(np.abs(data), (0, 128 * 8 - n)).reshape(8, 128)
+        assert np.array_equal(bits(scale), bits(blocks.max(axis=1)))
+        unpacked = ot.unpack(torch.from_numpy(codes), n).numpy()
+        assert np.array_equal(ot.pack(torch.from_numpy(unpacked), n).numpy(), codes)
+        assert codes[-1] >> 4 == 0                                      # odd tail
+        for b in range(8):
+            seg = slice(b * 128, min((b + 1) * 128, n))
+            if scale[b] == 0:
+                assert not unpacked[seg].any()
+                continue
+            k = int(np.argmax(np.abs(data[seg])))
+            assert unpacked[seg][k] == (15 if data[seg][k] > 0 else 0)
+        deq = oc.dequant(codes, scale, n, which)
+        codes2, scale2 = oc.quant(deq, which)
+        # requantizing a dequantized state changes nothing when the block's arg-max sits on
+        # +1.0 (always true for the second moment)
+        if which == 1:
+            assert np.array_equal(codes2, codes) and np.array_equal(bits(scale2), bits(scale))
+    # all-zero block: zero state, zero grads
+    p = (rng.standard_normal(256) * 0.02).astype(np.float32)
+    m, v, sm, sv = _zero_state(256)
+    for step in (1, 2, 3):
+        oc.step_quant(p, np.zeros(256, np.float32), m, v, sm, sv, step=step, **HP)
+        assert not m.any() and not v.any() and not sm.any() and not sv.any()
+    assert np.all(np.signbit(oc.dequant(m, sm, 256, 0)))               # -0.8875 * 0 = -0.0
+
+
+def test_unquantized_step_is_adamw():
+    """With fp32 moments the step is textbook AdamW with decoupled weight decay: it must
+    track torch.optim.AdamW (library routine).  The bound is set by the reference's fp32
+    derived scalars: 1.0f - 0.999f is 1.3e-5 (relative) away from the 0.001 that torch
+    uses, so the second moment may differ by that much and the parameters by a few 1e-6."""
+    gen = torch.Generator().manual_seed(2020)
+    n = 4096
+    for hp in (HP, HP_DRIVER):
+        p0 = torch.randn(n, generator=gen) * 0.1
+        ref = torch.nn.Parameter(p0.clone())
+        opt = torch.optim.AdamW([ref], lr=hp["lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["eps"],
+                                weight_decay=hp["weight_decay"])
+        p = p0.numpy().copy()
+        m = np.zeros(n, np.float32)
+        v = np.zeros(n, np.float32)
+        for step in range(1, 11):
+            g = torch.randn(n, generator=gen) * 1e-2
+            ref.grad = g.clone()
+            opt.step()
+            oc.step_unquant(p, g.numpy(), m, v, step=step, **hp)
+            st = opt.state[ref]
+            for got, want, tol in ((p, ref.detach().numpy(), 1e-5), (m, st["exp_avg"].numpy(), 1e-6),
+                                   (v, st["exp_avg_sq"].numpy(), 1e-4)):
+                assert np.abs(got - want).max() <= tol * np.abs(want).max()
+
+
+def test_quantized_step_tracks_adamw_like_the_reference_test():
+    """The reference's only live test (tests/driver.py:28-31, :70-71): 10 steps with betas
+    (0.8, 0.88), lr 5e-3, wd 0.03 stay within atol 0.025 / rtol 1e-5 of torch.optim.AdamW."""
+    gen = torch.Generator().manual_seed(2020)
+    n = 5000
+    p0 = torch.randn(n, generator=gen) * 0.3
+    ref = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([ref], lr=5e-3, betas=(0.8, 0.88), eps=1e-8, weight_decay=0.03)
+    p = p0.numpy().copy()
+    m, v, sm, sv = _zero_state(n)
+    for step in range(1, 11):
+        g = torch.randn(n, generator=gen)
+        ref.grad = g.clone()
+        opt.step()
+        oc.step_quant(p, g.numpy(), m, v, sm, sv, step=step, **HP_DRIVER)
+        torch.testing.assert_close(torch.from_numpy(p), ref.detach(), atol=0.025, rtol=1e-5)
+    assert not np.array_equal(p, p0.numpy())
