@@ -11,9 +11,10 @@
  * status comes back as an int instead of a C++ exception.
  *
  * All device pointers are borrowed for the duration of the call; tensors are
- * updated in place; nothing is retained except an internal descriptor cache that
- * q4adamw_release() frees.  Calls are asynchronous with respect to the host: work
- * is enqueued on `stream` (a hipStream_t; NULL is the default stream).
+ * updated in place; nothing is retained: tensor descriptors travel in kernel
+ * arguments and the library allocates no device or pinned memory.  Calls are
+ * asynchronous with respect to the host: work is enqueued on `stream` (a
+ * hipStream_t; NULL is the default stream).
  *
  * Return value: 0 on success, negative for an argument error, positive for a
  * hipError_t raised by the runtime.  q4adamw_last_error() describes the last
@@ -41,13 +42,13 @@ extern "C" {
 /*
  * One quantized tensor.  Field order follows the tensor arguments of
  * fused_4bit (optim/cuda_fused_interface.cc:19-21).
- *   p             numel elements, fp32 or bf16, 16-byte aligned
- *   g             numel elements, fp32 or bf16, 16-byte aligned
+ *   p             numel elements, fp32 (16-byte aligned) or bf16 (8-byte aligned)
+ *   g             numel elements, fp32 (16-byte aligned) or bf16 (8-byte aligned)
  *   exp_avg       (numel+1)/2 bytes; byte i = code(2i) | code(2i+1) << 4
  *   exp_avg_sq    same layout
  *   exp_avg_scale ceil(numel/128) fp32 block scales of exp_avg
  *   exp_avg_sq_scale  same for exp_avg_sq
- * Code buffers must be 4-byte aligned.
+ * Code buffers must be 2-byte aligned, scale buffers 4-byte aligned.
  */
 typedef struct q4adamw_tensor {
   void *p;
@@ -82,9 +83,10 @@ int q4adamw_fused_4bit(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_av
                        float weight_decay, float eps, float step, void *stream);
 
 /*
- * The same step over many tensors in one launch.  All tensors share dtypes,
- * hyper-parameters and step.  `tensors` is a host array.  Replaces the reference's
- * per-parameter Python loop around fused_4bit (optim/fused_quantfour.py:171-292).
+ * The same step over many tensors: one launch per batch of up to 48 tensors.  All
+ * tensors share dtypes, hyper-parameters and step.  `tensors` is a host array that
+ * is read before the call returns.  Replaces the reference's per-parameter Python
+ * loop around fused_4bit (optim/fused_quantfour.py:171-292).
  */
 int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dtype,
                              int g_dtype, float beta1, float beta2, float lr,
@@ -100,7 +102,7 @@ int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *e
                                 float beta2, float lr, float weight_decay, float eps,
                                 float step, void *stream);
 
-/* Many non-quantized tensors in one launch (`tensors` is a host array). */
+/* Many non-quantized tensors, one launch per batch of up to 80 (`tensors` is a host array). */
 int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int count,
                                       int p_dtype, int g_dtype, float beta1, float beta2,
                                       float lr, float weight_decay, float eps, float step,
@@ -127,7 +129,8 @@ void q4adamw_tables(int which, float *qmap16, float *qmid15);
  */
 int q4adamw_mtable_entry(uint32_t index, uint32_t *out2);
 
-/* Frees the cached descriptor buffers of every device.  Safe to call twice. */
+/* Kept for callers that pair an init with a release: the library holds no device
+ * memory, so this does nothing and returns 0. */
 int q4adamw_release(void);
 
 /* Message for the last non-zero status returned on this thread ("" if none). */

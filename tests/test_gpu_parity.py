@@ -241,3 +241,46 @@ def test_unquantized_step_vs_oracle(cuda):
             ok, worst = p_close(dp[i].cpu().numpy(), rp[i], prev)
             assert ok, f"unquant params worst {worst}"
             rp[i][:] = dp[i].cpu().numpy()
+
+
+def test_replay_under_graph_capture(cuda):
+    """The library allocates nothing and only launches kernels, so a step can be captured
+    into a graph; replays (same step number, refreshed inputs) must equal eager launches."""
+    gen = torch.Generator().manual_seed(77)
+    sizes = [70001, 4097, 128 * 40]
+    ps = [torch.randn(n, generator=gen) * 0.02 for n in sizes]
+    eager = [DeviceTensor(p, cuda) for p in ps]
+    graphed = [DeviceTensor(p, cuda) for p in ps]
+    gbuf = [torch.zeros(n, device=cuda) for n in sizes]
+    args = (HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"], HP["eps"], 3)
+
+    def launch(ts, gs):
+        q4.fused_4bit_multi([x.p for x in ts], gs, [x.m for x in ts], [x.v for x in ts],
+                            [x.sm for x in ts], [x.sv for x in ts], *args)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(graphed, gbuf)                      # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for x, p in zip(graphed, ps):                  # undo the warm-up step
+        x.p.copy_(p.to(cuda)); x.m.zero_(); x.v.zero_(); x.sm.zero_(); x.sv.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch(graphed, gbuf)
+    for x, p in zip(graphed, ps):                  # capture does not execute, but be explicit
+        x.p.copy_(p.to(cuda)); x.m.zero_(); x.v.zero_(); x.sm.zero_(); x.sv.zero_()
+    for rep in range(4):
+        gs = [grads_config3(gen, n).to(cuda) for n in sizes]
+        for b, g in zip(gbuf, gs):
+            b.copy_(g)
+        say(f"[graph] replay {rep}")
+        graph.replay()
+        launch(eager, gs)
+        torch.cuda.synchronize()
+        for x, y in zip(graphed, eager):
+            assert torch.equal(x.m, y.m) and torch.equal(x.v, y.v)
+            assert torch.equal(x.sm.view(torch.int32), y.sm.view(torch.int32))
+            assert torch.equal(x.sv.view(torch.int32), y.sv.view(torch.int32))
+            assert torch.equal(x.p.view(torch.int32), y.p.view(torch.int32))
