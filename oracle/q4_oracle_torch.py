@@ -17,6 +17,11 @@ midpoint table, which returns the same code for every non-NaN input.
 
 Every torch op below rounds once to fp32; none of them takes an ``alpha``/``value``
 multiplier, so no fused multiply-add hides in the update.
+
+The functions follow the device of their inputs.  On the CPU this is the timed
+baseline and the second restatement; on a GPU (plain torch element-wise kernels,
+nothing of this build's HIP code) it serves as the checker at sizes the CPU cannot
+finish in seconds, after the same test has checked it against the C oracle.
 """
 import math
 
@@ -69,7 +74,7 @@ def pack(q, numel):
 def dequantize(codes, scale, numel, which):
     """pass 1: materialise an fp32 moment (adamw_fourbit_triton.py:423-450)."""
     idx = unpack(codes, numel)
-    vals = QMAP[which][idx]
+    vals = QMAP[which].to(codes.device)[idx]
     s = scale.repeat_interleave(BLOCK)[:numel]
     return vals * s
 
@@ -78,23 +83,27 @@ def quantize(x, which):
     """pass 3: group abs-max, divide, nearest code, pack."""
     numel = x.numel()
     nblk = (numel + BLOCK - 1) // BLOCK
-    padded = torch.zeros(nblk * BLOCK, dtype=torch.float32)
+    padded = torch.zeros(nblk * BLOCK, dtype=torch.float32, device=x.device)
     padded[:numel] = x
     grouped = padded.view(nblk, BLOCK)
     max1 = grouped.abs().amax(dim=1, keepdim=True)          # :623-624, :1078-1087
     qx = grouped.div(max1)                                   # :625 (0/0 -> NaN)
     # number of midpoints strictly below x; NaN must land on 0
-    q = torch.bucketize(torch.nan_to_num(qx, nan=-2.0), QMID[which], right=False)
+    q = torch.bucketize(torch.nan_to_num(qx, nan=-2.0), QMID[which].to(x.device), right=False)
     return pack(q.reshape(-1)[:numel], numel), max1.reshape(-1)
 
 
 def adamw_update(p, g, m, v, sc, eps):
     """pass 2: cuda_adamw_kernels.cu:334-351 with separate, individually rounded ops."""
+    sc = {k: t.to(p.device) for k, t in sc.items()}
     m_new = sc["b1"] * m + sc["r1"] * g
     v_new = sc["b2"] * v + sc["r2"] * (g * g)
-    # torch.sqrt on CPU fp32 is not correctly rounded in every lane; numpy's is
-    root = torch.from_numpy(np.sqrt(v_new.numpy()))
-    denom = root / sc["c2s"] + torch.tensor(eps, dtype=torch.float32)
+    if v_new.is_cuda:
+        root = torch.sqrt(v_new)        # feeds only the parameters (tolerance class)
+    else:
+        # torch.sqrt on CPU fp32 is not correctly rounded in every lane; numpy's is
+        root = torch.from_numpy(np.sqrt(v_new.numpy()))
+    denom = root / sc["c2s"] + torch.tensor(eps, dtype=torch.float32, device=p.device)
     p_new = p * sc["wdu"] - sc["ss"] * (m_new / denom)
     return p_new, m_new, v_new
 

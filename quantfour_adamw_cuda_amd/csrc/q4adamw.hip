@@ -35,10 +35,7 @@
 namespace q4 {
 
 constexpr int kTile = 256;                 // elements per wave
-#ifndef Q4_WAVES
-#define Q4_WAVES 4
-#endif
-constexpr int kWaves = Q4_WAVES;           // waves per workgroup
+constexpr int kWaves = 4;                  // waves per workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kChunk = kTile * kWaves;     // elements per workgroup
 constexpr int kMaxTensors = 48;            // tensors per fused launch
@@ -374,9 +371,7 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     sm_old = as_global<const float>(sm_tile)[half];
     sv_old = as_global<const float>(sv_tile)[half];
   }
-#ifndef Q4_EARLY_BARRIER
   setup_tables(lds, tid, slot);
-#endif
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
   F4 mn, vn;
@@ -482,15 +477,10 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
   const int64_t begin = tile * kTile;
-#ifdef Q4_EARLY_BARRIER
-  setup_tables(lds, tid, slot);
-  if (begin >= T.numel) return;
-#else
   if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
     setup_tables(lds, tid, slot);
     return;
   }
-#endif
   if (begin + kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, tid, args.sc, lds, slot);
   else process_tile<PBF, GBF, false>(T, tile, lane, tid, args.sc, lds, slot);
 }

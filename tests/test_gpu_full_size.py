@@ -1,0 +1,162 @@
+"""Full-size checks of BASELINE configs[3] (Llama-3-8B: fp32 params, bf16 grads) and
+configs[4] (Llama-2-13B-shaped: bf16 params and grads): every tensor of the whole parameter
+set, every step, against the vectorised oracle run with plain torch ops on the GPU -- after
+that GPU run of the oracle has itself been checked against the C oracle -- plus format
+properties that hold at any size."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import q4_oracle as oc
+from oracle import q4_oracle_torch as ot
+from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+from tests.q4_testlib import HP, bits, to_np
+
+pytestmark = pytest.mark.gpu
+KW = dict(lr=HP["lr"], betas=(HP["beta1"], HP["beta2"]), eps=HP["eps"], weight_decay=HP["weight_decay"])
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def student_t(shape, gen, device, scale=1e-4):
+    z = torch.randn(shape, generator=gen, device=device)
+    c = torch.zeros(shape, device=device)
+    for _ in range(3):
+        c += torch.randn(shape, generator=gen, device=device).square_()
+    return (z * torch.rsqrt(c / 3.0) * scale).to(torch.bfloat16)
+
+
+def test_gpu_run_of_the_torch_oracle_matches_the_c_oracle(cuda):
+    """The checker used below: torch element-wise ops on the GPU must give the C oracle's
+    bits (IEEE division and individually rounded multiplies and adds on the device)."""
+    gen = torch.Generator().manual_seed(3)
+    n = 3 * 1000003
+    p = torch.randn(n, generator=gen) * 0.02
+    nb, nk = oc.state_sizes(n)
+    m, v = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8)
+    sm, sv = np.zeros(nk, np.float32), np.zeros(nk, np.float32)
+    pc = p.numpy().copy()
+    dp = p.to(cuda)
+    dm, dv, dsm, dsv = (torch.from_numpy(x.copy()).to(cuda) for x in (m, v, sm, sv))
+    for step in range(1, 4):
+        z = torch.randn(n, generator=gen)
+        g = (z / (torch.randn(3, n, generator=gen).square().sum(0) / 3).sqrt() * 1e-4).to(torch.bfloat16)
+        if step == 2:
+            g[1000:3000] = 0
+        oc.step_quant(pc, to_np(g), m, v, sm, sv, step=step, **HP)
+        dp, dm, dv, dsm, dsv = ot.step_quant(dp, g.to(cuda), dm, dv, dsm, dsv, step=step, **HP)
+        assert np.array_equal(dm.cpu().numpy(), m) and np.array_equal(dv.cpu().numpy(), v)
+        assert np.array_equal(bits(dsm.cpu().numpy()), bits(sm)) and np.array_equal(bits(dsv.cpu().numpy()), bits(sv))
+        assert np.allclose(dp.cpu().numpy(), pc, rtol=1e-6, atol=1e-9)
+        dp = torch.from_numpy(pc.copy()).to(cuda)
+
+
+def llama3_8b_shapes():
+    shapes = [(128256, 4096), (128256, 4096)]
+    for _ in range(32):
+        shapes += [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096),
+                   (4096, 14336), (4096,), (4096,)]
+    return shapes + [(4096,)]
+
+
+def llama2_13b_shapes():
+    shapes = [(32000, 5120), (32000, 5120)]
+    for _ in range(40):
+        shapes += [(5120, 5120)] * 4 + [(13824, 5120), (13824, 5120), (5120, 13824), (5120,), (5120,)]
+    return shapes
+
+
+def _check_tensor(p, st, before, g, step):
+    """One tensor after a step against the oracle applied to its state before the step."""
+    p0, m0, v0, sm0, sv0 = before
+    if st["momentum_qstate"]["enable"]:
+        rp, rm, rv, rsm, rsv = ot.step_quant(p0.reshape(-1), g.reshape(-1), m0, v0, sm0, sv0, step=step, **HP)
+        assert torch.equal(st["exp_avg"], rm), f"first-moment codes, shape {tuple(p.shape)}"
+        assert torch.equal(st["exp_avg_sq"], rv), f"second-moment codes, shape {tuple(p.shape)}"
+        assert torch.equal(st["momentum_qstate"]["overhead"]["max1"].view(torch.int32), rsm.view(torch.int32))
+        assert torch.equal(st["variance_qstate"]["overhead"]["max1"].view(torch.int32), rsv.view(torch.int32))
+        # format properties: a non-zero block holds code 15 (second moment) resp. 15 or 0
+        # (first moment) where its abs-max sits, an all-zero block holds only zero codes
+        n = p.numel()
+        if n % 256 == 0:
+            vcodes = torch.maximum(st["exp_avg_sq"] & 15, st["exp_avg_sq"] >> 4).view(-1, 64).amax(1)
+            sv = st["variance_qstate"]["overhead"]["max1"]
+            assert torch.equal(vcodes == 15, sv > 0) and bool((vcodes[sv == 0] == 0).all())
+    else:
+        rp, rm, rv = ot.step_unquant(p0, g, m0, v0, step=step, **HP)
+        assert torch.equal(st["exp_avg"].reshape(-1).view(torch.int32), rm.view(torch.int32))
+        assert torch.equal(st["exp_avg_sq"].reshape(-1).view(torch.int32), rv.view(torch.int32))
+    if p.dtype == torch.bfloat16:
+        d = (p.detach().reshape(-1).float() - rp.reshape(-1).float()).abs()
+        scale = torch.maximum(rp.reshape(-1).float().abs(), (rp.reshape(-1).float() - p0.reshape(-1).float()).abs())
+        ulp = torch.exp2(torch.floor(torch.log2(scale.clamp_min(1e-30))) - 7)
+        assert bool((d <= ulp).all()), f"bf16 params, shape {tuple(p.shape)}"
+    else:
+        d = (p.detach().reshape(-1).double() - rp.reshape(-1).double()).abs()
+        scale = torch.maximum(rp.reshape(-1).abs(), (rp.reshape(-1) - p0.reshape(-1)).abs()).double()
+        assert bool((d <= 1e-6 * scale.clamp_min(1e-30)).all()), f"params, shape {tuple(p.shape)}"
+
+
+def _run_config(shapes, p_dtype, cuda, steps, label):
+    gen = torch.Generator(device=cuda).manual_seed(0)
+    params = []
+    for s in shapes:
+        p = nn.Parameter((torch.randn(s, generator=gen, device=cuda) * 0.02).to(p_dtype))
+        if p_dtype != torch.bfloat16:
+            p.grad_dtype = torch.bfloat16
+        params.append(p)
+    total = sum(p.numel() for p in params)
+    opt = AdamWFused_QuantFour(params, **KW)
+    for step in range(1, steps + 1):
+        grads = [student_t(s, gen, cuda) for s in shapes]
+        if step == 2:
+            grads[0][5000:6000] = 0       # embedding rows without gradient: all-zero blocks
+        before = []
+        for p in params:
+            st = opt.state.get(p, {})
+            if st:
+                if st["momentum_qstate"]["enable"]:
+                    before.append((p.detach().clone(), st["exp_avg"].clone(), st["exp_avg_sq"].clone(),
+                                   st["momentum_qstate"]["overhead"]["max1"].clone(),
+                                   st["variance_qstate"]["overhead"]["max1"].clone()))
+                else:
+                    before.append((p.detach().clone(), st["exp_avg"].clone(), st["exp_avg_sq"].clone(), None, None))
+            else:
+                n = p.numel()
+                if n > 4096:
+                    nb, nk = oc.state_sizes(n)
+                    before.append((p.detach().clone(), torch.zeros(nb, dtype=torch.uint8, device=cuda),
+                                   torch.zeros(nb, dtype=torch.uint8, device=cuda),
+                                   torch.zeros(nk, device=cuda), torch.zeros(nk, device=cuda)))
+                else:
+                    before.append((p.detach().clone(), torch.zeros(n, device=cuda), torch.zeros(n, device=cuda), None, None))
+        for p, g in zip(params, grads):
+            p.grad = g
+        say(f"[{label}] step {step}: {len(params)} tensors, {total / 1e9:.2f} G params")
+        opt.step()
+        torch.cuda.synchronize()
+        for i, (p, g) in enumerate(zip(params, grads)):
+            _check_tensor(p, opt.state[p], before[i], g, step)
+            before[i] = None
+        say(f"[{label}] step {step}: all tensors match the oracle")
+        del before, grads
+    return total
+
+
+def test_llama3_8b_full_parameter_set(cuda):
+    shapes = llama3_8b_shapes()
+    assert len(shapes) == 291
+    total = _run_config(shapes, torch.float32, cuda, 3, "llama3-8b fp32/bf16")
+    assert total == 8030261248
+    torch.cuda.empty_cache()
+
+
+def test_llama2_13b_shaped_parameter_set_bf16(cuda):
+    shapes = llama2_13b_shapes()
+    assert len(shapes) == 362
+    total = _run_config(shapes, torch.bfloat16, cuda, 3, "llama2-13b bf16/bf16")
+    assert 13.0e9 < total < 13.1e9
+    torch.cuda.empty_cache()
