@@ -109,6 +109,26 @@ int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int c
                                       void *stream);
 
 /*
+ * Quantize one fp32 moment: per block of 128 consecutive elements the scale is the
+ * abs-max, every element is divided by it and mapped to the nearest code (ties go
+ * down), codes are packed two per byte.  which: 0 first moment (signed map),
+ * 1 second moment (unsigned map).  codes: (numel+1)/2 bytes, scales: ceil(numel/128).
+ * The device form of momentum_quant / variance_quant with per-block scaling
+ * (optim/adamw_fourbit_triton.py:556-588, :618-630) and of q_mapping
+ * (optim/cuda_adamw_kernels.cu:167-194); used to take over fp32 AdamW state.
+ */
+int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, float *scales,
+                     void *stream);
+
+/*
+ * Inverse layout step: out[i] = code_book[code(i)] * scales[i / 128], fp32.  The
+ * device form of the dequantize pass (optim/cuda_adamw_kernels.cu:329-343,
+ * optim/adamw_fourbit_triton.py:423-450); used to hand state back as fp32.
+ */
+int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel, int which,
+                       float *out, void *stream);
+
+/*
  * Host-only: the six fp32 scalars the launcher derives from the hyper-parameters
  * (optim/cuda_adamw_kernels.cu:435-440), in that order: correction1,
  * correction2_sqrt, step_size, weight_decay_update, resid_beta1, resid_beta2.

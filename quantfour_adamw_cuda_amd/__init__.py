@@ -7,8 +7,8 @@
 The step runs in csrc/libq4adamw.so (build: python -m quantfour_adamw_cuda_amd.build).
 """
 from .fused_quantfour import AdamWFused_QuantFour, enable_param_quantization
-from .quantfour_hip import (fused_4bit, fused_4bit_multi, fused_single_tensor,
-                            fused_single_tensor_multi, state_sizes)
+from .quantfour_hip import (dequantize_state, fused_4bit, fused_4bit_multi, fused_single_tensor,
+                            fused_single_tensor_multi, quantize_state, state_sizes)
 
 __all__ = [
     "AdamWFused_QuantFour",
@@ -18,4 +18,6 @@ __all__ = [
     "fused_single_tensor",
     "fused_single_tensor_multi",
     "state_sizes",
+    "quantize_state",
+    "dequantize_state",
 ]

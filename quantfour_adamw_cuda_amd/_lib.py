@@ -42,6 +42,8 @@ EXPORTS = (
     "q4adamw_fused_4bit_multi",
     "q4adamw_fused_single_tensor",
     "q4adamw_fused_single_tensor_multi",
+    "q4adamw_quantize",
+    "q4adamw_dequantize",
     "q4adamw_derive_scalars",
     "q4adamw_tables",
     "q4adamw_mtable_entry",
@@ -73,6 +75,10 @@ def load():
     L.q4adamw_fused_single_tensor.restype = i
     L.q4adamw_fused_single_tensor_multi.argtypes = [ctypes.POINTER(Q4SmallTensor), i, i, i] + hyper + [vp]
     L.q4adamw_fused_single_tensor_multi.restype = i
+    L.q4adamw_quantize.argtypes = [vp, i64, i, vp, vp, vp]
+    L.q4adamw_quantize.restype = i
+    L.q4adamw_dequantize.argtypes = [vp, vp, i64, i, vp, vp]
+    L.q4adamw_dequantize.restype = i
     L.q4adamw_derive_scalars.argtypes = [f, f, f, f, f, ctypes.POINTER(f)]
     L.q4adamw_derive_scalars.restype = None
     L.q4adamw_tables.argtypes = [i, ctypes.POINTER(f), ctypes.POINTER(f)]

@@ -99,6 +99,11 @@ static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096, "kernel ar
 // bucket table entries that hold a threshold and the two code books (see
 // q4adamw_tables.h), read by every workgroup at start-up
 __device__ const WorkgroupTables kWorkgroupTables = make_workgroup_tables();
+// first-moment code book for kernels that index it per lane
+__device__ const uint32_t kQmapMDev[16] = {
+    0xbf633333u, 0xbf29999au, 0xbee00000u, 0xbe59999au, 0xbd9eb852u, 0xbd051eb8u,
+    0xbbb43958u, 0x00000000u, 0x3bb43958u, 0x3d051eb8u, 0x3d9eb852u, 0x3e59999au,
+    0x3ee00000u, 0x3f29999au, 0x3f633333u, 0x3f800000u};
 
 // ---------------------------------------------------------------------------
 // device helpers
@@ -512,6 +517,64 @@ __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// stand-alone quantize / dequantize of one moment (checkpoint interchange)
+// ---------------------------------------------------------------------------
+// One wave per 128-element block, two elements (one packed byte) per lane.  These run
+// once per checkpoint, so they take the exact route only: IEEE division and the
+// 15-compare count (optim/adamw_fourbit_triton.py:618-630, cuda_adamw_kernels.cu:167-194).
+template <bool SECOND>
+__global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__ x_, int64_t numel,
+                                                       uint8_t *__restrict__ codes_,
+                                                       float *__restrict__ scale_) {
+  const gptr<const float> x = as_global<const float>(x_);
+  const int lane = threadIdx.x & 63;
+  const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t nblk = (numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
+  if (blk >= nblk) return;
+  const int64_t e = blk * Q4ADAMW_BLOCK + lane * 2;
+  const float a = e < numel ? x[e] : 0.0f;
+  const float b = e + 1 < numel ? x[e + 1] : 0.0f;
+  uint32_t u = f2bits(__builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b)));
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)u, off, 64);
+    u = u > o ? u : o;
+  }
+  const float s = bits2f(u);
+  if (lane == 0) as_global<float>(scale_)[blk] = s;
+  if (e < numel) {
+    uint32_t byte = 0;
+    const float q0 = a / s, q1 = b / s;
+#pragma unroll
+    for (int k = 0; k < 15; ++k) {
+      const float t = SECOND ? qmid_v(k) : bits2f(kQmidMBits[k]);
+      byte += (t < q0) ? 1u : 0u;
+      byte += (e + 1 < numel && t < q1) ? 16u : 0u;
+    }
+    as_global<uint8_t>(codes_)[e >> 1] = (uint8_t)byte;
+  }
+}
+
+// cuda_adamw_kernels.cu:329-343: code -> code-book entry * block scale
+template <bool SECOND>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t *__restrict__ codes_,
+                                                         const float *__restrict__ scale_,
+                                                         int64_t numel, float *__restrict__ out_) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (e >= numel) return;
+  const uint32_t byte = as_global<const uint8_t>(codes_)[e >> 1];
+  const float s = as_global<const float>(scale_)[e / Q4ADAMW_BLOCK];
+  const uint32_t c0 = byte & 15u, c1 = byte >> 4;
+  const float v0 = (SECOND ? qmap_v((int)c0) : bits2f(kQmapMDev[c0])) * s;
+  as_global<float>(out_)[e] = v0;
+  if (e + 1 < numel) {
+    const float v1 = (SECOND ? qmap_v((int)c1) : bits2f(kQmapMDev[c1])) * s;
+    as_global<float>(out_)[e + 1] = v1;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -761,10 +824,41 @@ int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *e
                                            weight_decay, eps, step, stream);
 }
 
+int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, float *scales,
+                     void *stream) {
+  if (numel < 0 || (which != 0 && which != 1)) return fail(Q4ADAMW_ERR_ARG, "bad numel or moment selector");
+  if (numel == 0) return 0;
+  if (!x || !codes || !scales) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+  if (!aligned(x, 4) || !aligned(scales, 4)) return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
+  const uint64_t blocks = (uint64_t)(numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
+  const uint64_t grid = (blocks + 3) / 4;
+  if (grid > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (which) hipLaunchKernelGGL(quantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, x, numel, codes, scales);
+  else hipLaunchKernelGGL(quantize_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, x, numel, codes, scales);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
+int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel, int which,
+                       float *out, void *stream) {
+  if (numel < 0 || (which != 0 && which != 1)) return fail(Q4ADAMW_ERR_ARG, "bad numel or moment selector");
+  if (numel == 0) return 0;
+  if (!out || !codes || !scales) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+  if (!aligned(out, 4) || !aligned(scales, 4)) return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
+  const uint64_t grid = ((uint64_t)(numel + 1) / 2 + 255) / 256;
+  if (grid > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (which) hipLaunchKernelGGL(dequantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, codes, scales, numel, out);
+  else hipLaunchKernelGGL(dequantize_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, codes, scales, numel, out);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1001; }
+int q4adamw_version(void) { return 1002; }
 
 }  // extern "C"

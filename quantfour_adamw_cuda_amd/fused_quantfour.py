@@ -160,6 +160,10 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             momentum_quant_enabled.append(state["momentum_qstate"]["enable"])
 
     def load_state_dict(self, state_dict):
+        """Accepts this optimizer's own state_dict and, as a migration path, the state_dict
+        of torch.optim.AdamW (fp32 `exp_avg` / `exp_avg_sq` shaped like the parameter):
+        moments of tensors above the quantization threshold are quantized on load
+        (per-128 abs-max scaling, nearest code), the others are kept in fp32."""
         super().load_state_dict(state_dict)
         # The base class casts every state tensor to the parameter's dtype.  Packed codes
         # are uint8, block scales and non-quantized moments fp32, whatever the parameter
@@ -179,7 +183,59 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 if torch.is_tensor(max1):
                     dst[key]["overhead"]["max1"] = max1.detach().to(
                         device=p.device, dtype=torch.float32, copy=True)
+            if "momentum_qstate" not in src:
+                self._adopt_adamw_state(p, dst)
         self._launch_cache = {}
+
+    def _adopt_adamw_state(self, p, state):
+        """Turns one parameter's torch.optim.AdamW state (step, exp_avg, exp_avg_sq in the
+        parameter's shape) into this optimizer's layout (optim/fused_quantfour.py:65-70,
+        :112-119, :199-204)."""
+        if "max_exp_avg_sq" in state:
+            raise ValueError("amsgrad state (max_exp_avg_sq) cannot be taken over")
+        if not torch.is_tensor(state["step"]):
+            state["step"] = torch.tensor(float(state["step"]))
+        state["step"] = state["step"].detach().to(device="cpu", dtype=torch.float32).reshape(())
+        exp_avg = state["exp_avg"].detach().to(device=p.device, dtype=torch.float32)
+        exp_avg_sq = state["exp_avg_sq"].detach().to(device=p.device, dtype=torch.float32)
+        if exp_avg.numel() != p.numel() or exp_avg_sq.numel() != p.numel():
+            raise ValueError("AdamW state does not match the parameter's size")
+        self.init_qstate(p, "momentum")
+        self.init_qstate(p, "variance")
+        if state["momentum_qstate"]["enable"]:
+            state["exp_avg"], state["momentum_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg, 0)
+            state["exp_avg_sq"], state["variance_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg_sq, 1)
+        else:
+            state["exp_avg"] = exp_avg.contiguous().clone()
+            state["exp_avg_sq"] = exp_avg_sq.contiguous().clone()
+
+    def adamw_state_dict(self):
+        """This optimizer's state in the layout of torch.optim.AdamW: fp32 moments shaped
+        like their parameter (quantized moments are dequantized: code-book entry times
+        block scale).  `torch.optim.AdamW(params).load_state_dict(opt.adamw_state_dict())`
+        continues training in full precision."""
+        sd = self.state_dict()
+        own = list(chain.from_iterable(g["params"] for g in self.param_groups))
+        ids = list(chain.from_iterable(g["params"] for g in sd["param_groups"]))
+        out_state = {}
+        for pid, p in zip(ids, own):
+            st = self.state.get(p)
+            if not st:
+                continue
+            if st["momentum_qstate"]["enable"]:
+                m = _q.dequantize_state(st["exp_avg"], st["momentum_qstate"]["overhead"]["max1"], p.numel(), 0)
+                v = _q.dequantize_state(st["exp_avg_sq"], st["variance_qstate"]["overhead"]["max1"], p.numel(), 1)
+            else:
+                m, v = st["exp_avg"].clone(), st["exp_avg_sq"].clone()
+            out_state[pid] = {"step": st["step"].detach().clone(),
+                              "exp_avg": m.view(p.shape), "exp_avg_sq": v.view(p.shape)}
+        groups = []
+        for g in sd["param_groups"]:
+            groups.append({"lr": g["lr"], "betas": g["betas"], "eps": g["eps"],
+                           "weight_decay": g["weight_decay"], "amsgrad": False, "maximize": False,
+                           "foreach": None, "capturable": False, "differentiable": False,
+                           "fused": None, "params": list(g["params"])})
+        return {"state": out_state, "param_groups": groups}
 
     # -- step -------------------------------------------------------------
     @torch.no_grad()

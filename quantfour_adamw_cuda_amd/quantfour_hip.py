@@ -150,3 +150,36 @@ def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, w
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
     launch_small_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step)
+
+
+def quantize_state(x, which):
+    """fp32 moment (any shape, on a GPU) -> (packed uint8 codes, fp32 block scales).
+    which: 0 first moment, 1 second moment.  Device form of momentum_quant /
+    variance_quant with per-block scaling (optim/adamw_fourbit_triton.py:556-630)."""
+    L = _lib.load()
+    assert x.is_cuda, "state must be on cuda"
+    x = x.detach().to(torch.float32).contiguous().reshape(-1)
+    nbytes, nblk = state_sizes(x.numel())
+    codes = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(nblk, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.q4adamw_quantize(x.data_ptr(), x.numel(), int(which), codes.data_ptr(),
+                                scales.data_ptr(), _stream(x.device))
+    _lib.check(rc, "quantize")
+    return codes, scales
+
+
+def dequantize_state(codes, scales, numel, which):
+    """(packed codes, block scales) -> flat fp32 moment of numel elements
+    (optim/cuda_adamw_kernels.cu:329-343)."""
+    L = _lib.load()
+    assert codes.is_cuda and scales.device == codes.device, "state must be on cuda"
+    nbytes, nblk = state_sizes(numel)
+    assert codes.dtype == torch.uint8 and codes.numel() == nbytes and codes.is_contiguous()
+    assert scales.dtype == torch.float32 and scales.numel() == nblk and scales.is_contiguous()
+    out = torch.empty(numel, dtype=torch.float32, device=codes.device)
+    with torch.cuda.device(codes.device):
+        rc = L.q4adamw_dequantize(codes.data_ptr(), scales.data_ptr(), numel, int(which),
+                                  out.data_ptr(), _stream(codes.device))
+    _lib.check(rc, "dequantize")
+    return out
