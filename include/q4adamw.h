@@ -42,13 +42,15 @@ extern "C" {
 /*
  * One quantized tensor.  Field order follows the tensor arguments of
  * fused_4bit (optim/cuda_fused_interface.cc:19-21).
- *   p             numel elements, fp32 (16-byte aligned) or bf16 (8-byte aligned)
- *   g             numel elements, fp32 (16-byte aligned) or bf16 (8-byte aligned)
+ *   p             numel elements, fp32 or bf16, 16-byte aligned
+ *   g             numel elements, fp32 or bf16, 16-byte aligned (8 bytes suffice for a
+ *                 bf16 gradient of an fp32 parameter)
  *   exp_avg       (numel+1)/2 bytes; byte i = code(2i) | code(2i+1) << 4
  *   exp_avg_sq    same layout
  *   exp_avg_scale ceil(numel/128) fp32 block scales of exp_avg
  *   exp_avg_sq_scale  same for exp_avg_sq
- * Code buffers must be 2-byte aligned, scale buffers 4-byte aligned.
+ * Code and scale buffers must be 4-byte aligned (2 bytes suffice for the codes of an
+ * fp32 parameter).
  */
 typedef struct q4adamw_tensor {
   void *p;

@@ -8,11 +8,13 @@
 // Work decomposition of the fused kernel (shaped by measurement: HBM on this part
 // streams best when every wave is short-lived, touches 1 KiB of the widest stream
 // with ONE 16-byte access per lane, and every access is marked non-temporal)
-//   tile    = 256 consecutive elements = 2 quantization blocks = one wave64, one
-//             pass: lane l owns elements [4l, 4l+4).  A block is 32 lanes: its
-//             abs-max is one v_permlane16_swap plus four DPP row steps, no LDS
-//             traffic and no barrier.
-//   chunk   = 4 tiles (1024 elements) of ONE tensor = one 256-thread workgroup.
+//   tile    = one wave64, one pass; a lane owns 16 bytes of the parameter stream:
+//             4 consecutive fp32 parameters (tile = 256 elements = 2 quantization
+//             blocks, a block = 32 lanes, abs-max by one v_permlane16_swap plus four
+//             DPP row steps) or 8 consecutive bf16 parameters (tile = 512 elements =
+//             4 blocks, a block = one 16-lane DPP row).  No LDS traffic and no
+//             barrier in the reduction.
+//   chunk   = 4 tiles of ONE tensor = one 256-thread workgroup.
 //   launch  = all chunks of up to kMaxTensors tensors.  The tensor descriptors and
 //             the per-tensor first-chunk prefix travel in the kernel arguments, so
 //             a workgroup finds its tensor with two scalar loads from the kernarg
@@ -34,10 +36,8 @@
 
 namespace q4 {
 
-constexpr int kTile = 256;                 // elements per wave
 constexpr int kWaves = 4;                  // waves per workgroup
 constexpr int kThreads = kWaves * 64;
-constexpr int kChunk = kTile * kWaves;     // elements per workgroup
 constexpr int kMaxTensors = 48;            // tensors per fused launch
 constexpr int kSmallChunk = 1024;          // elements per workgroup, non-quantized kernel
 constexpr int kMaxSmallTensors = 80;
@@ -158,27 +158,51 @@ __device__ __forceinline__ void block_max32_pair(float &am, float &av) {
   av = bits2f(s2[1]);
 }
 
+// Max of a non-negative float over the 16 lanes of a DPP row, result in every lane.
+__device__ __forceinline__ float row_max16(float x) {
+  uint32_t u = f2bits(x);
+  u = dpp_umax<0xB1>(u);
+  u = dpp_umax<0x4E>(u);
+  u = dpp_umax<0x141>(u);
+  u = dpp_umax<0x140>(u);
+  return bits2f(u);
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return bits2f(h << 16); }
 
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nearest even
   return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
-// four consecutive elements starting at element e0 (a multiple of 4) of the tile at base
-template <bool BF, bool FULL>
-__device__ __forceinline__ void load4(const void *base, uint32_t e0, int nv, float (&x)[4]) {
+__device__ __forceinline__ void widen_bf16_pair(uint32_t w, float &lo, float &hi) {
+  lo = bits2f(w << 16);
+  hi = bits2f(w & 0xffff0000u);
+}
+
+// N consecutive elements (N = 4 or 8) starting at element e0 of the tile at base
+template <bool BF, int N, bool FULL>
+__device__ __forceinline__ void load_elems(const void *base, uint32_t e0, int nv, float (&x)[N]) {
   if (FULL) {
-    if (BF) {
+    if (BF && N == 4) {
       const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(tile_rsrc(base), e0 * 2, 0, kNt);
-      x[0] = bits2f(w.x << 16); x[1] = bits2f(w.x & 0xffff0000u);
-      x[2] = bits2f(w.y << 16); x[3] = bits2f(w.y & 0xffff0000u);
+      widen_bf16_pair(w.x, x[0], x[1]);
+      widen_bf16_pair(w.y, x[2], x[3]);
+    } else if (BF) {
+      const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), e0 * 2, 0, kNt);
+      widen_bf16_pair(w.x, x[0], x[1]);
+      widen_bf16_pair(w.y, x[2], x[3]);
+      widen_bf16_pair(w.z, x[N - 4], x[N - 3]);
+      widen_bf16_pair(w.w, x[N - 2], x[N - 1]);
     } else {
-      const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), e0 * 4, 0, kNt);
-      x[0] = bits2f(a.x); x[1] = bits2f(a.y); x[2] = bits2f(a.z); x[3] = bits2f(a.w);
+#pragma unroll
+      for (int k = 0; k < N; k += 4) {
+        const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), (e0 + k) * 4, 0, kNt);
+        x[k] = bits2f(a.x); x[k + 1] = bits2f(a.y); x[k + 2] = bits2f(a.z); x[k + 3] = bits2f(a.w);
+      }
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < N; ++j) {
       x[j] = 0.0f;
       if (j < nv) {
         x[j] = BF ? bf16_bits_to_f32(as_global<const uint16_t>(base)[e0 + j])
@@ -188,21 +212,31 @@ __device__ __forceinline__ void load4(const void *base, uint32_t e0, int nv, flo
   }
 }
 
-template <bool BF, bool FULL>
-__device__ __forceinline__ void store4(void *base, uint32_t e0, int nv, const float (&x)[4]) {
+template <bool BF, int N, bool FULL>
+__device__ __forceinline__ void store_elems(void *base, uint32_t e0, int nv, const float (&x)[N]) {
   if (FULL) {
-    if (BF) {
+    if (BF && N == 4) {
       u32x2 w;
       w.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
       w.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
       __builtin_amdgcn_raw_buffer_store_b64(w, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else if (BF) {
+      u32x4 w;
+      w.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
+      w.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
+      w.z = f32_to_bf16_bits(x[N - 4]) | (f32_to_bf16_bits(x[N - 3]) << 16);
+      w.w = f32_to_bf16_bits(x[N - 2]) | (f32_to_bf16_bits(x[N - 1]) << 16);
+      __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), e0 * 2, 0, kNt);
     } else {
-      const u32x4 w = {f2bits(x[0]), f2bits(x[1]), f2bits(x[2]), f2bits(x[3])};
-      __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), e0 * 4, 0, kNt);
+#pragma unroll
+      for (int k = 0; k < N; k += 4) {
+        const u32x4 w = {f2bits(x[k]), f2bits(x[k + 1]), f2bits(x[k + 2]), f2bits(x[k + 3])};
+        __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), (e0 + k) * 4, 0, kNt);
+      }
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < N; ++j) {
       if (j < nv) {
         if (BF) as_global<uint16_t>(base)[e0 + j] = (uint16_t)f32_to_bf16_bits(x[j]);
         else as_global<float>(base)[e0 + j] = x[j];
@@ -211,18 +245,19 @@ __device__ __forceinline__ void store4(void *base, uint32_t e0, int nv, const fl
   }
 }
 
-struct F4 {
-  float x[4];
+template <int N>
+struct Vals {
+  float x[N];
 };
 
-// Exact quantization of four values of one state: IEEE division by the block
-// scale, then the number of thresholds strictly below the quotient
+// Exact quantization of N values of one state: IEEE division by the block scale,
+// then the number of thresholds strictly below the quotient
 // (cuda_adamw_kernels.cu:167-194 in closed form).  0/0 is NaN and gets code 0.
-template <bool SECOND>
-__device__ __forceinline__ uint32_t quantize4_exact(const F4 &v, float scale) {
+template <bool SECOND, int N>
+__device__ __forceinline__ uint32_t quantize_exact(const Vals<N> &v, float scale) {
   uint32_t word = 0;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < N; ++j) {
     const float q = v.x[j] / scale;
     uint32_t c = 0;
 #pragma unroll
@@ -279,88 +314,97 @@ constexpr uint32_t kLdsQm = kMtabEntries;
 constexpr uint32_t kLdsQv = kMtabEntries + 16;
 constexpr uint32_t kLdsEntries = kMtabEntries + 32;
 
-// The slots of the workgroup tables that this thread copies into LDS, requested
-// from memory as the very first thing a wave does.
-constexpr int kSlotsPerThread = (128 + kThreads - 1) / kThreads;
+// This thread's slot of the workgroup tables, requested from memory as the very
+// first thing a wave does (only the first two waves hold slots).
 struct TableSlot {
-  uint32_t a[kSlotsPerThread], b[kSlotsPerThread];
+  uint32_t a, b;
 };
 
 __device__ __forceinline__ TableSlot request_table_slot(int tid) {
-  TableSlot s;
-#pragma unroll
-  for (int i = 0; i < kSlotsPerThread; ++i) {
-    const int slot = tid + i * kThreads;
-    s.a[i] = s.b[i] = 0u;
-    if (slot < 128) {
-      s.a[i] = kWorkgroupTables.a[slot];
-      s.b[i] = kWorkgroupTables.b[slot];
-    }
+  TableSlot s{0u, 0u};
+  if (tid < 128) {
+    s.a = kWorkgroupTables.a[tid];
+    s.b = kWorkgroupTables.b[tid];
   }
   return s;
 }
 
-// Writes the slots into LDS and waits for the whole workgroup.  Called by every
-// wave exactly once.  The fences order LDS only: a full __syncthreads() would also
-// drain outstanding global loads.
+// Writes the slot into LDS and waits for the whole workgroup.  Called by every wave
+// exactly once, after it has issued its global loads, so that the latencies overlap.
+// The fences order LDS only: a full __syncthreads() would also drain the outstanding
+// global loads.
 __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
-#pragma unroll
-  for (int i = 0; i < kSlotsPerThread; ++i) {
-    const int slot = tid + i * kThreads;
-    if (slot < 128) {
-      // slots 0..37 -> positive buckets, 38..75 -> negative buckets, 76..95 -> unused
-      // entries 0..19 (below every bucket that is read), 96..127 -> the code books
-      const int entry = slot + (slot < (int)kBucketsPerSign       ? (int)kBucketFloor
-                                : slot < (int)(2 * kBucketsPerSign) ? (int)(kNegativeBuckets + kBucketFloor - kBucketsPerSign)
-                                : slot < 96                          ? -76
-                                                                     : (int)kLdsQm - 96);
-      lds[entry] = make_uint2(s.a[i], s.b[i]);
-    }
+  if (tid < 128) {
+    // slots 0..37 -> positive buckets, 38..75 -> negative buckets, 76..95 -> unused
+    // entries 0..19 (below every bucket that is read), 96..127 -> the code books
+    const int entry = tid + (tid < (int)kBucketsPerSign       ? (int)kBucketFloor
+                             : tid < (int)(2 * kBucketsPerSign) ? (int)(kNegativeBuckets + kBucketFloor - kBucketsPerSign)
+                             : tid < 96                          ? -76
+                                                                 : (int)kLdsQm - 96);
+    lds[entry] = make_uint2(s.a, s.b);
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  if (kWaves > 1) __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Geometry of the fused kernel: a lane owns 16 bytes of the parameter stream.
+template <bool PBF>
+struct Geometry {
+  static constexpr int kEpl = PBF ? 8 : 4;               // elements per lane
+  static constexpr int kTile = 64 * kEpl;                // elements per wave
+  static constexpr int kChunk = kTile * kWaves;          // elements per workgroup
+  static constexpr int kLanesPerBlock = Q4ADAMW_BLOCK / kEpl;   // 32 or 16
+  static constexpr int kBlocksPerTile = kTile / Q4ADAMW_BLOCK;  // 2 or 4
+};
+
 // ---------------------------------------------------------------------------
-// one tile (256 elements) of one tensor
+// one tile (256 or 512 elements) of one tensor
 // ---------------------------------------------------------------------------
 template <bool PBF, bool GBF, bool FULL>
 __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot) {
+  using G = Geometry<PBF>;
+  constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
   // block; the per-lane part is a small 32-bit offset.
   const int64_t numel = T.numel;
-  const int64_t tb = tile * kTile;
+  const int64_t tb = tile * G::kTile;
   const void *p_tile = static_cast<const char *>(T.p) + tb * (PBF ? 2 : 4);
   const void *g_tile = static_cast<const char *>(T.g) + tb * (GBF ? 2 : 4);
   const uint8_t *m_tile = T.m + (tb >> 1);
   const uint8_t *v_tile = T.v + (tb >> 1);
-  const float *sm_tile = T.sm + tile * 2;
-  const float *sv_tile = T.sv + tile * 2;
-  const uint32_t e0 = (uint32_t)lane * 4u;   // first element of this lane within the tile
-  const uint32_t half = (uint32_t)lane >> 5;  // which of the tile's two blocks
-  int nv = 4;
+  const float *sm_tile = T.sm + tile * G::kBlocksPerTile;
+  const float *sv_tile = T.sv + tile * G::kBlocksPerTile;
+  const uint32_t e0 = (uint32_t)lane * N;                          // first element of this lane in the tile
+  const uint32_t blk = (uint32_t)lane / G::kLanesPerBlock;         // which of the tile's blocks
+  const uint32_t code_off = (uint32_t)lane * (N / 2);              // byte offset of this lane's codes
+  int nv = N;
   bool blk_ok = true;
   if (!FULL) {
     const int64_t rem = numel - tb - (int64_t)e0;
-    nv = rem >= 4 ? 4 : (rem > 0 ? (int)rem : 0);
-    blk_ok = tb + (int64_t)half * 128 < numel;
+    nv = rem >= N ? N : (rem > 0 ? (int)rem : 0);
+    blk_ok = tb + (int64_t)blk * Q4ADAMW_BLOCK < numel;
   }
 
-  float p[4], g[4];
-  load4<PBF, FULL>(p_tile, e0, nv, p);
-  load4<GBF, FULL>(g_tile, e0, nv, g);
+  float p[N], g[N];
+  load_elems<PBF, N, FULL>(p_tile, e0, nv, p);
+  load_elems<GBF, N, FULL>(g_tile, e0, nv, g);
   uint32_t mw = 0, vw = 0;
   if (FULL) {
-    mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), (uint32_t)lane * 2u, 0, kNt);
-    vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), (uint32_t)lane * 2u, 0, kNt);
+    if (N == 4) {
+      mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), code_off, 0, kNt);
+      vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), code_off, 0, kNt);
+    } else {
+      mw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(m_tile), code_off, 0, kNt);
+      vw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_tile), code_off, 0, kNt);
+    }
   } else {
-    const gptr<const uint8_t> mb = as_global<const uint8_t>(m_tile) + (e0 >> 1);
-    const gptr<const uint8_t> vb = as_global<const uint8_t>(v_tile) + (e0 >> 1);
+    const gptr<const uint8_t> mb = as_global<const uint8_t>(m_tile) + code_off;
+    const gptr<const uint8_t> vb = as_global<const uint8_t>(v_tile) + code_off;
     const int nb = (nv + 1) >> 1;
 #pragma unroll
-    for (int k = 0; k < 2; ++k) {
+    for (int k = 0; k < N / 2; ++k) {
       if (k < nb) {
         mw |= (uint32_t)mb[k] << (8 * k);
         vw |= (uint32_t)vb[k] << (8 * k);
@@ -370,25 +414,25 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   float sm_old = 0.0f, sv_old = 0.0f;
   if (FULL) {
     // scales are 4 bytes per block: cached, so that neighbouring blocks share lines
-    sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), half * 4u, 0, 0));
-    sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), half * 4u, 0, 0));
+    sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0));
+    sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0));
   } else if (blk_ok) {
-    sm_old = as_global<const float>(sm_tile)[half];
-    sv_old = as_global<const float>(sv_tile)[half];
+    sm_old = as_global<const float>(sm_tile)[blk];
+    sv_old = as_global<const float>(sv_tile)[blk];
   }
   setup_tables(lds, tid, slot);
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
-  F4 mn, vn;
+  Vals<N> mn, vn;
   float am = 0.0f, av = 0.0f;
   const char *lds_bytes = reinterpret_cast<const char *>(lds);
-  const uint32_t mw8 = mw << 3, vw8 = vw << 3;  // nibble j * 8 = byte offset of its code-book entry
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float m_old =
-        *reinterpret_cast<const float *>(lds_bytes + kLdsQm * 8 + ((mw8 >> (4 * j)) & 0x78u)) * sm_old;
-    const float v_old =
-        *reinterpret_cast<const float *>(lds_bytes + kLdsQv * 8 + ((vw8 >> (4 * j)) & 0x78u)) * sv_old;
+  for (int j = 0; j < N; ++j) {
+    // nibble j * 8 = byte offset of its code-book entry
+    const uint32_t mo = (j == 0 ? (mw << 3) : (mw >> (4 * j - 3))) & 0x78u;
+    const uint32_t vo = (j == 0 ? (vw << 3) : (vw >> (4 * j - 3))) & 0x78u;
+    const float m_old = *reinterpret_cast<const float *>(lds_bytes + kLdsQm * 8 + mo) * sm_old;
+    const float v_old = *reinterpret_cast<const float *>(lds_bytes + kLdsQv * 8 + vo) * sv_old;
     const float gj = g[j];
     float m = sc.b1 * m_old + sc.r1 * gj;
     float v = sc.b2 * v_old + sc.r2 * (gj * gj);
@@ -402,17 +446,22 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
     av = __builtin_fmaxf(av, v);
   }
-  store4<PBF, FULL>(const_cast<void *>(p_tile), e0, nv, p);
+  store_elems<PBF, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
 
   // block scales (exact: max is order independent)
-  block_max32_pair(am, av);
-  if (blk_ok && (lane & 31) == 0) {
+  if (G::kLanesPerBlock == 32) {
+    block_max32_pair(am, av);
+  } else {
+    am = row_max16(am);
+    av = row_max16(av);
+  }
+  if (blk_ok && (lane & (G::kLanesPerBlock - 1)) == 0) {
     if (FULL) {
-      __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), half * 4u, 0, 0);
-      __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), half * 4u, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), blk * 4u, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), blk * 4u, 0, 0);
     } else {
-      as_global<float>(sm_tile)[half] = am;
-      as_global<float>(sv_tile)[half] = av;
+      as_global<float>(sm_tile)[blk] = am;
+      as_global<float>(sv_tile)[blk] = av;
     }
   }
 
@@ -425,13 +474,13 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   uint32_t mword = 0, vword = 0;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < N; ++j) {
     // first moment: bucket = top 11 bits of the quotient, clamped per sign to the
     // lowest bucket the workgroup built
     const float qm = mn.x[j] * rm;
     uint32_t a = (f2bits(qm) >> 18) & 0x3FF8u;
     a = clamp_bucket(a);
-    const uint2 ent = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(lds) + a);
+    const uint2 ent = *reinterpret_cast<const uint2 *>(lds_bytes + a);
     const bool above_hi = qm > bits2f(ent.y);
     const bool above_lo = qm > bits2f(ent.x);
     redo |= (above_hi != above_lo);
@@ -443,25 +492,30 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     vword |= (uint32_t)(int)t << (4 * j);  // t > -1, so truncation gives 0 for t < 0
   }
   if (__builtin_expect(redo, 0)) {
-    mword = quantize4_exact<false>(mn, am);
-    vword = quantize4_exact<true>(vn, av);
+    mword = quantize_exact<false, N>(mn, am);
+    vword = quantize_exact<true, N>(vn, av);
   }
   if (am == 0.0f) mword = 0;  // 0/0: code 0 for the whole block
   if (!FULL) {
-    const uint32_t keep = nv >= 4 ? 0xffffu : ((1u << (4 * nv)) - 1u);
+    const uint32_t keep = nv >= 8 ? 0xffffffffu : ((1u << (4 * nv)) - 1u);
     mword &= keep;
     vword &= keep;
   }
 
   if (FULL) {
-    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)mword, tile_rsrc(m_tile), (uint32_t)lane * 2u, 0, kNt);
-    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)vword, tile_rsrc(v_tile), (uint32_t)lane * 2u, 0, kNt);
+    if (N == 4) {
+      __builtin_amdgcn_raw_buffer_store_b16((uint16_t)mword, tile_rsrc(m_tile), code_off, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b16((uint16_t)vword, tile_rsrc(v_tile), code_off, 0, kNt);
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b32(mword, tile_rsrc(m_tile), code_off, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(vword, tile_rsrc(v_tile), code_off, 0, kNt);
+    }
   } else {
-    const gptr<uint8_t> mb = as_global<uint8_t>(m_tile) + (e0 >> 1);
-    const gptr<uint8_t> vb = as_global<uint8_t>(v_tile) + (e0 >> 1);
+    const gptr<uint8_t> mb = as_global<uint8_t>(m_tile) + code_off;
+    const gptr<uint8_t> vb = as_global<uint8_t>(v_tile) + code_off;
     const int nb = (nv + 1) >> 1;
 #pragma unroll
-    for (int k = 0; k < 2; ++k) {
+    for (int k = 0; k < N / 2; ++k) {
       if (k < nb) {
         mb[k] = (uint8_t)(mword >> (8 * k));
         vb[k] = (uint8_t)(vword >> (8 * k));
@@ -472,6 +526,7 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
 
 template <bool PBF, bool GBF>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
+  using G = Geometry<PBF>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot(tid);
@@ -481,12 +536,12 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const TensorDesc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
-  const int64_t begin = tile * kTile;
+  const int64_t begin = tile * G::kTile;
   if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
     setup_tables(lds, tid, slot);
     return;
   }
-  if (begin + kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, tid, args.sc, lds, slot);
+  if (begin + G::kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, tid, args.sc, lds, slot);
   else process_tile<PBF, GBF, false>(T, tile, lane, tid, args.sc, lds, slot);
 }
 
@@ -714,7 +769,11 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   FusedArgs a;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
-  const uintptr_t p_align = p_dtype == Q4ADAMW_BF16 ? 8 : 16, g_align = g_dtype == Q4ADAMW_BF16 ? 8 : 16;
+  // a lane reads 4 (fp32 parameters) or 8 (bf16 parameters) consecutive elements at once
+  const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
+  const int64_t chunk_elems = p_bf16 ? Geometry<true>::kChunk : Geometry<false>::kChunk;
+  const uintptr_t p_align = 16, g_align = g_dtype == Q4ADAMW_BF16 ? (p_bf16 ? 16 : 8) : 16;
+  const uintptr_t code_align = p_bf16 ? 4 : 2;
   // validate everything before the first launch
   for (int i = 0; i < count; ++i) {
     const q4adamw_tensor &t = tensors[i];
@@ -723,12 +782,11 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.exp_avg_sq_scale)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
     if (!aligned(t.p, p_align) || !aligned(t.g, g_align))
-      return fail(Q4ADAMW_ERR_ALIGN,
-                  "param and grad must be aligned to four elements (16 bytes fp32, 8 bytes bf16)");
-    if (!aligned(t.exp_avg, 2) || !aligned(t.exp_avg_sq, 2) || !aligned(t.exp_avg_scale, 4) ||
-        !aligned(t.exp_avg_sq_scale, 4))
-      return fail(Q4ADAMW_ERR_ALIGN, "code buffers must be 2-byte aligned, scale buffers 4-byte aligned");
-    if ((uint64_t)(t.numel + kChunk - 1) / kChunk > kMaxChunksPerLaunch)
+      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be 16-byte aligned");
+    if (!aligned(t.exp_avg, code_align) || !aligned(t.exp_avg_sq, code_align) ||
+        !aligned(t.exp_avg_scale, 4) || !aligned(t.exp_avg_sq_scale, 4))
+      return fail(Q4ADAMW_ERR_ALIGN, "code and scale buffers must be 4-byte aligned");
+    if ((uint64_t)(t.numel + chunk_elems - 1) / chunk_elems > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -738,7 +796,7 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
   for (int i = 0; i < count; ++i) {
     const q4adamw_tensor &t = tensors[i];
     if (t.numel == 0) continue;
-    const uint64_t c = (uint64_t)(t.numel + kChunk - 1) / kChunk;
+    const uint64_t c = (uint64_t)(t.numel + chunk_elems - 1) / chunk_elems;
     if (a.ntensors == kMaxTensors || chunks + c > kMaxChunksPerLaunch) {
       if (int rc = launch_fused_batch(a, chunks, kernel, s)) return rc;
       a.ntensors = 0;
