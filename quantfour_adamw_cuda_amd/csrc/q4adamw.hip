@@ -174,6 +174,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nea
   return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// two fp32 -> two bf16 (round to nearest even) in one 32-bit word, lo in the low half
+__device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+}
+
 __device__ __forceinline__ void widen_bf16_pair(uint32_t w, float &lo, float &hi) {
   lo = bits2f(w << 16);
   hi = bits2f(w & 0xffff0000u);
@@ -217,15 +225,15 @@ __device__ __forceinline__ void store_elems(void *base, uint32_t e0, int nv, con
   if (FULL) {
     if (BF && N == 4) {
       u32x2 w;
-      w.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
-      w.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
+      w.x = pack_bf16_pair(x[0], x[1]);
+      w.y = pack_bf16_pair(x[2], x[3]);
       __builtin_amdgcn_raw_buffer_store_b64(w, tile_rsrc(base), e0 * 2, 0, kNt);
     } else if (BF) {
       u32x4 w;
-      w.x = f32_to_bf16_bits(x[0]) | (f32_to_bf16_bits(x[1]) << 16);
-      w.y = f32_to_bf16_bits(x[2]) | (f32_to_bf16_bits(x[3]) << 16);
-      w.z = f32_to_bf16_bits(x[N - 4]) | (f32_to_bf16_bits(x[N - 3]) << 16);
-      w.w = f32_to_bf16_bits(x[N - 2]) | (f32_to_bf16_bits(x[N - 1]) << 16);
+      w.x = pack_bf16_pair(x[0], x[1]);
+      w.y = pack_bf16_pair(x[2], x[3]);
+      w.z = pack_bf16_pair(x[N - 4], x[N - 3]);
+      w.w = pack_bf16_pair(x[N - 2], x[N - 1]);
       __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), e0 * 2, 0, kNt);
     } else {
 #pragma unroll
@@ -270,13 +278,18 @@ __device__ __forceinline__ uint32_t quantize_exact(const Vals<N> &v, float scale
   return word;
 }
 
+// (x & mask) | base as one v_and_or_b32: the mask travels in a scalar register (the
+// compiler splits the operation when the mask is a literal, which a VOP3 encoding
+// cannot hold).
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t base) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(base));
+  return r;
+}
+
 // Per-sign lower clamp of a bucket byte offset: max(a, (a & sign bit) | floor).
-// Written as v_and_or_b32 because the compiler splits the and/or when both masks
-// are literals (a VOP3 encoding cannot hold two).
 __device__ __forceinline__ uint32_t clamp_bucket(uint32_t a) {
-  uint32_t floor_a;
-  const uint32_t sign_mask = kNegativeBuckets * 8u, floor_pos = kBucketFloor * 8u;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(floor_a) : "v"(a), "s"(sign_mask), "v"(floor_pos));
+  const uint32_t floor_a = and_or(a, kNegativeBuckets * 8u, kBucketFloor * 8u);
   return a > floor_a ? a : floor_a;
 }
 
@@ -305,27 +318,33 @@ __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
   return group * 8 + within - 1;
 }
 
-// LDS tables of a workgroup, one array of 8-byte entries:
-//   [0, 2048)     bucket table of the first-moment quantizer; only the 76 entries
-//                 that a clamped quotient can reach are written, the rest is never read
-//   [2048, 2064)  first-moment code book  (value in .x)
-//   [2064, 2080)  second-moment code book (value in .x)
-constexpr uint32_t kLdsQm = kMtabEntries;
-constexpr uint32_t kLdsQv = kMtabEntries + 16;
-constexpr uint32_t kLdsEntries = kMtabEntries + 32;
+// LDS of a workgroup, one array of 2048 8-byte entries: the bucket table of the
+// first-moment quantizer, of which only the 76 entries that a clamped quotient can
+// reach are written (the rest is never read).  A gap of that table, entries
+// [kLdsCodeBooks, kLdsCodeBooks + 256), holds the waves' private dequantization tables:
+// per wave 64 entries, per quantization block 16 entries {code_book_m[i] * scale_m,
+// code_book_v[i] * scale_v}, so that dequantizing an element is one LDS read.
+constexpr uint32_t kLdsEntries = kMtabEntries;
+constexpr uint32_t kLdsCodeBooks = 512;
+static_assert(kLdsCodeBooks > kBucketTop && kLdsCodeBooks + 64 * kWaves <= kNegativeBuckets + kBucketFloor,
+              "the code-book region must sit in a gap of the bucket table");
 
 // This thread's slot of the workgroup tables, requested from memory as the very
 // first thing a wave does (only the first two waves hold slots).
 struct TableSlot {
-  uint32_t a, b;
+  uint32_t a, b, entry;  // bucket table slot of this thread (first 76 threads)
+  float qm, qv;          // code-book entries (lane & 15) of both moments
 };
 
 __device__ __forceinline__ TableSlot request_table_slot(int tid) {
-  TableSlot s{0u, 0u};
-  if (tid < 128) {
+  TableSlot s{0u, 0u, 0u, 0.0f, 0.0f};
+  if (tid < (int)(2 * kBucketsPerSign)) {
     s.a = kWorkgroupTables.a[tid];
     s.b = kWorkgroupTables.b[tid];
+    s.entry = kWorkgroupTables.entry[tid];
   }
+  s.qm = bits2f(kWorkgroupTables.a[96 + (tid & 15)]);
+  s.qv = bits2f(kWorkgroupTables.a[112 + (tid & 15)]);
   return s;
 }
 
@@ -334,15 +353,7 @@ __device__ __forceinline__ TableSlot request_table_slot(int tid) {
 // The fences order LDS only: a full __syncthreads() would also drain the outstanding
 // global loads.
 __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
-  if (tid < 128) {
-    // slots 0..37 -> positive buckets, 38..75 -> negative buckets, 76..95 -> unused
-    // entries 0..19 (below every bucket that is read), 96..127 -> the code books
-    const int entry = tid + (tid < (int)kBucketsPerSign       ? (int)kBucketFloor
-                             : tid < (int)(2 * kBucketsPerSign) ? (int)(kNegativeBuckets + kBucketFloor - kBucketsPerSign)
-                             : tid < 96                          ? -76
-                                                                 : (int)kLdsQm - 96);
-    lds[entry] = make_uint2(s.a, s.b);
-  }
+  if (tid < (int)(2 * kBucketsPerSign)) lds[s.entry] = make_uint2(s.a, s.b);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -362,7 +373,7 @@ struct Geometry {
 // one tile (256 or 512 elements) of one tensor
 // ---------------------------------------------------------------------------
 template <bool PBF, bool GBF, bool FULL>
-__device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int tid,
+__device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot) {
   using G = Geometry<PBF>;
   constexpr int N = G::kEpl;
@@ -420,19 +431,25 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     sm_old = as_global<const float>(sm_tile)[blk];
     sv_old = as_global<const float>(sv_tile)[blk];
   }
+  // this block's dequantization table: entry i = {code_book_m[i] * scale_m,
+  // code_book_v[i] * scale_v} (cuda_adamw_kernels.cu:340,343), written by the block's
+  // lanes (lane & 15 = i) into the wave's private LDS region
+  char *lds_bytes = reinterpret_cast<char *>(lds);
+  const uint32_t cb_base = (kLdsCodeBooks + (uint32_t)wave * 64u + blk * 16u) * 8u;
+  *reinterpret_cast<float2 *>(lds_bytes + cb_base + ((uint32_t)lane & 15u) * 8u) =
+      make_float2(slot.qm * sm_old, slot.qv * sv_old);
   setup_tables(lds, tid, slot);
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
   Vals<N> mn, vn;
   float am = 0.0f, av = 0.0f;
-  const char *lds_bytes = reinterpret_cast<const char *>(lds);
 #pragma unroll
   for (int j = 0; j < N; ++j) {
-    // nibble j * 8 = byte offset of its code-book entry
-    const uint32_t mo = (j == 0 ? (mw << 3) : (mw >> (4 * j - 3))) & 0x78u;
-    const uint32_t vo = (j == 0 ? (vw << 3) : (vw >> (4 * j - 3))) & 0x78u;
-    const float m_old = *reinterpret_cast<const float *>(lds_bytes + kLdsQm * 8 + mo) * sm_old;
-    const float v_old = *reinterpret_cast<const float *>(lds_bytes + kLdsQv * 8 + vo) * sv_old;
+    // nibble j * 8 = byte offset of its entry in the block's table
+    const uint32_t mo = and_or(j == 0 ? (mw << 3) : (mw >> (4 * j - 3)), 0x78u, cb_base);
+    const uint32_t vo = and_or(j == 0 ? (vw << 3) : (vw >> (4 * j - 3)), 0x78u, cb_base);
+    const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
+    const float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
     const float gj = g[j];
     float m = sc.b1 * m_old + sc.r1 * gj;
     float v = sc.b2 * v_old + sc.r2 * (gj * gj);
@@ -541,8 +558,8 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
     setup_tables(lds, tid, slot);
     return;
   }
-  if (begin + G::kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, tid, args.sc, lds, slot);
-  else process_tile<PBF, GBF, false>(T, tile, lane, tid, args.sc, lds, slot);
+  if (begin + G::kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, wave, tid, args.sc, lds, slot);
+  else process_tile<PBF, GBF, false>(T, tile, lane, wave, tid, args.sc, lds, slot);
 }
 
 // Non-quantized step for small tensors (cuda_adamw_kernels.cu:100-133): fp32

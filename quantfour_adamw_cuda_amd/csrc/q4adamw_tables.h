@@ -117,13 +117,17 @@ constexpr uint32_t kBucketTop = 508;                                    // expon
 constexpr uint32_t kBucketsPerSign = kBucketTop - kBucketFloor + 1;     // 38
 constexpr uint32_t kNegativeBuckets = 1024;                             // index offset of the sign bit
 
-// What the first 128 threads of a workgroup copy into LDS, one slot each:
-// slots 0..75  : bucket entries (a = lo bound | base, b = hi bound)
-// slots 96..111: first-moment code book (a = fp32 bits)
-// slots 112..127: second-moment code book (a = fp32 bits)
+// What the first 128 threads of a workgroup copy into LDS, one 8-byte entry each:
+// slots 0..37   : positive buckets kBucketFloor.. (a = lo bound | base, b = hi bound)
+// slots 38..75  : negative buckets
+// slots 76..95  : padding (written to the unused entries 0..19)
+// slots 96..111 : first-moment code book  (a = fp32 bits) -> entries 2048..2063
+// slots 112..127: second-moment code book (a = fp32 bits) -> entries 2064..2079
+// entry[] is the index of the 8-byte LDS entry the slot goes to.
 struct WorkgroupTables {
   uint32_t a[128];
   uint32_t b[128];
+  uint32_t entry[128];
 };
 
 // slot j of the compact table <-> bucket index in the full table
@@ -142,6 +146,11 @@ constexpr WorkgroupTables make_workgroup_tables() {
   for (uint32_t k = 0; k < 16; ++k) {
     t.a[96 + k] = kQmapMBits[k];
     t.a[112 + k] = f2bits(qmap_v((int)k));
+  }
+  for (uint32_t j = 0; j < 128; ++j) {
+    t.entry[j] = j < 2 * kBucketsPerSign ? compact_slot_bucket(j)
+                 : j < 96                ? j - 2 * kBucketsPerSign
+                                         : kMtabEntries + (j - 96);
   }
   return t;
 }
