@@ -145,11 +145,20 @@ void q4adamw_derive_scalars(float beta1, float beta2, float lr, float weight_dec
 void q4adamw_tables(int which, float *qmap16, float *qmid15);
 
 /*
- * Host-only: entry `index` (0..2047) of the first-moment bucket table the fused
- * kernel builds in LDS; out2[0] = lower guard bound with the base code in its low
- * nibble, out2[1] = upper guard bound (fp32 bit patterns).  For tests.
+ * Host-only: entry `index` (0..2047) of the first-moment bucket table, indexed by
+ * the top eleven bits of a normalised value's fp32 pattern; out2[0] = lower guard
+ * bound with the base code in its low nibble, out2[1] = upper guard bound (fp32
+ * bit patterns).  For tests.
  */
 int q4adamw_mtable_entry(uint32_t index, uint32_t *out2);
+
+/*
+ * Host-only: the fused kernel holds 256 of those entries in LDS and indexes them
+ * by the high byte of the normalised value converted to half precision toward
+ * zero; this returns the index (0..2047) of the entry that `half_index` (0..255)
+ * stands for, or a negative status.  For tests.
+ */
+int q4adamw_mtable_half_bucket(uint32_t half_index);
 
 /* Kept for callers that pair an init with a release: the library holds no device
  * memory, so this does nothing and returns 0. */

@@ -47,6 +47,7 @@ EXPORTS = (
     "q4adamw_derive_scalars",
     "q4adamw_tables",
     "q4adamw_mtable_entry",
+    "q4adamw_mtable_half_bucket",
     "q4adamw_release",
     "q4adamw_last_error",
     "q4adamw_version",
@@ -85,6 +86,8 @@ def load():
     L.q4adamw_tables.restype = None
     L.q4adamw_mtable_entry.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
     L.q4adamw_mtable_entry.restype = i
+    L.q4adamw_mtable_half_bucket.argtypes = [ctypes.c_uint32]
+    L.q4adamw_mtable_half_bucket.restype = i
     L.q4adamw_release.argtypes = []
     L.q4adamw_release.restype = i
     L.q4adamw_last_error.argtypes = []

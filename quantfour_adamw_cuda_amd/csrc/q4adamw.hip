@@ -25,6 +25,7 @@
 // Per element the kernel reads p, g and one nibble of each moment, and writes p
 // and one nibble of each moment; per block it reads and writes two fp32 scales.
 #include <hip/hip_runtime.h>
+#include <float.h>
 #include <math.h>
 #include <stdint.h>
 #include <string.h>
@@ -46,8 +47,11 @@ constexpr int kMaxSmallTensors = 80;
 struct StepConsts {
   float b1, b2, r1, r2;  // beta1, beta2, 1-beta1, 1-beta2
   float wdu, ss;         // 1 - lr*wd, lr / (1 - beta1^t)
-  float c2s, inv_c2s;    // sqrt(1 - beta2^t) and its reciprocal
+  float c2s;             // sqrt(1 - beta2^t)
   float eps;
+  // the fused kernel's parameter update p*wdu - m'/(sqrt(v')*den_scale + den_eps), the
+  // step size folded into the denominator: 1/(c2s*ss) and eps/ss
+  float den_scale, den_eps;
 };
 
 struct TensorDesc {  // 56 bytes
@@ -96,9 +100,9 @@ struct SmallArgs {
 
 static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
-// bucket table entries that hold a threshold and the two code books (see
-// q4adamw_tables.h), read by every workgroup at start-up
-__device__ const WorkgroupTables kWorkgroupTables = make_workgroup_tables();
+// the first-moment bucket table (see q4adamw_tables.h), copied into LDS by every
+// workgroup at start-up, one entry per thread
+__device__ const HalfTable kHalfTable = make_half_table();
 // first-moment code book for kernels that index it per lane
 __device__ const uint32_t kQmapMDev[16] = {
     0xbf633333u, 0xbf29999au, 0xbee00000u, 0xbe59999au, 0xbd9eb852u, 0xbd051eb8u,
@@ -287,10 +291,19 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t b
   return r;
 }
 
-// Per-sign lower clamp of a bucket byte offset: max(a, (a & sign bit) | floor).
-__device__ __forceinline__ uint32_t clamp_bucket(uint32_t a) {
-  const uint32_t floor_a = and_or(a, kNegativeBuckets * 8u, kBucketFloor * 8u);
-  return a > floor_a ? a : floor_a;
+// Byte BYTE of x, times 8 (the byte offset of an 8-byte table entry), as one SDWA
+// shift; `three` is the shift amount in a register.
+template <int BYTE>
+__device__ __forceinline__ uint32_t byte_times8(uint32_t x, uint32_t three) {
+  static_assert(BYTE == 1 || BYTE == 3, "");
+  uint32_t r;
+  if (BYTE == 1)
+    asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1"
+        : "=v"(r) : "v"(three), "v"(x));
+  else
+    asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3"
+        : "=v"(r) : "v"(three), "v"(x));
+  return r;
 }
 
 // 1/s to within half an ulp for s in [2^-100, 2^100]: hardware estimate plus one
@@ -318,33 +331,27 @@ __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
   return group * 8 + within - 1;
 }
 
-// LDS of a workgroup, one array of 2048 8-byte entries: the bucket table of the
-// first-moment quantizer, of which only the 76 entries that a clamped quotient can
-// reach are written (the rest is never read).  A gap of that table, entries
-// [kLdsCodeBooks, kLdsCodeBooks + 256), holds the waves' private dequantization tables:
-// per wave 64 entries, per quantization block 16 entries {code_book_m[i] * scale_m,
-// code_book_v[i] * scale_v}, so that dequantizing an element is one LDS read.
-constexpr uint32_t kLdsEntries = kMtabEntries;
-constexpr uint32_t kLdsCodeBooks = 512;
-static_assert(kLdsCodeBooks > kBucketTop && kLdsCodeBooks + 64 * kWaves <= kNegativeBuckets + kBucketFloor,
-              "the code-book region must sit in a gap of the bucket table");
+// LDS of a workgroup, one array of 8-byte entries:
+//   [0, 256)    bucket table of the first-moment quantizer, indexed by the high byte
+//               of the quotient as a half
+//   [256, 512)  the waves' private dequantization tables: per wave 64 entries, per
+//               quantization block 16 entries {code_book_m[i] * scale_m,
+//               code_book_v[i] * scale_v}, so that dequantizing an element is one read
+constexpr uint32_t kLdsCodeBooks = kHalfTableEntries;
+constexpr uint32_t kLdsEntries = kLdsCodeBooks + 64 * kWaves;
+static_assert(kThreads == (int)kHalfTableEntries, "one bucket table entry per thread");
 
-// This thread's slot of the workgroup tables, requested from memory as the very
-// first thing a wave does (only the first two waves hold slots).
+// What a thread fetches from the constant tables as the very first thing it does.
 struct TableSlot {
-  uint32_t a, b, entry;  // bucket table slot of this thread (first 76 threads)
-  float qm, qv;          // code-book entries (lane & 15) of both moments
+  uint2 entry;  // bucket table entry number tid
+  float qm;     // first-moment code-book value number (lane & 15)
 };
 
 __device__ __forceinline__ TableSlot request_table_slot(int tid) {
-  TableSlot s{0u, 0u, 0u, 0.0f, 0.0f};
-  if (tid < (int)(2 * kBucketsPerSign)) {
-    s.a = kWorkgroupTables.a[tid];
-    s.b = kWorkgroupTables.b[tid];
-    s.entry = kWorkgroupTables.entry[tid];
-  }
-  s.qm = bits2f(kWorkgroupTables.a[96 + (tid & 15)]);
-  s.qv = bits2f(kWorkgroupTables.a[112 + (tid & 15)]);
+  TableSlot s;
+  const MtabEntry e = kHalfTable.e[tid];
+  s.entry = make_uint2(e.lo, e.hi);
+  s.qm = bits2f(kQmapMDev[tid & 15]);
   return s;
 }
 
@@ -353,7 +360,7 @@ __device__ __forceinline__ TableSlot request_table_slot(int tid) {
 // The fences order LDS only: a full __syncthreads() would also drain the outstanding
 // global loads.
 __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
-  if (tid < (int)(2 * kBucketsPerSign)) lds[s.entry] = make_uint2(s.a, s.b);
+  lds[tid] = s.entry;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -437,7 +444,7 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   char *lds_bytes = reinterpret_cast<char *>(lds);
   const uint32_t cb_base = (kLdsCodeBooks + (uint32_t)wave * 64u + blk * 16u) * 8u;
   *reinterpret_cast<float2 *>(lds_bytes + cb_base + ((uint32_t)lane & 15u) * 8u) =
-      make_float2(slot.qm * sm_old, slot.qv * sv_old);
+      make_float2(slot.qm * sm_old, qmap_v(lane & 15) * sv_old);
   setup_tables(lds, tid, slot);
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
@@ -455,9 +462,8 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     float v = sc.b2 * v_old + sc.r2 * (gj * gj);
     if (!FULL && j >= nv) { m = 0.0f; v = 0.0f; }
     // parameter: only this part may use the hardware's 1-ulp sqrt and reciprocal
-    const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.inv_c2s, sc.eps);
-    const float upd = m * __builtin_amdgcn_rcpf(den);
-    p[j] = __builtin_fmaf(-sc.ss, upd, p[j] * sc.wdu);
+    const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
+    p[j] = __builtin_fmaf(-m, __builtin_amdgcn_rcpf(den), p[j] * sc.wdu);
     mn.x[j] = m;
     vn.x[j] = v;
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
@@ -489,25 +495,37 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   const float rm = safe_m ? refined_rcp(am) : 0.0f;
   const float rv16 = safe_v ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
+  float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
   uint32_t mword = 0, vword = 0;
+  const uint32_t three = 3u;
 #pragma unroll
-  for (int j = 0; j < N; ++j) {
-    // first moment: bucket = top 11 bits of the quotient, clamped per sign to the
-    // lowest bucket the workgroup built
-    const float qm = mn.x[j] * rm;
-    uint32_t a = (f2bits(qm) >> 18) & 0x3FF8u;
-    a = clamp_bucket(a);
-    const uint2 ent = *reinterpret_cast<const uint2 *>(lds_bytes + a);
-    const bool above_hi = qm > bits2f(ent.y);
-    const bool above_lo = qm > bits2f(ent.x);
-    redo |= (above_hi != above_lo);
-    mword |= ((ent.x & 15u) + (above_hi ? 1u : 0u)) << (4 * j);
+  for (int j = 0; j < N; j += 2) {
+    // first moment: the quotients' bucket entries, two quotients per conversion
+    const float q0 = mn.x[j] * rm, q1 = mn.x[j + 1] * rm;
+    const uint32_t halves = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(q0, q1));
+    const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + byte_times8<1>(halves, three));
+    const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + byte_times8<3>(halves, three));
+    const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
+    redo |= (hi0 != (q0 > bits2f(ent0.x))) | (hi1 != (q1 > bits2f(ent1.x)));
+    // base code in the entry's low nibble, plus one above the threshold; every
+    // code enters the word at the top and moves down four bits per later element
+    mword = __builtin_amdgcn_alignbit(ent0.x + (hi0 ? 1u : 0u), mword, 4);
+    mword = __builtin_amdgcn_alignbit(ent1.x + (hi1 ? 1u : 0u), mword, 4);
 
     // second moment: thresholds at 16q = k + 0.5, k = 1..15
-    const float t = __builtin_fmaf(vn.x[j], rv16, kVGuard - 0.5f);
-    redo |= __builtin_amdgcn_fractf(t) < 2.0f * kVGuard;
-    vword |= (uint32_t)(int)t << (4 * j);  // t > -1, so truncation gives 0 for t < 0
+#pragma unroll
+    for (int k = j; k < j + 2; ++k) {
+      const float t = __builtin_fmaf(vn.x[k], rv16, kVGuard - 0.5f);
+      vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
+      // t > -1, so truncation gives 0 for t < 0
+      vword = __builtin_amdgcn_alignbit((uint32_t)(int)t, vword, 4);
+    }
   }
+  if (N == 4) {
+    mword >>= 16;
+    vword >>= 16;
+  }
+  redo |= vfrac < 2.0f * kVGuard;
   if (__builtin_expect(redo, 0)) {
     mword = quantize_exact<false, N>(mn, am);
     vword = quantize_exact<true, N>(vn, av);
@@ -683,8 +701,13 @@ static int make_consts(float beta1, float beta2, float lr, float wd, float eps, 
   out->wdu = s[3];
   out->ss = s[2];
   out->c2s = s[1];
-  out->inv_c2s = 1.0f / s[1];
   out->eps = eps;
+  // a step size so small that these overflow moves no parameter: a zero scale with
+  // an infinite offset makes the kernel's update term vanish
+  const double den_scale = 1.0 / ((double)s[1] * (double)s[2]), den_eps = (double)eps / (double)s[2];
+  const bool fits = den_scale <= (double)FLT_MAX && den_eps <= (double)FLT_MAX;
+  out->den_scale = fits ? (float)den_scale : 0.0f;
+  out->den_eps = fits ? (float)den_eps : INFINITY;
   return 0;
 }
 
@@ -777,6 +800,11 @@ int q4adamw_mtable_entry(uint32_t index, uint32_t *out2) {
   out2[0] = e.lo;
   out2[1] = e.hi;
   return 0;
+}
+
+int q4adamw_mtable_half_bucket(uint32_t half_index) {
+  if (half_index >= kHalfTableEntries) return fail(Q4ADAMW_ERR_ARG, "index out of range");
+  return (int)half_index_bucket(half_index);
 }
 
 int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,

@@ -45,7 +45,7 @@ Q4_HD constexpr float qmid_v(int k) { return (float)(2 * k + 3) * 0.03125f; }
 // with base = number of thresholds below the whole bucket and thr = the threshold
 // inside it, if any.
 //
-// The kernel's fast path knows q only to within three ulps (it multiplies by a
+// The fused kernel's fast path knows q only to within three ulps (it multiplies by a
 // refined reciprocal instead of dividing), so each entry stores a guard band
 // around thr instead of thr itself:
 //     x = fp32 "lo" bound, at least kGuardUlps below thr, low four bits = base
@@ -108,50 +108,36 @@ Q4_HD constexpr MtabEntry mtab_entry(uint32_t idx) {
   return out;
 }
 
-// Only the buckets that can hold a threshold differ from "no threshold, base 7":
-// per sign, buckets kBucketFloor .. kBucketTop (|q| from 1.75 * 2^-10 to 1.25).
-// The kernel clamps smaller magnitudes up to the floor bucket and builds just these
-// entries in LDS, at their natural index, leaving the rest of the table untouched.
-constexpr uint32_t kBucketFloor = 471;                                  // exponent 117, mantissa 11b
-constexpr uint32_t kBucketTop = 508;                                    // exponent 127, mantissa 00b
-constexpr uint32_t kBucketsPerSign = kBucketTop - kBucketFloor + 1;     // 38
-constexpr uint32_t kNegativeBuckets = 1024;                             // index offset of the sign bit
+// ---------------------------------------------------------------------------
+// The table a workgroup of the fused kernel holds in LDS: 256 entries.
+//
+// The kernel converts a quotient to half precision with round-toward-zero
+// (v_cvt_pkrtz_f16_f32, two quotients per instruction) and takes the high byte of
+// the half (sign, five exponent bits, two mantissa bits) as the entry index.
+// Truncation keeps the leading bits, so for |q| in [2^-14, 65536) that byte names
+// the same bucket as the top eleven bits of the fp32 pattern, with the exponent
+// re-biased by 112; every smaller magnitude (a subnormal half, exponent field 0) is
+// below the smallest threshold (2.7e-3) and shares the bucket of zero, which is why
+// the kernel needs no clamp.  Exponent field 31 (inf, nan) maps to the bucket of the
+// same fp32 class.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kHalfTableEntries = 256;
 
-// What the first 128 threads of a workgroup copy into LDS, one 8-byte entry each:
-// slots 0..37   : positive buckets kBucketFloor.. (a = lo bound | base, b = hi bound)
-// slots 38..75  : negative buckets
-// slots 76..95  : padding (written to the unused entries 0..19)
-// slots 96..111 : first-moment code book  (a = fp32 bits) -> entries 2048..2063
-// slots 112..127: second-moment code book (a = fp32 bits) -> entries 2064..2079
-// entry[] is the index of the 8-byte LDS entry the slot goes to.
-struct WorkgroupTables {
-  uint32_t a[128];
-  uint32_t b[128];
-  uint32_t entry[128];
+// bucket of the 2048-entry table that half-index h (0..255) stands for
+Q4_HD constexpr uint32_t half_index_bucket(uint32_t h) {
+  const uint32_t sign = (h >> 7) & 1u, e5 = (h >> 2) & 31u, m2 = h & 3u;
+  const uint32_t e8 = e5 == 0u ? 0u : e5 == 31u ? 255u : e5 + 112u;
+  return (sign << 10) | (e8 << 2) | (e5 == 0u ? 0u : m2);
+}
+static_assert((113u << 2) < 471u, "the lowest bucket that holds a threshold must be a normal half");
+
+struct HalfTable {
+  MtabEntry e[kHalfTableEntries];
 };
 
-// slot j of the compact table <-> bucket index in the full table
-Q4_HD constexpr uint32_t compact_slot_bucket(uint32_t j) {
-  return j < kBucketsPerSign ? kBucketFloor + j
-                             : kNegativeBuckets + kBucketFloor + (j - kBucketsPerSign);
-}
-
-constexpr WorkgroupTables make_workgroup_tables() {
-  WorkgroupTables t{};
-  for (uint32_t j = 0; j < 2 * kBucketsPerSign; ++j) {
-    const MtabEntry e = mtab_entry(compact_slot_bucket(j));
-    t.a[j] = e.lo;
-    t.b[j] = e.hi;
-  }
-  for (uint32_t k = 0; k < 16; ++k) {
-    t.a[96 + k] = kQmapMBits[k];
-    t.a[112 + k] = f2bits(qmap_v((int)k));
-  }
-  for (uint32_t j = 0; j < 128; ++j) {
-    t.entry[j] = j < 2 * kBucketsPerSign ? compact_slot_bucket(j)
-                 : j < 96                ? j - 2 * kBucketsPerSign
-                                         : kMtabEntries + (j - 96);
-  }
+constexpr HalfTable make_half_table() {
+  HalfTable t{};
+  for (uint32_t h = 0; h < kHalfTableEntries; ++h) t.e[h] = mtab_entry(half_index_bucket(h));
   return t;
 }
 

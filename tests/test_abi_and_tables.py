@@ -98,9 +98,9 @@ def test_bucket_table_properties(lib):
     mid_bits = mid.view(np.uint32)
     with_thr = np.flatnonzero(hi != NO_THR)
     assert with_thr.size == 15
-    # the kernel only builds buckets 471..508 per sign; everything a clamped quotient can
-    # reach outside the threshold buckets must say "base, no threshold"
-    assert set(with_thr.tolist()) <= set(range(471, 509)) | set(range(1024 + 471, 1024 + 509))
+    # every bucket that holds a threshold is one the kernel's 256-entry table carries
+    held = {lib.q4adamw_mtable_half_bucket(h) for h in range(256)}
+    assert set(with_thr.tolist()) <= held
     seen = []
     for i in range(2048):
         sign, mag = i >> 10, i & 1023
@@ -133,6 +133,47 @@ def test_bucket_table_properties(lib):
     assert sorted(seen) == list(range(15))
 
 
+def _half_index(q):
+    """High byte of q converted to half precision toward zero (what v_cvt_pkrtz_f16_f32
+    leaves in bits 8..15 / 24..31), for finite |q| < 65536: truncate, then convert exactly."""
+    q = np.asarray(q, np.float32)
+    bits = q.view(np.uint32)
+    normal = (bits & np.uint32(0xFFFFE000)).view(np.float32)               # keep 10 mantissa bits
+    tiny = (np.trunc(q.astype(np.float64) * 2.0 ** 24) / 2.0 ** 24).astype(np.float32)
+    tz = np.where(np.abs(q) >= np.float32(2.0 ** -14), normal, tiny)
+    h = tz.astype(np.float16).view(np.uint16)
+    assert np.array_equal(h.view(np.float16).astype(np.float32), tz)       # the conversion was exact
+    return (h >> 8).astype(np.int64) | np.where(np.signbit(q), 0x80, 0)    # -0.0 keeps its sign
+
+
+def test_half_index_names_the_same_entry(lib):
+    """The kernel indexes 256 entries by the high byte of the quotient as a half (round toward
+    zero); that entry must be the one the top eleven fp32 bits select in the full table, for
+    every magnitude a quotient can take (the approximate quotient never exceeds 1 by more than
+    a few ulps) and far beyond."""
+    lo, hi = _table(lib)
+    bucket_of = np.array([lib.q4adamw_mtable_half_bucket(h) for h in range(256)])
+    assert lib.q4adamw_mtable_half_bucket(256) < 0
+    rng = np.random.default_rng(5)
+    mag = np.concatenate([
+        10.0 ** rng.uniform(-44, 4.5, 200000),
+        2.0 ** np.arange(-30, 16, dtype=np.float64),                       # bucket edges
+        np.nextafter((2.0 ** np.arange(-30, 16)).astype(np.float32), np.float32(0)).astype(np.float64),
+        [0.0, 1.0, 1.0 + 2 ** -22, 65504.0, 65535.0],
+    ]).astype(np.float32)
+    # all four mantissa quarters of every exponent, and their lower neighbours
+    quarters = (2.0 ** np.arange(-20, 3))[:, None] * np.array([1.0, 1.25, 1.5, 1.75])[None, :]
+    q32 = quarters.astype(np.float32).ravel()
+    mag = np.concatenate([mag, q32, np.nextafter(q32, np.float32(0))])
+    q = np.concatenate([mag, -mag])
+    full = (q.view(np.uint32) >> 21).astype(np.int64)
+    via_half = bucket_of[_half_index(q)]
+    assert np.array_equal(lo[via_half], lo[full]) and np.array_equal(hi[via_half], hi[full])
+    # the buckets themselves coincide wherever the half is normal
+    normal = np.abs(q) >= np.float32(2.0 ** -14)
+    assert np.array_equal(via_half[normal], full[normal])
+
+
 def _nudge(x, d):
     """array of fp32 moved by d ulps in magnitude (d may be an array)."""
     return (x.view(np.uint32).astype(np.int64) + d).astype(np.uint32).view(np.float32)
@@ -144,10 +185,12 @@ def _rn32(x64):
 
 def test_fast_path_model_first_moment(lib):
     """Model of the kernel's first-moment fast path: q^ = RN(x * r) with r anywhere within one
-    ulp of 1/s, bucket lookup with the per-sign clamp, decision by the guard bounds.  Wherever
+    ulp of 1/s, entry lookup by the quotient's half-precision high byte, decision by the guard
+    bounds.  Wherever
     the model does not ask for the exact path its code must equal the exact code
     #{j : mid_j < RN(x / s)}, for x on and around every threshold times the scale."""
     lo, hi = _table(lib)
+    bucket_of = np.array([lib.q4adamw_mtable_half_bucket(h) for h in range(256)])
     _, mid = oc.tables(0)
     rng = np.random.default_rng(0)
     s = (10.0 ** rng.uniform(-25, 25, 4000)).astype(np.float32)
@@ -163,10 +206,8 @@ def test_fast_path_model_first_moment(lib):
         for dr in (-1, 0, 1):
             r = _nudge(r0, dr)
             q = _rn32(x.astype(np.float64) * r[:, None].astype(np.float64))
-            a = (q.view(np.uint32) >> 18) & 0x3FF8
-            floor_a = (a & (1024 * 8)) | (471 * 8)
-            a = np.maximum(a, floor_a)
-            e_lo, e_hi = lo[a >> 3], hi[a >> 3]
+            a = bucket_of[_half_index(q)]
+            e_lo, e_hi = lo[a], hi[a]
             above_hi = q > e_hi.view(np.float32)
             above_lo = q > (e_lo.view(np.float32))
             decided = above_hi == above_lo
