@@ -66,7 +66,7 @@ struct TensorDesc {  // 56 bytes
 
 // Kernel arguments of one fused launch (about 3 KiB, passed by value).
 // first_chunk[i] = index of tensor i's first chunk; entries past ntensors hold
-// 0xffffffff.  pivot[k] = first_chunk[8k] lets a workgroup find its tensor with two
+// 0x7fffffff (more than any chunk index).  pivot[k] = first_chunk[8k] lets a workgroup find its tensor with two
 // wide scalar loads.
 struct FusedArgs {
   static constexpr int kCapacity = kMaxTensors;
@@ -295,15 +295,27 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t b
 // shift; `three` is the shift amount in a register.
 template <int BYTE>
 __device__ __forceinline__ uint32_t byte_times8(uint32_t x, uint32_t three) {
-  static_assert(BYTE == 1 || BYTE == 3, "");
+  static_assert(BYTE >= 0 && BYTE <= 3, "");
   uint32_t r;
-  if (BYTE == 1)
-    asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1"
-        : "=v"(r) : "v"(three), "v"(x));
-  else
-    asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3"
-        : "=v"(r) : "v"(three), "v"(x));
+#define Q4_SDWA_SHIFT(SEL)                                                                          \
+  asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:" SEL \
+      : "=v"(r) : "v"(three), "v"(x))
+  if (BYTE == 0) Q4_SDWA_SHIFT("BYTE_0");
+  else if (BYTE == 1) Q4_SDWA_SHIFT("BYTE_1");
+  else if (BYTE == 2) Q4_SDWA_SHIFT("BYTE_2");
+  else Q4_SDWA_SHIFT("BYTE_3");
+#undef Q4_SDWA_SHIFT
   return r;
+}
+
+// byte_times8 with the byte chosen by a loop index of an unrolled loop
+__device__ __forceinline__ uint32_t entry_offset(uint32_t x, int byte, uint32_t three) {
+  switch (byte) {
+    case 0: return byte_times8<0>(x, three);
+    case 1: return byte_times8<1>(x, three);
+    case 2: return byte_times8<2>(x, three);
+    default: return byte_times8<3>(x, three);
+  }
 }
 
 // 1/s to within half an ulp for s in [2^-100, 2^100]: hardware estimate plus one
@@ -319,26 +331,30 @@ constexpr float kScaleHi = 1.2676506002282294e+30f;  // 2^100
 constexpr float kVGuard = 7.62939453125e-06f;        // 2^-17, in units of 16*q
 
 // Uniform search of the launch's tensor list: the last tensor whose first chunk is
-// <= chunk.  first_chunk[0] is 0, so the result is never negative.
+// <= chunk.  first_chunk[0] is 0, so the result is never negative.  Chunk indices and
+// table entries are below 2^31, so bit 31 of (x - chunk - 1) says x <= chunk: plain
+// integer arithmetic that stays on the scalar unit.
 template <typename Args>
 __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
-  int group = 0;
+  uint32_t group = 0;
 #pragma unroll
-  for (int k = 1; k < Args::kPivots; ++k) group += (a.pivot[k] <= chunk) ? 1 : 0;
-  int within = 0;
+  for (int k = 1; k < Args::kPivots; ++k) group += (a.pivot[k] - chunk - 1u) >> 31;
+  uint32_t within = 0;
 #pragma unroll
-  for (int k = 0; k < 8; ++k) within += (a.first_chunk[group * 8 + k] <= chunk) ? 1 : 0;
-  return group * 8 + within - 1;
+  for (int k = 0; k < 8; ++k) within += (a.first_chunk[group * 8 + k] - chunk - 1u) >> 31;
+  return (int)(group * 8 + within) - 1;
 }
 
 // LDS of a workgroup, one array of 8-byte entries:
-//   [0, 256)    bucket table of the first-moment quantizer, indexed by the high byte
-//               of the quotient as a half
-//   [256, 512)  the waves' private dequantization tables: per wave 64 entries, per
+//   [0, 256)    the waves' private dequantization tables: per wave 64 entries, per
 //               quantization block 16 entries {code_book_m[i] * scale_m,
 //               code_book_v[i] * scale_v}, so that dequantizing an element is one read
-constexpr uint32_t kLdsCodeBooks = kHalfTableEntries;
-constexpr uint32_t kLdsEntries = kLdsCodeBooks + 64 * kWaves;
+//               and an entry number fits a byte
+//   [256, 512)  bucket table of the first-moment quantizer, indexed by the high byte
+//               of the quotient as a half
+constexpr uint32_t kLdsBuckets = 64 * kWaves;
+constexpr uint32_t kLdsEntries = kLdsBuckets + kHalfTableEntries;
+static_assert(kLdsBuckets == 256, "dequantization entry numbers must fit a byte");
 static_assert(kThreads == (int)kHalfTableEntries, "one bucket table entry per thread");
 
 // What a thread fetches from the constant tables as the very first thing it does.
@@ -360,7 +376,7 @@ __device__ __forceinline__ TableSlot request_table_slot(int tid) {
 // The fences order LDS only: a full __syncthreads() would also drain the outstanding
 // global loads.
 __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
-  lds[tid] = s.entry;
+  lds[kLdsBuckets + tid] = s.entry;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -442,19 +458,24 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   // code_book_v[i] * scale_v} (cuda_adamw_kernels.cu:340,343), written by the block's
   // lanes (lane & 15 = i) into the wave's private LDS region
   char *lds_bytes = reinterpret_cast<char *>(lds);
-  const uint32_t cb_base = (kLdsCodeBooks + (uint32_t)wave * 64u + blk * 16u) * 8u;
-  *reinterpret_cast<float2 *>(lds_bytes + cb_base + ((uint32_t)lane & 15u) * 8u) =
+  const uint32_t cb_entry = (uint32_t)wave * 64u + blk * 16u;  // entry number of code 0
+  *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) =
       make_float2(slot.qm * sm_old, qmap_v(lane & 15) * sv_old);
   setup_tables(lds, tid, slot);
+
+  // entry numbers of the lane's codes, one per byte: even elements, odd elements
+  const uint32_t three = 3u;
+  const uint32_t cb_bytes = cb_entry * 0x01010101u;
+  const uint32_t m_even = and_or(mw, 0x0F0F0F0Fu, cb_bytes), m_odd = and_or(mw >> 4, 0x0F0F0F0Fu, cb_bytes);
+  const uint32_t v_even = and_or(vw, 0x0F0F0F0Fu, cb_bytes), v_odd = and_or(vw >> 4, 0x0F0F0F0Fu, cb_bytes);
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
   Vals<N> mn, vn;
   float am = 0.0f, av = 0.0f;
 #pragma unroll
   for (int j = 0; j < N; ++j) {
-    // nibble j * 8 = byte offset of its entry in the block's table
-    const uint32_t mo = and_or(j == 0 ? (mw << 3) : (mw >> (4 * j - 3)), 0x78u, cb_base);
-    const uint32_t vo = and_or(j == 0 ? (vw << 3) : (vw >> (4 * j - 3)), 0x78u, cb_base);
+    const uint32_t mo = entry_offset(j & 1 ? m_odd : m_even, j >> 1, three);
+    const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, three);
     const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
     const float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
     const float gj = g[j];
@@ -497,14 +518,13 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
   uint32_t mword = 0, vword = 0;
-  const uint32_t three = 3u;
 #pragma unroll
   for (int j = 0; j < N; j += 2) {
     // first moment: the quotients' bucket entries, two quotients per conversion
     const float q0 = mn.x[j] * rm, q1 = mn.x[j + 1] * rm;
     const uint32_t halves = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(q0, q1));
-    const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + byte_times8<1>(halves, three));
-    const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + byte_times8<3>(halves, three));
+    const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<1>(halves, three));
+    const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<3>(halves, three));
     const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
     redo |= (hi0 != (q0 > bits2f(ent0.x))) | (hi1 != (q1 > bits2f(ent1.x)));
     // base code in the entry's low nibble, plus one above the threshold; every
@@ -724,7 +744,7 @@ static int check_dtypes(int p_dtype, int g_dtype) {
 // or SmallArgs; `chunks` is the batch's total chunk count.
 template <typename Args>
 static void finish_prefix(Args &a) {
-  for (int i = a.ntensors; i < Args::kPivots * 8; ++i) a.first_chunk[i] = 0xffffffffu;
+  for (int i = a.ntensors; i < Args::kPivots * 8; ++i) a.first_chunk[i] = 0x7fffffffu;
   for (int k = 0; k < Args::kPivots; ++k) a.pivot[k] = a.first_chunk[k * 8];
 }
 
