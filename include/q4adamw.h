@@ -23,6 +23,7 @@
 #ifndef Q4ADAMW_H
 #define Q4ADAMW_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -75,6 +76,36 @@ typedef struct q4adamw_small_tensor {
 } q4adamw_small_tensor;
 
 /*
+ * What a step does to the gradients besides reading them.  The reference's caller
+ * pattern (tests/driver.py:53-59: zero_grad, backward, step) leaves loss-scale
+ * removal, clipping and zeroing to separate passes over the gradients; the `_ex`
+ * entry points fold them into the step's single read of g.
+ *   grad_scale       every gradient element is multiplied by
+ *   grad_scale_dev     s = grad_scale * (grad_scale_dev ? *grad_scale_dev : 1)
+ *                    in fp32 (one rounded multiplication per element) before the
+ *                    step uses it.  grad_scale_dev is a device fp32 scalar (e.g.
+ *                    1 / loss scale, a clip coefficient, q4adamw_grad_norm's
+ *                    out3[2]) or NULL.
+ *   skip_if_nonzero  device fp32 scalar or NULL: when it holds a non-zero value
+ *                    (an overflow flag) the call changes nothing.
+ *   zero_grad        non-zero: the gradients are overwritten with zeros once read
+ *                    (the `g` pointers are written in that case).
+ * The device scalars are read when the kernels run, not when the call returns.
+ */
+typedef struct q4adamw_grad_options {
+  float grad_scale;
+  int zero_grad;
+  const float *grad_scale_dev;
+  const float *skip_if_nonzero;
+} q4adamw_grad_options;
+
+/* One gradient tensor for q4adamw_grad_norm: numel elements, 16-byte aligned. */
+typedef struct q4adamw_grad {
+  const void *g;
+  int64_t numel;
+} q4adamw_grad;
+
+/*
  * Fused 4-bit AdamW step on one tensor.
  * Replaces fused_4bit (optim/cuda_fused_interface.cc:19-39) and its launcher
  * cuda_fused_4bit (optim/cuda_adamw_kernels.cu:422-469).
@@ -94,6 +125,12 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
                              int g_dtype, float beta1, float beta2, float lr,
                              float weight_decay, float eps, float step, void *stream);
 
+/* q4adamw_fused_4bit_multi with gradient options (NULL = none). */
+int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_dtype,
+                                int g_dtype, float beta1, float beta2, float lr,
+                                float weight_decay, float eps, float step,
+                                const q4adamw_grad_options *opt, void *stream);
+
 /*
  * Non-quantized AdamW step (fp32 moments) on one tensor.
  * Replaces fused_single_tensor (optim/cuda_fused_interface.cc:49-64) and
@@ -109,6 +146,31 @@ int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int c
                                       int p_dtype, int g_dtype, float beta1, float beta2,
                                       float lr, float weight_decay, float eps, float step,
                                       void *stream);
+
+/* q4adamw_fused_single_tensor_multi with gradient options (NULL = none). */
+int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, int count,
+                                         int p_dtype, int g_dtype, float beta1, float beta2,
+                                         float lr, float weight_decay, float eps, float step,
+                                         const q4adamw_grad_options *opt, void *stream);
+
+/*
+ * Global L2 norm of a set of gradient tensors and the clip coefficient that follows
+ * from it: what torch.nn.utils.clip_grad_norm_ computes before it rescales the
+ * gradients (the reference's callers clip between backward and step; the rescaling
+ * itself is the `_ex` entry points' multiplier).  With
+ *   s = grad_scale * (grad_scale_dev ? *grad_scale_dev : 1):
+ *   out3[0] = |s| * sqrt(sum g^2)               norm of the scaled gradients (fp32)
+ *   out3[1] = min(1, max_norm / (out3[0] + 1e-6))   clip coefficient; 1 if max_norm <= 0
+ *   out3[2] = s * out3[1]                       multiplier to hand to the step
+ * Squares are summed in fp64 in a fixed order (the result does not depend on
+ * scheduling).  `workspace` is device memory of Q4ADAMW_NORM_WORKSPACE_BYTES bytes,
+ * 8-byte aligned, overwritten by the call; out3 is three device floats.  All tensors
+ * share g_dtype.
+ */
+#define Q4ADAMW_NORM_WORKSPACE_BYTES 16384
+int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
+                      const float *grad_scale_dev, float max_norm, void *workspace,
+                      size_t workspace_bytes, float *out3, void *stream);
 
 /*
  * Quantize one fp32 moment: per block of 128 consecutive elements the scale is the

@@ -134,3 +134,46 @@ def quant(x, which):
     scale = np.zeros(nblk, np.float32)
     lib().q4o_quant(_ptr(x), x.size, which, _ptr(codes), _ptr(scale))
     return codes, scale
+
+
+# ---------------------------------------------------------------------------
+# gradient-side operations folded into the step
+#
+# The reference has no code for these: its callers zero, unscale and clip the
+# gradients around step() with torch's own routines (caller pattern:
+# tests/driver.py:53-59).  What is restated here is the published arithmetic of
+# those routines: GradScaler.unscale_ multiplies every gradient by a reciprocal
+# scale in fp32; torch.nn.utils.clip_grad_norm_ multiplies by
+# min(1, max_norm / (total_norm + 1e-6)).  Pinned against torch's routines on the
+# CPU (tests/test_oracle_pins.py); parity with the reference itself: UNPINNED, it
+# has no counterpart.
+# ---------------------------------------------------------------------------
+def as_f32(g):
+    """fp32 values of a gradient given as float32 or as bf16 bit patterns (uint16)."""
+    g = np.asarray(g)
+    if g.dtype == np.uint16:
+        return (g.astype(np.uint32) << 16).view(np.float32)
+    return g.astype(np.float32, copy=False)
+
+
+def scale_grad(g, s):
+    """The gradient a step with multiplier s works on: one rounded fp32 product per
+    element.  Feed the result to step_quant / step_unquant as a float32 gradient."""
+    return as_f32(g) * np.float32(s)
+
+
+def grad_norm(gs, s=1.0, max_norm=0.0):
+    """(norm of the gradients times s, clip coefficient, s * coefficient), fp32 each:
+    squares summed in fp64, the rest in fp32 in torch's order."""
+    total = 0.0
+    for g in gs:
+        x = as_f32(g).astype(np.float64)
+        total += float(np.dot(x, x))
+    s = np.float32(s)
+    norm = np.float32(np.abs(s) * np.float32(np.sqrt(total)))
+    coef = np.float32(1.0)
+    if max_norm > 0.0:
+        with np.errstate(over="ignore", invalid="ignore"):
+            coef = np.float32(max_norm) / (norm + np.float32(1e-6))
+        coef = np.float32(1.0) if coef > 1.0 else np.float32(coef)
+    return norm, coef, np.float32(s * coef)

@@ -37,11 +37,34 @@ class Q4SmallTensor(ctypes.Structure):
     ]
 
 
+class Q4GradOptions(ctypes.Structure):
+    """struct q4adamw_grad_options"""
+    _fields_ = [
+        ("grad_scale", ctypes.c_float),
+        ("zero_grad", ctypes.c_int),
+        ("grad_scale_dev", ctypes.c_void_p),
+        ("skip_if_nonzero", ctypes.c_void_p),
+    ]
+
+
+class Q4Grad(ctypes.Structure):
+    """struct q4adamw_grad"""
+    _fields_ = [
+        ("g", ctypes.c_void_p),
+        ("numel", ctypes.c_int64),
+    ]
+
+
+NORM_WORKSPACE_BYTES = 16384
+
 EXPORTS = (
     "q4adamw_fused_4bit",
     "q4adamw_fused_4bit_multi",
+    "q4adamw_fused_4bit_multi_ex",
     "q4adamw_fused_single_tensor",
     "q4adamw_fused_single_tensor_multi",
+    "q4adamw_fused_single_tensor_multi_ex",
+    "q4adamw_grad_norm",
     "q4adamw_quantize",
     "q4adamw_dequantize",
     "q4adamw_derive_scalars",
@@ -76,6 +99,13 @@ def load():
     L.q4adamw_fused_single_tensor.restype = i
     L.q4adamw_fused_single_tensor_multi.argtypes = [ctypes.POINTER(Q4SmallTensor), i, i, i] + hyper + [vp]
     L.q4adamw_fused_single_tensor_multi.restype = i
+    opt = ctypes.POINTER(Q4GradOptions)
+    L.q4adamw_fused_4bit_multi_ex.argtypes = [ctypes.POINTER(Q4Tensor), i, i, i] + hyper + [opt, vp]
+    L.q4adamw_fused_4bit_multi_ex.restype = i
+    L.q4adamw_fused_single_tensor_multi_ex.argtypes = [ctypes.POINTER(Q4SmallTensor), i, i, i] + hyper + [opt, vp]
+    L.q4adamw_fused_single_tensor_multi_ex.restype = i
+    L.q4adamw_grad_norm.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, ctypes.c_size_t, vp, vp]
+    L.q4adamw_grad_norm.restype = i
     L.q4adamw_quantize.argtypes = [vp, i64, i, vp, vp, vp]
     L.q4adamw_quantize.restype = i
     L.q4adamw_dequantize.argtypes = [vp, vp, i64, i, vp, vp]

@@ -54,6 +54,14 @@ struct StepConsts {
   float den_scale, den_eps;
 };
 
+// What a launch does to the gradients besides reading them (kernels with EXT only).
+struct GradOps {
+  float scale;             // host part of the multiplier
+  uint32_t zero;           // non-zero: overwrite the gradients with zeros once they are read
+  const float *scale_dev;  // device part of the multiplier, or null
+  const float *skip;       // device flag, or null: non-zero turns the launch into a no-op
+};
+
 struct TensorDesc {  // 56 bytes
   void *p;
   const void *g;
@@ -72,6 +80,7 @@ struct FusedArgs {
   static constexpr int kCapacity = kMaxTensors;
   static constexpr int kPivots = (kMaxTensors + 7) / 8;
   StepConsts sc;
+  GradOps go;
   int ntensors;
   uint32_t nchunks;        // chunks in this launch
   uint32_t chunks_per_xcd; // ceil(nchunks / 8); the grid has 8 * chunks_per_xcd workgroups
@@ -92,13 +101,37 @@ struct SmallArgs {
   static constexpr int kCapacity = kMaxSmallTensors;
   static constexpr int kPivots = (kMaxSmallTensors + 7) / 8;
   StepConsts sc;
+  GradOps go;
   int ntensors;
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
   SmallDesc desc[kMaxSmallTensors];
 };
 
-static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+// Gradient-norm launch: every workgroup walks chunks of 32 KiB with a grid stride.
+constexpr int kMaxNormTensors = 160;
+constexpr int kNormPartials = Q4ADAMW_NORM_WORKSPACE_BYTES / 8;  // workgroups = fp64 partial sums
+constexpr int kNormChunkBytes = 32768;                          // 8 16-byte loads per thread
+
+struct NormDesc {
+  const void *g;
+  int64_t numel;
+};
+
+struct NormArgs {
+  static constexpr int kCapacity = kMaxNormTensors;
+  static constexpr int kPivots = (kMaxNormTensors + 7) / 8;
+  double *partials;   // kNormPartials sums, one per workgroup
+  uint32_t nchunks;
+  uint32_t first;     // non-zero: the partial sums are overwritten, otherwise added to
+  int ntensors;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  NormDesc desc[kMaxNormTensors];
+};
+
+static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(NormArgs) <= 4096,
+              "kernel arguments are limited to 4 KiB");
 
 // the first-moment bucket table (see q4adamw_tables.h), copied into LDS by every
 // workgroup at start-up, one entry per thread
@@ -257,6 +290,32 @@ __device__ __forceinline__ void store_elems(void *base, uint32_t e0, int nv, con
   }
 }
 
+// zeros over the N elements that load_elems<BF, N, FULL> read
+template <bool BF, int N, bool FULL>
+__device__ __forceinline__ void zero_elems(void *base, uint32_t e0, int nv) {
+  if (FULL) {
+    const u32x4 z4 = {0u, 0u, 0u, 0u};
+    if (BF && N == 4) {
+      const u32x2 z2 = {0u, 0u};
+      __builtin_amdgcn_raw_buffer_store_b64(z2, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else if (BF) {
+      __builtin_amdgcn_raw_buffer_store_b128(z4, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else {
+#pragma unroll
+      for (int k = 0; k < N; k += 4)
+        __builtin_amdgcn_raw_buffer_store_b128(z4, tile_rsrc(base), (e0 + k) * 4, 0, kNt);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      if (j < nv) {
+        if (BF) as_global<uint16_t>(base)[e0 + j] = 0;
+        else as_global<float>(base)[e0 + j] = 0.0f;
+      }
+    }
+  }
+}
+
 template <int N>
 struct Vals {
   float x[N];
@@ -395,9 +454,12 @@ struct Geometry {
 // ---------------------------------------------------------------------------
 // one tile (256 or 512 elements) of one tensor
 // ---------------------------------------------------------------------------
-template <bool PBF, bool GBF, bool FULL>
+// EXT: gradients are multiplied by gscale (one rounded fp32 multiplication per
+// element, before anything else uses them) and, if zero_g, overwritten with zeros.
+template <bool PBF, bool GBF, bool FULL, bool EXT>
 __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int wave, int tid,
-                                             const StepConsts &sc, uint2 *lds, const TableSlot &slot) {
+                                             const StepConsts &sc, uint2 *lds, const TableSlot &slot,
+                                             float gscale, bool zero_g) {
   using G = Geometry<PBF>;
   constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
@@ -424,6 +486,11 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   float p[N], g[N];
   load_elems<PBF, N, FULL>(p_tile, e0, nv, p);
   load_elems<GBF, N, FULL>(g_tile, e0, nv, g);
+  if (EXT) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) g[j] *= gscale;
+    if (zero_g) zero_elems<GBF, N, FULL>(const_cast<void *>(g_tile), e0, nv);
+  }
   uint32_t mw = 0, vw = 0;
   if (FULL) {
     if (N == 4) {
@@ -579,7 +646,15 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   }
 }
 
-template <bool PBF, bool GBF>
+// The launch's gradient multiplier; false if the launch is to do nothing.
+__device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale) {
+  if (go.skip && *as_global<const float>(go.skip) != 0.0f) return false;
+  gscale = go.scale;
+  if (go.scale_dev) gscale *= *as_global<const float>(go.scale_dev);
+  return true;
+}
+
+template <bool PBF, bool GBF, bool EXT>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
   using G = Geometry<PBF>;
   __shared__ uint2 lds[kLdsEntries];
@@ -587,6 +662,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const TableSlot slot = request_table_slot(tid);
   const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;  // whole workgroup: the grid is padded to a multiple of 8
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;  // whole grid
+  const bool zero_g = EXT && args.go.zero != 0u;
   const int t = find_tensor(args, chunk);
   const TensorDesc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -596,23 +674,35 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
     setup_tables(lds, tid, slot);
     return;
   }
-  if (begin + G::kTile <= T.numel) process_tile<PBF, GBF, true>(T, tile, lane, wave, tid, args.sc, lds, slot);
-  else process_tile<PBF, GBF, false>(T, tile, lane, wave, tid, args.sc, lds, slot);
+  if (begin + G::kTile <= T.numel)
+    process_tile<PBF, GBF, true, EXT>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+  else
+    process_tile<PBF, GBF, false, EXT>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
 }
 
 // Non-quantized step for small tensors (cuda_adamw_kernels.cu:100-133): fp32
 // moments in place, same derived scalars and operation order as the fused path.
-template <bool PBF, bool GBF>
+template <bool PBF, bool GBF, bool EXT>
 __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args) {
   const uint32_t chunk = blockIdx.x;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const bool zero_g = EXT && args.go.zero != 0u;
   const int t = find_tensor(args, chunk);
   const SmallDesc &T = args.desc[t];
   const StepConsts &sc = args.sc;
   const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kSmallChunk;
   const int64_t end = base + kSmallChunk < T.numel ? base + kSmallChunk : T.numel;
   for (int64_t i = base + threadIdx.x; i < end; i += 256) {
-    const float gi = GBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.g)[i])
-                         : as_global<const float>(T.g)[i];
+    float gi = GBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.g)[i])
+                   : as_global<const float>(T.g)[i];
+    if (EXT) {
+      gi *= gscale;
+      if (zero_g) {
+        if (GBF) as_global<uint16_t>(const_cast<void *>(T.g))[i] = 0;
+        else as_global<float>(const_cast<void *>(T.g))[i] = 0.0f;
+      }
+    }
     const float pi = PBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.p)[i])
                          : as_global<const float>(T.p)[i];
     const float m = sc.b1 * as_global<const float>(T.m)[i] + sc.r1 * gi;
@@ -627,6 +717,96 @@ __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// global gradient norm (what a caller computes before it clips)
+// ---------------------------------------------------------------------------
+// Sum over a 256-thread workgroup in a fixed order; the result is valid in thread 0.
+__device__ __forceinline__ double workgroup_sum(double x, double *lds4) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, 64);
+  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = x;
+  __syncthreads();
+  return (lds4[0] + lds4[1]) + (lds4[2] + lds4[3]);
+}
+
+// Squares are exact in fp64 and summed there: four accumulators per thread, chunks in
+// grid-stride order, so the sum depends on the tensor list only, not on scheduling.
+template <bool GBF>
+__global__ __launch_bounds__(256) void grad_sumsq_kernel(const NormArgs args) {
+  constexpr int kElemBytes = GBF ? 2 : 4;
+  constexpr int64_t kChunkElems = kNormChunkBytes / kElemBytes;
+  __shared__ double lds4[4];
+  const int tid = threadIdx.x;
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  for (uint32_t chunk = blockIdx.x; chunk < args.nchunks; chunk += kNormPartials) {
+    const int t = find_tensor(args, chunk);
+    const NormDesc &T = args.desc[t];
+    const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kChunkElems;
+    const void *cb = static_cast<const char *>(T.g) + base * kElemBytes;
+    const int64_t rem = T.numel - base;
+    if (rem >= kChunkElems) {
+      u32x4 w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        w[k] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(cb), (uint32_t)(k * 256 + tid) * 16u, 0, kNt);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t u[4] = {w[k].x, w[k].y, w[k].z, w[k].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          if (GBF) {
+            float lo, hi;
+            widen_bf16_pair(u[c], lo, hi);
+            acc[c] = __builtin_fma((double)lo, (double)lo, acc[c]);
+            acc[c] = __builtin_fma((double)hi, (double)hi, acc[c]);
+          } else {
+            const double x = (double)bits2f(u[c]);
+            acc[c] = __builtin_fma(x, x, acc[c]);
+          }
+        }
+      }
+    } else {
+      for (int64_t i = tid; i < rem; i += 256) {
+        const double x = GBF ? (double)bf16_bits_to_f32(as_global<const uint16_t>(cb)[i])
+                             : (double)as_global<const float>(cb)[i];
+        acc[0] = __builtin_fma(x, x, acc[0]);
+      }
+    }
+  }
+  const double total = workgroup_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), lds4);
+  if (tid == 0) {
+    const gptr<double> out = as_global<double>(args.partials) + blockIdx.x;
+    *out = args.first ? total : *out + total;
+  }
+}
+
+__global__ __launch_bounds__(256) void grad_norm_finish_kernel(const double *partials_, float scale,
+                                                               const float *scale_dev, float max_norm,
+                                                               float *out3_) {
+  __shared__ double lds4[4];
+  const gptr<const double> partials = as_global<const double>(partials_);
+  double a = 0.0;
+#pragma unroll
+  for (int k = 0; k < kNormPartials / 256; ++k) a += partials[threadIdx.x * (kNormPartials / 256) + k];
+  const double total = workgroup_sum(a, lds4);
+  if (threadIdx.x == 0) {
+    float s = scale;
+    if (scale_dev) s *= *as_global<const float>(scale_dev);
+    const float norm = __builtin_fabsf(s) * (float)__builtin_sqrt(total);
+    // torch.nn.utils.clip_grad_norm_: max_norm / (total_norm + 1e-6), clamped to 1
+    // (a NaN stays a NaN)
+    float coef = 1.0f;
+    if (max_norm > 0.0f) {
+      coef = max_norm / (norm + 1e-6f);
+      coef = coef > 1.0f ? 1.0f : coef;
+    }
+    const gptr<float> out3 = as_global<float>(out3_);
+    out3[0] = norm;
+    out3[1] = coef;
+    out3[2] = s * coef;
+  }
+}
 
 // ---------------------------------------------------------------------------
 // stand-alone quantize / dequantize of one moment (checkpoint interchange)
@@ -769,20 +949,51 @@ static int launch_small_batch(SmallArgs &a, uint64_t chunks, void (*kernel)(cons
 typedef void (*FusedKernel)(const FusedArgs);
 typedef void (*SmallKernel)(const SmallArgs);
 
-static FusedKernel pick_fused(int p_dtype, int g_dtype) {
-  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  if (!pb && !gb) return fused_4bit_kernel<false, false>;
-  if (!pb && gb) return fused_4bit_kernel<false, true>;
-  if (pb && !gb) return fused_4bit_kernel<true, false>;
-  return fused_4bit_kernel<true, true>;
+template <bool EXT>
+static FusedKernel pick_fused_ext(bool pb, bool gb) {
+  if (!pb && !gb) return fused_4bit_kernel<false, false, EXT>;
+  if (!pb && gb) return fused_4bit_kernel<false, true, EXT>;
+  if (pb && !gb) return fused_4bit_kernel<true, false, EXT>;
+  return fused_4bit_kernel<true, true, EXT>;
 }
 
-static SmallKernel pick_small(int p_dtype, int g_dtype) {
+static FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext) {
   const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  if (!pb && !gb) return single_tensor_kernel<false, false>;
-  if (!pb && gb) return single_tensor_kernel<false, true>;
-  if (pb && !gb) return single_tensor_kernel<true, false>;
-  return single_tensor_kernel<true, true>;
+  return ext ? pick_fused_ext<true>(pb, gb) : pick_fused_ext<false>(pb, gb);
+}
+
+template <bool EXT>
+static SmallKernel pick_small_ext(bool pb, bool gb) {
+  if (!pb && !gb) return single_tensor_kernel<false, false, EXT>;
+  if (!pb && gb) return single_tensor_kernel<false, true, EXT>;
+  if (pb && !gb) return single_tensor_kernel<true, false, EXT>;
+  return single_tensor_kernel<true, true, EXT>;
+}
+
+static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
+  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
+  return ext ? pick_small_ext<true>(pb, gb) : pick_small_ext<false>(pb, gb);
+}
+
+// Fills the kernels' view of the caller's gradient options; returns whether the
+// launch needs the EXT kernels (false: the options change nothing).
+static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext) {
+  go->scale = 1.0f;
+  go->zero = 0u;
+  go->scale_dev = nullptr;
+  go->skip = nullptr;
+  *ext = false;
+  if (!opt) return 0;
+  if (opt->grad_scale_dev && (reinterpret_cast<uintptr_t>(opt->grad_scale_dev) & 3))
+    return fail(Q4ADAMW_ERR_ALIGN, "grad_scale_dev must be 4-byte aligned");
+  if (opt->skip_if_nonzero && (reinterpret_cast<uintptr_t>(opt->skip_if_nonzero) & 3))
+    return fail(Q4ADAMW_ERR_ALIGN, "skip_if_nonzero must be 4-byte aligned");
+  go->scale = opt->grad_scale;
+  go->zero = opt->zero_grad ? 1u : 0u;
+  go->scale_dev = opt->grad_scale_dev;
+  go->skip = opt->skip_if_nonzero;
+  *ext = opt->grad_scale != 1.0f || opt->zero_grad || opt->grad_scale_dev || opt->skip_if_nonzero;
+  return 0;
 }
 
 constexpr uint64_t kMaxChunksPerLaunch = 0x7ffffff0ull;  // grid.x limit, with room for padding to 8
@@ -830,10 +1041,19 @@ int q4adamw_mtable_half_bucket(uint32_t half_index) {
 int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,
                              float beta1, float beta2, float lr, float weight_decay, float eps,
                              float step, void *stream) {
+  return q4adamw_fused_4bit_multi_ex(tensors, count, p_dtype, g_dtype, beta1, beta2, lr,
+                                     weight_decay, eps, step, nullptr, stream);
+}
+
+int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,
+                                float beta1, float beta2, float lr, float weight_decay, float eps,
+                                float step, const q4adamw_grad_options *opt, void *stream) {
   if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   FusedArgs a;
+  bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
+  if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
   // a lane reads 4 (fp32 parameters) or 8 (bf16 parameters) consecutive elements at once
   const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
   const int64_t chunk_elems = p_bf16 ? Geometry<true>::kChunk : Geometry<false>::kChunk;
@@ -855,7 +1075,7 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const FusedKernel kernel = pick_fused(p_dtype, g_dtype);
+  const FusedKernel kernel = pick_fused(p_dtype, g_dtype, ext);
   a.ntensors = 0;
   uint64_t chunks = 0;
   for (int i = 0; i < count; ++i) {
@@ -895,10 +1115,20 @@ int q4adamw_fused_4bit(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_av
 int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int count, int p_dtype,
                                       int g_dtype, float beta1, float beta2, float lr,
                                       float weight_decay, float eps, float step, void *stream) {
+  return q4adamw_fused_single_tensor_multi_ex(tensors, count, p_dtype, g_dtype, beta1, beta2, lr,
+                                              weight_decay, eps, step, nullptr, stream);
+}
+
+int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, int count,
+                                         int p_dtype, int g_dtype, float beta1, float beta2,
+                                         float lr, float weight_decay, float eps, float step,
+                                         const q4adamw_grad_options *opt, void *stream) {
   if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   SmallArgs a;
+  bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
+  if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
   const uintptr_t pa = p_dtype == Q4ADAMW_BF16 ? 2 : 4, ga = g_dtype == Q4ADAMW_BF16 ? 2 : 4;
   for (int i = 0; i < count; ++i) {
     const q4adamw_small_tensor &t = tensors[i];
@@ -912,7 +1142,7 @@ int q4adamw_fused_single_tensor_multi(const q4adamw_small_tensor *tensors, int c
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const SmallKernel kernel = pick_small(p_dtype, g_dtype);
+  const SmallKernel kernel = pick_small(p_dtype, g_dtype, ext);
   a.ntensors = 0;
   uint64_t chunks = 0;
   for (int i = 0; i < count; ++i) {
@@ -945,6 +1175,65 @@ int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *e
   q4adamw_small_tensor t = {p, g, exp_avg, exp_avg_sq, numel};
   return q4adamw_fused_single_tensor_multi(&t, 1, p_dtype, g_dtype, beta1, beta2, lr,
                                            weight_decay, eps, step, stream);
+}
+
+int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
+                      const float *grad_scale_dev, float max_norm, void *workspace,
+                      size_t workspace_bytes, float *out3, void *stream) {
+  if (count < 0 || (count > 0 && !grads)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
+  if (int rc = check_dtypes(Q4ADAMW_FP32, g_dtype)) return rc;
+  if (!workspace || !out3) return fail(Q4ADAMW_ERR_ARG, "null workspace or output");
+  if (workspace_bytes < Q4ADAMW_NORM_WORKSPACE_BYTES)
+    return fail(Q4ADAMW_ERR_ARG, "workspace smaller than Q4ADAMW_NORM_WORKSPACE_BYTES");
+  if (!aligned(workspace, 8) || !aligned(out3, 4) || (grad_scale_dev && !aligned(grad_scale_dev, 4)))
+    return fail(Q4ADAMW_ERR_ALIGN, "workspace must be 8-byte, scalars 4-byte aligned");
+  const bool bf16 = g_dtype == Q4ADAMW_BF16;
+  const int64_t chunk_elems = kNormChunkBytes / (bf16 ? 2 : 4);
+  for (int i = 0; i < count; ++i) {
+    if (grads[i].numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
+    if (grads[i].numel == 0) continue;
+    if (!grads[i].g) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+    if (!aligned(grads[i].g, 16)) return fail(Q4ADAMW_ERR_ALIGN, "gradients must be 16-byte aligned");
+    if ((uint64_t)(grads[i].numel + chunk_elems - 1) / chunk_elems > kMaxChunksPerLaunch)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  NormArgs a;
+  a.partials = static_cast<double *>(workspace);
+  a.first = 1u;
+  a.ntensors = 0;
+  uint64_t chunks = 0;
+  auto launch = [&]() -> int {
+    finish_prefix(a);
+    a.nchunks = (uint32_t)chunks;
+    if (bf16) hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(kNormPartials), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(kNormPartials), dim3(256), 0, s, a);
+    Q4_HIP(hipGetLastError());
+    a.first = 0u;
+    a.ntensors = 0;
+    chunks = 0;
+    return 0;
+  };
+  for (int i = 0; i < count; ++i) {
+    if (grads[i].numel == 0) continue;
+    const uint64_t c = (uint64_t)(grads[i].numel + chunk_elems - 1) / chunk_elems;
+    if (a.ntensors == kMaxNormTensors || chunks + c > kMaxChunksPerLaunch) {
+      if (int rc = launch()) return rc;
+    }
+    a.desc[a.ntensors].g = grads[i].g;
+    a.desc[a.ntensors].numel = grads[i].numel;
+    a.first_chunk[a.ntensors] = (uint32_t)chunks;
+    ++a.ntensors;
+    chunks += c;
+  }
+  // the first launch also defines every partial sum, so an empty list still takes one
+  if (a.ntensors > 0 || a.first) {
+    if (int rc = launch()) return rc;
+  }
+  hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(256), 0, s,
+                     static_cast<const double *>(workspace), grad_scale, grad_scale_dev, max_norm, out3);
+  Q4_HIP(hipGetLastError());
+  return 0;
 }
 
 int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, float *scales,
@@ -982,6 +1271,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1002; }
+int q4adamw_version(void) { return 1003; }
 
 }  // extern "C"

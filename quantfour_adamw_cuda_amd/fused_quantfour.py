@@ -17,6 +17,12 @@ behaviour where the reference's draft is unfinished:
     of one launch plus one device synchronisation per tensor
     (fused_quantfour.py:171-292)
 
+Beyond the reference's `step(closure)`: keyword arguments fold what its callers do
+to the gradients between backward and step (tests/driver.py:53-59) into the step's
+single read of them -- a multiplier (loss-scale removal), global-norm clipping, an
+overflow flag that skips the step, and zeroing.  torch.amp.GradScaler.step() drives
+the same path through the `grad_scale` / `found_inf` attributes it sets.
+
 The step itself runs only in the HIP library (csrc/libq4adamw.so); without it,
 or with parameters that are not on a GPU, `step()` raises.
 """
@@ -77,6 +83,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         )
         super().__init__(params, defaults)
         self._launch_cache: Dict[Any, Any] = {}
+        # global gradient norm of the last step(max_grad_norm=...), a device scalar
+        self.last_grad_norm = None
+        self._norm_buffers: Dict[Any, Any] = {}
         # set to a list to collect ("fused_4bit" | "fused_single_tensor", start, end)
         # event triples around every launch, recorded on the launch stream
         self.kernel_timing = None
@@ -97,7 +106,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         """optim/fused_quantfour.py:73-84"""
         super().__setstate__(state)
         self._launch_cache = {}
+        self._norm_buffers = {}
         self.__dict__.setdefault("kernel_timing", None)
+        self.__dict__.setdefault("last_grad_norm", None)
         for group in self.param_groups:
             group.setdefault("fused", None)
         state_values = list(self.state.values())
@@ -238,13 +249,79 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         return {"state": out_state, "param_groups": groups}
 
     # -- step -------------------------------------------------------------
+    # torch.amp.GradScaler.step() hands its scale and overflow flag to an optimizer that
+    # declares this, as attributes `grad_scale` and `found_inf`, instead of unscaling
+    # the gradients in a pass of its own
+    _step_supports_amp_scaling = True
+
+    def _grad_multiplier(self, grad_scale, max_grad_norm):
+        """(host float, device float32 scalar or None): the factor every gradient is
+        multiplied by inside the step."""
+        host, dev = 1.0, None
+        if torch.is_tensor(grad_scale):
+            dev = grad_scale.detach().to(torch.float32).reshape(1)
+        elif grad_scale is not None:
+            host = float(grad_scale)
+        amp_scale = getattr(self, "grad_scale", None)   # set by GradScaler: divide by it
+        if amp_scale is not None:
+            inv = amp_scale.detach().double().reciprocal().float().reshape(1)
+            dev = inv if dev is None else dev * inv
+        if max_grad_norm is None:
+            return host, dev
+        # global norm of the multiplied gradients, per dtype on the device, combined there
+        by_dtype: Dict[Any, list] = {}
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.grad is not None:
+                    by_dtype.setdefault((p.grad.device, p.grad.dtype), []).append(p.grad)
+        if not by_dtype:
+            return host, dev
+        devices = {d for d, _ in by_dtype}
+        assert len(devices) == 1, "max_grad_norm needs all gradients on one device"
+        device = devices.pop()
+        outs = []
+        for key, gs in by_dtype.items():
+            bufs = self._norm_buffers.get(key)
+            if bufs is None:
+                bufs = (torch.empty(3, dtype=torch.float32, device=device),
+                        torch.empty(_lib.NORM_WORKSPACE_BYTES // 8, dtype=torch.float64, device=device))
+                self._norm_buffers[key] = bufs
+            outs.append(_q.grad_norm(gs, host, dev, float(max_grad_norm), out=bufs[0], workspace=bufs[1]))
+        if len(outs) == 1:
+            self.last_grad_norm = outs[0][0]
+            return 1.0, outs[0][2:3]
+        total = torch.linalg.vector_norm(torch.stack([o[0] for o in outs]))
+        coef = torch.clamp(float(max_grad_norm) / (total + 1e-6), max=1.0)
+        self.last_grad_norm = total
+        mult = coef * host if dev is None else coef * host * dev
+        return 1.0, mult.reshape(1)
+
     @torch.no_grad()
-    def step(self, closure=None):
-        """single optimization step"""
+    def step(self, closure=None, *, grad_scale=None, found_inf=None, max_grad_norm=None,
+             zero_grad=False):
+        """single optimization step
+
+        grad_scale     number or one-element tensor: every gradient is multiplied by it
+                       inside the step (e.g. 1 / loss scale); the stored gradients stay
+                       as they are
+        max_grad_norm  clip the (multiplied) gradients to this global L2 norm, as
+                       torch.nn.utils.clip_grad_norm_ would, without rewriting them;
+                       the norm is left in `last_grad_norm` (a device scalar)
+        found_inf      one-element float32 device tensor: a non-zero value makes the
+                       step a no-op on the device, without synchronising; the step
+                       counters advance regardless
+        zero_grad      overwrite the gradients with zeros once the step has read them
+        """
         loss = None
         if closure:
             with torch.enable_grad():
                 loss = closure()
+
+        if found_inf is None:
+            found_inf = getattr(self, "found_inf", None)    # set by GradScaler
+        if found_inf is not None:
+            found_inf = found_inf.detach().to(torch.float32).reshape(1)
+        host_mult, dev_mult = self._grad_multiplier(grad_scale, max_grad_norm)
 
         _lib.load()  # raises if the HIP library has not been built
 
@@ -311,14 +388,15 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                     self._launch_cache[cache_key] = cached
                 _, arr, (p_tag, g_tag) = cached
                 launch = _q.launch_table if quantized else _q.launch_small_table
+                options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad)
                 if self.kernel_timing is None:
-                    launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step)
+                    launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                 else:
                     with torch.cuda.device(device):
                         start = torch.cuda.Event(enable_timing=True)
                         end = torch.cuda.Event(enable_timing=True)
                         start.record()
-                        launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step)
+                        launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                         end.record()
                     kind = "fused_4bit" if quantized else "fused_single_tensor"
                     self.kernel_timing.append((kind, start, end))

@@ -110,25 +110,49 @@ def make_small_table(ps, gs, exp_avgs, exp_avg_sqs):
     return arr
 
 
-def launch_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step):
+def _device_scalar(t, device, what):
+    assert t.is_cuda and t.device == device, f"{what} must be on the tensors' device"
+    assert t.dtype == torch.float32 and t.numel() == 1, f"{what} must hold one float32"
+    return t.data_ptr()
+
+
+def grad_options(device, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False):
+    """struct q4adamw_grad_options, or None when the arguments change nothing.  The device
+    scalars are referenced, not copied: keep the tensors alive until the step has run."""
+    if grad_scale == 1.0 and grad_scale_dev is None and found_inf is None and not zero_grad:
+        return None
+    o = _lib.Q4GradOptions()
+    o.grad_scale = float(grad_scale)
+    o.zero_grad = 1 if zero_grad else 0
+    o.grad_scale_dev = None if grad_scale_dev is None else _device_scalar(grad_scale_dev, device, "grad_scale_dev")
+    o.skip_if_nonzero = None if found_inf is None else _device_scalar(found_inf, device, "found_inf")
+    return o
+
+
+def launch_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options=None):
     L = _lib.load()
     with torch.cuda.device(device):
-        rc = L.q4adamw_fused_4bit_multi(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
-                                        weight_decay, eps, float(step), _stream(device))
+        rc = L.q4adamw_fused_4bit_multi_ex(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
+                                           weight_decay, eps, float(step), options, _stream(device))
     _lib.check(rc, "fused_4bit_multi")
 
 
-def launch_small_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step):
+def launch_small_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step,
+                       options=None):
     L = _lib.load()
     with torch.cuda.device(device):
-        rc = L.q4adamw_fused_single_tensor_multi(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
-                                                 weight_decay, eps, float(step), _stream(device))
+        rc = L.q4adamw_fused_single_tensor_multi_ex(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
+                                                    weight_decay, eps, float(step), options,
+                                                    _stream(device))
     _lib.check(rc, "fused_single_tensor_multi")
 
 
 def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr, weight_decay,
-                     eps, step):
-    """One launch over many quantized tensors that share device, dtypes and step."""
+                     eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False):
+    """One launch over many quantized tensors that share device, dtypes and step.  The
+    gradients enter the step multiplied by grad_scale * grad_scale_dev (a device float32
+    scalar); found_inf (a device float32 scalar) turns the call into a no-op when it holds a
+    non-zero value; zero_grad overwrites the gradients with zeros once they are read."""
     if not ps:
         return
     arr = make_table(ps, gs, exps, sqs, exp_scales, sq_scales)
@@ -136,12 +160,15 @@ def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr,
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    launch_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    launch_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
 
 
 def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, weight_decay,
-                              eps, step):
-    """One launch over many non-quantized tensors that share device, dtypes and step."""
+                              eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None,
+                              zero_grad=False):
+    """One launch over many non-quantized tensors that share device, dtypes and step; gradient
+    options as for fused_4bit_multi."""
     if not ps:
         return
     arr = make_small_table(ps, gs, exp_avgs, exp_avg_sqs)
@@ -149,7 +176,50 @@ def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, w
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    launch_small_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    launch_small_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step,
+                       options)
+
+
+def make_grad_table(gs):
+    """ctypes descriptor array for grad_norm_table (gradients validated)."""
+    arr = (_lib.Q4Grad * len(gs))()
+    for i, g in enumerate(gs):
+        assert g.is_cuda and g.device == gs[0].device, "gradients must share a cuda device"
+        assert g.is_contiguous(), "grad must be contiguous"
+        assert g.dtype == gs[0].dtype, "gradients of one call must share a dtype"
+        arr[i].g, arr[i].numel = g.data_ptr(), g.numel()
+    return arr
+
+
+def grad_norm_table(arr, device, g_tag, out3, workspace, grad_scale=1.0, grad_scale_dev=None,
+                    max_norm=0.0):
+    L = _lib.load()
+    assert out3.dtype == torch.float32 and out3.numel() >= 3 and out3.device == device
+    assert workspace.device == device and workspace.numel() * workspace.element_size() >= _lib.NORM_WORKSPACE_BYTES
+    dev_ptr = None if grad_scale_dev is None else _device_scalar(grad_scale_dev, device, "grad_scale_dev")
+    with torch.cuda.device(device):
+        rc = L.q4adamw_grad_norm(arr, len(arr), g_tag, float(grad_scale), dev_ptr, float(max_norm),
+                                 workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+                                 out3.data_ptr(), _stream(device))
+    _lib.check(rc, "grad_norm")
+
+
+def grad_norm(gs, grad_scale=1.0, grad_scale_dev=None, max_norm=0.0, out=None, workspace=None):
+    """Global L2 norm of the gradients `gs` (one dtype, one device) and the clip coefficient of
+    torch.nn.utils.clip_grad_norm_.  Returns a device float32[3]: the norm of the gradients
+    times s = grad_scale * grad_scale_dev, min(1, max_norm / (norm + 1e-6)) (1 when max_norm
+    <= 0), and s times that coefficient -- the multiplier to pass to a step as
+    grad_scale_dev.  Nothing is synchronised."""
+    assert len(gs) > 0, "no gradients"
+    device = gs[0].device
+    if out is None:
+        out = torch.empty(3, dtype=torch.float32, device=device)
+    if workspace is None:
+        workspace = torch.empty(_lib.NORM_WORKSPACE_BYTES // 8, dtype=torch.float64, device=device)
+    grad_norm_table(make_grad_table(gs), device, _tag(gs[0], "grad"), out, workspace, grad_scale,
+                    grad_scale_dev, max_norm)
+    return out
 
 
 def quantize_state(x, which):

@@ -257,3 +257,55 @@ def test_quantized_step_tracks_adamw_like_the_reference_test():
         oc.step_quant(p, g.numpy(), m, v, sm, sv, step=step, **HP_DRIVER)
         torch.testing.assert_close(torch.from_numpy(p), ref.detach(), atol=0.025, rtol=1e-5)
     assert not np.array_equal(p, p0.numpy())
+
+
+# ---------------------------------------------------------------------------
+# gradient-side operations: pinned against torch's own routines on the CPU
+# ---------------------------------------------------------------------------
+def test_grad_norm_matches_torch_clip_grad_norm():
+    gen = torch.Generator().manual_seed(11)
+    for max_norm in (0.05, 1.0, 1e3):
+        params = [torch.nn.Parameter(torch.zeros(n)) for n in (1, 127, 4096, 100003)]
+        for p in params:
+            p.grad = torch.randn(p.numel(), generator=gen) * 1e-2
+        before = [p.grad.clone() for p in params]
+        total = torch.nn.utils.clip_grad_norm_(params, max_norm)
+        norm, coef, mult = oc.grad_norm([g.numpy() for g in before], 1.0, max_norm)
+        assert abs(float(norm) - float(total)) <= 2e-6 * float(total)
+        assert mult == coef
+        # what the routine did to the gradients is a multiplication by the coefficient
+        for p, g0 in zip(params, before):
+            want = g0 * float(coef)
+            assert torch.allclose(p.grad, want, rtol=3e-6, atol=0.0)
+        assert (float(coef) == 1.0) == (float(total) + 1e-6 <= max_norm)
+
+
+def test_grad_norm_closed_forms():
+    ones = np.ones(1 << 20, np.float32)
+    norm, coef, mult = oc.grad_norm([ones, ones[:3]], s=-0.5, max_norm=0.0)
+    assert norm == np.float32(0.5 * np.sqrt((1 << 20) + 3)) and coef == 1.0 and mult == np.float32(-0.5)
+    # bf16 bit patterns: 0x4000 = 2.0
+    twos = np.full(9, 0x4000, np.uint16)
+    norm, coef, mult = oc.grad_norm([twos], s=1.0, max_norm=3.0)
+    assert norm == np.float32(6.0)
+    assert coef == np.float32(3.0) / (np.float32(6.0) + np.float32(1e-6)) and mult == coef
+    assert oc.grad_norm([np.zeros(5, np.float32)], 1.0, 1.0)[1] == 1.0      # 1 / 1e-6 clamps to 1
+    n, c, _ = oc.grad_norm([np.array([np.inf], np.float32)], 1.0, 1.0)
+    assert np.isinf(n) and c == 0.0
+    n, c, _ = oc.grad_norm([np.array([np.nan], np.float32)], 1.0, 1.0)
+    assert np.isnan(n) and np.isnan(c)
+
+
+def test_scale_grad_is_unscale():
+    """GradScaler.unscale_ multiplies by the fp32 reciprocal of the scale; for the power-of-two
+    scales it uses that equals dividing, and for bf16 bit patterns the widening is exact."""
+    gen = torch.Generator().manual_seed(12)
+    g = torch.randn(5000, generator=gen)
+    for scale in (65536.0, 2.0 ** 10):
+        inv = torch.tensor(scale).double().reciprocal().float()
+        want = (g * inv).numpy()
+        assert np.array_equal(oc.scale_grad(g.numpy(), float(inv)), want)
+        assert np.array_equal(want, (g / scale).numpy())
+    gb = g.to(torch.bfloat16)
+    got = oc.scale_grad(gb.view(torch.int16).numpy().view(np.uint16), 0.3)
+    assert np.array_equal(got, (gb.float() * np.float32(0.3)).numpy())
