@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # WRITE_SIZE (each scaled by what the same counter reads for a 4 GiB device copy: 2.0 and 1.0);
 # summary in profiles/fused_4bit_kernel_llama3_8b_hbm_counters.txt.  Workloads that have not
 # been profiled report null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {"llama3-8b": 9.7364e10}
+MEASURED_TRAFFIC_BYTES_PER_STEP = {"llama3-8b": 9.7365e10}
 HP = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 
 
@@ -275,10 +275,15 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_STEP.get(args.workload),
+            # per launch, averaged over the step's launches (they differ in size): measured
+            # HBM bytes, algorithmic bytes, duration; achieved = algorithmic bytes / duration
+            "traffic": (MEASURED_TRAFFIC_BYTES_PER_STEP[args.workload] / launches_per_step
+                        if args.workload in MEASURED_TRAFFIC_BYTES_PER_STEP else None),
+            "algorithmic_bytes_per_launch": algo_bytes / launches_per_step,
+            "kernel_ms_per_launch": avg_kernel_s * 1e3 / launches_per_step,
+            "kernel_launches_per_step": launches_per_step,
             "algorithmic_bytes_per_step": algo_bytes,
             "kernel_ms_per_step": avg_kernel_s * 1e3,
-            "kernel_launches_per_step": launches_per_step,
         },
     }
     if not args.no_cpu_baseline:
