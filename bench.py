@@ -175,6 +175,10 @@ def main():
     ap.add_argument("--workload", default="llama3-8b", choices=sorted(WORKLOADS))
     ap.add_argument("--grad-sets", type=int, default=2,
                     help="distinct pre-generated gradient sets rotated over the steps")
+    ap.add_argument("--clip", choices=["none", "fused", "separate"], default="none",
+                    help="also unscale the gradients by 1/1024 and clip them to a global norm of 1.0 "
+                         "in every step: 'fused' = norm kernel + multiplier inside the step, "
+                         "'separate' = torch's foreach multiply and clip_grad_norm_ passes, then the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, run a plain 4 GiB device copy three times, so that "
@@ -216,7 +220,14 @@ def main():
         gs = grad_sets[i % len(grad_sets)]
         for p, g in zip(params, gs):
             p.grad = g
-        opt.step()
+        if args.clip == "fused":
+            opt.step(grad_scale=1.0 / 1024.0, max_grad_norm=1.0)
+        elif args.clip == "separate":
+            torch._foreach_mul_(gs, 1.0 / 1024.0)
+            torch.nn.utils.clip_grad_norm_(params, 1.0, foreach=True)
+            opt.step()
+        else:
+            opt.step()
 
     for i in range(args.warmup):
         one_step(i)
@@ -286,6 +297,15 @@ def main():
             "kernel_ms_per_step": avg_kernel_s * 1e3,
         },
     }
+    if args.clip != "none":
+        out["config"]["workload"] += f"; gradients unscaled by 1/1024 and clipped to norm 1.0 ({args.clip})"
+        norm_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "grad_norm"]
+        if norm_ms:
+            g_bytes = sum(g.numel() * g.element_size() for g in grad_sets[0])
+            norm_s = sum(norm_ms) / args.steps / 1e3
+            out["grad_norm"] = {"bound": "hbm", "kernel": "grad_sumsq_kernel", "ms_per_step": norm_s * 1e3,
+                                "algorithmic_bytes_per_step": g_bytes, "achieved": g_bytes / norm_s / 1e9,
+                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g_bytes / norm_s / 1e9 / HBM_PEAK_GBS}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, params, grad_sets[0], HP)
     print(json.dumps(out), flush=True)

@@ -86,7 +86,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # global gradient norm of the last step(max_grad_norm=...), a device scalar
         self.last_grad_norm = None
         self._norm_buffers: Dict[Any, Any] = {}
-        # set to a list to collect ("fused_4bit" | "fused_single_tensor", start, end)
+        # set to a list to collect ("fused_4bit" | "fused_single_tensor" | "grad_norm", start, end)
         # event triples around every launch, recorded on the launch stream
         self.kernel_timing = None
 
@@ -286,7 +286,16 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 bufs = (torch.empty(3, dtype=torch.float32, device=device),
                         torch.empty(_lib.NORM_WORKSPACE_BYTES // 8, dtype=torch.float64, device=device))
                 self._norm_buffers[key] = bufs
-            outs.append(_q.grad_norm(gs, host, dev, float(max_grad_norm), out=bufs[0], workspace=bufs[1]))
+            if self.kernel_timing is None:
+                outs.append(_q.grad_norm(gs, host, dev, float(max_grad_norm), out=bufs[0], workspace=bufs[1]))
+            else:
+                with torch.cuda.device(device):
+                    start = torch.cuda.Event(enable_timing=True)
+                    end = torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    outs.append(_q.grad_norm(gs, host, dev, float(max_grad_norm), out=bufs[0], workspace=bufs[1]))
+                    end.record()
+                self.kernel_timing.append(("grad_norm", start, end))
         if len(outs) == 1:
             self.last_grad_norm = outs[0][0]
             return 1.0, outs[0][2:3]
