@@ -132,6 +132,45 @@ int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_
                                 const q4adamw_grad_options *opt, void *stream);
 
 /*
+ * One quantized matrix whose second moment is rank-1 scaled: the scale of element
+ * (i, j) is min(row_max[i], col_max[j]), the maxima of the second moment over row i
+ * and over column j (get_variance_tensor_statistics / compute_variance_tensor_scale,
+ * optim/adamw_fourbit_triton.py:738-755; scale_type "rank1", :124).  The first moment
+ * keeps its per-128 block scales.  row_max/col_max (rows and cols floats) are
+ * updated by the call; row_max_next/col_max_next are state-owned scratch of the same
+ * sizes that must hold zeros on entry and holds zeros again afterwards.
+ * rows x cols, row-major, cols a multiple of 8 and at least 512; p, g, col_max and
+ * col_max_next 16-byte aligned, the rest 4-byte aligned.
+ */
+typedef struct q4adamw_rank1_tensor {
+  void *p;
+  const void *g;
+  uint8_t *exp_avg;
+  uint8_t *exp_avg_sq;
+  float *exp_avg_scale;
+  float *row_max;
+  float *col_max;
+  float *row_max_next;
+  float *col_max_next;
+  int64_t rows;
+  int64_t cols;
+} q4adamw_rank1_tensor;
+
+/*
+ * The fused step with a rank-1-scaled second moment, per batch of up to 32 tensors
+ * three launches: new second moments reduced to row and column maxima, the update
+ * (dequantize with the old maxima, quantize with the new ones), and the commit of the
+ * new maxima.  Everything else as q4adamw_fused_4bit_multi_ex (opt may be NULL).  The
+ * device form of variance_quant / variance_dequant with scale_type "rank1"
+ * (optim/adamw_fourbit_triton.py:498-527, :803-863) inside the fused step
+ * (optim/cuda_adamw_kernels.cu:266-419).
+ */
+int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
+                                   int g_dtype, float beta1, float beta2, float lr,
+                                   float weight_decay, float eps, float step,
+                                   const q4adamw_grad_options *opt, void *stream);
+
+/*
  * Non-quantized AdamW step (fp32 moments) on one tensor.
  * Replaces fused_single_tensor (optim/cuda_fused_interface.cc:49-64) and
  * cuda_fused_single_tensor (optim/cuda_adamw_kernels.cu:136-164).

@@ -128,6 +128,56 @@ def step_unquant(p, g, m, v, *, beta1, beta2, lr, weight_decay, eps, step):
     return p_new.to(p.dtype).view_as(p), m_new, v_new
 
 
+# ---------------------------------------------------------------------------
+# rank-1 scaling of the second moment (2-D tensors)
+#
+# The reference sketches it in its PyTorch draft only: statistics = per-row and
+# per-column maxima (get_variance_tensor_statistics / max_reduce_except_dim,
+# optim/adamw_fourbit_triton.py:738-746, :1080-1090), scale tensor = their
+# broadcast minimum (compute_variance_tensor_scale, :749-755; sqs_scale_tensor,
+# :537-545), quantize x.div(scale) (:834-863), dequantize x.mul(scale) (:520-527).
+# The code book stays the fused path's linear map.  The draft never runs this
+# against data, so parity with the reference is UNPINNED; the functions are pinned
+# by brute force on small matrices and by closed forms (tests/test_oracle_pins.py).
+# ---------------------------------------------------------------------------
+def rank1_scale(row_max, col_max):
+    """compute_variance_tensor_scale for a matrix: min(row_max[i], col_max[j])."""
+    return torch.minimum(row_max.reshape(-1, 1), col_max.reshape(1, -1))
+
+
+def dequantize_rank1(codes, row_max, col_max):
+    rows, cols = row_max.numel(), col_max.numel()
+    idx = unpack(codes, rows * cols)
+    vals = QMAP[1].to(codes.device)[idx].view(rows, cols)
+    return vals * rank1_scale(row_max, col_max)
+
+
+def quantize_rank1(x):
+    """x: fp32 matrix (non-negative).  Returns (packed codes, row_max, col_max)."""
+    ax = x.abs()
+    row_max = ax.amax(dim=1)                                 # max over all dims except 0
+    col_max = ax.amax(dim=0)                                 # max over all dims except 1
+    qx = x.div(rank1_scale(row_max, col_max))                # 0/0 -> NaN -> code 0
+    q = torch.bucketize(torch.nan_to_num(qx, nan=-2.0), QMID[1].to(x.device), right=False)
+    return pack(q.reshape(-1), x.numel()), row_max, col_max
+
+
+def step_quant_rank1(p, g, m_codes, v_codes, m_scale, row_max, col_max, *, beta1, beta2, lr,
+                     weight_decay, eps, step):
+    """The fused step with block-scaled first moment and rank-1-scaled second moment.
+    p, g: matrices [rows, cols].  Returns new (p, m_codes, v_codes, m_scale, row_max,
+    col_max)."""
+    rows, cols = p.shape
+    numel = p.numel()
+    sc = derive_scalars(beta1, beta2, lr, weight_decay, step)
+    m = dequantize(m_codes, m_scale, numel, 0)
+    v = dequantize_rank1(v_codes, row_max, col_max).reshape(-1)
+    p_new, m_new, v_new = adamw_update(p.reshape(-1).float(), g.reshape(-1).float(), m, v, sc, eps)
+    mc, ms = quantize(m_new, 0)
+    vc, rmax, cmax = quantize_rank1(v_new.view(rows, cols))
+    return p_new.to(p.dtype).view_as(p), mc, vc, ms, rmax, cmax
+
+
 def closed_form_tables():
     """Independent constructions of the four tables (double precision, then fp32):
     second moment k/16 and (2k+1)/32 (quant_opt_base.py:88-102); first moment from

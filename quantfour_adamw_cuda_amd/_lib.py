@@ -37,6 +37,23 @@ class Q4SmallTensor(ctypes.Structure):
     ]
 
 
+class Q4Rank1Tensor(ctypes.Structure):
+    """struct q4adamw_rank1_tensor"""
+    _fields_ = [
+        ("p", ctypes.c_void_p),
+        ("g", ctypes.c_void_p),
+        ("exp_avg", ctypes.c_void_p),
+        ("exp_avg_sq", ctypes.c_void_p),
+        ("exp_avg_scale", ctypes.c_void_p),
+        ("row_max", ctypes.c_void_p),
+        ("col_max", ctypes.c_void_p),
+        ("row_max_next", ctypes.c_void_p),
+        ("col_max_next", ctypes.c_void_p),
+        ("rows", ctypes.c_int64),
+        ("cols", ctypes.c_int64),
+    ]
+
+
 class Q4GradOptions(ctypes.Structure):
     """struct q4adamw_grad_options"""
     _fields_ = [
@@ -61,6 +78,7 @@ EXPORTS = (
     "q4adamw_fused_4bit",
     "q4adamw_fused_4bit_multi",
     "q4adamw_fused_4bit_multi_ex",
+    "q4adamw_fused_4bit_rank1_multi",
     "q4adamw_fused_single_tensor",
     "q4adamw_fused_single_tensor_multi",
     "q4adamw_fused_single_tensor_multi_ex",
@@ -104,6 +122,8 @@ def load():
     L.q4adamw_fused_4bit_multi_ex.restype = i
     L.q4adamw_fused_single_tensor_multi_ex.argtypes = [ctypes.POINTER(Q4SmallTensor), i, i, i] + hyper + [opt, vp]
     L.q4adamw_fused_single_tensor_multi_ex.restype = i
+    L.q4adamw_fused_4bit_rank1_multi.argtypes = [ctypes.POINTER(Q4Rank1Tensor), i, i, i] + hyper + [opt, vp]
+    L.q4adamw_fused_4bit_rank1_multi.restype = i
     L.q4adamw_grad_norm.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, ctypes.c_size_t, vp, vp]
     L.q4adamw_grad_norm.restype = i
     L.q4adamw_quantize.argtypes = [vp, i64, i, vp, vp, vp]

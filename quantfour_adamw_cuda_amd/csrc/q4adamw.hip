@@ -108,6 +108,63 @@ struct SmallArgs {
   SmallDesc desc[kMaxSmallTensors];
 };
 
+// One tensor whose second moment is rank-1 scaled (a rows x cols matrix, row-major).
+struct Rank1Desc {  // 104 bytes
+  void *p;
+  const void *g;
+  uint8_t *m;
+  uint8_t *v;
+  float *sm;          // block scales of the first moment
+  float *rmax;        // current statistics of the second moment: rows, cols floats
+  float *cmax;
+  float *rmax_next;   // the step's new statistics (all zero between steps)
+  float *cmax_next;
+  int64_t numel;      // rows * cols
+  int64_t rows;
+  int64_t cols;
+  double inv_cols;    // 1.0 / cols
+};
+
+constexpr int kMaxRank1Tensors = 32;
+
+// Kernel arguments of the rank-1 launches.  The update kernel indexes chunks of
+// kChunk flat elements like FusedArgs; the statistics kernel indexes tiles of
+// kStatRows rows x kStatCols columns (stat_first_chunk, stat_col_groups).
+struct Rank1Args {
+  static constexpr int kCapacity = kMaxRank1Tensors;
+  static constexpr int kPivots = (kMaxRank1Tensors + 7) / 8;
+  StepConsts sc;
+  GradOps go;
+  int ntensors;
+  uint32_t nchunks;
+  uint32_t chunks_per_xcd;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  Rank1Desc desc[kMaxRank1Tensors];
+};
+
+struct Rank1StatArgs {
+  static constexpr int kCapacity = kMaxRank1Tensors;
+  static constexpr int kPivots = (kMaxRank1Tensors + 7) / 8;
+  float b2, r2;
+  GradOps go;
+  int ntensors;
+  uint32_t nchunks;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  uint32_t col_groups[kMaxRank1Tensors];   // column groups per row group of tensor t
+  struct Desc {
+    const void *g;
+    const uint8_t *v;
+    const float *rmax;
+    const float *cmax;
+    float *rmax_next;
+    float *cmax_next;
+    int64_t rows;
+    int64_t cols;
+  } desc[kMaxRank1Tensors];
+};
+
 // Gradient-norm launch: every workgroup walks chunks of 32 KiB with a grid stride.
 constexpr int kMaxNormTensors = 160;
 constexpr int kNormPartials = Q4ADAMW_NORM_WORKSPACE_BYTES / 8;  // workgroups = fp64 partial sums
@@ -130,7 +187,8 @@ struct NormArgs {
   NormDesc desc[kMaxNormTensors];
 };
 
-static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(NormArgs) <= 4096,
+static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(NormArgs) <= 4096 &&
+                  sizeof(Rank1Args) <= 4096 && sizeof(Rank1StatArgs) <= 4096,
               "kernel arguments are limited to 4 KiB");
 
 // the first-moment bucket table (see q4adamw_tables.h), copied into LDS by every
@@ -341,6 +399,21 @@ __device__ __forceinline__ uint32_t quantize_exact(const Vals<N> &v, float scale
   return word;
 }
 
+// The same for the second moment with a scale per element (rank-1 scaling).
+template <int N>
+__device__ __forceinline__ uint32_t quantize_exact_scales(const Vals<N> &v, const Vals<N> &scale) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float q = v.x[j] / scale.x[j];
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < 15; ++k) c += (qmid_v(k) < q) ? 1u : 0u;
+    word |= c << (4 * j);
+  }
+  return word;
+}
+
 // (x & mask) | base as one v_and_or_b32: the mask travels in a scalar register (the
 // compiler splits the operation when the mask is a literal, which a VOP3 encoding
 // cannot hold).
@@ -456,8 +529,11 @@ struct Geometry {
 // ---------------------------------------------------------------------------
 // EXT: gradients are multiplied by gscale (one rounded fp32 multiplication per
 // element, before anything else uses them) and, if zero_g, overwritten with zeros.
-template <bool PBF, bool GBF, bool FULL, bool EXT>
-__device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, int lane, int wave, int tid,
+// RANK1 (Desc = Rank1Desc): the second moment's scale is min(row maximum, column
+// maximum) per element instead of one value per block: old statistics dequantize, the
+// step's new statistics (complete before this kernel starts) quantize.
+template <bool PBF, bool GBF, bool FULL, bool EXT, bool RANK1, typename Desc>
+__device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g) {
   using G = Geometry<PBF>;
@@ -471,7 +547,8 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   const uint8_t *m_tile = T.m + (tb >> 1);
   const uint8_t *v_tile = T.v + (tb >> 1);
   const float *sm_tile = T.sm + tile * G::kBlocksPerTile;
-  const float *sv_tile = T.sv + tile * G::kBlocksPerTile;
+  const float *sv_tile = nullptr;
+  if constexpr (!RANK1) sv_tile = T.sv + tile * G::kBlocksPerTile;
   const uint32_t e0 = (uint32_t)lane * N;                          // first element of this lane in the tile
   const uint32_t blk = (uint32_t)lane / G::kLanesPerBlock;         // which of the tile's blocks
   const uint32_t code_off = (uint32_t)lane * (N / 2);              // byte offset of this lane's codes
@@ -481,6 +558,35 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     const int64_t rem = numel - tb - (int64_t)e0;
     nv = rem >= N ? N : (rem > 0 ? (int)rem : 0);
     blk_ok = tb + (int64_t)blk * Q4ADAMW_BLOCK < numel;
+  }
+
+  // rank-1: this lane's row maxima (old, new) and its N column maxima (old, new)
+  float r_old = 0.0f, r_new = 0.0f;
+  Vals<N> c_old, c_new;
+  if constexpr (RANK1) {
+    // (row, column) of the tile's first element; the quotient estimate is at most
+    // one off and corrected.  A tile is shorter than a row, so a lane is in that row
+    // or in the next one.
+    int64_t row = (int64_t)((double)tb * T.inv_cols);
+    int64_t col0 = tb - row * T.cols;
+    if (col0 < 0) { row -= 1; col0 += T.cols; }
+    if (col0 >= T.cols) { row += 1; col0 -= T.cols; }
+    uint32_t col = (uint32_t)col0 + e0;
+    const bool wrapped = col >= (uint32_t)T.cols;
+    if (wrapped) col -= (uint32_t)T.cols;
+    const int64_t last = T.rows - 1;
+    const int64_t ra = row < last ? row : last, rb = row + 1 < last ? row + 1 : last;  // past-the-end lanes stay in bounds
+    const float r_old_a = as_global<const float>(T.rmax)[ra], r_old_b = as_global<const float>(T.rmax)[rb];
+    const float r_new_a = as_global<const float>(T.rmax_next)[ra], r_new_b = as_global<const float>(T.rmax_next)[rb];
+    r_old = wrapped ? r_old_b : r_old_a;
+    r_new = wrapped ? r_new_b : r_new_a;
+#pragma unroll
+    for (int k = 0; k < N; k += 4) {
+      const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax), (col + k) * 4u, 0, 0);
+      const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax_next), (col + k) * 4u, 0, 0);
+      c_old.x[k] = bits2f(a.x); c_old.x[k + 1] = bits2f(a.y); c_old.x[k + 2] = bits2f(a.z); c_old.x[k + 3] = bits2f(a.w);
+      c_new.x[k] = bits2f(b.x); c_new.x[k + 1] = bits2f(b.y); c_new.x[k + 2] = bits2f(b.z); c_new.x[k + 3] = bits2f(b.w);
+    }
   }
 
   float p[N], g[N];
@@ -516,11 +622,12 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   if (FULL) {
     // scales are 4 bytes per block: cached, so that neighbouring blocks share lines
     sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0));
-    sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0));
+    if (!RANK1) sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0));
   } else if (blk_ok) {
     sm_old = as_global<const float>(sm_tile)[blk];
-    sv_old = as_global<const float>(sv_tile)[blk];
+    if (!RANK1) sv_old = as_global<const float>(sv_tile)[blk];
   }
+  if (RANK1) sv_old = 1.0f;  // the table holds the bare code book; the scale follows per element
   // this block's dequantization table: entry i = {code_book_m[i] * scale_m,
   // code_book_v[i] * scale_v} (cuda_adamw_kernels.cu:340,343), written by the block's
   // lanes (lane & 15 = i) into the wave's private LDS region
@@ -544,7 +651,8 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     const uint32_t mo = entry_offset(j & 1 ? m_odd : m_even, j >> 1, three);
     const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, three);
     const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
-    const float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
+    float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
+    if constexpr (RANK1) v_old *= __builtin_fminf(r_old, c_old.x[j]);  // adamw_fourbit_triton.py:520-527
     const float gj = g[j];
     float m = sc.b1 * m_old + sc.r1 * gj;
     float v = sc.b2 * v_old + sc.r2 * (gj * gj);
@@ -560,30 +668,49 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   store_elems<PBF, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
 
   // block scales (exact: max is order independent)
+  const float v_lane_max = av;
   if (G::kLanesPerBlock == 32) {
     block_max32_pair(am, av);
   } else {
     am = row_max16(am);
-    av = row_max16(av);
+    if (!RANK1) av = row_max16(av);
   }
   if (blk_ok && (lane & (G::kLanesPerBlock - 1)) == 0) {
     if (FULL) {
       __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), blk * 4u, 0, 0);
-      __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), blk * 4u, 0, 0);
+      if (!RANK1) __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), blk * 4u, 0, 0);
     } else {
       as_global<float>(sm_tile)[blk] = am;
-      as_global<float>(sv_tile)[blk] = av;
+      if (!RANK1) as_global<float>(sv_tile)[blk] = av;
     }
   }
 
   // fast quantization: multiply by a refined reciprocal, decide every code whose
   // quotient is clear of all thresholds, flag the rest
   const bool safe_m = am >= kScaleLo && am <= kScaleHi;
-  const bool safe_v = av >= kScaleLo && av <= kScaleHi;
+  const bool safe_v = RANK1 || (av >= kScaleLo && av <= kScaleHi);
   const float rm = safe_m ? refined_rcp(am) : 0.0f;
-  const float rv16 = safe_v ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
+  const float rv16 = (safe_v && !RANK1) ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
+  // rank-1: the new scale of every element and 16 / scale.  The hardware reciprocal's
+  // one ulp is well inside the second moment's guard band (2^-17 in units of 16 q), so
+  // it goes unrefined.  Scales below the safe range are clamped for the reciprocal: a
+  // zero value under a zero scale then still gets code 0; any other value under such a
+  // scale sends the lane to the exact path.
+  Vals<N> s_new, inv16;
+  if constexpr (RANK1) {
+    float s_min = kScaleHi, s_max = 0.0f;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float sj = __builtin_fminf(r_new, c_new.x[j]);   // adamw_fourbit_triton.py:749-755
+      s_new.x[j] = sj;
+      s_min = __builtin_fminf(s_min, sj);
+      s_max = __builtin_fmaxf(s_max, sj);
+      inv16.x[j] = __builtin_amdgcn_rcpf(__builtin_fmaxf(sj, kScaleLo)) * 16.0f;
+    }
+    redo |= s_max > kScaleHi || (s_min < kScaleLo && v_lane_max != 0.0f);
+  }
   uint32_t mword = 0, vword = 0;
 #pragma unroll
   for (int j = 0; j < N; j += 2) {
@@ -602,7 +729,7 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
     // second moment: thresholds at 16q = k + 0.5, k = 1..15
 #pragma unroll
     for (int k = j; k < j + 2; ++k) {
-      const float t = __builtin_fmaf(vn.x[k], rv16, kVGuard - 0.5f);
+      const float t = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, kVGuard - 0.5f);
       vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
       // t > -1, so truncation gives 0 for t < 0
       vword = __builtin_amdgcn_alignbit((uint32_t)(int)t, vword, 4);
@@ -615,7 +742,8 @@ __device__ __forceinline__ void process_tile(const TensorDesc &T, int64_t tile, 
   redo |= vfrac < 2.0f * kVGuard;
   if (__builtin_expect(redo, 0)) {
     mword = quantize_exact<false, N>(mn, am);
-    vword = quantize_exact<true, N>(vn, av);
+    if constexpr (RANK1) vword = quantize_exact_scales<N>(vn, s_new);
+    else vword = quantize_exact<true, N>(vn, av);
   }
   if (am == 0.0f) mword = 0;  // 0/0: code 0 for the whole block
   if (!FULL) {
@@ -675,9 +803,145 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
     return;
   }
   if (begin + G::kTile <= T.numel)
-    process_tile<PBF, GBF, true, EXT>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+    process_tile<PBF, GBF, true, EXT, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
   else
-    process_tile<PBF, GBF, false, EXT>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+    process_tile<PBF, GBF, false, EXT, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+}
+
+// ---------------------------------------------------------------------------
+// rank-1 scaling of the second moment: statistics, update, commit
+// ---------------------------------------------------------------------------
+constexpr int kStatRows = 64;            // rows per workgroup of the statistics kernel
+constexpr int kStatColsPerWave = 512;    // 8 columns per lane
+constexpr int kStatCols = kStatColsPerWave * kWaves;
+
+__device__ __forceinline__ void atomic_max_nonneg(const float *addr, float x) {
+  // non-negative floats order like their bit patterns
+  atomicMax(reinterpret_cast<unsigned int *>(const_cast<float *>(addr)), f2bits(x));
+}
+
+// New second moments of a tile of kStatRows x kStatCols elements, reduced to row and
+// column maxima (get_variance_tensor_statistics, adamw_fourbit_triton.py:738-746).  The
+// arithmetic is the update kernel's, operation for operation, so the maxima are maxima
+// of exactly the values that kernel quantizes.  Every lane keeps 8 columns over the
+// tile's rows: one atomic per column per tile, one per row per wave.
+template <bool GBF, bool EXT>
+__global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
+  const uint32_t chunk = blockIdx.x;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const int t = find_tensor(args, chunk);
+  const auto &T = args.desc[t];
+  const uint32_t local = chunk - args.first_chunk[t];
+  const uint32_t groups = args.col_groups[t];
+  const uint32_t rg = local / groups, cg = local - rg * groups;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t col = (int64_t)cg * kStatCols + wave * kStatColsPerWave + lane * 8;
+  const bool active = col < T.cols;  // cols is a multiple of 8: all 8 columns or none
+  const int64_t row0 = (int64_t)rg * kStatRows;
+  const int64_t row_end = row0 + kStatRows < T.rows ? row0 + kStatRows : T.rows;
+  if ((int64_t)cg * kStatCols + wave * kStatColsPerWave >= T.cols) return;  // whole wave
+  float c_old[8], c_max[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    c_old[k] = active ? as_global<const float>(T.cmax)[col + k] : 0.0f;
+    c_max[k] = 0.0f;
+  }
+  for (int64_t row = row0; row < row_end; ++row) {
+    const float r_old = as_global<const float>(T.rmax)[row];
+    const int64_t e = row * T.cols + col;
+    float g[8];
+    uint32_t vw = 0;
+    if (active) {
+      vw = *as_global<const uint32_t>(T.v + (e >> 1));
+      if (GBF) {
+        const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 2);
+        widen_bf16_pair(w.x, g[0], g[1]);
+        widen_bf16_pair(w.y, g[2], g[3]);
+        widen_bf16_pair(w.z, g[4], g[5]);
+        widen_bf16_pair(w.w, g[6], g[7]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; k += 4) {
+          const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + (e + k) * 4);
+          g[k] = bits2f(w.x); g[k + 1] = bits2f(w.y); g[k + 2] = bits2f(w.z); g[k + 3] = bits2f(w.w);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) g[k] = 0.0f;
+    }
+    float r_max = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float gk = EXT ? g[k] * gscale : g[k];
+      const float code_value = qmap_v((int)((vw >> (4 * k)) & 15u));
+      const float v_old = code_value * __builtin_fminf(r_old, c_old[k]);
+      float v = args.b2 * v_old + args.r2 * (gk * gk);
+      if (!active) v = 0.0f;
+      c_max[k] = __builtin_fmaxf(c_max[k], v);
+      r_max = __builtin_fmaxf(r_max, v);
+    }
+    uint32_t u = f2bits(r_max);
+    u = dpp_umax<0xB1>(u);
+    u = dpp_umax<0x4E>(u);
+    u = dpp_umax<0x141>(u);
+    u = dpp_umax<0x140>(u);           // maximum of each 16-lane row, in all its lanes
+    const uint32_t u1 = (uint32_t)__shfl_xor((int)u, 16, 64);
+    u = u > u1 ? u : u1;
+    const uint32_t u2 = (uint32_t)__shfl_xor((int)u, 32, 64);
+    u = u > u2 ? u : u2;
+    if (lane == 0 && u != 0u) atomic_max_nonneg(T.rmax_next + row, bits2f(u));
+  }
+  if (active) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
+  }
+}
+
+template <bool PBF, bool GBF, bool EXT>
+__global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
+  using G = Geometry<PBF>;
+  __shared__ uint2 lds[kLdsEntries];
+  const int tid = threadIdx.x;
+  const TableSlot slot = request_table_slot(tid);
+  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  if (chunk >= args.nchunks) return;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const bool zero_g = EXT && args.go.zero != 0u;
+  const int t = find_tensor(args, chunk);
+  const Rank1Desc &T = args.desc[t];
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
+  const int64_t begin = tile * G::kTile;
+  if (begin >= T.numel) {
+    setup_tables(lds, tid, slot);
+    return;
+  }
+  if (begin + G::kTile <= T.numel)
+    process_tile<PBF, GBF, true, EXT, true>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+  else
+    process_tile<PBF, GBF, false, EXT, true>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+}
+
+// After the update: the new statistics become the current ones and the buffers that
+// received them go back to zero for the next step's maxima.  One workgroup column per
+// tensor (blockIdx.y), grid-stride over rows + cols floats.
+__global__ __launch_bounds__(256) void rank1_commit_kernel(const Rank1Args args) {
+  float gscale;
+  if (!grad_ops_begin(args.go, gscale)) return;
+  const Rank1Desc &T = args.desc[blockIdx.y];
+  const int64_t total = T.rows + T.cols;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const bool is_row = i < T.rows;
+    const gptr<float> cur = as_global<float>(is_row ? T.rmax : T.cmax) + (is_row ? i : i - T.rows);
+    const gptr<float> next = as_global<float>(is_row ? T.rmax_next : T.cmax_next) + (is_row ? i : i - T.rows);
+    *cur = *next;
+    *next = 0.0f;
+  }
 }
 
 // Non-quantized step for small tensors (cuda_adamw_kernels.cu:100-133): fp32
@@ -975,6 +1239,27 @@ static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
   return ext ? pick_small_ext<true>(pb, gb) : pick_small_ext<false>(pb, gb);
 }
 
+typedef void (*Rank1Kernel)(const Rank1Args);
+typedef void (*Rank1StatKernel)(const Rank1StatArgs);
+
+template <bool EXT>
+static Rank1Kernel pick_rank1_ext(bool pb, bool gb) {
+  if (!pb && !gb) return fused_4bit_rank1_kernel<false, false, EXT>;
+  if (!pb && gb) return fused_4bit_rank1_kernel<false, true, EXT>;
+  if (pb && !gb) return fused_4bit_rank1_kernel<true, false, EXT>;
+  return fused_4bit_rank1_kernel<true, true, EXT>;
+}
+
+static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext) {
+  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
+  return ext ? pick_rank1_ext<true>(pb, gb) : pick_rank1_ext<false>(pb, gb);
+}
+
+static Rank1StatKernel pick_rank1_stats(int g_dtype, bool ext) {
+  if (g_dtype == Q4ADAMW_BF16) return ext ? rank1_stats_kernel<true, true> : rank1_stats_kernel<true, false>;
+  return ext ? rank1_stats_kernel<false, true> : rank1_stats_kernel<false, false>;
+}
+
 // Fills the kernels' view of the caller's gradient options; returns whether the
 // launch needs the EXT kernels (false: the options change nothing).
 static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext) {
@@ -1100,6 +1385,115 @@ int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_
     chunks += c;
   }
   if (a.ntensors > 0) return launch_fused_batch(a, chunks, kernel, s);
+  return 0;
+}
+
+int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
+                                   int g_dtype, float beta1, float beta2, float lr,
+                                   float weight_decay, float eps, float step,
+                                   const q4adamw_grad_options *opt, void *stream) {
+  if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
+  if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
+  Rank1Args a;
+  Rank1StatArgs sa;
+  bool ext = false;
+  if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
+  if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
+  sa.go = a.go;
+  sa.b2 = a.sc.b2;
+  sa.r2 = a.sc.r2;
+  const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
+  const int64_t chunk_elems = p_bf16 ? Geometry<true>::kChunk : Geometry<false>::kChunk;
+  for (int i = 0; i < count; ++i) {
+    const q4adamw_rank1_tensor &t = tensors[i];
+    if (t.rows < 0 || t.cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
+    if (t.rows == 0 || t.cols == 0) continue;
+    if (t.cols % 8 != 0 || t.cols < 512)
+      return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8 and at least 512");
+    if (t.cols > 0x40000000ll || t.rows > 0x7fffffffffffll / t.cols)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+    if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.row_max || !t.col_max ||
+        !t.row_max_next || !t.col_max_next)
+      return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+    if (!aligned(t.p, 16) || !aligned(t.g, 16))
+      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be 16-byte aligned");
+    if (!aligned(t.exp_avg, 4) || !aligned(t.exp_avg_sq, 4) || !aligned(t.exp_avg_scale, 4) ||
+        !aligned(t.row_max, 4) || !aligned(t.row_max_next, 4))
+      return fail(Q4ADAMW_ERR_ALIGN, "code, scale and row buffers must be 4-byte aligned");
+    if (!aligned(t.col_max, 16) || !aligned(t.col_max_next, 16))
+      return fail(Q4ADAMW_ERR_ALIGN, "column buffers must be 16-byte aligned");
+    const uint64_t numel = (uint64_t)t.rows * (uint64_t)t.cols;
+    const uint64_t stat_chunks = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) *
+                                 (uint64_t)((t.cols + kStatCols - 1) / kStatCols);
+    if ((numel + chunk_elems - 1) / chunk_elems > kMaxChunksPerLaunch || stat_chunks > kMaxChunksPerLaunch)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const Rank1Kernel kernel = pick_rank1(p_dtype, g_dtype, ext);
+  const Rank1StatKernel stat_kernel = pick_rank1_stats(g_dtype, ext);
+  a.ntensors = 0;
+  uint64_t chunks = 0, stat_chunks = 0;
+  // statistics of every tensor of the batch, then the update, then the commit
+  auto launch = [&]() -> int {
+    sa.ntensors = a.ntensors;
+    finish_prefix(sa);
+    sa.nchunks = (uint32_t)stat_chunks;
+    hipLaunchKernelGGL(stat_kernel, dim3(sa.nchunks), dim3(kThreads), 0, s, sa);
+    Q4_HIP(hipGetLastError());
+    finish_prefix(a);
+    a.nchunks = (uint32_t)chunks;
+    a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
+    hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, s, a);
+    Q4_HIP(hipGetLastError());
+    hipLaunchKernelGGL(rank1_commit_kernel, dim3(8, (unsigned)a.ntensors), dim3(256), 0, s, a);
+    Q4_HIP(hipGetLastError());
+    a.ntensors = 0;
+    chunks = 0;
+    stat_chunks = 0;
+    return 0;
+  };
+  for (int i = 0; i < count; ++i) {
+    const q4adamw_rank1_tensor &t = tensors[i];
+    if (t.rows == 0 || t.cols == 0) continue;
+    const int64_t numel = t.rows * t.cols;
+    const uint64_t c = (uint64_t)(numel + chunk_elems - 1) / chunk_elems;
+    const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
+    const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
+    if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
+        stat_chunks + sc_ > kMaxChunksPerLaunch) {
+      if (int rc = launch()) return rc;
+    }
+    Rank1Desc &d = a.desc[a.ntensors];
+    d.p = t.p;
+    d.g = t.g;
+    d.m = t.exp_avg;
+    d.v = t.exp_avg_sq;
+    d.sm = t.exp_avg_scale;
+    d.rmax = t.row_max;
+    d.cmax = t.col_max;
+    d.rmax_next = t.row_max_next;
+    d.cmax_next = t.col_max_next;
+    d.numel = numel;
+    d.rows = t.rows;
+    d.cols = t.cols;
+    d.inv_cols = 1.0 / (double)t.cols;
+    a.first_chunk[a.ntensors] = (uint32_t)chunks;
+    Rank1StatArgs::Desc &sd = sa.desc[a.ntensors];
+    sd.g = t.g;
+    sd.v = t.exp_avg_sq;
+    sd.rmax = t.row_max;
+    sd.cmax = t.col_max;
+    sd.rmax_next = t.row_max_next;
+    sd.cmax_next = t.col_max_next;
+    sd.rows = t.rows;
+    sd.cols = t.cols;
+    sa.first_chunk[a.ntensors] = (uint32_t)stat_chunks;
+    sa.col_groups[a.ntensors] = groups;
+    ++a.ntensors;
+    chunks += c;
+    stat_chunks += sc_;
+  }
+  if (a.ntensors > 0) return launch();
   return 0;
 }
 
@@ -1271,6 +1665,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1003; }
+int q4adamw_version(void) { return 1004; }
 
 }  // extern "C"

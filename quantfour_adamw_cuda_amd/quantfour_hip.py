@@ -181,6 +181,73 @@ def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, w
                        options)
 
 
+RANK1_MIN_COLS = 512
+
+
+def rank1_eligible(p):
+    """Whether a parameter's second moment can take rank-1 scaling: a matrix whose rows hold a
+    multiple of 8 and at least 512 elements (other tensors keep per-128 block scales, as 1-D
+    tensors do in the reference's draft, optim/adamw_fourbit_triton.py:841-846)."""
+    return p.dim() == 2 and p.shape[1] % 8 == 0 and p.shape[1] >= RANK1_MIN_COLS
+
+
+def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next):
+    _check_common(p, g)
+    assert rank1_eligible(p), "rank-1 scaling needs a matrix with cols % 8 == 0 and cols >= 512"
+    rows, cols = p.shape
+    nbytes, nblk = state_sizes(p.numel())
+    assert exp.dtype == torch.uint8 and sq.dtype == torch.uint8, "moments must be packed uint8"
+    assert exp.numel() == nbytes and sq.numel() == nbytes, f"packed moments must hold {nbytes} bytes"
+    assert exp_scale.dtype == torch.float32 and exp_scale.numel() == nblk, f"exp_avg scales must hold {nblk} blocks"
+    for t, n, what in ((row_max, rows, "row"), (row_next, rows, "row"), (col_max, cols, "column"),
+                       (col_next, cols, "column")):
+        assert t.dtype == torch.float32 and t.numel() == n, f"{what} maxima must be {n} float32"
+    for t in (exp, sq, exp_scale, row_max, col_max, row_next, col_next):
+        assert t.device == p.device and t.is_contiguous(), "state must be contiguous on the param's device"
+
+
+def make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts):
+    n = len(ps)
+    arr = (_lib.Q4Rank1Tensor * n)()
+    for i in range(n):
+        check_rank1(ps[i], gs[i], exps[i], sqs[i], exp_scales[i], row_maxes[i], col_maxes[i],
+                    row_nexts[i], col_nexts[i])
+        a = arr[i]
+        a.p, a.g = ps[i].data_ptr(), gs[i].data_ptr()
+        a.exp_avg, a.exp_avg_sq = exps[i].data_ptr(), sqs[i].data_ptr()
+        a.exp_avg_scale = exp_scales[i].data_ptr()
+        a.row_max, a.col_max = row_maxes[i].data_ptr(), col_maxes[i].data_ptr()
+        a.row_max_next, a.col_max_next = row_nexts[i].data_ptr(), col_nexts[i].data_ptr()
+        a.rows, a.cols = ps[i].shape
+    return arr
+
+
+def launch_rank1_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step,
+                       options=None):
+    L = _lib.load()
+    with torch.cuda.device(device):
+        rc = L.q4adamw_fused_4bit_rank1_multi(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
+                                              weight_decay, eps, float(step), options, _stream(device))
+    _lib.check(rc, "fused_4bit_rank1_multi")
+
+
+def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts,
+                           beta1, beta2, lr, weight_decay, eps, step, grad_scale=1.0,
+                           grad_scale_dev=None, found_inf=None, zero_grad=False):
+    """The fused step over matrices whose second moment is rank-1 scaled: scale of element
+    (i, j) = min(row_maxes[i], col_maxes[j]).  row_nexts / col_nexts are state-owned scratch
+    that holds zeros between steps.  Gradient options as for fused_4bit_multi."""
+    if not ps:
+        return
+    arr = make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts)
+    p_tag, g_tag = _tag(ps[0], "param"), _tag(gs[0], "grad")
+    for p, g in zip(ps, gs):
+        assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
+            "tensors of one launch must share device and dtypes"
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    launch_rank1_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
+
+
 def make_grad_table(gs):
     """ctypes descriptor array for grad_norm_table (gradients validated)."""
     arr = (_lib.Q4Grad * len(gs))()

@@ -309,3 +309,75 @@ def test_scale_grad_is_unscale():
     gb = g.to(torch.bfloat16)
     got = oc.scale_grad(gb.view(torch.int16).numpy().view(np.uint16), 0.3)
     assert np.array_equal(got, (gb.float() * np.float32(0.3)).numpy())
+
+
+# ---------------------------------------------------------------------------
+# rank-1 scaling of the second moment
+# ---------------------------------------------------------------------------
+def test_rank1_quantizer_brute_force():
+    """small matrices, plain Python loops: scale_ij = min(max of row i, max of column j), code =
+    number of thresholds strictly below x_ij / scale_ij, 0/0 -> 0; dequantize multiplies back"""
+    gen = torch.Generator().manual_seed(21)
+    _, mid = oc.tables(1)
+    qmap, _ = oc.tables(1)
+    for rows, cols in ((1, 8), (8, 1), (5, 6), (7, 16)):
+        x = torch.rand(rows, cols, generator=gen) ** 4
+        x[rows // 2] = 0.0                                  # a zero row
+        if cols > 2:
+            x[:, 1] = 0.0                                   # a zero column
+        codes, rmax, cmax = ot.quantize_rank1(x)
+        un = ot.unpack(codes, rows * cols).view(rows, cols)
+        back = ot.dequantize_rank1(codes, rmax, cmax)
+        for i in range(rows):
+            for j in range(cols):
+                r = max(float(x[i, k]) for k in range(cols))
+                c = max(float(x[k, j]) for k in range(rows))
+                s = np.float32(min(r, c))
+                assert float(rmax[i]) == r and float(cmax[j]) == c
+                if s == 0:
+                    want = 0
+                else:
+                    q = np.float32(x[i, j].item()) / s
+                    want = sum(1 for t in mid if t < q)
+                assert int(un[i, j]) == want, (rows, cols, i, j)
+                assert float(back[i, j]) == float(np.float32(qmap[want]) * s)
+
+
+def test_rank1_closed_forms():
+    # one row: every column maximum is the element itself, so every non-zero element gets the
+    # top code; one column likewise
+    x = torch.tensor([[0.3, 0.0, 7.0, 1e-20]])
+    codes, _, _ = ot.quantize_rank1(x)
+    assert ot.unpack(codes, 4).tolist() == [15, 0, 15, 15]
+    codes, _, _ = ot.quantize_rank1(x.t().contiguous())
+    assert ot.unpack(codes, 4).tolist() == [15, 0, 15, 15]
+    # outer product of powers of two a_i * b_j: scale_ij = min(a_i * max b, b_j * max a) and
+    # the quotient is max(b_j / max b, a_i / max a) exactly
+    a = torch.tensor([1.0, 0.5, 0.25, 0.125])
+    b = torch.tensor([1.0, 0.5, 0.25, 2.0 ** -5, 2.0 ** -6, 0.125])
+    x = a[:, None] * b[None, :]
+    codes, rmax, cmax = ot.quantize_rank1(x)
+    assert torch.equal(rmax, a) and torch.equal(cmax, b)
+    q = torch.maximum((b / b.max())[None, :].expand(4, 6), (a / a.max())[:, None].expand(4, 6))
+    want = torch.bucketize(q, ot.QMID[1], right=False)
+    assert torch.equal(ot.unpack(codes, 24).view(4, 6), want)
+    # the step on an all-zero state keeps the arg-max of every row and column at code 15
+    gen = torch.Generator().manual_seed(22)
+    rows, cols = 16, 128
+    g = torch.randn(rows, cols, generator=gen)
+    p = torch.zeros(rows, cols)
+    z8 = torch.zeros(rows * cols // 2, dtype=torch.uint8)
+    out = ot.step_quant_rank1(p, g, z8, z8.clone(), torch.zeros(rows * cols // 128), torch.zeros(rows),
+                              torch.zeros(cols), step=1, **HP)
+    vc = ot.unpack(out[2], rows * cols).view(rows, cols)
+    v_new = (1 - np.float32(HP["beta2"])) * (g * g)
+    assert torch.equal(out[4], v_new.amax(1)) and torch.equal(out[5], v_new.amax(0))
+    # an element that is the maximum of its row or of its column has quotient >= ... 1 only
+    # when it is the smaller of the two maxima; the global maximum always is
+    i, j = divmod(int(v_new.argmax()), cols)
+    assert int(vc[i, j]) == 15
+    # m-part and parameters agree with the block-scaled step (same first moment arithmetic)
+    ref = ot.step_quant(p.reshape(-1), g.reshape(-1), z8, z8.clone(), torch.zeros(rows * cols // 128),
+                        torch.zeros(rows * cols // 128), step=1, **HP)
+    assert torch.equal(out[1], ref[1]) and torch.equal(out[3], ref[3])
+    assert torch.equal(out[0].reshape(-1), ref[0])
