@@ -232,6 +232,19 @@ int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel,
                        float *out, void *stream);
 
 /*
+ * The same pair for a second moment with rank-1 scaling: x is a rows x cols fp32
+ * matrix (cols a multiple of 8); row_max[i] / col_max[j] receive the abs-maxima of
+ * row i / column j, every element is divided by min(row_max[i], col_max[j]) and
+ * mapped to the nearest code of the second moment's map (variance_quant_scaling and
+ * variance_quant, optim/adamw_fourbit_triton.py:803-863); dequantize multiplies back
+ * (:520-527).
+ */
+int q4adamw_quantize_rank1(const float *x, int64_t rows, int64_t cols, uint8_t *codes,
+                           float *row_max, float *col_max, void *stream);
+int q4adamw_dequantize_rank1(const uint8_t *codes, const float *row_max, const float *col_max,
+                             int64_t rows, int64_t cols, float *out, void *stream);
+
+/*
  * Host-only: the six fp32 scalars the launcher derives from the hyper-parameters
  * (optim/cuda_adamw_kernels.cu:435-440), in that order: correction1,
  * correction2_sqrt, step_size, weight_decay_update, resid_beta1, resid_beta2.

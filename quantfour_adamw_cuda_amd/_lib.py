@@ -85,6 +85,8 @@ EXPORTS = (
     "q4adamw_grad_norm",
     "q4adamw_quantize",
     "q4adamw_dequantize",
+    "q4adamw_quantize_rank1",
+    "q4adamw_dequantize_rank1",
     "q4adamw_derive_scalars",
     "q4adamw_tables",
     "q4adamw_mtable_entry",
@@ -130,6 +132,10 @@ def load():
     L.q4adamw_quantize.restype = i
     L.q4adamw_dequantize.argtypes = [vp, vp, i64, i, vp, vp]
     L.q4adamw_dequantize.restype = i
+    L.q4adamw_quantize_rank1.argtypes = [vp, i64, i64, vp, vp, vp, vp]
+    L.q4adamw_quantize_rank1.restype = i
+    L.q4adamw_dequantize_rank1.argtypes = [vp, vp, vp, i64, i64, vp, vp]
+    L.q4adamw_dequantize_rank1.restype = i
     L.q4adamw_derive_scalars.argtypes = [f, f, f, f, f, ctypes.POINTER(f)]
     L.q4adamw_derive_scalars.restype = None
     L.q4adamw_tables.argtypes = [i, ctypes.POINTER(f), ctypes.POINTER(f)]

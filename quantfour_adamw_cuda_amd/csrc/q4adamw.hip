@@ -122,8 +122,34 @@ struct Rank1Desc {  // 104 bytes
   int64_t numel;      // rows * cols
   int64_t rows;
   int64_t cols;
-  double inv_cols;    // 1.0 / cols
+  // division of a 32-bit number by cols / 8 as multiply-high, add and shifts
+  // (round-up method: exact for every 32-bit dividend)
+  uint32_t div_magic;
+  uint32_t div_shift;
 };
+
+struct FastDiv {
+  uint32_t magic, shift;
+};
+
+// n / d for the divisor the pair was made for
+__host__ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t shift) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t t = __umulhi(n, magic);
+#else
+  const uint32_t t = (uint32_t)(((uint64_t)n * magic) >> 32);
+#endif
+  return (t + ((n - t) >> 1)) >> shift;
+}
+
+static FastDiv make_fast_div(uint32_t d) {  // d >= 2
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;                     // ceil(log2 d) >= 1
+  FastDiv f;
+  f.magic = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+  f.shift = l - 1;
+  return f;
+}
 
 constexpr int kMaxRank1Tensors = 32;
 
@@ -564,14 +590,14 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   float r_old = 0.0f, r_new = 0.0f;
   Vals<N> c_old, c_new;
   if constexpr (RANK1) {
-    // (row, column) of the tile's first element; the quotient estimate is at most
-    // one off and corrected.  A tile is shorter than a row, so a lane is in that row
-    // or in the next one.
-    int64_t row = (int64_t)((double)tb * T.inv_cols);
-    int64_t col0 = tb - row * T.cols;
-    if (col0 < 0) { row -= 1; col0 += T.cols; }
-    if (col0 >= T.cols) { row += 1; col0 -= T.cols; }
-    uint32_t col = (uint32_t)col0 + e0;
+    // (row, column) of the tile's first element, in units of 8 elements so that the
+    // division is a 32-bit one.  A tile is shorter than a row, so a lane is in that
+    // row or in the next one.
+    const uint32_t tb8 = (uint32_t)(tb >> 3), cols8 = (uint32_t)(T.cols >> 3);  // numel < 2^35
+    const uint32_t row32 = fast_div(tb8, T.div_magic, T.div_shift);
+    const int64_t row = row32;
+    const uint32_t col0 = (tb8 - row32 * cols8) << 3;
+    uint32_t col = col0 + e0;
     const bool wrapped = col >= (uint32_t)T.cols;
     if (wrapped) col -= (uint32_t)T.cols;
     const int64_t last = T.rows - 1;
@@ -700,16 +726,16 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   // scale sends the lane to the exact path.
   Vals<N> s_new, inv16;
   if constexpr (RANK1) {
-    float s_min = kScaleHi, s_max = 0.0f;
+    float c_min = c_new.x[0];
 #pragma unroll
     for (int j = 0; j < N; ++j) {
       const float sj = __builtin_fminf(r_new, c_new.x[j]);   // adamw_fourbit_triton.py:749-755
       s_new.x[j] = sj;
-      s_min = __builtin_fminf(s_min, sj);
-      s_max = __builtin_fmaxf(s_max, sj);
+      c_min = __builtin_fminf(c_min, c_new.x[j]);
       inv16.x[j] = __builtin_amdgcn_rcpf(__builtin_fmaxf(sj, kScaleLo)) * 16.0f;
     }
-    redo |= s_max > kScaleHi || (s_min < kScaleLo && v_lane_max != 0.0f);
+    // every scale is at most r_new and at least min(r_new, c_min)
+    redo |= r_new > kScaleHi || (__builtin_fminf(r_new, c_min) < kScaleLo && v_lane_max != 0.0f);
   }
   uint32_t mword = 0, vword = 0;
 #pragma unroll
@@ -827,6 +853,7 @@ __device__ __forceinline__ void atomic_max_nonneg(const float *addr, float x) {
 // tile's rows: one atomic per column per tile, one per row per wave.
 template <bool GBF, bool EXT>
 __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
+  __shared__ uint32_t row_bits[kStatRows];
   const uint32_t chunk = blockIdx.x;
   float gscale = 1.0f;
   if (EXT && !grad_ops_begin(args.go, gscale)) return;
@@ -840,65 +867,71 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   const int64_t col = (int64_t)cg * kStatCols + wave * kStatColsPerWave + lane * 8;
   const bool active = col < T.cols;  // cols is a multiple of 8: all 8 columns or none
   const int64_t row0 = (int64_t)rg * kStatRows;
-  const int64_t row_end = row0 + kStatRows < T.rows ? row0 + kStatRows : T.rows;
-  if ((int64_t)cg * kStatCols + wave * kStatColsPerWave >= T.cols) return;  // whole wave
+  const int nrows = (int)(row0 + kStatRows < T.rows ? kStatRows : T.rows - row0);
+  if (tid < kStatRows) row_bits[tid] = 0u;
+  __syncthreads();
+  // lanes past the last column work on zeros: code 0 under a zero scale and a zero
+  // gradient give a zero second moment, which leaves every maximum alone
   float c_old[8], c_max[8];
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     c_old[k] = active ? as_global<const float>(T.cmax)[col + k] : 0.0f;
     c_max[k] = 0.0f;
   }
-  for (int64_t row = row0; row < row_end; ++row) {
-    const float r_old = as_global<const float>(T.rmax)[row];
-    const int64_t e = row * T.cols + col;
-    float g[8];
-    uint32_t vw = 0;
-    if (active) {
-      vw = *as_global<const uint32_t>(T.v + (e >> 1));
-      if (GBF) {
-        const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 2);
-        widen_bf16_pair(w.x, g[0], g[1]);
-        widen_bf16_pair(w.y, g[2], g[3]);
-        widen_bf16_pair(w.z, g[4], g[5]);
-        widen_bf16_pair(w.w, g[6], g[7]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < 8; k += 4) {
-          const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + (e + k) * 4);
-          g[k] = bits2f(w.x); g[k + 1] = bits2f(w.y); g[k + 2] = bits2f(w.z); g[k + 3] = bits2f(w.w);
-        }
-      }
-    } else {
+  const bool wave_active = (int64_t)cg * kStatCols + wave * kStatColsPerWave < T.cols;
+  if (wave_active) {
+
+    for (int r = 0; r < nrows; ++r) {
+      const int64_t row = row0 + r;
+      const float r_old = as_global<const float>(T.rmax)[row];
+      const int64_t e = row * T.cols + col;
+      float g[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) g[k] = 0.0f;
-    }
-    float r_max = 0.0f;
+      uint32_t vw = 0;
+      if (active) {
+        vw = *as_global<const uint32_t>(T.v + (e >> 1));
+        if (GBF) {
+          const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 2);
+          widen_bf16_pair(w.x, g[0], g[1]);
+          widen_bf16_pair(w.y, g[2], g[3]);
+          widen_bf16_pair(w.z, g[4], g[5]);
+          widen_bf16_pair(w.w, g[6], g[7]);
+        } else {
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const float gk = EXT ? g[k] * gscale : g[k];
-      const float code_value = qmap_v((int)((vw >> (4 * k)) & 15u));
-      const float v_old = code_value * __builtin_fminf(r_old, c_old[k]);
-      float v = args.b2 * v_old + args.r2 * (gk * gk);
-      if (!active) v = 0.0f;
-      c_max[k] = __builtin_fmaxf(c_max[k], v);
-      r_max = __builtin_fmaxf(r_max, v);
-    }
-    uint32_t u = f2bits(r_max);
-    u = dpp_umax<0xB1>(u);
-    u = dpp_umax<0x4E>(u);
-    u = dpp_umax<0x141>(u);
-    u = dpp_umax<0x140>(u);           // maximum of each 16-lane row, in all its lanes
-    const uint32_t u1 = (uint32_t)__shfl_xor((int)u, 16, 64);
-    u = u > u1 ? u : u1;
-    const uint32_t u2 = (uint32_t)__shfl_xor((int)u, 32, 64);
-    u = u > u2 ? u : u2;
-    if (lane == 0 && u != 0u) atomic_max_nonneg(T.rmax_next + row, bits2f(u));
-  }
-  if (active) {
+          for (int k = 0; k < 8; k += 4) {
+            const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + (e + k) * 4);
+            g[k] = bits2f(w.x); g[k + 1] = bits2f(w.y); g[k + 2] = bits2f(w.z); g[k + 3] = bits2f(w.w);
+          }
+        }
+      }
+      const uint32_t even = vw & 0x0F0F0F0Fu, odd = (vw >> 4) & 0x0F0F0F0Fu;  // one code per byte
+      float r_max = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
-      if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
+      for (int k = 0; k < 8; ++k) {
+        const float gk = EXT ? g[k] * gscale : g[k];
+        const uint32_t code = ((k & 1 ? odd : even) >> (8 * (k >> 1))) & 0xffu;
+        const float code_value = __builtin_fmaf((float)code, 0.0625f, 0.0625f);  // (code + 1) / 16, exact
+        const float v_old = code_value * __builtin_fminf(r_old, c_old[k]);
+        const float v = args.b2 * v_old + args.r2 * (gk * gk);
+        c_max[k] = __builtin_fmaxf(c_max[k], v);
+        r_max = __builtin_fmaxf(r_max, v);
+      }
+      uint32_t u = f2bits(r_max);
+      u = dpp_umax<0xB1>(u);
+      u = dpp_umax<0x4E>(u);
+      u = dpp_umax<0x141>(u);
+      u = dpp_umax<0x140>(u);           // maximum of each 16-lane row, in all its lanes
+      if ((lane & 15) == 0 && u != 0u) atomicMax(&row_bits[r], u);
+    }
+    if (active) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
+    }
   }
+  __syncthreads();
+  if (tid < nrows && row_bits[tid] != 0u) atomic_max_nonneg(T.rmax_next + row0 + tid, bits2f(row_bits[tid]));
 }
 
 template <bool PBF, bool GBF, bool EXT>
@@ -1109,6 +1142,73 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__
     }
     as_global<uint8_t>(codes_)[e >> 1] = (uint8_t)byte;
   }
+}
+
+// Rank-1 forms for the second moment of a rows x cols matrix (run once per
+// checkpoint).  Statistics: a workgroup takes 64 rows x 256 columns, a thread one
+// column; row maxima meet in LDS, then one atomic per row and per column.
+__global__ __launch_bounds__(256) void fill_zero_kernel(float *x_, int64_t n) {
+  const gptr<float> x = as_global<float>(x_);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) x[i] = 0.0f;
+}
+
+__global__ __launch_bounds__(256) void rank1_absmax_kernel(const float *x_, int64_t rows, int64_t cols,
+                                                           float *row_max, float *col_max) {
+  __shared__ uint32_t row_bits[64];
+  const gptr<const float> x = as_global<const float>(x_);
+  const int tid = threadIdx.x;
+  const int64_t col = (int64_t)blockIdx.x * 256 + tid;
+  const int64_t row0 = (int64_t)blockIdx.y * 64;
+  const int nrows = (int)(row0 + 64 < rows ? 64 : rows - row0);
+  if (tid < 64) row_bits[tid] = 0u;
+  __syncthreads();
+  float c_max = 0.0f;
+  for (int r = 0; r < nrows; ++r) {
+    const float a = col < cols ? __builtin_fabsf(x[(row0 + r) * cols + col]) : 0.0f;
+    c_max = __builtin_fmaxf(c_max, a);
+    uint32_t u = f2bits(a);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const uint32_t o = (uint32_t)__shfl_xor((int)u, off, 64);
+      u = u > o ? u : o;
+    }
+    if ((tid & 63) == 0 && u != 0u) atomicMax(&row_bits[r], u);
+  }
+  if (col < cols && c_max != 0.0f) atomic_max_nonneg(col_max + col, c_max);
+  __syncthreads();
+  if (tid < nrows && row_bits[tid] != 0u) atomic_max_nonneg(row_max + row0 + tid, bits2f(row_bits[tid]));
+}
+
+// one thread per packed byte: x / min(row maximum, column maximum), IEEE division, the
+// 15-compare count (optim/adamw_fourbit_triton.py:834-863)
+__global__ __launch_bounds__(256) void quantize_rank1_kernel(const float *x_, int64_t rows, int64_t cols,
+                                                             const float *row_max, const float *col_max,
+                                                             uint8_t *codes_) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (e >= rows * cols) return;
+  const int64_t i = e / cols, j = e - i * cols;  // cols is even: both elements in row i
+  const float r = as_global<const float>(row_max)[i];
+  uint32_t byte = 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float q = as_global<const float>(x_)[e + h] / __builtin_fminf(r, as_global<const float>(col_max)[j + h]);
+#pragma unroll
+    for (int k = 0; k < 15; ++k) byte += (qmid_v(k) < q) ? (1u << (4 * h)) : 0u;
+  }
+  as_global<uint8_t>(codes_)[e >> 1] = (uint8_t)byte;
+}
+
+// optim/adamw_fourbit_triton.py:520-527: code-book entry times min(row, column maximum)
+__global__ __launch_bounds__(256) void dequantize_rank1_kernel(const uint8_t *codes_, const float *row_max,
+                                                               const float *col_max, int64_t rows,
+                                                               int64_t cols, float *out_) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (e >= rows * cols) return;
+  const int64_t i = e / cols, j = e - i * cols;
+  const float r = as_global<const float>(row_max)[i];
+  const uint32_t byte = as_global<const uint8_t>(codes_)[e >> 1];
+  as_global<float>(out_)[e] = qmap_v((int)(byte & 15u)) * __builtin_fminf(r, as_global<const float>(col_max)[j]);
+  as_global<float>(out_)[e + 1] = qmap_v((int)(byte >> 4)) * __builtin_fminf(r, as_global<const float>(col_max)[j + 1]);
 }
 
 // cuda_adamw_kernels.cu:329-343: code -> code-book entry * block scale
@@ -1410,8 +1510,8 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
     if (t.rows == 0 || t.cols == 0) continue;
     if (t.cols % 8 != 0 || t.cols < 512)
       return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8 and at least 512");
-    if (t.cols > 0x40000000ll || t.rows > 0x7fffffffffffll / t.cols)
-      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+    if (t.cols > 0x40000000ll || t.rows > 0x7ffffffffll / t.cols)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "rank-1 scaling handles matrices of up to 2^35 - 1 elements");
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.row_max || !t.col_max ||
         !t.row_max_next || !t.col_max_next)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
@@ -1445,7 +1545,7 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
     a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
     hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, s, a);
     Q4_HIP(hipGetLastError());
-    hipLaunchKernelGGL(rank1_commit_kernel, dim3(8, (unsigned)a.ntensors), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(rank1_commit_kernel, dim3(64, (unsigned)a.ntensors), dim3(256), 0, s, a);
     Q4_HIP(hipGetLastError());
     a.ntensors = 0;
     chunks = 0;
@@ -1476,7 +1576,9 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
     d.numel = numel;
     d.rows = t.rows;
     d.cols = t.cols;
-    d.inv_cols = 1.0 / (double)t.cols;
+    const FastDiv fd = make_fast_div((uint32_t)(t.cols >> 3));
+    d.div_magic = fd.magic;
+    d.div_shift = fd.shift;
     a.first_chunk[a.ntensors] = (uint32_t)chunks;
     Rank1StatArgs::Desc &sd = sa.desc[a.ntensors];
     sd.g = t.g;
@@ -1646,6 +1748,48 @@ int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, f
   return 0;
 }
 
+static int check_rank1_shape(int64_t rows, int64_t cols) {
+  if (rows < 0 || cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
+  if (cols % 8 != 0) return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8");
+  if (rows > 0 && cols > 0 && (cols > 0x40000000ll || rows > 0x7ffffffffll / cols))
+    return fail(Q4ADAMW_ERR_TOO_LARGE, "rank-1 scaling handles matrices of up to 2^35 - 1 elements");
+  return 0;
+}
+
+int q4adamw_quantize_rank1(const float *x, int64_t rows, int64_t cols, uint8_t *codes,
+                           float *row_max, float *col_max, void *stream) {
+  if (int rc = check_rank1_shape(rows, cols)) return rc;
+  if (rows == 0 || cols == 0) return 0;
+  if (!x || !codes || !row_max || !col_max) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+  if (!aligned(x, 4) || !aligned(row_max, 4) || !aligned(col_max, 4))
+    return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, row_max, rows);
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, col_max, cols);
+  const dim3 tiles((unsigned)((cols + 255) / 256), (unsigned)((rows + 63) / 64));
+  if (tiles.y > 65535u) return fail(Q4ADAMW_ERR_TOO_LARGE, "more than 4194240 rows");
+  hipLaunchKernelGGL(rank1_absmax_kernel, tiles, dim3(256), 0, s, x, rows, cols, row_max, col_max);
+  const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
+  hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, rows, cols,
+                     static_cast<const float *>(row_max), static_cast<const float *>(col_max), codes);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
+int q4adamw_dequantize_rank1(const uint8_t *codes, const float *row_max, const float *col_max,
+                             int64_t rows, int64_t cols, float *out, void *stream) {
+  if (int rc = check_rank1_shape(rows, cols)) return rc;
+  if (rows == 0 || cols == 0) return 0;
+  if (!codes || !row_max || !col_max || !out) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+  if (!aligned(out, 4) || !aligned(row_max, 4) || !aligned(col_max, 4))
+    return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
+  const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
+  hipLaunchKernelGGL(dequantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), codes, row_max, col_max, rows, cols, out);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel, int which,
                        float *out, void *stream) {
   if (numel < 0 || (which != 0 && which != 1)) return fail(Q4ADAMW_ERR_ARG, "bad numel or moment selector");
@@ -1665,6 +1809,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1004; }
+int q4adamw_version(void) { return 1005; }
 
 }  // extern "C"

@@ -57,6 +57,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         weight_decay=1e-2,
         *,
         fused: Optional[bool] = False,
+        variance_scale_type: str = "group",
     ):
         # optim/fused_quantfour.py:38-47
         if not 0.0 < lr:
@@ -69,6 +70,15 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             raise ValueError(f"Invalid Beta[1]: {betas[1]=}")
         if not 0.0 <= weight_decay:
             raise ValueError(f"Invalid weight_decay value: {weight_decay=}")
+
+        # how the second moment is scaled before it is quantized: "group" = one abs-max per
+        # 128 consecutive elements, what the fused CUDA path does (cuda_adamw_kernels.cu:353-383);
+        # "rank1" = min(row maximum, column maximum) for matrices, the draft's SecondMoment
+        # setting (adamw_fourbit_triton.py:124, :834-863); tensors that are not matrices with
+        # cols % 8 == 0 and cols >= 512 keep group scaling, as 1-D tensors do there (:841-846)
+        if variance_scale_type not in ("group", "rank1"):
+            raise ValueError(f"Invalid variance_scale_type: {variance_scale_type=}")
+        self.variance_scale_type = variance_scale_type
 
         # tensors with numel <= threshold are not quantized
         # (FirstMoment.threshold / SecondMoment.threshold, adamw_fourbit_triton.py:118, :128)
@@ -109,6 +119,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self._norm_buffers = {}
         self.__dict__.setdefault("kernel_timing", None)
         self.__dict__.setdefault("last_grad_norm", None)
+        self.__dict__.setdefault("variance_scale_type", "group")
         for group in self.param_groups:
             group.setdefault("fused", None)
         state_values = list(self.state.values())
@@ -130,13 +141,33 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             state["exp_avg_sq"] = torch.zeros((nbytes,), dtype=torch.uint8, device=p.device)
             state["momentum_qstate"]["overhead"]["max1"] = torch.zeros(
                 (nblk,), dtype=torch.float32, device=p.device)
-            state["variance_qstate"]["overhead"]["max1"] = torch.zeros(
-                (nblk,), dtype=torch.float32, device=p.device)
+            if self._use_rank1(p):
+                self._init_rank1_overhead(p, state["variance_qstate"]["overhead"])
+            else:
+                state["variance_qstate"]["overhead"]["max1"] = torch.zeros(
+                    (nblk,), dtype=torch.float32, device=p.device)
         else:
             state["exp_avg"] = torch.zeros_like(p, dtype=torch.float32,
                                                 memory_format=torch.contiguous_format)
             state["exp_avg_sq"] = torch.zeros_like(p, dtype=torch.float32,
                                                    memory_format=torch.contiguous_format)
+
+    def _use_rank1(self, p):
+        return self.variance_scale_type == "rank1" and _q.rank1_eligible(p)
+
+    @staticmethod
+    def _init_rank1_overhead(p, overhead, row_max=None, col_max=None):
+        """Statistics of a rank-1-scaled second moment, keys as in the draft's metadata
+        (adamw_fourbit_triton.py:846-852): max_dims = [row maxima [rows, 1], column maxima
+        [1, cols]], max1 = None; scratch_dims are same-sized buffers the step accumulates
+        the new maxima in (zeros between steps)."""
+        rows, cols = p.shape
+        z = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=p.device)
+        overhead["dim"] = 2
+        overhead["max1"] = None
+        overhead["max_dims"] = [z(rows, 1) if row_max is None else row_max.reshape(rows, 1),
+                                z(1, cols) if col_max is None else col_max.reshape(1, cols)]
+        overhead["scratch_dims"] = [z(rows, 1), z(1, cols)]
 
     def _init_group(
         self,
@@ -186,14 +217,22 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             if src is None:
                 continue
             dst = self.state[p]
+            if torch.is_tensor(dst.get("step")):
+                # the base class hands the source's own tensor on; step() advances it in place
+                dst["step"] = dst["step"].detach().clone()
             for key in ("exp_avg", "exp_avg_sq"):
                 if torch.is_tensor(src.get(key)):
                     dst[key] = src[key].detach().to(device=p.device, copy=True)
             for key in ("momentum_qstate", "variance_qstate"):
-                max1 = src.get(key, {}).get("overhead", {}).get("max1")
+                overhead = src.get(key, {}).get("overhead", {})
+                max1 = overhead.get("max1")
                 if torch.is_tensor(max1):
                     dst[key]["overhead"]["max1"] = max1.detach().to(
                         device=p.device, dtype=torch.float32, copy=True)
+                if "max_dims" in overhead:      # rank-1 statistics; the scratch restarts from zero
+                    rmax, cmax = (t.detach().to(device=p.device, dtype=torch.float32, copy=True)
+                                  for t in overhead["max_dims"])
+                    self._init_rank1_overhead(p, dst[key]["overhead"], rmax, cmax)
             if "momentum_qstate" not in src:
                 self._adopt_adamw_state(p, dst)
         self._launch_cache = {}
@@ -215,7 +254,12 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self.init_qstate(p, "variance")
         if state["momentum_qstate"]["enable"]:
             state["exp_avg"], state["momentum_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg, 0)
-            state["exp_avg_sq"], state["variance_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg_sq, 1)
+            if self._use_rank1(p):
+                codes, rmax, cmax = _q.quantize_state_rank1(exp_avg_sq.reshape(p.shape))
+                state["exp_avg_sq"] = codes
+                self._init_rank1_overhead(p, state["variance_qstate"]["overhead"], rmax, cmax)
+            else:
+                state["exp_avg_sq"], state["variance_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg_sq, 1)
         else:
             state["exp_avg"] = exp_avg.contiguous().clone()
             state["exp_avg_sq"] = exp_avg_sq.contiguous().clone()
@@ -235,7 +279,12 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 continue
             if st["momentum_qstate"]["enable"]:
                 m = _q.dequantize_state(st["exp_avg"], st["momentum_qstate"]["overhead"]["max1"], p.numel(), 0)
-                v = _q.dequantize_state(st["exp_avg_sq"], st["variance_qstate"]["overhead"]["max1"], p.numel(), 1)
+                v_meta = st["variance_qstate"]["overhead"]
+                if "max_dims" in v_meta:
+                    v = _q.dequantize_state_rank1(st["exp_avg_sq"], v_meta["max_dims"][0].reshape(-1),
+                                                  v_meta["max_dims"][1].reshape(-1))
+                else:
+                    v = _q.dequantize_state(st["exp_avg_sq"], v_meta["max1"], p.numel(), 1)
             else:
                 m, v = st["exp_avg"].clone(), st["exp_avg_sq"].clone()
             out_state[pid] = {"step": st["step"].detach().clone(),
@@ -371,7 +420,10 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             buckets: Dict[Any, list] = {}
             for i, param in enumerate(params_with_grad):
                 assert param.is_cuda, "param must be on cuda"
-                key = (momentum_quant_enabled[i], param.device, param.dtype, grads[i].dtype, steps[i])
+                kind = momentum_quant_enabled[i]
+                if kind and "max_dims" in variance_meta[i]:
+                    kind = "rank1"
+                key = (kind, param.device, param.dtype, grads[i].dtype, steps[i])
                 buckets.setdefault(key, []).append(i)
 
             for (quantized, device, p_dtype, g_dtype, t_step), idx in buckets.items():
@@ -379,7 +431,12 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 gs = [grads[i] for i in idx]
                 ms = [exp_avgs[i] for i in idx]
                 vs = [exp_avg_sqs[i] for i in idx]
-                if quantized:
+                if quantized == "rank1":
+                    sms = [momentum_meta[i]["max1"] for i in idx]
+                    stats = [[variance_meta[i][k][d] for i in idx]
+                             for k in ("max_dims", "scratch_dims") for d in (0, 1)]
+                    ptrs = tuple(t.data_ptr() for ts in (ps, gs, ms, vs, sms, *stats) for t in ts)
+                elif quantized:
                     sms = [momentum_meta[i]["max1"] for i in idx]
                     svs = [variance_meta[i]["max1"] for i in idx]
                     ptrs = tuple(t.data_ptr() for ts in (ps, gs, ms, vs, sms, svs) for t in ts)
@@ -388,7 +445,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 cache_key = (gi, quantized, device, p_dtype, g_dtype)
                 cached = self._launch_cache.get(cache_key)
                 if cached is None or cached[0] != ptrs:
-                    if quantized:
+                    if quantized == "rank1":
+                        arr = _q.make_rank1_table(ps, gs, ms, vs, sms, stats[0], stats[1], stats[2], stats[3])
+                    elif quantized:
                         arr = _q.make_table(ps, gs, ms, vs, sms, svs)
                     else:
                         arr = _q.make_small_table(ps, gs, ms, vs)
@@ -396,7 +455,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                     cached = (ptrs, arr, tags)
                     self._launch_cache[cache_key] = cached
                 _, arr, (p_tag, g_tag) = cached
-                launch = _q.launch_table if quantized else _q.launch_small_table
+                launch = (_q.launch_rank1_table if quantized == "rank1" else
+                          _q.launch_table if quantized else _q.launch_small_table)
                 options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad)
                 if self.kernel_timing is None:
                     launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
@@ -407,7 +467,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                         start.record()
                         launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                         end.record()
-                    kind = "fused_4bit" if quantized else "fused_single_tensor"
+                    kind = ("fused_4bit_rank1" if quantized == "rank1" else
+                            "fused_4bit" if quantized else "fused_single_tensor")
                     self.kernel_timing.append((kind, start, end))
 
         return loss

@@ -320,3 +320,37 @@ def dequantize_state(codes, scales, numel, which):
                                   out.data_ptr(), _stream(codes.device))
     _lib.check(rc, "dequantize")
     return out
+
+
+def quantize_state_rank1(x):
+    """fp32 second moment of a matrix (on a GPU) -> (packed uint8 codes, row maxima [rows],
+    column maxima [cols]); element (i, j) is divided by min(row_max[i], col_max[j]).  Device
+    form of variance_quant with rank-1 scaling (optim/adamw_fourbit_triton.py:803-863)."""
+    L = _lib.load()
+    assert x.is_cuda and x.dim() == 2 and x.shape[1] % 8 == 0, "needs a cuda matrix with cols % 8 == 0"
+    x = x.detach().to(torch.float32).contiguous()
+    rows, cols = x.shape
+    codes = torch.empty((rows * cols + 1) // 2, dtype=torch.uint8, device=x.device)
+    row_max = torch.empty(rows, dtype=torch.float32, device=x.device)
+    col_max = torch.empty(cols, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.q4adamw_quantize_rank1(x.data_ptr(), rows, cols, codes.data_ptr(), row_max.data_ptr(),
+                                      col_max.data_ptr(), _stream(x.device))
+    _lib.check(rc, "quantize_rank1")
+    return codes, row_max, col_max
+
+
+def dequantize_state_rank1(codes, row_max, col_max):
+    """(packed codes, row maxima, column maxima) -> fp32 matrix [rows, cols]
+    (optim/adamw_fourbit_triton.py:520-527)."""
+    L = _lib.load()
+    rows, cols = row_max.numel(), col_max.numel()
+    assert codes.is_cuda and codes.dtype == torch.uint8 and codes.numel() == (rows * cols + 1) // 2
+    for t in (row_max, col_max):
+        assert t.dtype == torch.float32 and t.device == codes.device and t.is_contiguous()
+    out = torch.empty(rows, cols, dtype=torch.float32, device=codes.device)
+    with torch.cuda.device(codes.device):
+        rc = L.q4adamw_dequantize_rank1(codes.data_ptr(), row_max.data_ptr(), col_max.data_ptr(), rows, cols,
+                                        out.data_ptr(), _stream(codes.device))
+    _lib.check(rc, "dequantize_rank1")
+    return out

@@ -162,3 +162,87 @@ def test_rank1_argument_errors(cuda):
     with pytest.raises(AssertionError, match="rank-1"):
         q.make_rank1_table([torch.zeros(4, 100, device=cuda)], [torch.zeros(4, 100, device=cuda)], [d.m], [d.v],
                            [d.sm], [d.r], [d.c], [d.rn], [d.cn])
+
+
+# ---------------------------------------------------------------------------
+# interchange kernels and the optimizer class
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(1, 8), (7, 24), (64, 512), (130, 1032), (300, 264)])
+def test_rank1_quantize_dequantize_against_oracle(cuda, shape):
+    gen = torch.Generator().manual_seed(shape[0] + shape[1])
+    x = torch.rand(shape, generator=gen) ** 6
+    x[shape[0] // 2] = 0.0
+    x[:, 3] = 0.0
+    codes, rmax, cmax = q.quantize_state_rank1(x.to(cuda))
+    rc, rr, rcm = ot.quantize_rank1(x)
+    assert torch.equal(codes.cpu(), rc) and torch.equal(rmax.cpu(), rr) and torch.equal(cmax.cpu(), rcm)
+    back = q.dequantize_state_rank1(codes, rmax, cmax)
+    want = ot.dequantize_rank1(rc, rr, rcm)
+    assert torch.equal(back.cpu().view(torch.int32), want.view(torch.int32))
+    # signed input: statistics are maxima of magnitudes
+    y = x.clone()
+    y[0] = -y[0]
+    _, r2, c2 = q.quantize_state_rank1(y.to(cuda))
+    assert torch.equal(r2.cpu(), rr) and torch.equal(c2.cpu(), rcm)
+
+
+def _mlp(cuda, seed):
+    torch.manual_seed(seed)
+    return torch.nn.Sequential(torch.nn.Linear(512, 96), torch.nn.Tanh(), torch.nn.Linear(96, 1024),
+                               torch.nn.Tanh(), torch.nn.Linear(1024, 16)).to(cuda)
+
+
+def test_optimizer_rank1_layout_tracking_and_resume(cuda):
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+    with pytest.raises(ValueError, match="variance_scale_type"):
+        AdamWFused_QuantFour([torch.nn.Parameter(torch.zeros(2, device=cuda))], variance_scale_type="rank2")
+    model, twin = _mlp(cuda, 3), _mlp(cuda, 3)
+    opt = AdamWFused_QuantFour(model.parameters(), lr=1e-3, weight_decay=0.01, variance_scale_type="rank1")
+    ref = torch.optim.AdamW(twin.parameters(), lr=1e-3, weight_decay=0.01)
+    for it in range(10):
+        x = torch.randn(32, 512, device=cuda)
+        for m_, o_ in ((model, opt), (twin, ref)):
+            o_.zero_grad(set_to_none=True)
+            m_(x).square().mean().backward()
+            o_.step()
+    # layout: [96, 512] and [16, 1024] are rank-1 (cols >= 512), [1024, 96] keeps block scales
+    w0, w1, w2 = model[0].weight, model[2].weight, model[4].weight
+    ov = lambda p: opt.state[p]["variance_qstate"]["overhead"]
+    assert [tuple(t.shape) for t in ov(w0)["max_dims"]] == [(96, 1), (1, 512)] and ov(w0)["max1"] is None
+    assert [tuple(t.shape) for t in ov(w2)["max_dims"]] == [(16, 1), (1, 1024)]
+    assert "max_dims" not in ov(w1) and ov(w1)["max1"].numel() == 1024 * 96 // 128
+    assert all(not t.any() for t in ov(w0)["scratch_dims"])
+    assert opt.state[model[0].bias]["exp_avg_sq"].dtype == torch.float32      # below the threshold
+    # the draft's own bar against AdamW (tests/driver.py:70-71)
+    for a, b in zip(model.parameters(), twin.parameters()):
+        torch.testing.assert_close(a, b, atol=0.025, rtol=1e-5)
+    # export: dequantized second moment is close to AdamW's (4-bit resolution of its scale)
+    exported = opt.adamw_state_dict()["state"]
+    v4 = exported[0]["exp_avg_sq"]
+    v32 = ref.state[twin[0].weight]["exp_avg_sq"]
+    scale = torch.minimum(v32.amax(1, keepdim=True), v32.amax(0, keepdim=True))
+    assert float(((v4 - v32).abs() / scale).max()) < 0.2
+    # resume from a state_dict: bit-identical continuation
+    sd = opt.state_dict()
+    model2 = _mlp(cuda, 4)
+    model2.load_state_dict(model.state_dict())
+    opt2 = AdamWFused_QuantFour(model2.parameters(), lr=1e-3, weight_decay=0.01, variance_scale_type="rank1")
+    opt2.load_state_dict(sd)
+    x = torch.randn(32, 512, device=cuda)
+    for m_, o_ in ((model, opt), (model2, opt2)):
+        o_.zero_grad(set_to_none=True)
+        m_(x).square().mean().backward()
+        o_.step()
+    for a, b in zip(model.parameters(), model2.parameters()):
+        assert torch.equal(a, b)
+    for pa, pb in zip(model.parameters(), model2.parameters()):
+        sa, sb = opt.state[pa], opt2.state[pb]
+        assert torch.equal(sa["exp_avg_sq"], sb["exp_avg_sq"]) and torch.equal(sa["exp_avg"], sb["exp_avg"])
+    # adopting torch.optim.AdamW's state quantizes the second moment with rank-1 statistics
+    opt3 = AdamWFused_QuantFour(_mlp(cuda, 3).parameters(), lr=1e-3, variance_scale_type="rank1")
+    opt3.load_state_dict(ref.state_dict())
+    p3 = opt3.param_groups[0]["params"][0]
+    md = opt3.state[p3]["variance_qstate"]["overhead"]["max_dims"]
+    assert torch.equal(md[0].reshape(-1), v32.amax(1)) and torch.equal(md[1].reshape(-1), v32.amax(0))
+    want_codes, _, _ = ot.quantize_rank1(v32.cpu())
+    assert torch.equal(opt3.state[p3]["exp_avg_sq"].cpu(), want_codes)
