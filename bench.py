@@ -179,6 +179,9 @@ def main():
                     help="also unscale the gradients by 1/1024 and clip them to a global norm of 1.0 "
                          "in every step: 'fused' = norm kernel + multiplier inside the step, "
                          "'separate' = torch's foreach multiply and clip_grad_norm_ passes, then the step")
+    ap.add_argument("--variance-scale", choices=["group", "rank1"], default="group",
+                    help="scaling of the second moment: per-128 block maxima (the fused CUDA path) or "
+                         "rank-1 row/column maxima for matrices (a statistics pass precedes the update)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, run a plain 4 GiB device copy three times, so that "
@@ -213,7 +216,7 @@ def main():
     total_params = sum(p.numel() for p in params)
     quant_params = sum(p.numel() for p in params if p.numel() > 4096)
 
-    opt = AdamWFused_QuantFour(params, **HP)
+    opt = AdamWFused_QuantFour(params, variance_scale_type=args.variance_scale, **HP)
     opt.kernel_timing = []  # (kind, start event, end event) per launch
 
     def one_step(i):
@@ -242,9 +245,13 @@ def main():
 
     # one entry per step: the step's fused launches (one kernel per batch of up to 48
     # tensors, back to back on the stream) between two events
-    fused_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "fused_4bit"]
-    avg_kernel_s = sum(fused_ms) / len(fused_ms) / 1e3
-    launches_per_step = -(-sum(1 for p in params if p.numel() > 4096) // 48)
+    fused_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind.startswith("fused_4bit")]
+    avg_kernel_s = sum(fused_ms) / args.steps / 1e3
+    rank1 = [p for p in params if opt.state[p]["variance_qstate"]["overhead"].get("max_dims") is not None]
+    grouped = sum(1 for p in params if p.numel() > 4096) - len(rank1)
+    # kernels per step: one per batch of 48 block-scaled tensors; statistics + update +
+    # commit per batch of 32 rank-1 tensors
+    launches_per_step = -(-grouped // 48) + 3 * -(-len(rank1) // 32)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.float32, device=device).normal_()
@@ -253,6 +260,12 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
     algo_bytes = quant_params * bytes_per_param(p_dtype_s, g_dtype_s)
+    if rank1:
+        # the statistics pass reads g and the second moment's codes once more; no block scales
+        # for the second moment, row and column maxima instead (read twice, written twice)
+        gb = 4 if g_dtype_s == "float32" else 2
+        n1 = sum(p.numel() for p in rank1)
+        algo_bytes += n1 * (gb + 0.5 - 2 * 4 / 128.0) + sum(16 * (p.shape[0] + p.shape[1]) for p in rank1)
     achieved = algo_bytes / avg_kernel_s / 1e9
 
     out = {
@@ -281,7 +294,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "fused_4bit_kernel",
+            "kernel": "fused_4bit_kernel" if not rank1 else "rank1_stats_kernel + fused_4bit_rank1_kernel",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -289,7 +302,7 @@ def main():
             # per launch, averaged over the step's launches (they differ in size): measured
             # HBM bytes, algorithmic bytes, duration; achieved = algorithmic bytes / duration
             "traffic": (MEASURED_TRAFFIC_BYTES_PER_STEP[args.workload] / launches_per_step
-                        if args.workload in MEASURED_TRAFFIC_BYTES_PER_STEP else None),
+                        if args.workload in MEASURED_TRAFFIC_BYTES_PER_STEP and not rank1 else None),
             "algorithmic_bytes_per_launch": algo_bytes / launches_per_step,
             "kernel_ms_per_launch": avg_kernel_s * 1e3 / launches_per_step,
             "kernel_launches_per_step": launches_per_step,
@@ -297,6 +310,8 @@ def main():
             "kernel_ms_per_step": avg_kernel_s * 1e3,
         },
     }
+    if rank1:
+        out["config"]["workload"] += f"; rank-1 scaled second moment on {len(rank1)} matrices"
     if args.clip != "none":
         out["config"]["workload"] += f"; gradients unscaled by 1/1024 and clipped to norm 1.0 ({args.clip})"
         norm_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "grad_norm"]

@@ -135,6 +135,55 @@ def test_state_dict_round_trip_keeps_dtypes():
     assert s_big["momentum_qstate"]["enable"] is True and s_small["momentum_qstate"]["enable"] is False
 
 
+def test_loaded_state_shares_nothing_with_its_source():
+    """load_state_dict(opt.state_dict()) must not leave the two optimizers advancing one step
+    counter or writing one moment buffer"""
+    (big,) = params((50, 130))
+    opt = AdamWFused_QuantFour([big])
+    opt._init_state(big)
+    big2 = torch.nn.Parameter(big.detach().clone())
+    opt2 = AdamWFused_QuantFour([big2])
+    opt2.load_state_dict(opt.state_dict())
+    a, b = opt.state[big], opt2.state[big2]
+    assert a["step"].data_ptr() != b["step"].data_ptr()
+    assert a["exp_avg"].data_ptr() != b["exp_avg"].data_ptr()
+    assert (a["momentum_qstate"]["overhead"]["max1"].data_ptr()
+            != b["momentum_qstate"]["overhead"]["max1"].data_ptr())
+
+
+def test_rank1_state_layout_and_round_trip():
+    """variance_scale_type="rank1": matrices with cols % 8 == 0 and cols >= 512 keep row and
+    column maxima (the draft's max_dims, keepdim shapes) instead of block scales; everything
+    else keeps block scales; a state_dict round trip keeps layout, values and dtypes"""
+    wide, narrow, vec = [torch.nn.Parameter(torch.randn(s).to(torch.bfloat16))
+                         for s in ((12, 1024), (1024, 96), (8192,))]
+    opt = AdamWFused_QuantFour([wide, narrow, vec], variance_scale_type="rank1")
+    for p in (wide, narrow, vec):
+        opt._init_state(p)
+    ov = opt.state[wide]["variance_qstate"]["overhead"]
+    assert ov["max1"] is None and ov["dim"] == 2
+    assert [tuple(t.shape) for t in ov["max_dims"]] == [(12, 1), (1, 1024)]
+    assert [tuple(t.shape) for t in ov["scratch_dims"]] == [(12, 1), (1, 1024)]
+    assert all(t.dtype == torch.float32 and not t.any() for t in ov["max_dims"] + ov["scratch_dims"])
+    assert opt.state[wide]["momentum_qstate"]["overhead"]["max1"].shape == (12 * 1024 // 128,)
+    for p in (narrow, vec):
+        o = opt.state[p]["variance_qstate"]["overhead"]
+        assert "max_dims" not in o and o["max1"].shape == (p.numel() // 128,)
+    ov["max_dims"][0].fill_(1.0 + 2.0 ** -20)            # not a bf16 value
+    ov["max_dims"][1].fill_(3.0)
+    ov["scratch_dims"][1].fill_(9.0)                     # scratch is not state: it restarts from zero
+    wide2, narrow2, vec2 = [torch.nn.Parameter(p.detach().clone()) for p in (wide, narrow, vec)]
+    opt2 = AdamWFused_QuantFour([wide2, narrow2, vec2])  # the layout follows the checkpoint
+    opt2.load_state_dict(opt.state_dict())
+    o2 = opt2.state[wide2]["variance_qstate"]["overhead"]
+    assert o2["max_dims"][0].dtype == torch.float32 and bool((o2["max_dims"][0] == 1.0 + 2.0 ** -20).all())
+    assert bool((o2["max_dims"][1] == 3.0).all()) and tuple(o2["max_dims"][1].shape) == (1, 1024)
+    assert all(not t.any() for t in o2["scratch_dims"])
+    assert o2["max_dims"][0].data_ptr() != ov["max_dims"][0].data_ptr()
+    with pytest.raises(ValueError, match="variance_scale_type"):
+        AdamWFused_QuantFour([wide], variance_scale_type="rank2")
+
+
 def test_setstate_backfills():
     (p,) = params((4, 4))
     opt = AdamWFused_QuantFour([p])
