@@ -853,7 +853,9 @@ __device__ __forceinline__ void atomic_max_nonneg(const float *addr, float x) {
 // tile's rows: one atomic per column per tile, one per row per wave.
 template <bool GBF, bool EXT>
 __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
-  __shared__ uint32_t row_bits[kStatRows];
+  constexpr int kAhead = 4;  // rows whose loads are in flight together
+  // row maxima of each 16-lane quarter of each wave; reduced by the last phase
+  __shared__ uint32_t row_bits[kWaves * 4][kStatRows];
   const uint32_t chunk = blockIdx.x;
   float gscale = 1.0f;
   if (EXT && !grad_ops_begin(args.go, gscale)) return;
@@ -868,8 +870,6 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   const bool active = col < T.cols;  // cols is a multiple of 8: all 8 columns or none
   const int64_t row0 = (int64_t)rg * kStatRows;
   const int nrows = (int)(row0 + kStatRows < T.rows ? kStatRows : T.rows - row0);
-  if (tid < kStatRows) row_bits[tid] = 0u;
-  __syncthreads();
   // lanes past the last column work on zeros: code 0 under a zero scale and a zero
   // gradient give a zero second moment, which leaves every maximum alone
   float c_old[8], c_max[8];
@@ -878,41 +878,52 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
     c_old[k] = active ? as_global<const float>(T.cmax)[col + k] : 0.0f;
     c_max[k] = 0.0f;
   }
-  const bool wave_active = (int64_t)cg * kStatCols + wave * kStatColsPerWave < T.cols;
-  if (wave_active) {
-
-    for (int r = 0; r < nrows; ++r) {
+  const uint32_t quarter = (uint32_t)wave * 4u + ((uint32_t)lane >> 4);
+  for (int r0 = 0; r0 < nrows; r0 += kAhead) {
+    // a group past the tile's last row repeats that row: maxima do not mind
+    u32x4 gw[kAhead][GBF ? 1 : 2];
+    uint32_t vw[kAhead];
+    float r_old[kAhead];
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      const int r = r0 + i < nrows ? r0 + i : nrows - 1;
       const int64_t row = row0 + r;
-      const float r_old = as_global<const float>(T.rmax)[row];
+      r_old[i] = as_global<const float>(T.rmax)[row];
       const int64_t e = row * T.cols + col;
-      float g[8];
+      vw[i] = 0u;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) g[k] = 0.0f;
-      uint32_t vw = 0;
+      for (int h = 0; h < (GBF ? 1 : 2); ++h) gw[i][h] = u32x4{0u, 0u, 0u, 0u};
       if (active) {
-        vw = *as_global<const uint32_t>(T.v + (e >> 1));
+        vw[i] = *as_global<const uint32_t>(T.v + (e >> 1));
         if (GBF) {
-          const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 2);
-          widen_bf16_pair(w.x, g[0], g[1]);
-          widen_bf16_pair(w.y, g[2], g[3]);
-          widen_bf16_pair(w.z, g[4], g[5]);
-          widen_bf16_pair(w.w, g[6], g[7]);
+          gw[i][0] = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 2);
         } else {
-#pragma unroll
-          for (int k = 0; k < 8; k += 4) {
-            const u32x4 w = *as_global<const u32x4>(static_cast<const char *>(T.g) + (e + k) * 4);
-            g[k] = bits2f(w.x); g[k + 1] = bits2f(w.y); g[k + 2] = bits2f(w.z); g[k + 3] = bits2f(w.w);
-          }
+          gw[i][0] = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 4);
+          gw[i][GBF ? 0 : 1] = *as_global<const u32x4>(static_cast<const char *>(T.g) + (e + 4) * 4);
         }
       }
-      const uint32_t even = vw & 0x0F0F0F0Fu, odd = (vw >> 4) & 0x0F0F0F0Fu;  // one code per byte
+    }
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      float g[8];
+      if (GBF) {
+        widen_bf16_pair(gw[i][0].x, g[0], g[1]);
+        widen_bf16_pair(gw[i][0].y, g[2], g[3]);
+        widen_bf16_pair(gw[i][0].z, g[4], g[5]);
+        widen_bf16_pair(gw[i][0].w, g[6], g[7]);
+      } else {
+        const u32x4 lo = gw[i][0], hi = gw[i][GBF ? 0 : 1];
+        g[0] = bits2f(lo.x); g[1] = bits2f(lo.y); g[2] = bits2f(lo.z); g[3] = bits2f(lo.w);
+        g[4] = bits2f(hi.x); g[5] = bits2f(hi.y); g[6] = bits2f(hi.z); g[7] = bits2f(hi.w);
+      }
+      const uint32_t even = vw[i] & 0x0F0F0F0Fu, odd = (vw[i] >> 4) & 0x0F0F0F0Fu;  // one code per byte
       float r_max = 0.0f;
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const float gk = EXT ? g[k] * gscale : g[k];
         const uint32_t code = ((k & 1 ? odd : even) >> (8 * (k >> 1))) & 0xffu;
         const float code_value = __builtin_fmaf((float)code, 0.0625f, 0.0625f);  // (code + 1) / 16, exact
-        const float v_old = code_value * __builtin_fminf(r_old, c_old[k]);
+        const float v_old = code_value * __builtin_fminf(r_old[i], c_old[k]);
         const float v = args.b2 * v_old + args.r2 * (gk * gk);
         c_max[k] = __builtin_fmaxf(c_max[k], v);
         r_max = __builtin_fmaxf(r_max, v);
@@ -921,17 +932,22 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
       u = dpp_umax<0xB1>(u);
       u = dpp_umax<0x4E>(u);
       u = dpp_umax<0x141>(u);
-      u = dpp_umax<0x140>(u);           // maximum of each 16-lane row, in all its lanes
-      if ((lane & 15) == 0 && u != 0u) atomicMax(&row_bits[r], u);
-    }
-    if (active) {
-#pragma unroll
-      for (int k = 0; k < 8; ++k)
-        if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
+      u = dpp_umax<0x140>(u);           // maximum of each 16-lane quarter, in all its lanes
+      if ((lane & 15) == 0) row_bits[quarter][r0 + i] = u;   // slots past nrows are not read
     }
   }
+  if (active) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
+  }
   __syncthreads();
-  if (tid < nrows && row_bits[tid] != 0u) atomic_max_nonneg(T.rmax_next + row0 + tid, bits2f(row_bits[tid]));
+  if (tid < nrows) {
+    uint32_t u = 0u;
+#pragma unroll
+    for (int qi = 0; qi < kWaves * 4; ++qi) u = u > row_bits[qi][tid] ? u : row_bits[qi][tid];
+    if (u != 0u) atomic_max_nonneg(T.rmax_next + row0 + tid, bits2f(u));
+  }
 }
 
 template <bool PBF, bool GBF, bool EXT>
