@@ -132,6 +132,27 @@ int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_
                                 const q4adamw_grad_options *opt, void *stream);
 
 /*
+ * q4adamw_fused_4bit_multi_ex with stochastic rounding in the quantizer of both
+ * moments: a normalised value between two neighbouring code-book entries Q[k] and
+ * Q[k+1] takes the upper one with probability (x - Q[k]) / (Q[k+1] - Q[k]) instead of
+ * the nearer one; values at or beyond the ends of the code book take the end codes.
+ * The rule of quantize_bsearch<STOCHASTIC> quoted at
+ * optim/adamw_fourbit_triton.py:1050-1075, evaluated without its division as
+ * noise * (Q[k+1] - Q[k]) < x - Q[k].  The noise of an element is a hash of its index
+ * and of q4adamw_sr_tensor_salt(seed, step, salts[i]) (salts == NULL: the tensor's
+ * position in the list), so a call is reproducible and two steps, tensors or seeds
+ * draw different noise; the reference's optimizers agree on such a seed across ranks
+ * (optim/adamw_fourbit_triton.py:163-165).  Scales stay the blocks' abs-maxima.
+ */
+int q4adamw_fused_4bit_multi_sr(const q4adamw_tensor *tensors, int count, const uint32_t *salts,
+                                uint64_t seed, int p_dtype, int g_dtype, float beta1, float beta2,
+                                float lr, float weight_decay, float eps, float step,
+                                const q4adamw_grad_options *opt, void *stream);
+
+/* Host-only: the 32-bit noise salt of one tensor in one step (for tests). */
+uint32_t q4adamw_sr_tensor_salt(uint64_t seed, float step, uint32_t tensor_salt);
+
+/*
  * One quantized matrix whose second moment is rank-1 scaled: the scale of element
  * (i, j) is min(row_max[i], col_max[j]), the maxima of the second moment over row i
  * and over column j (get_variance_tensor_statistics / compute_variance_tensor_scale,

@@ -178,6 +178,102 @@ def step_quant_rank1(p, g, m_codes, v_codes, m_scale, row_max, col_max, *, beta1
     return p_new.to(p.dtype).view_as(p), mc, vc, ms, rmax, cmax
 
 
+# ---------------------------------------------------------------------------
+# stochastic rounding in the quantizer
+#
+# The reference quotes lpmm's quantizer in a docstring and never runs it
+# (optim/adamw_fourbit_triton.py:969-997 kernel with Philox noise, :1050-1075
+# quantize_bsearch<STOCHASTIC>): the value's interval [Q[k], Q[k+1]) of the code book is
+# found, proba = (x - Q[k]) / (Q[k+1] - Q[k]), and the upper code is taken when
+# rn(proba + noise - 0.5) is non-zero, i.e. with probability proba; values at or beyond the
+# ends of the code book take the end codes.  This build's statement of it avoids the
+# division and fixes the noise as a function of (seed, step, tensor, element), so that the
+# result is reproducible bit for bit:
+#     up  <=>  RN(u * w[k]) < RN(q - Q[k]),   w[k] = RN(Q[k+1] - Q[k]),
+#     u = (2 n + 1) / 2^17 with n a 16-bit hash value (never 0, never 1).
+# Parity with the reference is UNPINNED (it has no runnable counterpart); pinned by
+# brute force, by exactness on code-book values and by the rounding's mean
+# (tests/test_oracle_pins.py).
+# ---------------------------------------------------------------------------
+_M32 = np.uint64(0xFFFFFFFF)
+
+
+def lowbias32(x):
+    """A 32-bit integer mixer (two multiply-xorshift rounds); x: numpy array of uint32
+    values held in uint64."""
+    x = np.asarray(x, np.uint64) & _M32
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7FEB352D)) & _M32
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846CA68B)) & _M32
+    x ^= x >> np.uint64(16)
+    return x
+
+
+def sr_tensor_salt(seed, step, tensor_salt):
+    """32-bit salt of one tensor in one step: nested mixes of the tensor's salt, the step
+    number and the two halves of the 64-bit seed."""
+    h = lowbias32(np.uint64(int(tensor_salt) & 0xFFFFFFFF))
+    h = lowbias32(h ^ np.uint64(int(step) & 0xFFFFFFFF))
+    h = lowbias32(h ^ np.uint64((int(seed) >> 32) & 0xFFFFFFFF))
+    h = lowbias32(h ^ np.uint64(int(seed) & 0xFFFFFFFF))
+    return int(h)
+
+
+def sr_noise(numel, salt):
+    """(u_first_moment, u_second_moment) for elements 0..numel-1 of a tensor: float32 arrays
+    of values (2 n + 1) / 2^17, n = high / low half of the element's hash."""
+    e = np.arange(numel, dtype=np.uint64)
+    key = (e & _M32) ^ np.uint64(salt) ^ (((e >> np.uint64(32)) * np.uint64(0x9E3779B9)) & _M32)
+    h = lowbias32(key)
+    to_u = lambda n: ((2.0 * n.astype(np.float64) + 1.0) / 2.0 ** 17).astype(np.float32)   # exact
+    return to_u(h >> np.uint64(16)), to_u(h & np.uint64(0xFFFF))
+
+
+def quantize_sr(x, which, u):
+    """Per-128 abs-max scale, then stochastic rounding between the two neighbouring code-book
+    values.  x: fp32 torch vector, u: float32 numpy noise per element.  Returns (packed
+    codes, scales)."""
+    numel = x.numel()
+    nblk = (numel + BLOCK - 1) // BLOCK
+    padded = np.zeros(nblk * BLOCK, np.float32)
+    padded[:numel] = x.numpy()
+    noise = np.zeros(nblk * BLOCK, np.float32)
+    noise[:numel] = u
+    grouped = padded.reshape(nblk, BLOCK)
+    max1 = np.abs(grouped).max(axis=1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        q = (grouped / max1).reshape(-1)                     # 0/0 -> NaN -> code 0
+    Q = QMAP[which].numpy()
+    # k_raw = number of code-book values <= q; the tables are extended so that both ends
+    # need no special case: below Q[0] the "gap" is 0 (always up, from -1 to 0), at or
+    # above Q[15] it is infinite (never up)
+    k_raw = np.searchsorted(Q, np.nan_to_num(q, nan=-4.0), side="right")
+    lower = np.concatenate(([-np.finfo(np.float32).max], Q)).astype(np.float32)
+    gap = np.concatenate(([0.0], (Q[1:] - Q[:-1]).astype(np.float32), [np.inf])).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        d = q - lower[k_raw]
+        t = noise * gap[k_raw]
+        up = t < d
+    code = np.clip(k_raw - 1 + up, 0, 15)
+    code[np.isnan(q)] = 0
+    return pack(torch.from_numpy(code.astype(np.int64))[:numel], numel), torch.from_numpy(max1.reshape(-1))
+
+
+def step_quant_sr(p, g, m_codes, v_codes, m_scale, v_scale, *, seed, tensor_salt, beta1, beta2, lr,
+                  weight_decay, eps, step):
+    """step_quant with stochastic rounding of both moments (CPU tensors)."""
+    numel = p.numel()
+    sc = derive_scalars(beta1, beta2, lr, weight_decay, step)
+    m = dequantize(m_codes, m_scale, numel, 0)
+    v = dequantize(v_codes, v_scale, numel, 1)
+    p_new, m_new, v_new = adamw_update(p.reshape(-1).float(), g.reshape(-1).float(), m, v, sc, eps)
+    um, uv = sr_noise(numel, sr_tensor_salt(seed, step, tensor_salt))
+    mc, ms = quantize_sr(m_new, 0, um)
+    vc, vs = quantize_sr(v_new, 1, uv)
+    return p_new.to(p.dtype).view_as(p), mc, vc, ms, vs
+
+
 def closed_form_tables():
     """Independent constructions of the four tables (double precision, then fp32):
     second moment k/16 and (2k+1)/32 (quant_opt_base.py:88-102); first moment from

@@ -78,6 +78,8 @@ EXPORTS = (
     "q4adamw_fused_4bit",
     "q4adamw_fused_4bit_multi",
     "q4adamw_fused_4bit_multi_ex",
+    "q4adamw_fused_4bit_multi_sr",
+    "q4adamw_sr_tensor_salt",
     "q4adamw_fused_4bit_rank1_multi",
     "q4adamw_fused_single_tensor",
     "q4adamw_fused_single_tensor_multi",
@@ -124,6 +126,11 @@ def load():
     L.q4adamw_fused_4bit_multi_ex.restype = i
     L.q4adamw_fused_single_tensor_multi_ex.argtypes = [ctypes.POINTER(Q4SmallTensor), i, i, i] + hyper + [opt, vp]
     L.q4adamw_fused_single_tensor_multi_ex.restype = i
+    L.q4adamw_fused_4bit_multi_sr.argtypes = ([ctypes.POINTER(Q4Tensor), i, ctypes.POINTER(ctypes.c_uint32),
+                                               ctypes.c_uint64, i, i] + hyper + [opt, vp])
+    L.q4adamw_fused_4bit_multi_sr.restype = i
+    L.q4adamw_sr_tensor_salt.argtypes = [ctypes.c_uint64, f, ctypes.c_uint32]
+    L.q4adamw_sr_tensor_salt.restype = ctypes.c_uint32
     L.q4adamw_fused_4bit_rank1_multi.argtypes = [ctypes.POINTER(Q4Rank1Tensor), i, i, i] + hyper + [opt, vp]
     L.q4adamw_fused_4bit_rank1_multi.restype = i
     L.q4adamw_grad_norm.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, ctypes.c_size_t, vp, vp]

@@ -87,6 +87,7 @@ struct FusedArgs {
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
   TensorDesc desc[kMaxTensors];
+  uint32_t sr_salt[kMaxTensors];  // stochastic rounding: the tensors' noise salts of this step
 };
 
 struct SmallDesc {  // 40 bytes
@@ -220,6 +221,9 @@ static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(N
 // the first-moment bucket table (see q4adamw_tables.h), copied into LDS by every
 // workgroup at start-up, one entry per thread
 __device__ const HalfTable kHalfTable = make_half_table();
+// stochastic rounding: code-book entries per bucket and the 17 intervals between them
+__device__ const SrHalfTable kSrHalfTable = make_sr_half_table();
+__device__ const SrIntervalTable kSrIntervals = make_sr_interval_table();
 // first-moment code book for kernels that index it per lane
 __device__ const uint32_t kQmapMDev[16] = {
     0xbf633333u, 0xbf29999au, 0xbee00000u, 0xbe59999au, 0xbd9eb852u, 0xbd051eb8u,
@@ -440,6 +444,54 @@ __device__ __forceinline__ uint32_t quantize_exact_scales(const Vals<N> &v, cons
   return word;
 }
 
+// A 32-bit integer mixer (two multiply-xorshift rounds) for the rounding noise.
+__host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7FEB352Du;
+  x ^= x >> 15;
+  x *= 0x846CA68Bu;
+  x ^= x >> 16;
+  return x;
+}
+
+// noise in (0, 1) from a 16-bit number: (2 n + 1) / 2^17, exact
+__device__ __forceinline__ float sr_noise_value(uint32_t n16) {
+  return __builtin_fmaf((float)n16, 1.52587890625e-05f, 7.62939453125e-06f);
+}
+
+// Stochastic rounding, exact form (the closed form of quantize_bsearch<STOCHASTIC>,
+// optim/adamw_fourbit_triton.py:1050-1075, without its division): IEEE quotient, its
+// interval [Q[k], Q[k+1]) among the code-book entries, upper code iff
+// noise * (Q[k+1] - Q[k]) < q - Q[k].  0/0 is NaN and gets code 0.
+template <bool SECOND, int N>
+__device__ __forceinline__ uint32_t quantize_exact_sr(const Vals<N> &v, float scale, const Vals<N> &noise) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float q = v.x[j] / scale;
+    uint32_t k_raw = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float t = SECOND ? qmap_v(k) : bits2f(kQmapMBits[k]);
+      k_raw += (t <= q) ? 1u : 0u;
+    }
+    float lower, width;
+    if (SECOND) {
+      lower = k_raw == 0u ? -3.4028234663852886e38f : (float)k_raw * 0.0625f;
+      width = k_raw == 0u ? 0.0f : (k_raw == 16u ? __builtin_inff() : 0.0625f);
+    } else {
+      const SrInterval iv = kSrIntervals.e[k_raw];
+      lower = iv.lower;
+      width = iv.width;
+    }
+    const bool up = noise.x[j] * width < q - lower;
+    int c = (int)k_raw - 1 + (up ? 1 : 0);
+    c = c < 0 ? 0 : (c > 15 ? 15 : c);
+    word |= (uint32_t)c << (4 * j);
+  }
+  return word;
+}
+
 // (x & mask) | base as one v_and_or_b32: the mask travels in a scalar register (the
 // compiler splits the operation when the mask is a literal, which a VOP3 encoding
 // cannot hold).
@@ -510,21 +562,33 @@ __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
 //               and an entry number fits a byte
 //   [256, 512)  bucket table of the first-moment quantizer, indexed by the high byte
 //               of the quotient as a half
+//   [512, 529)  stochastic rounding only: the first moment's interval table
 constexpr uint32_t kLdsBuckets = 64 * kWaves;
-constexpr uint32_t kLdsEntries = kLdsBuckets + kHalfTableEntries;
+constexpr uint32_t kLdsIntervals = kLdsBuckets + kHalfTableEntries;
+constexpr uint32_t kLdsEntries = kLdsIntervals + 32;
 static_assert(kLdsBuckets == 256, "dequantization entry numbers must fit a byte");
 static_assert(kThreads == (int)kHalfTableEntries, "one bucket table entry per thread");
 
 // What a thread fetches from the constant tables as the very first thing it does.
 struct TableSlot {
-  uint2 entry;  // bucket table entry number tid
-  float qm;     // first-moment code-book value number (lane & 15)
+  uint2 entry;     // bucket table entry number tid
+  float qm;        // first-moment code-book value number (lane & 15)
+  uint2 interval;  // stochastic rounding: interval table entry number tid (tid < 17)
 };
 
+template <bool SR>
 __device__ __forceinline__ TableSlot request_table_slot(int tid) {
   TableSlot s;
-  const MtabEntry e = kHalfTable.e[tid];
-  s.entry = make_uint2(e.lo, e.hi);
+  if (SR) {
+    const SrEntry e = kSrHalfTable.e[tid];
+    s.entry = make_uint2(e.thr, e.base);
+    const SrInterval iv = kSrIntervals.e[tid < 17 ? tid : 0];
+    s.interval = make_uint2(f2bits(iv.lower), f2bits(iv.width));
+  } else {
+    const MtabEntry e = kHalfTable.e[tid];
+    s.entry = make_uint2(e.lo, e.hi);
+    s.interval = make_uint2(0u, 0u);
+  }
   s.qm = bits2f(kQmapMDev[tid & 15]);
   return s;
 }
@@ -533,8 +597,10 @@ __device__ __forceinline__ TableSlot request_table_slot(int tid) {
 // exactly once, after it has issued its global loads, so that the latencies overlap.
 // The fences order LDS only: a full __syncthreads() would also drain the outstanding
 // global loads.
+template <bool SR>
 __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
   lds[kLdsBuckets + tid] = s.entry;
+  if (SR && tid < 17) lds[kLdsIntervals + tid] = s.interval;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -558,10 +624,13 @@ struct Geometry {
 // RANK1 (Desc = Rank1Desc): the second moment's scale is min(row maximum, column
 // maximum) per element instead of one value per block: old statistics dequantize, the
 // step's new statistics (complete before this kernel starts) quantize.
-template <bool PBF, bool GBF, bool FULL, bool EXT, bool RANK1, typename Desc>
+// SR: both moments are rounded stochastically between the two neighbouring code-book
+// entries; the noise of element e is a hash of e and the tensor's salt of this step.
+template <bool PBF, bool GBF, bool FULL, bool EXT, bool RANK1, bool SR, typename Desc>
 __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
-                                             float gscale, bool zero_g) {
+                                             float gscale, bool zero_g, uint32_t salt) {
+  static_assert(!(SR && RANK1), "stochastic rounding is built for block scaling only");
   using G = Geometry<PBF>;
   constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
@@ -661,7 +730,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   const uint32_t cb_entry = (uint32_t)wave * 64u + blk * 16u;  // entry number of code 0
   *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) =
       make_float2(slot.qm * sm_old, qmap_v(lane & 15) * sv_old);
-  setup_tables(lds, tid, slot);
+  setup_tables<SR>(lds, tid, slot);
 
   // entry numbers of the lane's codes, one per byte: even elements, odd elements
   const uint32_t three = 3u;
@@ -738,6 +807,18 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     redo |= r_new > kScaleHi || (__builtin_fminf(r_new, c_min) < kScaleLo && v_lane_max != 0.0f);
   }
   uint32_t mword = 0, vword = 0;
+  Vals<N> um, uv;  // stochastic rounding: the elements' noise
+  if constexpr (SR) {
+    // key = low half of the element index, xor the salt, xor the mixed high half
+    const uint32_t tile_salt = salt ^ ((uint32_t)((uint64_t)tb >> 32) * 0x9E3779B9u);
+    const uint32_t first = (uint32_t)tb + e0;   // a tile never straddles a multiple of 2^32
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const uint32_t h = lowbias32((first + (uint32_t)j) ^ tile_salt);
+      um.x[j] = sr_noise_value(h >> 16);
+      uv.x[j] = sr_noise_value(h & 0xffffu);
+    }
+  }
 #pragma unroll
   for (int j = 0; j < N; j += 2) {
     // first moment: the quotients' bucket entries, two quotients per conversion
@@ -745,20 +826,45 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint32_t halves = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(q0, q1));
     const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<1>(halves, three));
     const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<3>(halves, three));
-    const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
-    redo |= (hi0 != (q0 > bits2f(ent0.x))) | (hi1 != (q1 > bits2f(ent1.x)));
-    // base code in the entry's low nibble, plus one above the threshold; every
-    // code enters the word at the top and moves down four bits per later element
-    mword = __builtin_amdgcn_alignbit(ent0.x + (hi0 ? 1u : 0u), mword, 4);
-    mword = __builtin_amdgcn_alignbit(ent1.x + (hi1 ? 1u : 0u), mword, 4);
+    if constexpr (SR) {
+      // interval among the code-book entries, then up iff noise * width < q - lower end;
+      // a comparison closer than the quotient's error goes to the exact path
+      const float qq[2] = {q0, q1};
+      const uint2 ent[2] = {ent0, ent1};
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t k_raw = ent[h].y + (qq[h] >= bits2f(ent[h].x) ? 1u : 0u);
+        const uint2 iv = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsIntervals * 8u + k_raw * 8u);
+        const float d = qq[h] - bits2f(iv.x), t = um.x[j + h] * bits2f(iv.y);
+        redo |= __builtin_fabsf(t - d) <= __builtin_fabsf(qq[h]) * 4.76837158203125e-07f;  // 2^-21: 4 ulps
+        mword = __builtin_amdgcn_alignbit(k_raw - 1u + (t < d ? 1u : 0u), mword, 4);
+      }
+    } else {
+      const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
+      redo |= (hi0 != (q0 > bits2f(ent0.x))) | (hi1 != (q1 > bits2f(ent1.x)));
+      // base code in the entry's low nibble, plus one above the threshold; every
+      // code enters the word at the top and moves down four bits per later element
+      mword = __builtin_amdgcn_alignbit(ent0.x + (hi0 ? 1u : 0u), mword, 4);
+      mword = __builtin_amdgcn_alignbit(ent1.x + (hi1 ? 1u : 0u), mword, 4);
+    }
 
     // second moment: thresholds at 16q = k + 0.5, k = 1..15
 #pragma unroll
     for (int k = j; k < j + 2; ++k) {
-      const float t = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, kVGuard - 0.5f);
-      vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
-      // t > -1, so truncation gives 0 for t < 0
-      vword = __builtin_amdgcn_alignbit((uint32_t)(int)t, vword, 4);
+      if constexpr (SR) {
+        // code-book entries at 16 q = 1..16: interval number floor(16 q), position in
+        // it fract(16 q), up iff noise < position; the ends clamp
+        const float q16 = vn.x[k] * rv16;
+        const float kf = __builtin_floorf(q16), d16 = q16 - kf;
+        redo |= __builtin_fabsf(uv.x[k] - d16) <= kVGuard;
+        const float cf = __builtin_amdgcn_fmed3f(kf + (uv.x[k] < d16 ? 0.0f : -1.0f), 0.0f, 15.0f);
+        vword = __builtin_amdgcn_alignbit((uint32_t)(int)cf, vword, 4);
+      } else {
+        const float t = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, kVGuard - 0.5f);
+        vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
+        // t > -1, so truncation gives 0 for t < 0
+        vword = __builtin_amdgcn_alignbit((uint32_t)(int)t, vword, 4);
+      }
     }
   }
   if (N == 4) {
@@ -767,9 +873,14 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   }
   redo |= vfrac < 2.0f * kVGuard;
   if (__builtin_expect(redo, 0)) {
-    mword = quantize_exact<false, N>(mn, am);
-    if constexpr (RANK1) vword = quantize_exact_scales<N>(vn, s_new);
-    else vword = quantize_exact<true, N>(vn, av);
+    if constexpr (SR) {
+      mword = quantize_exact_sr<false, N>(mn, am, um);
+      vword = quantize_exact_sr<true, N>(vn, av, uv);
+    } else {
+      mword = quantize_exact<false, N>(mn, am);
+      if constexpr (RANK1) vword = quantize_exact_scales<N>(vn, s_new);
+      else vword = quantize_exact<true, N>(vn, av);
+    }
   }
   if (am == 0.0f) mword = 0;  // 0/0: code 0 for the whole block
   if (!FULL) {
@@ -808,12 +919,12 @@ __device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale)
   return true;
 }
 
-template <bool PBF, bool GBF, bool EXT>
+template <bool PBF, bool GBF, bool EXT, bool SR>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
   using G = Geometry<PBF>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
-  const TableSlot slot = request_table_slot(tid);
+  const TableSlot slot = request_table_slot<SR>(tid);
   const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;  // whole workgroup: the grid is padded to a multiple of 8
   float gscale = 1.0f;
@@ -825,13 +936,14 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
   const int64_t begin = tile * G::kTile;
   if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
-    setup_tables(lds, tid, slot);
+    setup_tables<SR>(lds, tid, slot);
     return;
   }
+  const uint32_t salt = SR ? args.sr_salt[t] : 0u;
   if (begin + G::kTile <= T.numel)
-    process_tile<PBF, GBF, true, EXT, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+    process_tile<PBF, GBF, true, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PBF, GBF, false, EXT, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+    process_tile<PBF, GBF, false, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
@@ -955,7 +1067,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   using G = Geometry<PBF>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
-  const TableSlot slot = request_table_slot(tid);
+  const TableSlot slot = request_table_slot<false>(tid);
   const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;
   float gscale = 1.0f;
@@ -967,13 +1079,13 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
   const int64_t begin = tile * G::kTile;
   if (begin >= T.numel) {
-    setup_tables(lds, tid, slot);
+    setup_tables<false>(lds, tid, slot);
     return;
   }
   if (begin + G::kTile <= T.numel)
-    process_tile<PBF, GBF, true, EXT, true>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+    process_tile<PBF, GBF, true, EXT, true, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, 0u);
   else
-    process_tile<PBF, GBF, false, EXT, true>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g);
+    process_tile<PBF, GBF, false, EXT, true, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, 0u);
 }
 
 // After the update: the new statistics become the current ones and the buffers that
@@ -1329,17 +1441,19 @@ static int launch_small_batch(SmallArgs &a, uint64_t chunks, void (*kernel)(cons
 typedef void (*FusedKernel)(const FusedArgs);
 typedef void (*SmallKernel)(const SmallArgs);
 
-template <bool EXT>
+template <bool EXT, bool SR>
 static FusedKernel pick_fused_ext(bool pb, bool gb) {
-  if (!pb && !gb) return fused_4bit_kernel<false, false, EXT>;
-  if (!pb && gb) return fused_4bit_kernel<false, true, EXT>;
-  if (pb && !gb) return fused_4bit_kernel<true, false, EXT>;
-  return fused_4bit_kernel<true, true, EXT>;
+  if (!pb && !gb) return fused_4bit_kernel<false, false, EXT, SR>;
+  if (!pb && gb) return fused_4bit_kernel<false, true, EXT, SR>;
+  if (pb && !gb) return fused_4bit_kernel<true, false, EXT, SR>;
+  return fused_4bit_kernel<true, true, EXT, SR>;
 }
 
-static FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext) {
+// stochastic rounding comes with the gradient options' kernels only
+static FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext, bool sr = false) {
   const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  return ext ? pick_fused_ext<true>(pb, gb) : pick_fused_ext<false>(pb, gb);
+  if (sr) return pick_fused_ext<true, true>(pb, gb);
+  return ext ? pick_fused_ext<true, false>(pb, gb) : pick_fused_ext<false, false>(pb, gb);
 }
 
 template <bool EXT>
@@ -1403,6 +1517,11 @@ constexpr uint64_t kMaxChunksPerLaunch = 0x7ffffff0ull;  // grid.x limit, with r
 
 using namespace q4;
 
+static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,
+                                 float beta1, float beta2, float lr, float weight_decay, float eps,
+                                 float step, const q4adamw_grad_options *opt, bool sr,
+                                 const uint32_t *salts, uint64_t seed, void *stream);
+
 extern "C" {
 
 void q4adamw_derive_scalars(float beta1, float beta2, float lr, float weight_decay, float step,
@@ -1449,6 +1568,31 @@ int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dty
 int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,
                                 float beta1, float beta2, float lr, float weight_decay, float eps,
                                 float step, const q4adamw_grad_options *opt, void *stream) {
+  return fused_4bit_multi_impl(tensors, count, p_dtype, g_dtype, beta1, beta2, lr, weight_decay, eps,
+                               step, opt, false, nullptr, 0, stream);
+}
+
+int q4adamw_fused_4bit_multi_sr(const q4adamw_tensor *tensors, int count, const uint32_t *salts,
+                                uint64_t seed, int p_dtype, int g_dtype, float beta1, float beta2,
+                                float lr, float weight_decay, float eps, float step,
+                                const q4adamw_grad_options *opt, void *stream) {
+  return fused_4bit_multi_impl(tensors, count, p_dtype, g_dtype, beta1, beta2, lr, weight_decay, eps,
+                               step, opt, true, salts, seed, stream);
+}
+
+uint32_t q4adamw_sr_tensor_salt(uint64_t seed, float step, uint32_t tensor_salt) {
+  uint32_t h = lowbias32(tensor_salt);
+  h = lowbias32(h ^ (uint32_t)step);
+  h = lowbias32(h ^ (uint32_t)(seed >> 32));
+  return lowbias32(h ^ (uint32_t)seed);
+}
+
+}  // extern "C"
+
+static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,
+                                 float beta1, float beta2, float lr, float weight_decay, float eps,
+                                 float step, const q4adamw_grad_options *opt, bool sr,
+                                 const uint32_t *salts, uint64_t seed, void *stream) {
   if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   FusedArgs a;
@@ -1476,7 +1620,7 @@ int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const FusedKernel kernel = pick_fused(p_dtype, g_dtype, ext);
+  const FusedKernel kernel = pick_fused(p_dtype, g_dtype, ext, sr);
   a.ntensors = 0;
   uint64_t chunks = 0;
   for (int i = 0; i < count; ++i) {
@@ -1496,6 +1640,7 @@ int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_
     d.sm = t.exp_avg_scale;
     d.sv = t.exp_avg_sq_scale;
     d.numel = t.numel;
+    a.sr_salt[a.ntensors] = sr ? q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i) : 0u;
     a.first_chunk[a.ntensors] = (uint32_t)chunks;
     ++a.ntensors;
     chunks += c;
@@ -1503,6 +1648,8 @@ int q4adamw_fused_4bit_multi_ex(const q4adamw_tensor *tensors, int count, int p_
   if (a.ntensors > 0) return launch_fused_batch(a, chunks, kernel, s);
   return 0;
 }
+
+extern "C" {
 
 int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
                                    int g_dtype, float beta1, float beta2, float lr,
@@ -1825,6 +1972,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1005; }
+int q4adamw_version(void) { return 1006; }
 
 }  // extern "C"

@@ -141,4 +141,86 @@ constexpr HalfTable make_half_table() {
   return t;
 }
 
+// ---------------------------------------------------------------------------
+// Stochastic rounding (first moment): the interval of a normalised value among the code
+// book's entries.  k_raw = number of entries <= q (0..16); entry [k_raw] of the interval
+// table holds the interval's lower end and its width, extended at both ends so that no
+// case split is needed: below the first entry the width is 0 (always "up", from code -1
+// to code 0), at or above the last one it is infinite (never "up").
+//
+// The half-indexed table gives k_raw as base + (q >= thr): thr is the code-book entry
+// inside the bucket, if any (no bucket holds two).  No guard band: a value within a few
+// ulps of an entry gets the same final code from either neighbouring interval.
+// ---------------------------------------------------------------------------
+struct SrEntry {
+  uint32_t thr;   // fp32 bits of the entry inside the bucket; kNoThr if none
+  uint32_t base;  // number of entries below the whole bucket
+};
+
+Q4_HD constexpr SrEntry sr_entry(uint32_t half_index) {
+  const uint32_t idx = half_index_bucket(half_index);
+  const uint32_t sign = (idx >> 10) & 1u, mag = idx & 1023u, e = mag >> 2;
+  SrEntry out{kNoThr, 0u};
+  if (e >= 128u) {            // |q| >= 2, inf, nan
+    out.base = sign ? 0u : 16u;
+    return out;
+  }
+  if (mag == 0u) {            // the bucket of zero and of every |q| < 2^-14
+    out.base = sign ? 7u : 8u;
+    return out;
+  }
+  const float lo = bits2f(mag << 21), hi = bits2f((mag + 1u) << 21);
+  for (int j = 0; j < 16; ++j) {
+    const float t = bits2f(kQmapMBits[j]);
+    if (!sign) {              // bucket holds q in [lo, hi)
+      if (t < lo) ++out.base;
+      else if (t < hi) out.thr = kQmapMBits[j];
+    } else {                  // bucket holds q in (-hi, -lo]
+      if (t <= -hi) ++out.base;
+      else if (t <= -lo) out.thr = kQmapMBits[j];
+    }
+  }
+  return out;
+}
+
+struct SrHalfTable {
+  SrEntry e[kHalfTableEntries];
+};
+
+constexpr SrHalfTable make_sr_half_table() {
+  SrHalfTable t{};
+  for (uint32_t h = 0; h < kHalfTableEntries; ++h) t.e[h] = sr_entry(h);
+  return t;
+}
+
+// number of code-book entries that some bucket names as its threshold: must be all that
+// are not zero (zero sits on the boundary between the two zero buckets)
+constexpr int sr_thresholds_found() {
+  int n = 0;
+  for (uint32_t h = 0; h < kHalfTableEntries; ++h) n += sr_entry(h).thr != kNoThr ? 1 : 0;
+  return n;
+}
+static_assert(sr_thresholds_found() == 15, "every non-zero code-book entry needs a bucket of its own");
+
+struct SrInterval {
+  float lower, width;
+};
+
+Q4_HD constexpr SrInterval sr_interval_m(uint32_t k_raw) {  // k_raw 0..16
+  if (k_raw == 0u) return SrInterval{-3.4028234663852886e38f, 0.0f};
+  const float lower = bits2f(kQmapMBits[k_raw - 1u]);
+  if (k_raw == 16u) return SrInterval{lower, __builtin_inff()};
+  return SrInterval{lower, bits2f(kQmapMBits[k_raw]) - lower};
+}
+
+struct SrIntervalTable {
+  SrInterval e[17];
+};
+
+constexpr SrIntervalTable make_sr_interval_table() {
+  SrIntervalTable t{};
+  for (uint32_t k = 0; k < 17; ++k) t.e[k] = sr_interval_m(k);
+  return t;
+}
+
 }  // namespace q4

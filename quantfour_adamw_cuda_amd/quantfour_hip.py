@@ -181,6 +181,41 @@ def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, w
                        options)
 
 
+def make_salts(salts):
+    """ctypes uint32 array of per-tensor noise salts for launch_table_sr."""
+    import ctypes
+    return (ctypes.c_uint32 * len(salts))(*[int(x) & 0xFFFFFFFF for x in salts])
+
+
+def launch_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps,
+                    step, options=None):
+    L = _lib.load()
+    assert salts_arr is None or len(salts_arr) == len(arr), "one salt per tensor"
+    with torch.cuda.device(device):
+        rc = L.q4adamw_fused_4bit_multi_sr(arr, len(arr), salts_arr, int(seed) & (2 ** 64 - 1), p_tag, g_tag,
+                                           beta1, beta2, lr, weight_decay, eps, float(step), options,
+                                           _stream(device))
+    _lib.check(rc, "fused_4bit_multi_sr")
+
+
+def fused_4bit_multi_sr(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr, weight_decay, eps,
+                        step, seed, salts=None, grad_scale=1.0, grad_scale_dev=None, found_inf=None,
+                        zero_grad=False):
+    """fused_4bit_multi with stochastic rounding of both moments (the rule quoted at
+    optim/adamw_fourbit_triton.py:1050-1075).  The noise is a function of (seed, step, the
+    tensor's salt, element index): salts defaults to the tensors' positions in the list."""
+    if not ps:
+        return
+    arr = make_table(ps, gs, exps, sqs, exp_scales, sq_scales)
+    p_tag, g_tag = _tag(ps[0], "param"), _tag(gs[0], "grad")
+    for p, g in zip(ps, gs):
+        assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
+            "tensors of one launch must share device and dtypes"
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    launch_table_sr(arr, None if salts is None else make_salts(salts), seed, ps[0].device, p_tag, g_tag,
+                    beta1, beta2, lr, weight_decay, eps, step, options)
+
+
 RANK1_MIN_COLS = 512
 
 

@@ -1,0 +1,116 @@
+"""GPU parity of the fused step with stochastic rounding, through the C ABI, against
+oracle/q4_oracle_torch.py step_quant_sr (pinned in tests/test_oracle_pins.py): the noise is a
+function of (seed, step, tensor salt, element), so codes and scales must agree bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import q4_oracle_torch as ot
+from quantfour_adamw_cuda_amd import _lib
+from quantfour_adamw_cuda_amd import quantfour_hip as q
+from tests.q4_testlib import HP, DeviceTensor, grads_config1, grads_config3, grads_student_t, p_close, to_np
+
+pytestmark = pytest.mark.gpu
+
+DT = {"fp32": torch.float32, "bf16": torch.bfloat16}
+HPA = (HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"], HP["eps"])
+SEED = 0x1234_5678_9ABC_DEF0
+
+
+def _check(dev, ref, prev, what):
+    for name, d, r in (("m codes", dev.m, ref[1]), ("v codes", dev.v, ref[2])):
+        d = d.cpu()
+        bad = torch.nonzero(d != r).reshape(-1)
+        assert bad.numel() == 0, f"{what}: {name} differ at bytes {bad[:5].tolist()}: {d[bad[:5]].tolist()} vs {r[bad[:5]].tolist()} ({bad.numel()} bytes)"
+    for name, d, r in (("m scales", dev.sm, ref[3]), ("v scales", dev.sv, ref[4])):
+        assert torch.equal(d.cpu().view(torch.int32), r.view(torch.int32)), f"{what}: {name} differ"
+    ok, worst = p_close(to_np(dev.p), to_np(ref[0]), to_np(prev), bf16=dev.p.dtype == torch.bfloat16)
+    assert ok, f"{what}: parameters out of tolerance (worst {worst})"
+
+
+def test_salt_function_matches_oracle():
+    L = _lib.load()
+    for seed, step, salt in ((0, 1, 0), (SEED, 7, 3), (2 ** 64 - 1, 123456, 2 ** 32 - 1), (1 << 32, 2, 5)):
+        assert L.q4adamw_sr_tensor_salt(seed, float(step), salt) == ot.sr_tensor_salt(seed, step, salt)
+
+
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32")])
+@pytest.mark.parametrize("n", [128 * 300 + 77, 4097, 1 << 18])
+def test_sr_against_oracle(cuda, p_dt, g_dt, n):
+    gen = torch.Generator().manual_seed(n % 1000)
+    p0 = (torch.randn(n, generator=gen) * 0.05).to(DT[p_dt])
+    dev = DeviceTensor(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.sv.cpu())
+    makers = (grads_config1, grads_config3, grads_student_t, grads_config1)
+    for step in range(1, 5):
+        g = makers[step - 1](gen, n).to(DT[g_dt])
+        prev = ref[0]
+        ref = ot.step_quant_sr(ref[0], g, *ref[1:], seed=SEED, tensor_salt=11, step=step, **HP)
+        q.fused_4bit_multi_sr([dev.p], [g.to(cuda)], [dev.m], [dev.v], [dev.sm], [dev.sv], *HPA, step,
+                              SEED, salts=[11])
+        _check(dev, ref, prev, f"{p_dt}/{g_dt} n={n} step {step}")
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
+
+
+def test_sr_multi_tensor_salts_reproducibility_and_options(cuda):
+    gen = torch.Generator().manual_seed(5)
+    sizes = [5000 + 131 * i for i in range(60)]          # more than one launch batch
+    ps = [torch.randn(n, generator=gen) * 0.05 for n in sizes]
+    gs = [grads_config1(gen, n).to(torch.bfloat16) for n in sizes]
+
+    def run(seed, salts, **kw):
+        devs = [DeviceTensor(p, cuda) for p in ps]
+        q.fused_4bit_multi_sr([d.p for d in devs], [g.to(cuda) for g in gs], [d.m for d in devs],
+                              [d.v for d in devs], [d.sm for d in devs], [d.sv for d in devs], *HPA, 1, seed,
+                              salts=salts, **kw)
+        return devs
+
+    a = run(SEED, None)
+    for i in (0, 1, 47, 48, 59):                          # default salt = position in the list
+        z8 = torch.zeros((sizes[i] + 1) // 2, dtype=torch.uint8)
+        zs = torch.zeros((sizes[i] + 127) // 128)
+        ref = ot.step_quant_sr(ps[i], gs[i], z8, z8.clone(), zs, zs.clone(), seed=SEED, tensor_salt=i, step=1, **HP)
+        _check(a[i], ref, ps[i], f"tensor {i}")
+    b = run(SEED, list(range(60)))
+    assert all(torch.equal(x.m, y.m) and torch.equal(x.v, y.v) for x, y in zip(a, b)), "a call must be reproducible"
+    c = run(SEED + 1, None)
+    assert all(not torch.equal(x.m, y.m) for x, y in zip(a, c)), "another seed must draw other noise"
+    d = run(SEED, [7] * 60)
+    assert not torch.equal(a[3].m, d[3].m)
+    # gradient multiplier: same as pre-multiplied fp32 gradients
+    e = run(SEED, None, grad_scale_dev=torch.tensor([0.5], device=cuda))
+    z8 = torch.zeros((sizes[2] + 1) // 2, dtype=torch.uint8)
+    zs = torch.zeros((sizes[2] + 127) // 128)
+    ref = ot.step_quant_sr(ps[2], gs[2].float() * 0.5, z8, z8.clone(), zs, zs.clone(), seed=SEED, tensor_salt=2,
+                           step=1, **HP)
+    _check(e[2], ref, ps[2], "with multiplier")
+
+
+def test_sr_is_unbiased_at_scale(cuda):
+    """one step from zero state on 2^24 elements: inside the code book's range (values beyond its
+    ends clamp under either rounding) the dequantized moments average to the exact moments,
+    which nearest rounding does not achieve"""
+    n = 1 << 24
+    gen = torch.Generator(device=cuda).manual_seed(6)
+    g = torch.randn(n, generator=gen, device=cuda) * 1e-3
+    p = torch.zeros(n, device=cuda)
+    m_exact = (1 - np.float32(HP["beta1"])) * g
+    v_exact = (1 - np.float32(HP["beta2"])) * (g * g)
+    out = {}
+    for name in ("sr", "nearest"):
+        d = DeviceTensor(p, cuda)
+        if name == "sr":
+            q.fused_4bit_multi_sr([d.p], [g], [d.m], [d.v], [d.sm], [d.sv], *HPA, 1, SEED)
+        else:
+            q.fused_4bit_multi([d.p], [g], [d.m], [d.v], [d.sm], [d.sv], *HPA, 1)
+        m = q.dequantize_state(d.m, d.sm, n, 0)
+        v = q.dequantize_state(d.v, d.sv, n, 1)
+        sm = d.sm.repeat_interleave(128)[:n]
+        sv = d.sv.repeat_interleave(128)[:n]
+        in_m = (m_exact / sm >= -0.8875)
+        in_v = (v_exact / sv >= 0.0625)
+        # signed error relative to the block scale, averaged over the in-range elements: bias
+        out[name] = (float((((m - m_exact) / sm)[in_m]).double().mean()),
+                     float((((v - v_exact) / sv)[in_v]).double().mean()))
+    assert abs(out["sr"][0]) < 1e-4 and abs(out["sr"][1]) < 1e-4, out
+    assert abs(out["nearest"][0]) > 5 * abs(out["sr"][0]) or abs(out["nearest"][1]) > 5 * abs(out["sr"][1]), out

@@ -381,3 +381,67 @@ def test_rank1_closed_forms():
                         torch.zeros(rows * cols // 128), step=1, **HP)
     assert torch.equal(out[1], ref[1]) and torch.equal(out[3], ref[3])
     assert torch.equal(out[0].reshape(-1), ref[0])
+
+
+# ---------------------------------------------------------------------------
+# stochastic rounding
+# ---------------------------------------------------------------------------
+def test_sr_quantizer_brute_force_and_exact_values():
+    """scalar restatement with plain Python floats rounded through numpy.float32; code-book
+    values themselves are never moved, whatever the noise"""
+    rng = np.random.default_rng(31)
+    f32 = np.float32
+    for which in (0, 1):
+        Q, _ = oc.tables(which)
+        x = (rng.standard_normal(1024) * (0.3 if which == 0 else 1.0)).astype(np.float32)
+        if which:
+            x = np.abs(x)
+        x[5] = 0.0
+        x[128:256] = 0.0                                     # an all-zero block
+        x[300] = -x[256:384].max() if which == 0 else x[300]  # the most negative value of a block
+        u = ((2 * rng.integers(0, 65536, 1024) + 1) / 2.0 ** 17).astype(np.float32)
+        codes, scales = ot.quantize_sr(torch.from_numpy(x), which, u)
+        got = ot.unpack(codes, 1024).numpy()
+        for i in range(1024):
+            s = f32(np.abs(x[i // 128 * 128:(i // 128 + 1) * 128]).max())
+            assert scales[i // 128] == s
+            if s == 0:
+                want = 0
+            else:
+                q = f32(x[i] / s)
+                if q <= Q[0]:
+                    want = 0
+                elif q >= Q[15]:
+                    want = 15
+                else:
+                    k = max(j for j in range(16) if Q[j] <= q)
+                    want = k + (1 if f32(u[i] * f32(Q[k + 1] - Q[k])) < f32(q - Q[k]) else 0)
+            assert got[i] == want, (which, i)
+        # exact code-book values times a power-of-two scale
+        blk = np.tile(Q, 8).astype(np.float32) * f32(0.25)
+        codes, _ = ot.quantize_sr(torch.from_numpy(blk), which, u[:128])
+        assert ot.unpack(codes, 128).tolist() == list(range(16)) * 8
+
+
+def test_sr_is_unbiased_and_noise_is_uniform():
+    um, uv = ot.sr_noise(1 << 20, ot.sr_tensor_salt(1234567890123, 7, 3))
+    for u in (um, uv):
+        assert u.min() >= 2.0 ** -17 and u.max() <= 1.0 - 2.0 ** -17
+        assert abs(float(u.astype(np.float64).mean()) - 0.5) < 2e-3
+        hist = np.histogram(u, bins=64, range=(0.0, 1.0))[0]
+        assert hist.min() > 0.9 * (1 << 20) / 64 and hist.max() < 1.1 * (1 << 20) / 64
+    assert abs(np.corrcoef(um, uv)[0, 1]) < 5e-3 and abs(np.corrcoef(um[:-1], um[1:])[0, 1]) < 5e-3
+    # different steps, tensors and seeds draw different noise
+    salts = {ot.sr_tensor_salt(s, t, k) for s in (1, 2, 1 << 40) for t in (1, 2) for k in (0, 1)}
+    assert len(salts) == 12
+    # the dequantized mean of many roundings of one value is that value (nearest rounding would
+    # be off by up to half a gap)
+    for which, x0 in ((0, 0.1234), (0, -0.5), (1, 0.4321)):
+        n = 1 << 18
+        x = np.full(n, x0, np.float32)
+        x[::128] = 1.0                                       # every block's scale is 1
+        u = ot.sr_noise(n, 99)[which]
+        codes, scales = ot.quantize_sr(torch.from_numpy(x), which, u)
+        back = ot.dequantize(codes, scales, n, which).numpy().astype(np.float64)
+        keep = np.arange(n) % 128 != 0
+        assert abs(back[keep].mean() - x0) < 2e-3 * abs(x0) + 1e-4
