@@ -182,6 +182,8 @@ def main():
     ap.add_argument("--variance-scale", choices=["group", "rank1"], default="group",
                     help="scaling of the second moment: per-128 block maxima (the fused CUDA path) or "
                          "rank-1 row/column maxima for matrices (a statistics pass precedes the update)")
+    ap.add_argument("--round-type", choices=["real-nearest", "stochastic"], default="real-nearest",
+                    help="rounding of the quantizer (stochastic: hash noise per element, block scaling only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, run a plain 4 GiB device copy three times, so that "
@@ -216,7 +218,8 @@ def main():
     total_params = sum(p.numel() for p in params)
     quant_params = sum(p.numel() for p in params if p.numel() > 4096)
 
-    opt = AdamWFused_QuantFour(params, variance_scale_type=args.variance_scale, **HP)
+    opt = AdamWFused_QuantFour(params, variance_scale_type=args.variance_scale,
+                               round_type=args.round_type, seed=0, **HP)
     opt.kernel_timing = []  # (kind, start event, end event) per launch
 
     def one_step(i):
@@ -310,6 +313,8 @@ def main():
             "kernel_ms_per_step": avg_kernel_s * 1e3,
         },
     }
+    if args.round_type == "stochastic":
+        out["config"]["workload"] += "; stochastic rounding"
     if rank1:
         out["config"]["workload"] += f"; rank-1 scaled second moment on {len(rank1)} matrices"
     if args.clip != "none":

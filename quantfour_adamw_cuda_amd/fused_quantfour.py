@@ -58,6 +58,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         *,
         fused: Optional[bool] = False,
         variance_scale_type: str = "group",
+        round_type: str = "real-nearest",
+        seed: Optional[int] = None,
     ):
         # optim/fused_quantfour.py:38-47
         if not 0.0 < lr:
@@ -80,6 +82,24 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             raise ValueError(f"Invalid variance_scale_type: {variance_scale_type=}")
         self.variance_scale_type = variance_scale_type
 
+        # rounding of the quantizer: "real-nearest" (the fused CUDA path and the draft's setting,
+        # quant_opt_base.py:28) or "stochastic" (the quantize_bsearch<STOCHASTIC> rule the draft
+        # quotes, adamw_fourbit_triton.py:1050-1075).  The noise seed is drawn once and, as in the
+        # draft (adamw_fourbit_triton.py:163-165), agreed on across ranks; it travels in the
+        # param groups, so a resumed run continues the same noise sequence.
+        if round_type not in ("real-nearest", "stochastic"):
+            raise ValueError(f"Invalid round_type: {round_type=}")
+        if round_type == "stochastic" and variance_scale_type == "rank1":
+            raise ValueError("stochastic rounding is built for variance_scale_type='group' only")
+        if round_type == "stochastic" and seed is None:
+            seed_t = torch.randint(1 << 31, size=[1])
+            if torch.distributed.is_available() and torch.distributed.is_initialized():
+                on_gpu = torch.distributed.get_backend() == "nccl"
+                seed_t = seed_t.cuda() if on_gpu else seed_t
+                torch.distributed.broadcast(seed_t, src=0)
+                seed_t = seed_t.cpu()
+            seed = int(seed_t)
+
         # tensors with numel <= threshold are not quantized
         # (FirstMoment.threshold / SecondMoment.threshold, adamw_fourbit_triton.py:118, :128)
         self.param_quant_threshold = 4096
@@ -90,6 +110,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             eps=eps,
             weight_decay=weight_decay,
             fused=fused,
+            round_type=round_type,
+            seed=seed,
         )
         super().__init__(params, defaults)
         self._launch_cache: Dict[Any, Any] = {}
@@ -122,6 +144,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self.__dict__.setdefault("variance_scale_type", "group")
         for group in self.param_groups:
             group.setdefault("fused", None)
+            group.setdefault("round_type", "real-nearest")
+            group.setdefault("seed", None)
         state_values = list(self.state.values())
         step_is_tensor = len(state_values) != 0 and torch.is_tensor(state_values[0]["step"])
         if not step_is_tensor:
@@ -151,6 +175,14 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                                                 memory_format=torch.contiguous_format)
             state["exp_avg_sq"] = torch.zeros_like(p, dtype=torch.float32,
                                                    memory_format=torch.contiguous_format)
+
+    def _param_position(self, p):
+        """Index of p among all parameters of all groups (stable across runs and resumes)."""
+        pos = self.__dict__.get("_positions")
+        if pos is None or p not in pos:
+            pos = {q_: i for i, q_ in enumerate(chain.from_iterable(g["params"] for g in self.param_groups))}
+            self._positions = pos
+        return pos[p]
 
     def _use_rank1(self, p):
         return self.variance_scale_type == "rank1" and _q.rank1_eligible(p)
@@ -411,6 +443,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             lr = group["lr"]
             weight_decay = group["weight_decay"]
             eps = group["eps"]
+            stochastic = group.get("round_type", "real-nearest") == "stochastic"
 
             # update step (optim/fused_quantfour.py:178)
             torch._foreach_add_(state_steps, 1)
@@ -423,6 +456,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 kind = momentum_quant_enabled[i]
                 if kind and "max_dims" in variance_meta[i]:
                     kind = "rank1"
+                elif kind and stochastic:
+                    kind = "sr"
                 key = (kind, param.device, param.dtype, grads[i].dtype, steps[i])
                 buckets.setdefault(key, []).append(i)
 
@@ -452,11 +487,17 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                     else:
                         arr = _q.make_small_table(ps, gs, ms, vs)
                     tags = (_q._tag(ps[0], "param"), _q._tag(gs[0], "grad"))
+                    if quantized == "sr":   # noise salt of a tensor: its position among all parameters
+                        tags += (_q.make_salts([self._param_position(p) for p in ps]),)
                     cached = (ptrs, arr, tags)
                     self._launch_cache[cache_key] = cached
-                _, arr, (p_tag, g_tag) = cached
-                launch = (_q.launch_rank1_table if quantized == "rank1" else
-                          _q.launch_table if quantized else _q.launch_small_table)
+                _, arr, (p_tag, g_tag, *extra) = cached
+                if quantized == "sr":
+                    salts_arr, sr_seed = extra[0], group["seed"]
+                    launch = lambda *a: _q.launch_table_sr(a[0], salts_arr, sr_seed, *a[1:])
+                else:
+                    launch = (_q.launch_rank1_table if quantized == "rank1" else
+                              _q.launch_table if quantized else _q.launch_small_table)
                 options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad)
                 if self.kernel_timing is None:
                     launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
@@ -468,7 +509,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                         launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                         end.record()
                     kind = ("fused_4bit_rank1" if quantized == "rank1" else
-                            "fused_4bit" if quantized else "fused_single_tensor")
+                            "fused_4bit" if quantized else "fused_single_tensor")   # "sr" counts as fused_4bit
                     self.kernel_timing.append((kind, start, end))
 
         return loss

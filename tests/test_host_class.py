@@ -184,6 +184,29 @@ def test_rank1_state_layout_and_round_trip():
         AdamWFused_QuantFour([wide], variance_scale_type="rank2")
 
 
+def test_round_type_and_seed_travel_in_the_param_groups():
+    (p,) = params((64, 130))
+    with pytest.raises(ValueError, match="round_type"):
+        AdamWFused_QuantFour([p], round_type="nearest-even")
+    with pytest.raises(ValueError, match="stochastic rounding"):
+        AdamWFused_QuantFour([p], round_type="stochastic", variance_scale_type="rank1")
+    assert AdamWFused_QuantFour([p]).param_groups[0]["round_type"] == "real-nearest"
+    torch.manual_seed(5)
+    a = AdamWFused_QuantFour([p], round_type="stochastic")
+    torch.manual_seed(5)
+    b = AdamWFused_QuantFour([p], round_type="stochastic")
+    seed = a.param_groups[0]["seed"]
+    assert isinstance(seed, int) and 0 <= seed < 1 << 31 and seed == b.param_groups[0]["seed"]
+    assert AdamWFused_QuantFour([p], round_type="stochastic", seed=77).param_groups[0]["seed"] == 77
+    # a resumed optimizer continues with the checkpoint's seed and rounding
+    c = AdamWFused_QuantFour([torch.nn.Parameter(p.detach().clone())])
+    c.load_state_dict(a.state_dict())
+    assert c.param_groups[0]["seed"] == seed and c.param_groups[0]["round_type"] == "stochastic"
+    q0, q1 = params((8, 8), (9, 9))
+    d = AdamWFused_QuantFour([{"params": [q0]}, {"params": [q1]}])
+    assert d._param_position(q0) == 0 and d._param_position(q1) == 1
+
+
 def test_setstate_backfills():
     (p,) = params((4, 4))
     opt = AdamWFused_QuantFour([p])
