@@ -1005,17 +1005,21 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
       const int r = r0 + i < nrows ? r0 + i : nrows - 1;
       const int64_t row = row0 + r;
       r_old[i] = as_global<const float>(T.rmax)[row];
-      const int64_t e = row * T.cols + col;
+      // row bases are uniform; the lane's column is a 32-bit offset
+      const int64_t row_first = row * T.cols + ((int64_t)cg * kStatCols + wave * kStatColsPerWave);
+      const uint32_t lane_elem = (uint32_t)lane * 8u;
+      const void *g_row = static_cast<const char *>(T.g) + row_first * (GBF ? 2 : 4);
+      const void *v_row = T.v + (row_first >> 1);
       vw[i] = 0u;
 #pragma unroll
       for (int h = 0; h < (GBF ? 1 : 2); ++h) gw[i][h] = u32x4{0u, 0u, 0u, 0u};
       if (active) {
-        vw[i] = *as_global<const uint32_t>(T.v + (e >> 1));
+        vw[i] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_row), lane_elem >> 1, 0, kNtReadOnly);
         if (GBF) {
-          gw[i][0] = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 2);
+          gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 2u, 0, kNtReadOnly);
         } else {
-          gw[i][0] = *as_global<const u32x4>(static_cast<const char *>(T.g) + e * 4);
-          gw[i][GBF ? 0 : 1] = *as_global<const u32x4>(static_cast<const char *>(T.g) + (e + 4) * 4);
+          gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u, 0, kNtReadOnly);
+          gw[i][GBF ? 0 : 1] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u + 16u, 0, kNtReadOnly);
         }
       }
     }
