@@ -160,3 +160,54 @@ def test_llama2_13b_shaped_parameter_set_bf16(cuda):
     total = _run_config(shapes, torch.bfloat16, cuda, 3, "llama2-13b bf16/bf16")
     assert 13.0e9 < total < 13.1e9
     torch.cuda.empty_cache()
+
+
+def test_more_than_2_to_32_elements_in_one_tensor(cuda):
+    """element indices and byte offsets beyond 32 bits: a tensor of 2^32 + 2^20 + 77 elements in one
+    call equals, bit for bit, the same data stepped as two tensors split at a block boundary
+    (blocks are independent), for the plain step and for stochastic rounding with the salts and
+    element offsets that make the noise line up only where it must"""
+    from quantfour_adamw_cuda_amd import quantfour_hip as q
+    n = (1 << 32) + (1 << 20) + 77
+    cut = (1 << 32) - 5 * 128 * 1024            # multiple of 128 and of both chunk sizes
+    gen = torch.Generator(device=cuda).manual_seed(12)
+    hp = (0.9, 0.999, 1e-3, 0.01, 1e-8)
+
+    def fresh():
+        g_ = torch.Generator(device=cuda).manual_seed(13)
+        p = torch.empty(n, dtype=torch.bfloat16, device=cuda).normal_(0, 0.05, generator=g_)
+        m = torch.zeros((n + 1) // 2, dtype=torch.uint8, device=cuda)
+        v = torch.zeros_like(m)
+        sm = torch.zeros((n + 127) // 128, device=cuda)
+        sv = torch.zeros_like(sm)
+        return p, m, v, sm, sv
+
+    g = torch.empty(n, dtype=torch.bfloat16, device=cuda).normal_(0, 1e-3, generator=gen)
+    whole, parts = fresh(), fresh()
+    for step in (1, 2):
+        q.fused_4bit_multi([whole[0]], [g], [whole[1]], [whole[2]], [whole[3]], [whole[4]], *hp, step)
+        a = [t[:c] for t, c in zip(parts, (cut, cut // 2, cut // 2, cut // 128, cut // 128))]
+        b = [t[c:] for t, c in zip(parts, (cut, cut // 2, cut // 2, cut // 128, cut // 128))]
+        q.fused_4bit_multi([a[0], b[0]], [g[:cut], g[cut:]], [a[1], b[1]], [a[2], b[2]], [a[3], b[3]],
+                           [a[4], b[4]], *hp, step)
+        for name, x, y in zip(("p", "m", "v", "sm", "sv"), whole, parts):
+            assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), f"step {step}: {name} differs"
+    assert whole[1][-1] < 16 and whole[1][cut // 2:].any()      # odd tail: high nibble stays clear
+    # stochastic rounding: the noise of element e depends on e itself, so only the first part
+    # of a split run sees the same noise; check that part, and that the tail beyond 2^32 is not
+    # a repeat of the head (its hash mixes the high half of the index)
+    sr_whole, sr_head = fresh(), fresh()
+    q.fused_4bit_multi_sr([sr_whole[0]], [g], [sr_whole[1]], [sr_whole[2]], [sr_whole[3]], [sr_whole[4]],
+                          *hp, 1, 42, salts=[3])
+    h = [t[:c] for t, c in zip(sr_head, (cut, cut // 2, cut // 2, cut // 128, cut // 128))]
+    q.fused_4bit_multi_sr([h[0]], [g[:cut]], [h[1]], [h[2]], [h[3]], [h[4]], *hp, 1, 42, salts=[3])
+    assert torch.equal(sr_whole[1][:cut // 2], h[1]) and torch.equal(sr_whole[2][:cut // 2], h[2])
+    # elements 2^32 .. 2^32 + 2^20 carry the gradients and parameters of elements 0 .. 2^20 in a
+    # second run; with identical inputs only the noise can make their codes differ
+    g2, rep = g.clone(), fresh()
+    g2[1 << 32:(1 << 32) + (1 << 20)] = g[:1 << 20]
+    rep[0][1 << 32:(1 << 32) + (1 << 20)] = rep[0][:1 << 20]
+    q.fused_4bit_multi_sr([rep[0]], [g2], [rep[1]], [rep[2]], [rep[3]], [rep[4]], *hp, 1, 42, salts=[3])
+    lo, hi = rep[1][:1 << 19], rep[1][1 << 31:(1 << 31) + (1 << 19)]
+    assert torch.equal(rep[3][:1 << 13], rep[3][1 << 25:(1 << 25) + (1 << 13)])      # same block scales
+    assert 0.01 < float((lo != hi).float().mean()) < 0.9

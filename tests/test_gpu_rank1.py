@@ -246,3 +246,27 @@ def test_optimizer_rank1_layout_tracking_and_resume(cuda):
     assert torch.equal(md[0].reshape(-1), v32.amax(1)) and torch.equal(md[1].reshape(-1), v32.amax(0))
     want_codes, _, _ = ot.quantize_rank1(v32.cpu())
     assert torch.equal(opt3.state[p3]["exp_avg_sq"].cpu(), want_codes)
+
+
+def test_rank1_more_than_2_to_32_elements(cuda):
+    """a matrix of 2 x 33000 x 65536 elements (4.3e9) whose lower half repeats the upper half:
+    row and column maxima of the whole equal those of a half, so the run on the whole matrix
+    must reproduce, in both halves, the run on one half -- rows whose flat indices lie beyond
+    2^32 included"""
+    half_rows, cols = 33000, 65536
+    gen = torch.Generator(device=cuda).manual_seed(14)
+    p_half = torch.empty(half_rows, cols, dtype=torch.bfloat16, device=cuda).normal_(0, 0.05, generator=gen)
+    half, whole = Rank1State(p_half, cuda), Rank1State(torch.cat([p_half, p_half]), cuda)
+    for step in (1, 2):
+        g_half = torch.empty(half_rows, cols, dtype=torch.bfloat16, device=cuda).normal_(0, 1e-3, generator=gen)
+        g_half *= torch.rand(half_rows, 1, device=cuda, generator=gen).to(torch.bfloat16)
+        half.step(g_half, step)
+        whole.step(torch.cat([g_half, g_half]), step)
+        n2 = half_rows * cols // 2
+        for name, w, h in (("p", whole.p.view(-1), half.p.view(-1)), ("m", whole.m, half.m), ("v", whole.v, half.v),
+                           ("sm", whole.sm, half.sm), ("r", whole.r, half.r)):
+            k = h.numel()
+            assert torch.equal(w[:k].view(torch.uint8), h.view(torch.uint8)), f"step {step}: upper half {name}"
+            assert torch.equal(w[k:].view(torch.uint8), h.view(torch.uint8)), f"step {step}: lower half {name}"
+        assert torch.equal(whole.c, half.c)
+    assert whole.v.any() and whole.r.min() > 0
