@@ -86,7 +86,8 @@ def quantize(x, which):
     padded = torch.zeros(nblk * BLOCK, dtype=torch.float32, device=x.device)
     padded[:numel] = x
     grouped = padded.view(nblk, BLOCK)
-    max1 = grouped.abs().amax(dim=1, keepdim=True)          # :623-624, :1078-1087
+    # :623-624, :1078-1087; like the C oracle's running maximum, a NaN never becomes the scale
+    max1 = torch.nan_to_num(grouped.abs(), nan=0.0, posinf=float("inf")).amax(dim=1, keepdim=True)
     qx = grouped.div(max1)                                   # :625 (0/0 -> NaN)
     # number of midpoints strictly below x; NaN must land on 0
     q = torch.bucketize(torch.nan_to_num(qx, nan=-2.0), QMID[which].to(x.device), right=False)
@@ -154,7 +155,7 @@ def dequantize_rank1(codes, row_max, col_max):
 
 def quantize_rank1(x):
     """x: fp32 matrix (non-negative).  Returns (packed codes, row_max, col_max)."""
-    ax = x.abs()
+    ax = torch.nan_to_num(x.abs(), nan=0.0, posinf=float("inf"))   # a NaN never becomes a maximum
     row_max = ax.amax(dim=1)                                 # max over all dims except 0
     col_max = ax.amax(dim=0)                                 # max over all dims except 1
     qx = x.div(rank1_scale(row_max, col_max))                # 0/0 -> NaN -> code 0
@@ -241,7 +242,7 @@ def quantize_sr(x, which, u):
     noise = np.zeros(nblk * BLOCK, np.float32)
     noise[:numel] = u
     grouped = padded.reshape(nblk, BLOCK)
-    max1 = np.abs(grouped).max(axis=1, keepdims=True)
+    max1 = np.fmax.reduce(np.abs(grouped), axis=1, initial=0.0, keepdims=True)   # a NaN never becomes the scale
     with np.errstate(invalid="ignore", divide="ignore"):
         q = (grouped / max1).reshape(-1)                     # 0/0 -> NaN -> code 0
     Q = QMAP[which].numpy()

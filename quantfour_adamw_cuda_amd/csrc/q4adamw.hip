@@ -1259,7 +1259,9 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__
   const int64_t e = blk * Q4ADAMW_BLOCK + lane * 2;
   const float a = e < numel ? x[e] : 0.0f;
   const float b = e + 1 < numel ? x[e + 1] : 0.0f;
-  uint32_t u = f2bits(__builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b)));
+  // fmaxf drops a NaN next to a number; two NaN count as 0: a NaN never becomes the scale
+  const float lane_max = __builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b));
+  uint32_t u = lane_max == lane_max ? f2bits(lane_max) : 0u;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const uint32_t o = (uint32_t)__shfl_xor((int)u, off, 64);
@@ -1300,7 +1302,8 @@ __global__ __launch_bounds__(256) void rank1_absmax_kernel(const float *x_, int6
   __syncthreads();
   float c_max = 0.0f;
   for (int r = 0; r < nrows; ++r) {
-    const float a = col < cols ? __builtin_fabsf(x[(row0 + r) * cols + col]) : 0.0f;
+    float a = col < cols ? __builtin_fabsf(x[(row0 + r) * cols + col]) : 0.0f;
+    a = a == a ? a : 0.0f;  // a NaN never becomes a maximum
     c_max = __builtin_fmaxf(c_max, a);
     uint32_t u = f2bits(a);
 #pragma unroll

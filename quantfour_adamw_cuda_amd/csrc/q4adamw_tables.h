@@ -68,7 +68,9 @@ Q4_HD constexpr MtabEntry mtab_entry(uint32_t idx) {
   const uint32_t sign = (idx >> 10) & 1u, mag = idx & 1023u, e = mag >> 2;
   uint32_t base = 0, thr = 0;
   bool has = false;
-  if (e >= 128u) {           // |q| >= 2, inf, nan: beyond every threshold
+  if (e == 255u) {           // nan (an infinite quotient only occurs in blocks that take the
+    base = 0u;               // exact path): no threshold is below a nan
+  } else if (e >= 128u) {    // |q| >= 2: beyond every threshold
     base = sign ? 0u : 15u;
   } else if (e < 118u) {     // |q| < 2^-9 < 0.00275: the seven negative thresholds are below
     base = 7u;
@@ -161,7 +163,11 @@ Q4_HD constexpr SrEntry sr_entry(uint32_t half_index) {
   const uint32_t idx = half_index_bucket(half_index);
   const uint32_t sign = (idx >> 10) & 1u, mag = idx & 1023u, e = mag >> 2;
   SrEntry out{kNoThr, 0u};
-  if (e >= 128u) {            // |q| >= 2, inf, nan
+  if (e == 255u) {            // nan: interval 1 makes "up" false and the code 1 - 1 + 0 = 0
+    out.base = 1u;
+    return out;
+  }
+  if (e >= 128u) {            // |q| >= 2
     out.base = sign ? 0u : 16u;
     return out;
   }

@@ -106,3 +106,31 @@ def test_take_over_adamw_state_and_hand_it_back(cuda):
     for f in fresh:
         f.grad = torch.zeros_like(f)
     adamw2.step()                                # the library routine runs on it
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_quantize_non_finite_values(cuda, which):
+    """a NaN never becomes a block's scale (the oracle's running maximum skips it) and gets code 0;
+    an infinite scale sends the block's finite values to x / inf = 0"""
+    from oracle import q4_oracle_torch as ot
+    from quantfour_adamw_cuda_amd import quantfour_hip as q
+    gen = torch.Generator().manual_seed(23 + which)
+    x = torch.randn(128 * 12, generator=gen)
+    x = x * x if which else x
+    x[3] = float("nan")
+    x[128:256] = float("nan")
+    x[256 + 4] = float("inf")
+    x[384 + 5], x[384 + 6] = float("inf"), float("nan")
+    x[512 + 64], x[512 + 65] = float("nan"), float("nan")          # one lane's both values
+    codes, scales = q4.quantize_state(x.to(cuda), which)
+    rc, rs = oc.quant(x.numpy(), which)
+    assert np.array_equal(bits(scales.cpu().numpy()), bits(rs)), (scales.cpu().numpy(), rs)
+    assert np.array_equal(codes.cpu().numpy(), rc)
+    if which:
+        m = x.view(12, 128).clone()
+        m = torch.cat([m] * 5, dim=1)[:, :512].contiguous()           # 12 x 512 with the same oddities
+        c1, r1, k1 = q.quantize_state_rank1(m.to(cuda))
+        c2, r2, k2 = ot.quantize_rank1(m)
+        assert torch.equal(r1.cpu().view(torch.int32), r2.view(torch.int32))
+        assert torch.equal(k1.cpu().view(torch.int32), k2.view(torch.int32))
+        assert torch.equal(c1.cpu(), c2)

@@ -284,3 +284,42 @@ def test_replay_under_graph_capture(cuda):
             assert torch.equal(x.sm.view(torch.int32), y.sm.view(torch.int32))
             assert torch.equal(x.sv.view(torch.int32), y.sv.view(torch.int32))
             assert torch.equal(x.p.view(torch.int32), y.p.view(torch.int32))
+
+
+@pytest.mark.parametrize("p_dtype,g_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.bfloat16)])
+def test_non_finite_gradients(cuda, p_dtype, g_dtype):
+    """inf, -inf and NaN gradients in some blocks: codes and scales still match the oracle bit
+    for bit (a block's scale is the maximum over its non-NaN magnitudes, an infinite scale sends
+    finite values to the code of zero, inf/inf and NaN get code 0); the blocks without such
+    values are untouched by their neighbours; parameters agree where the oracle's are finite
+    and are non-finite where the oracle's are"""
+    n = 128 * 64 + 50
+    gen = torch.Generator().manual_seed(17)
+    p0 = (torch.randn(n, generator=gen) * 0.05).to(p_dtype)
+    dev, ref = DeviceTensor(p0, cuda), OracleTensor(p0)
+    inf, nan = float("inf"), float("nan")
+    for step in (1, 2, 3):
+        g = grads_config1(gen, n)
+        if step == 2:
+            g[5] = inf                     # one inf in block 0
+            g[128 + 7] = -inf              # block 1
+            g[256 + 9] = nan               # block 2
+            g[384:512] = nan               # block 3: nothing but NaN
+            g[512 + 1], g[512 + 2] = inf, nan   # block 4: both
+            g[n - 3] = inf                 # the ragged last block
+        g = g.to(g_dtype)
+        q4.fused_4bit(dev.p, g.to(cuda), dev.m, dev.v, dev.sm, dev.sv, HP["beta1"], HP["beta2"], HP["lr"],
+                      HP["weight_decay"], HP["eps"], step)
+        prev = ref.step(g, step)
+        for name, d, r in (("sm", dev.sm, ref.sm), ("sv", dev.sv, ref.sv)):
+            assert np.array_equal(bits(d.cpu().numpy()), bits(r)), f"step {step}: {name}: {d.cpu().numpy()[:6]} vs {r[:6]}"
+        assert np.array_equal(dev.m.cpu().numpy(), ref.m), f"step {step}: m codes"
+        assert np.array_equal(dev.v.cpu().numpy(), ref.v), f"step {step}: v codes"
+        p_dev = dev.p.float().cpu().numpy()
+        p_ref = ref.p if ref.p.dtype == np.float32 else (ref.p.astype(np.uint32) << 16).view(np.float32)
+        finite = np.isfinite(p_ref)
+        assert np.array_equal(np.isfinite(p_dev), finite), f"step {step}: finiteness of the parameters"
+        ok, worst = p_close(to_np(dev.p)[finite], ref.p[finite], prev[finite], bf16=p_dtype == torch.bfloat16)
+        assert ok, f"step {step}: parameters out of tolerance (worst {worst})"
+        ref.resync(dev.p)

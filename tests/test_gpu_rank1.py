@@ -270,3 +270,28 @@ def test_rank1_more_than_2_to_32_elements(cuda):
             assert torch.equal(w[k:].view(torch.uint8), h.view(torch.uint8)), f"step {step}: lower half {name}"
         assert torch.equal(whole.c, half.c)
     assert whole.v.any() and whole.r.min() > 0
+
+
+def test_rank1_non_finite_gradients(cuda):
+    """inf and NaN gradients: maxima are taken over the non-NaN values, an infinite scale sends
+    finite values to code 0 (x / inf = 0), NaN and inf / inf get code 0"""
+    rows, cols = 40, 1024
+    gen = torch.Generator().manual_seed(19)
+    p0 = torch.randn(rows, cols, generator=gen) * 0.05
+    dev = Rank1State(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.r.cpu(), dev.c.cpu())
+    for step in (1, 2, 3):
+        g = grads_config1(gen, rows * cols).view(rows, cols)
+        if step == 2:
+            g[3, 5] = float("inf")
+            g[7, 100] = float("nan")
+            g[9] = float("nan")
+            g[11, 5], g[11, 6] = float("-inf"), float("nan")
+        ref = ot.step_quant_rank1(ref[0], g, *ref[1:], step=step, **HP)
+        dev.step(g.to(cuda), step)
+        for name, d, r in list(zip(("p", "m codes", "v codes", "m scales", "row maxima", "column maxima"),
+                                   dev.tensors(), ref))[1:]:
+            d = d.cpu()
+            same = torch.equal(d.view(torch.int32), r.view(torch.int32)) if d.dtype == torch.float32 else torch.equal(d, r)
+            assert same, f"step {step}: {name} differ at {torch.nonzero(d != r).reshape(-1)[:6].tolist()}"
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])

@@ -163,3 +163,30 @@ def test_optimizer_stochastic_rounding(cuda):
         m_res(x).square().mean().backward()
         o_res.step()
     assert all(torch.equal(a, b) for a, b in zip(m1.parameters(), m_res.parameters()))
+
+
+def test_sr_non_finite_gradients(cuda):
+    """inf and NaN gradients: a NaN moment gets code 0, an infinite block scale sends finite
+    values to the code of zero, as the oracle has it"""
+    n = 128 * 40 + 9
+    gen = torch.Generator().manual_seed(18)
+    p0 = torch.randn(n, generator=gen) * 0.05
+    dev = DeviceTensor(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.sv.cpu())
+    for step in (1, 2, 3):
+        g = grads_config1(gen, n)
+        if step == 2:
+            g[5] = float("inf")
+            g[128 + 7] = float("-inf")
+            g[256 + 9] = float("nan")
+            g[384:512] = float("nan")
+            g[512 + 1], g[512 + 2] = float("inf"), float("nan")
+        with np.errstate(invalid="ignore"):
+            ref = ot.step_quant_sr(ref[0], g, *ref[1:], seed=SEED, tensor_salt=0, step=step, **HP)
+        q.fused_4bit_multi_sr([dev.p], [g.to(cuda)], [dev.m], [dev.v], [dev.sm], [dev.sv], *HPA, step, SEED)
+        for name, d, r in (("m codes", dev.m, ref[1]), ("v codes", dev.v, ref[2])):
+            bad = torch.nonzero(d.cpu() != r).reshape(-1)
+            assert bad.numel() == 0, f"step {step}: {name} differ at bytes {bad[:8].tolist()}: {d.cpu()[bad[:8]].tolist()} vs {r[bad[:8]].tolist()}"
+        for name, d, r in (("m scales", dev.sm, ref[3]), ("v scales", dev.sv, ref[4])):
+            assert torch.equal(d.cpu().view(torch.int32), r.view(torch.int32)), f"step {step}: {name}"
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
