@@ -35,6 +35,36 @@ def test_library_exports_every_declared_symbol(lib):
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(_lib.Q4Tensor) == 56 and ctypes.sizeof(_lib.Q4SmallTensor) == 40
     assert _lib.Q4Tensor.numel.offset == 48 and _lib.Q4SmallTensor.numel.offset == 32
+    assert ctypes.sizeof(_lib.Q4Rank1Tensor) == 88 and _lib.Q4Rank1Tensor.rows.offset == 72
+    assert ctypes.sizeof(_lib.Q4GradOptions) == 24 and _lib.Q4GradOptions.grad_scale_dev.offset == 8
+    assert ctypes.sizeof(_lib.Q4Grad) == 16 and _lib.NORM_WORKSPACE_BYTES == 16384
+    header = open(os.path.join(ROOT, "include", "q4adamw.h")).read()
+    assert "#define Q4ADAMW_NORM_WORKSPACE_BYTES 16384" in header
+
+
+def test_new_entry_points_validate_before_any_gpu_call(lib):
+    z = ctypes.c_void_p(0)
+    hp = (0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0)
+    t = (_lib.Q4Tensor * 1)()
+    t[0].numel = 128
+    assert lib.q4adamw_fused_4bit_multi_sr(t, 1, None, 7, 0, 0, *hp, None, z) == -1      # null pointers
+    assert lib.q4adamw_fused_4bit_multi_ex(t, 1, 0, 5, *hp, None, z) == -1               # dtype tag
+    r = (_lib.Q4Rank1Tensor * 1)()
+    r[0].rows, r[0].cols = 4, 500
+    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -1 and b"cols" in lib.q4adamw_last_error()
+    r[0].cols = 1 << 31
+    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -4
+    r[0].rows, r[0].cols = 0, 512                                                        # empty: nothing to do
+    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == 0
+    g = (_lib.Q4Grad * 1)()
+    g[0].numel = 16
+    assert lib.q4adamw_grad_norm(g, 1, 0, 1.0, None, 0.0, z, 16384, z, z) == -1
+    assert lib.q4adamw_quantize_rank1(z, 4, 12, z, z, z, z) == -1 and b"multiple of 8" in lib.q4adamw_last_error()
+    assert lib.q4adamw_dequantize_rank1(z, z, z, 0, 512, z, z) == 0
+    # hyper-parameter domain, shared by every step entry point
+    t[0].numel = 0
+    assert lib.q4adamw_fused_4bit_multi_sr(t, 1, None, 7, 0, 0, 0.9, 1.0, 1e-3, 0.01, 1e-8, 1.0, None, z) == -3
+    assert lib.q4adamw_sr_tensor_salt(0, 1.0, 0) != lib.q4adamw_sr_tensor_salt(0, 2.0, 0)
 
 
 def test_host_helpers_match_oracle(lib):
