@@ -470,13 +470,18 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                     sms = [momentum_meta[i]["max1"] for i in idx]
                     stats = [[variance_meta[i][k][d] for i in idx]
                              for k in ("max_dims", "scratch_dims") for d in (0, 1)]
-                    ptrs = tuple(t.data_ptr() for ts in (ps, gs, ms, vs, sms, *stats) for t in ts)
+                    fixed = (ps, ms, vs, sms, *stats)
                 elif quantized:
                     sms = [momentum_meta[i]["max1"] for i in idx]
                     svs = [variance_meta[i]["max1"] for i in idx]
-                    ptrs = tuple(t.data_ptr() for ts in (ps, gs, ms, vs, sms, svs) for t in ts)
+                    fixed = (ps, ms, vs, sms, svs)
                 else:
-                    ptrs = tuple(t.data_ptr() for ts in (ps, gs, ms, vs) for t in ts)
+                    fixed = (ps, ms, vs)
+                # parameters and state stay where they are from step to step; gradients
+                # usually do not: a descriptor table is rebuilt (and everything validated)
+                # only when a parameter or state pointer changed, otherwise the gradients'
+                # pointers are refreshed in place
+                ptrs = tuple(t.data_ptr() for ts in fixed for t in ts)
                 cache_key = (gi, quantized, device, p_dtype, g_dtype)
                 cached = self._launch_cache.get(cache_key)
                 if cached is None or cached[0] != ptrs:
@@ -491,6 +496,14 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                         tags += (_q.make_salts([self._param_position(p) for p in ps]),)
                     cached = (ptrs, arr, tags)
                     self._launch_cache[cache_key] = cached
+                else:
+                    arr = cached[1]
+                    for i, (p, g) in enumerate(zip(ps, gs)):
+                        # dtype and device are part of the bucket key (optim/fused_quantfour.py:255-261)
+                        assert g.device == device, "grad must be on the param's device"
+                        assert g.is_contiguous(), "grad must be contiguous"
+                        assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
+                        arr[i].g = g.data_ptr()
                 _, arr, (p_tag, g_tag, *extra) = cached
                 if quantized == "sr":
                     salts_arr, sr_seed = extra[0], group["seed"]
