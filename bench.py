@@ -87,16 +87,16 @@ def gpt2_small_shapes():
 WORKLOADS = {
     # name: (shapes, param dtype, grad dtype, grad distribution, description)
     "llama3-8b": (llama3_8b_shapes, "float32", "bfloat16", "student_t",
-                  "Llama-3-8B parameter set (BASELINE configs[3]): 291 tensors, fp32 master "
+                  "Llama-3-8B parameter set (benchmark configuration 3): 291 tensors, fp32 master "
                   "params, bf16 grads, 4-bit m/v, block 128"),
     "llama2-13b": (llama2_13b_shapes, "bfloat16", "bfloat16", "student_t",
-                   "Llama-2-13B-shaped parameter set (BASELINE configs[4]): 362 tensors, bf16 "
+                   "Llama-2-13B-shaped parameter set (benchmark configuration 4): 362 tensors, bf16 "
                    "params, bf16 grads, 4-bit m/v, block 128"),
     "gpt2-small": (gpt2_small_shapes, "float32", "float32", "normal_outliers",
-                   "GPT-2-small parameter set (BASELINE configs[1]): 148 tensors, fp32 params and "
+                   "GPT-2-small parameter set (benchmark configuration 1): 148 tensors, fp32 params and "
                    "grads, 4-bit m/v, block 128"),
     "single-4096": (lambda: [("w", (4096, 4096))], "float32", "float32", "normal_outliers",
-                    "single fp32 4096x4096 tensor (BASELINE configs[0])"),
+                    "single fp32 4096x4096 tensor (benchmark configuration 0)"),
 }
 
 

@@ -1,4 +1,4 @@
-"""Full-size checks of BASELINE configs[3] (Llama-3-8B: fp32 params, bf16 grads) and
+"""Full-size checks of benchmark configuration 3 (Llama-3-8B: fp32 params, bf16 grads) and
 configs[4] (Llama-2-13B-shaped: bf16 params and grads): every tensor of the whole parameter
 set, every step, against the vectorised oracle run with plain torch ops on the GPU -- after
 that GPU run of the oracle has itself been checked against the C oracle -- plus format
