@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # WRITE_SIZE (each scaled by what the same counter reads for a 4 GiB device copy: 2.0 and 1.0);
 # summary in profiles/fused_4bit_kernel_llama3_8b_hbm_counters.txt.  Workloads that have not
 # been profiled report null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {"llama3-8b": 9.7365e10}
+MEASURED_TRAFFIC_BYTES_PER_STEP = {"llama3-8b": 9.7374e10}
 HP = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 
 
