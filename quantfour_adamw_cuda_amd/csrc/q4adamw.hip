@@ -610,10 +610,11 @@ __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlo
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-// Geometry of the fused kernel: a lane owns 16 bytes of the parameter stream.
-template <bool PBF>
+// Geometry of the fused kernel: a lane owns 16 bytes of the widest of the parameter and
+// gradient streams, so that no stream needs two accesses per lane.
+template <bool PBF, bool GBF>
 struct Geometry {
-  static constexpr int kEpl = PBF ? 8 : 4;               // elements per lane
+  static constexpr int kEpl = (PBF && GBF) ? 8 : 4;      // elements per lane
   static constexpr int kTile = 64 * kEpl;                // elements per wave
   static constexpr int kChunk = kTile * kWaves;          // elements per workgroup
   static constexpr int kLanesPerBlock = Q4ADAMW_BLOCK / kEpl;   // 32 or 16
@@ -635,7 +636,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g, uint32_t salt) {
   static_assert(!(SR && RANK1), "stochastic rounding is built for block scaling only");
-  using G = Geometry<PBF>;
+  using G = Geometry<PBF, GBF>;
   constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
   // block; the per-lane part is a small 32-bit offset.
@@ -925,7 +926,7 @@ __device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale)
 
 template <bool PBF, bool GBF, bool EXT, bool SR>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
-  using G = Geometry<PBF>;
+  using G = Geometry<PBF, GBF>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
@@ -1072,7 +1073,7 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
 
 template <bool PBF, bool GBF, bool EXT>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
-  using G = Geometry<PBF>;
+  using G = Geometry<PBF, GBF>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<false>(tid);
@@ -1610,11 +1611,12 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
-  // a lane reads 4 (fp32 parameters) or 8 (bf16 parameters) consecutive elements at once
+  // a lane reads 8 consecutive elements at once when parameters and gradients are bf16, else 4
   const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
-  const int64_t chunk_elems = p_bf16 ? Geometry<true>::kChunk : Geometry<false>::kChunk;
+  const bool wide = p_bf16 && g_dtype == Q4ADAMW_BF16;   // 8 elements per lane
+  const int64_t chunk_elems = wide ? Geometry<true, true>::kChunk : Geometry<false, false>::kChunk;
   const uintptr_t p_align = 16, g_align = g_dtype == Q4ADAMW_BF16 ? (p_bf16 ? 16 : 8) : 16;
-  const uintptr_t code_align = p_bf16 ? 4 : 2;
+  const uintptr_t code_align = wide ? 4 : 2;
   // validate everything before the first launch
   for (int i = 0; i < count; ++i) {
     const q4adamw_tensor &t = tensors[i];
@@ -1677,7 +1679,8 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
   sa.b2 = a.sc.b2;
   sa.r2 = a.sc.r2;
   const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
-  const int64_t chunk_elems = p_bf16 ? Geometry<true>::kChunk : Geometry<false>::kChunk;
+  const bool wide = p_bf16 && g_dtype == Q4ADAMW_BF16;   // 8 elements per lane
+  const int64_t chunk_elems = wide ? Geometry<true, true>::kChunk : Geometry<false, false>::kChunk;
   for (int i = 0; i < count; ++i) {
     const q4adamw_rank1_tensor &t = tensors[i];
     if (t.rows < 0 || t.cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
