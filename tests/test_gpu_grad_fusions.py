@@ -287,3 +287,68 @@ def test_grad_scaler_drives_the_fused_path(cuda):
     scaler.update()
     assert all(torch.equal(p, q0) for p, q0 in zip(m.parameters(), before))
     assert scaler.get_scale() == s0 * 0.5
+
+
+def test_clip_pipeline_and_rank1_replay_under_graph_capture(cuda):
+    """norm kernel -> step with the device multiplier -> rank-1 step (atomics, three launches):
+    nothing allocates, synchronises or uses a memset, so the sequence can be captured; replays
+    with refreshed gradients and eager work in between must equal eager launches bit for bit"""
+    gen = torch.Generator().manual_seed(31)
+    sizes = [70001, 4097, 128 * 40]
+    ps = [torch.randn(n, generator=gen) * 0.02 for n in sizes]
+    mat = torch.randn(24, 1024, generator=gen) * 0.02
+
+    class Rank1:
+        def __init__(self):
+            self.p = mat.clone().to(cuda)
+            n = mat.numel()
+            self.m = torch.zeros(n // 2, dtype=torch.uint8, device=cuda)
+            self.v = torch.zeros_like(self.m)
+            self.sm = torch.zeros(n // 128, device=cuda)
+            self.r, self.c = torch.zeros(24, device=cuda), torch.zeros(1024, device=cuda)
+            self.rn, self.cn = torch.zeros(24, device=cuda), torch.zeros(1024, device=cuda)
+
+        def all(self):
+            return (self.p, self.m, self.v, self.sm, self.r, self.c, self.rn, self.cn)
+
+    def fresh():
+        return [DeviceTensor(p, cuda) for p in ps], Rank1()
+
+    eager, graphed = fresh(), fresh()
+    gbuf = [torch.zeros(n, device=cuda) for n in sizes] + [torch.zeros(24, 1024, device=cuda)]
+    out = [torch.zeros(3, device=cuda) for _ in range(2)]
+    ws = [torch.zeros(_lib.NORM_WORKSPACE_BYTES // 8, dtype=torch.float64, device=cuda) for _ in range(2)]
+
+    def launch(state, gs, which):
+        ts, r1 = state
+        q.grad_norm(gs, grad_scale=0.5, max_norm=1e-3, out=out[which], workspace=ws[which])
+        mult = out[which][2:3]
+        q.fused_4bit_multi([x.p for x in ts], gs[:3], [x.m for x in ts], [x.v for x in ts], [x.sm for x in ts],
+                           [x.sv for x in ts], *HPA, 2, grad_scale_dev=mult)
+        q.fused_4bit_rank1_multi([r1.p], gs[3:], [r1.m], [r1.v], [r1.sm], [r1.r], [r1.c], [r1.rn], [r1.cn],
+                                 *HPA, 2, grad_scale_dev=mult)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(graphed, gbuf, 1)                   # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graphed = fresh()                              # new state: re-capture against its pointers
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch(graphed, gbuf, 1)
+    for rep in range(4):
+        gs = [grads_config1(gen, n).to(cuda) for n in sizes] + [grads_config1(gen, 24 * 1024).view(24, 1024).to(cuda)]
+        for b, g in zip(gbuf, gs):
+            b.copy_(g)
+        graph.replay()
+        launch(eager, gs, 0)
+        torch.cuda.synchronize()
+        assert torch.equal(out[0].view(torch.int32), out[1].view(torch.int32)), f"replay {rep}: norm outputs"
+        assert float(out[0][1]) < 1.0, "the pipeline must actually clip"
+        for x, y in zip(graphed[0], eager[0]):
+            for a, b in ((x.p, y.p), (x.m, y.m), (x.v, y.v), (x.sm, y.sm), (x.sv, y.sv)):
+                assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"replay {rep}"
+        for a, b in zip(graphed[1].all(), eager[1].all()):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"replay {rep}: rank-1 state"
