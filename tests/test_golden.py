@@ -13,7 +13,9 @@ from oracle import q4_oracle_torch as ot
 from tests.q4_testlib import p_close
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
+FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "quant_*.npz")))
+SR_FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "sr_*.npz")))
+RANK1_FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "rank1_*.npz")))
 
 
 def load(path):
@@ -25,7 +27,7 @@ def load(path):
 
 
 def test_fixtures_exist():
-    assert len(FIXTURES) >= 4
+    assert len(FIXTURES) >= 4 and len(SR_FIXTURES) >= 2 and len(RANK1_FIXTURES) >= 2
 
 
 @pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p) for p in FIXTURES])
@@ -85,3 +87,90 @@ def test_device_replays_fixture(path, cuda):
         # continue from the fixture's parameters so that the bound stays a per-step bound
         prev = z[f"p{t}"]
         p.copy_(to_t(prev).to(cuda))
+
+
+# ---------------------------------------------------------------------------
+# stochastic rounding and rank-1 fixtures (written from oracle/q4_oracle_torch.py)
+# ---------------------------------------------------------------------------
+def _t(a):
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16) if a.dtype == np.uint16 else torch.from_numpy(a.copy())
+
+
+def _bits(t):
+    if t.dtype == torch.bfloat16:
+        return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1)
+    if t.dtype == torch.float32:
+        return t.contiguous().cpu().numpy().view(np.uint32).reshape(-1)
+    return t.cpu().numpy().reshape(-1)
+
+
+@pytest.mark.parametrize("path", SR_FIXTURES, ids=[os.path.basename(p) for p in SR_FIXTURES])
+def test_oracle_replays_sr_fixture(path):
+    z, hp, steps = load(path)
+    seed, salt = (int(x) for x in z["sr"])
+    n = z["p0"].size
+    nb, nk = oc.state_sizes(n)
+    st = (_t(z["p0"]), torch.zeros(nb, dtype=torch.uint8), torch.zeros(nb, dtype=torch.uint8), torch.zeros(nk), torch.zeros(nk))
+    for t in range(1, steps + 1):
+        st = ot.step_quant_sr(st[0], _t(z[f"g{t}"]), *st[1:], seed=seed, tensor_salt=salt, step=t, **hp)
+        for key, got in zip(("p", "m", "v", "sm", "sv"), st):
+            assert np.array_equal(_bits(got), z[f"{key}{t}"].view(_bits(got).dtype)), (key, t)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", SR_FIXTURES, ids=[os.path.basename(p) for p in SR_FIXTURES])
+def test_device_replays_sr_fixture(path, cuda):
+    from quantfour_adamw_cuda_amd import quantfour_hip as q
+    z, hp, steps = load(path)
+    seed, salt = (int(x) for x in z["sr"])
+    n = z["p0"].size
+    nb, nk = oc.state_sizes(n)
+    p = _t(z["p0"]).to(cuda)
+    m, v = torch.zeros(nb, dtype=torch.uint8, device=cuda), torch.zeros(nb, dtype=torch.uint8, device=cuda)
+    sm, sv = torch.zeros(nk, device=cuda), torch.zeros(nk, device=cuda)
+    prev = z["p0"]
+    for t in range(1, steps + 1):
+        q.fused_4bit_multi_sr([p], [_t(z[f"g{t}"]).to(cuda)], [m], [v], [sm], [sv], hp["beta1"], hp["beta2"], hp["lr"],
+                              hp["weight_decay"], hp["eps"], t, seed, salts=[salt])
+        for key, got in (("m", m), ("v", v), ("sm", sm), ("sv", sv)):
+            assert np.array_equal(_bits(got), z[f"{key}{t}"].view(_bits(got).dtype)), (key, t)
+        ok, worst = p_close(_bits(p).view(z["p0"].dtype), z[f"p{t}"], prev, bf16=z["p0"].dtype == np.uint16)
+        assert ok, worst
+        prev = z[f"p{t}"]
+        p.copy_(_t(prev).to(cuda))
+
+
+@pytest.mark.parametrize("path", RANK1_FIXTURES, ids=[os.path.basename(p) for p in RANK1_FIXTURES])
+def test_oracle_replays_rank1_fixture(path):
+    z, hp, steps = load(path)
+    rows, cols = (int(x) for x in z["shape"])
+    nb, nk = oc.state_sizes(rows * cols)
+    st = (_t(z["p0"]).view(rows, cols), torch.zeros(nb, dtype=torch.uint8), torch.zeros(nb, dtype=torch.uint8),
+          torch.zeros(nk), torch.zeros(rows), torch.zeros(cols))
+    for t in range(1, steps + 1):
+        st = ot.step_quant_rank1(st[0], _t(z[f"g{t}"]).view(rows, cols), *st[1:], step=t, **hp)
+        for key, got in zip(("p", "m", "v", "sm", "r", "c"), st):
+            assert np.array_equal(_bits(got), z[f"{key}{t}"].view(_bits(got).dtype)), (key, t)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", RANK1_FIXTURES, ids=[os.path.basename(p) for p in RANK1_FIXTURES])
+def test_device_replays_rank1_fixture(path, cuda):
+    from quantfour_adamw_cuda_amd import quantfour_hip as q
+    z, hp, steps = load(path)
+    rows, cols = (int(x) for x in z["shape"])
+    nb, nk = oc.state_sizes(rows * cols)
+    p = _t(z["p0"]).view(rows, cols).to(cuda)
+    m, v = torch.zeros(nb, dtype=torch.uint8, device=cuda), torch.zeros(nb, dtype=torch.uint8, device=cuda)
+    sm = torch.zeros(nk, device=cuda)
+    r, c, rn, cn = (torch.zeros(k, device=cuda) for k in (rows, cols, rows, cols))
+    prev = z["p0"]
+    for t in range(1, steps + 1):
+        q.fused_4bit_rank1_multi([p], [_t(z[f"g{t}"]).view(rows, cols).to(cuda)], [m], [v], [sm], [r], [c], [rn], [cn],
+                                 hp["beta1"], hp["beta2"], hp["lr"], hp["weight_decay"], hp["eps"], t)
+        for key, got in (("m", m), ("v", v), ("sm", sm), ("r", r), ("c", c)):
+            assert np.array_equal(_bits(got), z[f"{key}{t}"].view(_bits(got).dtype)), (key, t)
+        ok, worst = p_close(_bits(p).view(z["p0"].dtype), z[f"p{t}"], prev, bf16=z["p0"].dtype == np.uint16)
+        assert ok, worst
+        prev = z[f"p{t}"]
+        p.copy_(_t(prev).view(rows, cols).to(cuda))
