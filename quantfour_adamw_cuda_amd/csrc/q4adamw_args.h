@@ -1,0 +1,206 @@
+// Launch arguments of the kernels (passed by value in the kernarg segment) and the constant
+// tables they read.  Shared by the kernels and the host launchers of q4adamw.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/q4adamw.h"
+#include "q4adamw_tables.h"
+
+namespace q4 {
+
+
+constexpr int kWaves = 4;                  // waves per workgroup
+constexpr int kThreads = kWaves * 64;
+constexpr int kMaxTensors = 48;            // tensors per fused launch
+constexpr int kSmallChunk = 1024;          // elements per workgroup, non-quantized kernel
+constexpr int kMaxSmallTensors = 80;
+
+// derived on the host exactly as optim/cuda_adamw_kernels.cu:435-440
+struct StepConsts {
+  float b1, b2, r1, r2;  // beta1, beta2, 1-beta1, 1-beta2
+  float wdu, ss;         // 1 - lr*wd, lr / (1 - beta1^t)
+  float c2s;             // sqrt(1 - beta2^t)
+  float eps;
+  // the fused kernel's parameter update p*wdu - m'/(sqrt(v')*den_scale + den_eps), the
+  // step size folded into the denominator: 1/(c2s*ss) and eps/ss
+  float den_scale, den_eps;
+};
+
+// What a launch does to the gradients besides reading them (kernels with EXT only).
+struct GradOps {
+  float scale;             // host part of the multiplier
+  uint32_t zero;           // non-zero: overwrite the gradients with zeros once they are read
+  const float *scale_dev;  // device part of the multiplier, or null
+  const float *skip;       // device flag, or null: non-zero turns the launch into a no-op
+};
+
+struct TensorDesc {  // 56 bytes
+  void *p;
+  const void *g;
+  uint8_t *m;
+  uint8_t *v;
+  float *sm;
+  float *sv;
+  int64_t numel;
+};
+
+// Kernel arguments of one fused launch (about 3 KiB, passed by value).
+// first_chunk[i] = index of tensor i's first chunk; entries past ntensors hold
+// 0x7fffffff (more than any chunk index).  pivot[k] = first_chunk[8k] lets a workgroup find its tensor with two
+// wide scalar loads.
+struct FusedArgs {
+  static constexpr int kCapacity = kMaxTensors;
+  static constexpr int kPivots = (kMaxTensors + 7) / 8;
+  StepConsts sc;
+  GradOps go;
+  int ntensors;
+  uint32_t nchunks;        // chunks in this launch
+  uint32_t chunks_per_xcd; // ceil(nchunks / 8); the grid has 8 * chunks_per_xcd workgroups
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  TensorDesc desc[kMaxTensors];
+  uint32_t sr_salt[kMaxTensors];  // stochastic rounding: the tensors' noise salts of this step
+};
+
+struct SmallDesc {  // 40 bytes
+  void *p;
+  const void *g;
+  float *m;
+  float *v;
+  int64_t numel;
+};
+
+struct SmallArgs {
+  static constexpr int kCapacity = kMaxSmallTensors;
+  static constexpr int kPivots = (kMaxSmallTensors + 7) / 8;
+  StepConsts sc;
+  GradOps go;
+  int ntensors;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  SmallDesc desc[kMaxSmallTensors];
+};
+
+// One tensor whose second moment is rank-1 scaled (a rows x cols matrix, row-major).
+struct Rank1Desc {  // 104 bytes
+  void *p;
+  const void *g;
+  uint8_t *m;
+  uint8_t *v;
+  float *sm;          // block scales of the first moment
+  float *rmax;        // current statistics of the second moment: rows, cols floats
+  float *cmax;
+  float *rmax_next;   // the step's new statistics (all zero between steps)
+  float *cmax_next;
+  int64_t numel;      // rows * cols
+  int64_t rows;
+  int64_t cols;
+  // division of a 32-bit number by cols / 8 as multiply-high, add and shifts
+  // (round-up method: exact for every 32-bit dividend)
+  uint32_t div_magic;
+  uint32_t div_shift;
+};
+
+struct FastDiv {
+  uint32_t magic, shift;
+};
+
+// n / d for the divisor the pair was made for
+__host__ __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t shift) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t t = __umulhi(n, magic);
+#else
+  const uint32_t t = (uint32_t)(((uint64_t)n * magic) >> 32);
+#endif
+  return (t + ((n - t) >> 1)) >> shift;
+}
+
+static FastDiv make_fast_div(uint32_t d) {  // d >= 2
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;                     // ceil(log2 d) >= 1
+  FastDiv f;
+  f.magic = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+  f.shift = l - 1;
+  return f;
+}
+
+constexpr int kMaxRank1Tensors = 32;
+
+// Kernel arguments of the rank-1 launches.  The update kernel indexes chunks of
+// kChunk flat elements like FusedArgs; the statistics kernel indexes tiles of
+// kStatRows rows x kStatCols columns (stat_first_chunk, stat_col_groups).
+struct Rank1Args {
+  static constexpr int kCapacity = kMaxRank1Tensors;
+  static constexpr int kPivots = (kMaxRank1Tensors + 7) / 8;
+  StepConsts sc;
+  GradOps go;
+  int ntensors;
+  uint32_t nchunks;
+  uint32_t chunks_per_xcd;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  Rank1Desc desc[kMaxRank1Tensors];
+};
+
+struct Rank1StatArgs {
+  static constexpr int kCapacity = kMaxRank1Tensors;
+  static constexpr int kPivots = (kMaxRank1Tensors + 7) / 8;
+  float b2, r2;
+  GradOps go;
+  int ntensors;
+  uint32_t nchunks;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  uint32_t col_groups[kMaxRank1Tensors];   // column groups per row group of tensor t
+  struct Desc {
+    const void *g;
+    const uint8_t *v;
+    const float *rmax;
+    const float *cmax;
+    float *rmax_next;
+    float *cmax_next;
+    int64_t rows;
+    int64_t cols;
+  } desc[kMaxRank1Tensors];
+};
+
+// Gradient-norm launch: every workgroup walks chunks of 32 KiB with a grid stride.
+constexpr int kMaxNormTensors = 160;
+constexpr int kNormPartials = Q4ADAMW_NORM_WORKSPACE_BYTES / 8;  // workgroups = fp64 partial sums
+constexpr int kNormChunkBytes = 32768;                          // 8 16-byte loads per thread
+
+struct NormDesc {
+  const void *g;
+  int64_t numel;
+};
+
+struct NormArgs {
+  static constexpr int kCapacity = kMaxNormTensors;
+  static constexpr int kPivots = (kMaxNormTensors + 7) / 8;
+  double *partials;   // kNormPartials sums, one per workgroup
+  uint32_t nchunks;
+  uint32_t first;     // non-zero: the partial sums are overwritten, otherwise added to
+  int ntensors;
+  uint32_t pivot[kPivots];
+  uint32_t first_chunk[kPivots * 8];
+  NormDesc desc[kMaxNormTensors];
+};
+
+static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(NormArgs) <= 4096 &&
+                  sizeof(Rank1Args) <= 4096 && sizeof(Rank1StatArgs) <= 4096,
+              "kernel arguments are limited to 4 KiB");
+
+// the first-moment bucket table (see q4adamw_tables.h), copied into LDS by every
+// workgroup at start-up, one entry per thread
+__device__ const HalfTable kHalfTable = make_half_table();
+// stochastic rounding: code-book entries per bucket and the 17 intervals between them
+__device__ const SrHalfTable kSrHalfTable = make_sr_half_table();
+__device__ const SrIntervalTable kSrIntervals = make_sr_interval_table();
+// first-moment code book for kernels that index it per lane
+__device__ const uint32_t kQmapMDev[16] = {
+    0xbf633333u, 0xbf29999au, 0xbee00000u, 0xbe59999au, 0xbd9eb852u, 0xbd051eb8u,
+    0xbbb43958u, 0x00000000u, 0x3bb43958u, 0x3d051eb8u, 0x3d9eb852u, 0x3e59999au,
+    0x3ee00000u, 0x3f29999au, 0x3f633333u, 0x3f800000u};
+
+}  // namespace q4

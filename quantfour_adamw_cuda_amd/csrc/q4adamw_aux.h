@@ -1,0 +1,263 @@
+// Kernels around the fused step: the non-quantized step of small tensors, the global
+// gradient norm, stand-alone quantize / dequantize for checkpoint interchange.
+#pragma once
+#include "q4adamw_device.h"
+
+namespace q4 {
+
+// Non-quantized step for small tensors (cuda_adamw_kernels.cu:100-133): fp32
+// moments in place, same derived scalars and operation order as the fused path.
+template <bool PBF, bool GBF, bool EXT>
+__global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args) {
+  const uint32_t chunk = blockIdx.x;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const bool zero_g = EXT && args.go.zero != 0u;
+  const int t = find_tensor(args, chunk);
+  const SmallDesc &T = args.desc[t];
+  const StepConsts &sc = args.sc;
+  const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kSmallChunk;
+  const int64_t end = base + kSmallChunk < T.numel ? base + kSmallChunk : T.numel;
+  for (int64_t i = base + threadIdx.x; i < end; i += 256) {
+    float gi = GBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.g)[i])
+                   : as_global<const float>(T.g)[i];
+    if (EXT) {
+      gi *= gscale;
+      if (zero_g) {
+        if (GBF) as_global<uint16_t>(const_cast<void *>(T.g))[i] = 0;
+        else as_global<float>(const_cast<void *>(T.g))[i] = 0.0f;
+      }
+    }
+    const float pi = PBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.p)[i])
+                         : as_global<const float>(T.p)[i];
+    const float m = sc.b1 * as_global<const float>(T.m)[i] + sc.r1 * gi;
+    const float v = sc.b2 * as_global<const float>(T.v)[i] + sc.r2 * (gi * gi);
+    as_global<float>(T.m)[i] = m;
+    as_global<float>(T.v)[i] = v;
+    // exact form here: these tensors are tiny, so the divisions cost nothing
+    const float den = __builtin_sqrtf(v) / sc.c2s + sc.eps;
+    const float pn = pi * sc.wdu - sc.ss * (m / den);
+    if (PBF) as_global<uint16_t>(T.p)[i] = (uint16_t)f32_to_bf16_bits(pn);
+    else as_global<float>(T.p)[i] = pn;
+  }
+}
+
+
+// ---------------------------------------------------------------------------
+// global gradient norm (what a caller computes before it clips)
+// ---------------------------------------------------------------------------
+// Sum over a 256-thread workgroup in a fixed order; the result is valid in thread 0.
+__device__ __forceinline__ double workgroup_sum(double x, double *lds4) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, 64);
+  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = x;
+  __syncthreads();
+  return (lds4[0] + lds4[1]) + (lds4[2] + lds4[3]);
+}
+
+// Squares are exact in fp64 and summed there: four accumulators per thread, chunks in
+// grid-stride order, so the sum depends on the tensor list only, not on scheduling.
+template <bool GBF>
+__global__ __launch_bounds__(256) void grad_sumsq_kernel(const NormArgs args) {
+  constexpr int kElemBytes = GBF ? 2 : 4;
+  constexpr int64_t kChunkElems = kNormChunkBytes / kElemBytes;
+  __shared__ double lds4[4];
+  const int tid = threadIdx.x;
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  for (uint32_t chunk = blockIdx.x; chunk < args.nchunks; chunk += kNormPartials) {
+    const int t = find_tensor(args, chunk);
+    const NormDesc &T = args.desc[t];
+    const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kChunkElems;
+    const void *cb = static_cast<const char *>(T.g) + base * kElemBytes;
+    const int64_t rem = T.numel - base;
+    if (rem >= kChunkElems) {
+      u32x4 w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        w[k] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(cb), (uint32_t)(k * 256 + tid) * 16u, 0, kNtReadOnly);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t u[4] = {w[k].x, w[k].y, w[k].z, w[k].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          if (GBF) {
+            float lo, hi;
+            widen_bf16_pair(u[c], lo, hi);
+            acc[c] = __builtin_fma((double)lo, (double)lo, acc[c]);
+            acc[c] = __builtin_fma((double)hi, (double)hi, acc[c]);
+          } else {
+            const double x = (double)bits2f(u[c]);
+            acc[c] = __builtin_fma(x, x, acc[c]);
+          }
+        }
+      }
+    } else {
+      for (int64_t i = tid; i < rem; i += 256) {
+        const double x = GBF ? (double)bf16_bits_to_f32(as_global<const uint16_t>(cb)[i])
+                             : (double)as_global<const float>(cb)[i];
+        acc[0] = __builtin_fma(x, x, acc[0]);
+      }
+    }
+  }
+  const double total = workgroup_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), lds4);
+  if (tid == 0) {
+    const gptr<double> out = as_global<double>(args.partials) + blockIdx.x;
+    *out = args.first ? total : *out + total;
+  }
+}
+
+__global__ __launch_bounds__(256) void grad_norm_finish_kernel(const double *partials_, float scale,
+                                                               const float *scale_dev, float max_norm,
+                                                               float *out3_) {
+  __shared__ double lds4[4];
+  const gptr<const double> partials = as_global<const double>(partials_);
+  double a = 0.0;
+#pragma unroll
+  for (int k = 0; k < kNormPartials / 256; ++k) a += partials[threadIdx.x * (kNormPartials / 256) + k];
+  const double total = workgroup_sum(a, lds4);
+  if (threadIdx.x == 0) {
+    float s = scale;
+    if (scale_dev) s *= *as_global<const float>(scale_dev);
+    const float norm = __builtin_fabsf(s) * (float)__builtin_sqrt(total);
+    // torch.nn.utils.clip_grad_norm_: max_norm / (total_norm + 1e-6), clamped to 1
+    // (a NaN stays a NaN)
+    float coef = 1.0f;
+    if (max_norm > 0.0f) {
+      coef = max_norm / (norm + 1e-6f);
+      coef = coef > 1.0f ? 1.0f : coef;
+    }
+    const gptr<float> out3 = as_global<float>(out3_);
+    out3[0] = norm;
+    out3[1] = coef;
+    out3[2] = s * coef;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// stand-alone quantize / dequantize of one moment (checkpoint interchange)
+// ---------------------------------------------------------------------------
+// One wave per 128-element block, two elements (one packed byte) per lane.  These run
+// once per checkpoint, so they take the exact route only: IEEE division and the
+// 15-compare count (optim/adamw_fourbit_triton.py:618-630, cuda_adamw_kernels.cu:167-194).
+template <bool SECOND>
+__global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__ x_, int64_t numel,
+                                                       uint8_t *__restrict__ codes_,
+                                                       float *__restrict__ scale_) {
+  const gptr<const float> x = as_global<const float>(x_);
+  const int lane = threadIdx.x & 63;
+  const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t nblk = (numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
+  if (blk >= nblk) return;
+  const int64_t e = blk * Q4ADAMW_BLOCK + lane * 2;
+  const float a = e < numel ? x[e] : 0.0f;
+  const float b = e + 1 < numel ? x[e + 1] : 0.0f;
+  // fmaxf drops a NaN next to a number; two NaN count as 0: a NaN never becomes the scale
+  const float lane_max = __builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b));
+  uint32_t u = lane_max == lane_max ? f2bits(lane_max) : 0u;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)u, off, 64);
+    u = u > o ? u : o;
+  }
+  const float s = bits2f(u);
+  if (lane == 0) as_global<float>(scale_)[blk] = s;
+  if (e < numel) {
+    uint32_t byte = 0;
+    const float q0 = a / s, q1 = b / s;
+#pragma unroll
+    for (int k = 0; k < 15; ++k) {
+      const float t = SECOND ? qmid_v(k) : bits2f(kQmidMBits[k]);
+      byte += (t < q0) ? 1u : 0u;
+      byte += (e + 1 < numel && t < q1) ? 16u : 0u;
+    }
+    as_global<uint8_t>(codes_)[e >> 1] = (uint8_t)byte;
+  }
+}
+
+// Rank-1 forms for the second moment of a rows x cols matrix (run once per
+// checkpoint).  Statistics: a workgroup takes 64 rows x 256 columns, a thread one
+// column; row maxima meet in LDS, then one atomic per row and per column.
+__global__ __launch_bounds__(256) void fill_zero_kernel(float *x_, int64_t n) {
+  const gptr<float> x = as_global<float>(x_);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) x[i] = 0.0f;
+}
+
+__global__ __launch_bounds__(256) void rank1_absmax_kernel(const float *x_, int64_t rows, int64_t cols,
+                                                           float *row_max, float *col_max) {
+  __shared__ uint32_t row_bits[64];
+  const gptr<const float> x = as_global<const float>(x_);
+  const int tid = threadIdx.x;
+  const int64_t col = (int64_t)blockIdx.x * 256 + tid;
+  const int64_t row0 = (int64_t)blockIdx.y * 64;
+  const int nrows = (int)(row0 + 64 < rows ? 64 : rows - row0);
+  if (tid < 64) row_bits[tid] = 0u;
+  __syncthreads();
+  float c_max = 0.0f;
+  for (int r = 0; r < nrows; ++r) {
+    float a = col < cols ? __builtin_fabsf(x[(row0 + r) * cols + col]) : 0.0f;
+    a = a == a ? a : 0.0f;  // a NaN never becomes a maximum
+    c_max = __builtin_fmaxf(c_max, a);
+    uint32_t u = f2bits(a);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const uint32_t o = (uint32_t)__shfl_xor((int)u, off, 64);
+      u = u > o ? u : o;
+    }
+    if ((tid & 63) == 0 && u != 0u) atomicMax(&row_bits[r], u);
+  }
+  if (col < cols && c_max != 0.0f) atomic_max_nonneg(col_max + col, c_max);
+  __syncthreads();
+  if (tid < nrows && row_bits[tid] != 0u) atomic_max_nonneg(row_max + row0 + tid, bits2f(row_bits[tid]));
+}
+
+// one thread per packed byte: x / min(row maximum, column maximum), IEEE division, the
+// 15-compare count (optim/adamw_fourbit_triton.py:834-863)
+__global__ __launch_bounds__(256) void quantize_rank1_kernel(const float *x_, int64_t rows, int64_t cols,
+                                                             const float *row_max, const float *col_max,
+                                                             uint8_t *codes_) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (e >= rows * cols) return;
+  const int64_t i = e / cols, j = e - i * cols;  // cols is even: both elements in row i
+  const float r = as_global<const float>(row_max)[i];
+  uint32_t byte = 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float q = as_global<const float>(x_)[e + h] / __builtin_fminf(r, as_global<const float>(col_max)[j + h]);
+#pragma unroll
+    for (int k = 0; k < 15; ++k) byte += (qmid_v(k) < q) ? (1u << (4 * h)) : 0u;
+  }
+  as_global<uint8_t>(codes_)[e >> 1] = (uint8_t)byte;
+}
+
+// optim/adamw_fourbit_triton.py:520-527: code-book entry times min(row, column maximum)
+__global__ __launch_bounds__(256) void dequantize_rank1_kernel(const uint8_t *codes_, const float *row_max,
+                                                               const float *col_max, int64_t rows,
+                                                               int64_t cols, float *out_) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (e >= rows * cols) return;
+  const int64_t i = e / cols, j = e - i * cols;
+  const float r = as_global<const float>(row_max)[i];
+  const uint32_t byte = as_global<const uint8_t>(codes_)[e >> 1];
+  as_global<float>(out_)[e] = qmap_v((int)(byte & 15u)) * __builtin_fminf(r, as_global<const float>(col_max)[j]);
+  as_global<float>(out_)[e + 1] = qmap_v((int)(byte >> 4)) * __builtin_fminf(r, as_global<const float>(col_max)[j + 1]);
+}
+
+// cuda_adamw_kernels.cu:329-343: code -> code-book entry * block scale
+template <bool SECOND>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t *__restrict__ codes_,
+                                                         const float *__restrict__ scale_,
+                                                         int64_t numel, float *__restrict__ out_) {
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (e >= numel) return;
+  const uint32_t byte = as_global<const uint8_t>(codes_)[e >> 1];
+  const float s = as_global<const float>(scale_)[e / Q4ADAMW_BLOCK];
+  const uint32_t c0 = byte & 15u, c1 = byte >> 4;
+  const float v0 = (SECOND ? qmap_v((int)c0) : bits2f(kQmapMDev[c0])) * s;
+  as_global<float>(out_)[e] = v0;
+  if (e + 1 < numel) {
+    const float v1 = (SECOND ? qmap_v((int)c1) : bits2f(kQmapMDev[c1])) * s;
+    as_global<float>(out_)[e + 1] = v1;
+  }
+}
+
+}  // namespace q4

@@ -1,0 +1,403 @@
+// Device helpers of the 4-bit AdamW kernels: address spaces and buffer resources, wave
+// reductions, bf16 conversion, element loads and stores, the exact quantizers, the rounding
+// noise, the tensor search.
+#pragma once
+#include "q4adamw_args.h"
+
+namespace q4 {
+
+// ---------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------
+// Pointers that arrive inside a descriptor are generic; every tensor lives in
+// global memory, so say so and get global_load/global_store instead of flat ones.
+template <typename T>
+using gptr = __attribute__((address_space(1))) T *;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+__device__ __forceinline__ gptr<T> as_global(const void *p) {
+  return (gptr<T>)(uintptr_t)p;
+}
+
+// Full tiles go through buffer instructions: the tile's base address sits in a
+// scalar resource descriptor and each lane supplies a 32-bit byte offset, so no
+// vector ALU work goes into addresses.  Cache policy of the streamed tensors: the
+// non-temporal hint (bit 1) plus system scope (sc1, bit 4); every datum is touched
+// once, and with the wider scope the streams measure 1.5 % faster than with the hint
+// alone (and 11 % faster than without either).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kNt = 2 | 16;
+constexpr int kNtReadOnly = 2;  // a pure read stream (the gradient norm) measures the same with and without sc1
+
+__device__ __forceinline__ rsrc_t tile_rsrc(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, -1, 0x00020000);
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_umax(uint32_t x) {
+  const uint32_t y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, true);
+  return x > y ? x : y;
+}
+
+// Abs-max of both moments over the 32 lanes of a quantization block (lanes 0-31 or
+// 32-63), results in every lane of the block.  The inputs are non-negative floats,
+// so their bit patterns order like unsigned integers.  One v_permlane16_swap pairs
+// lane i of the block's first row with lane i of its second row and leaves the
+// first-moment partial max in the first row and the second-moment partial max in
+// the second row; four DPP steps then reduce both rows at once; a second swap
+// hands each row the other row's result.
+__device__ __forceinline__ void block_max32_pair(float &am, float &av) {
+  // after the swap: a = [am.r0, av.r0, am.r2, av.r2], b = [am.r1, av.r1, am.r3, av.r3]
+  const auto s1 = __builtin_amdgcn_permlane16_swap(f2bits(am), f2bits(av), false, false);
+  uint32_t u = s1[0] > s1[1] ? s1[0] : s1[1];
+  u = dpp_umax<0xB1>(u);   // quad_perm [1,0,3,2]
+  u = dpp_umax<0x4E>(u);   // quad_perm [2,3,0,1]
+  u = dpp_umax<0x141>(u);  // row_half_mirror
+  u = dpp_umax<0x140>(u);  // row_mirror
+  // u = [max am, max av, max am, max av] per row; spread: a = rows (0,0,2,2), b = rows (1,1,3,3)
+  const auto s2 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  am = bits2f(s2[0]);
+  av = bits2f(s2[1]);
+}
+
+// Max of a non-negative float over the 16 lanes of a DPP row, result in every lane.
+__device__ __forceinline__ float row_max16(float x) {
+  uint32_t u = f2bits(x);
+  u = dpp_umax<0xB1>(u);
+  u = dpp_umax<0x4E>(u);
+  u = dpp_umax<0x141>(u);
+  u = dpp_umax<0x140>(u);
+  return bits2f(u);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return bits2f(h << 16); }
+
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nearest even
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// two fp32 -> two bf16 (round to nearest even) in one 32-bit word, lo in the low half
+__device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+}
+
+__device__ __forceinline__ void widen_bf16_pair(uint32_t w, float &lo, float &hi) {
+  lo = bits2f(w << 16);
+  hi = bits2f(w & 0xffff0000u);
+}
+
+// N consecutive elements (N = 4 or 8) starting at element e0 of the tile at base
+template <bool BF, int N, bool FULL>
+__device__ __forceinline__ void load_elems(const void *base, uint32_t e0, int nv, float (&x)[N]) {
+  if (FULL) {
+    if (BF && N == 4) {
+      const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(tile_rsrc(base), e0 * 2, 0, kNt);
+      widen_bf16_pair(w.x, x[0], x[1]);
+      widen_bf16_pair(w.y, x[2], x[3]);
+    } else if (BF) {
+      const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), e0 * 2, 0, kNt);
+      widen_bf16_pair(w.x, x[0], x[1]);
+      widen_bf16_pair(w.y, x[2], x[3]);
+      widen_bf16_pair(w.z, x[N - 4], x[N - 3]);
+      widen_bf16_pair(w.w, x[N - 2], x[N - 1]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < N; k += 4) {
+        const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), (e0 + k) * 4, 0, kNt);
+        x[k] = bits2f(a.x); x[k + 1] = bits2f(a.y); x[k + 2] = bits2f(a.z); x[k + 3] = bits2f(a.w);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      x[j] = 0.0f;
+      if (j < nv) {
+        x[j] = BF ? bf16_bits_to_f32(as_global<const uint16_t>(base)[e0 + j])
+                  : as_global<const float>(base)[e0 + j];
+      }
+    }
+  }
+}
+
+template <bool BF, int N, bool FULL>
+__device__ __forceinline__ void store_elems(void *base, uint32_t e0, int nv, const float (&x)[N]) {
+  if (FULL) {
+    if (BF && N == 4) {
+      u32x2 w;
+      w.x = pack_bf16_pair(x[0], x[1]);
+      w.y = pack_bf16_pair(x[2], x[3]);
+      __builtin_amdgcn_raw_buffer_store_b64(w, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else if (BF) {
+      u32x4 w;
+      w.x = pack_bf16_pair(x[0], x[1]);
+      w.y = pack_bf16_pair(x[2], x[3]);
+      w.z = pack_bf16_pair(x[N - 4], x[N - 3]);
+      w.w = pack_bf16_pair(x[N - 2], x[N - 1]);
+      __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else {
+#pragma unroll
+      for (int k = 0; k < N; k += 4) {
+        const u32x4 w = {f2bits(x[k]), f2bits(x[k + 1]), f2bits(x[k + 2]), f2bits(x[k + 3])};
+        __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), (e0 + k) * 4, 0, kNt);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      if (j < nv) {
+        if (BF) as_global<uint16_t>(base)[e0 + j] = (uint16_t)f32_to_bf16_bits(x[j]);
+        else as_global<float>(base)[e0 + j] = x[j];
+      }
+    }
+  }
+}
+
+// zeros over the N elements that load_elems<BF, N, FULL> read
+template <bool BF, int N, bool FULL>
+__device__ __forceinline__ void zero_elems(void *base, uint32_t e0, int nv) {
+  if (FULL) {
+    const u32x4 z4 = {0u, 0u, 0u, 0u};
+    if (BF && N == 4) {
+      const u32x2 z2 = {0u, 0u};
+      __builtin_amdgcn_raw_buffer_store_b64(z2, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else if (BF) {
+      __builtin_amdgcn_raw_buffer_store_b128(z4, tile_rsrc(base), e0 * 2, 0, kNt);
+    } else {
+#pragma unroll
+      for (int k = 0; k < N; k += 4)
+        __builtin_amdgcn_raw_buffer_store_b128(z4, tile_rsrc(base), (e0 + k) * 4, 0, kNt);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      if (j < nv) {
+        if (BF) as_global<uint16_t>(base)[e0 + j] = 0;
+        else as_global<float>(base)[e0 + j] = 0.0f;
+      }
+    }
+  }
+}
+
+template <int N>
+struct Vals {
+  float x[N];
+};
+
+// Exact quantization of N values of one state: IEEE division by the block scale,
+// then the number of thresholds strictly below the quotient
+// (cuda_adamw_kernels.cu:167-194 in closed form).  0/0 is NaN and gets code 0.
+template <bool SECOND, int N>
+__device__ __forceinline__ uint32_t quantize_exact(const Vals<N> &v, float scale) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float q = v.x[j] / scale;
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < 15; ++k) {
+      const float t = SECOND ? qmid_v(k) : bits2f(kQmidMBits[k]);
+      c += (t < q) ? 1u : 0u;
+    }
+    word |= c << (4 * j);
+  }
+  return word;
+}
+
+// The same for the second moment with a scale per element (rank-1 scaling).
+template <int N>
+__device__ __forceinline__ uint32_t quantize_exact_scales(const Vals<N> &v, const Vals<N> &scale) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float q = v.x[j] / scale.x[j];
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < 15; ++k) c += (qmid_v(k) < q) ? 1u : 0u;
+    word |= c << (4 * j);
+  }
+  return word;
+}
+
+// A 32-bit integer mixer (two multiply-xorshift rounds) for the rounding noise.
+__host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7FEB352Du;
+  x ^= x >> 15;
+  x *= 0x846CA68Bu;
+  x ^= x >> 16;
+  return x;
+}
+
+// noise in (0, 1) from a 16-bit number: (2 n + 1) / 2^17, exact
+__device__ __forceinline__ float sr_noise_value(uint32_t n16) {
+  return __builtin_fmaf((float)n16, 1.52587890625e-05f, 7.62939453125e-06f);
+}
+
+// Stochastic rounding, exact form (the closed form of quantize_bsearch<STOCHASTIC>,
+// optim/adamw_fourbit_triton.py:1050-1075, without its division): IEEE quotient, its
+// interval [Q[k], Q[k+1]) among the code-book entries, upper code iff
+// noise * (Q[k+1] - Q[k]) < q - Q[k].  0/0 is NaN and gets code 0.
+template <bool SECOND, int N>
+__device__ __forceinline__ uint32_t quantize_exact_sr(const Vals<N> &v, float scale, const Vals<N> &noise) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float q = v.x[j] / scale;
+    uint32_t k_raw = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float t = SECOND ? qmap_v(k) : bits2f(kQmapMBits[k]);
+      k_raw += (t <= q) ? 1u : 0u;
+    }
+    float lower, width;
+    if (SECOND) {
+      lower = k_raw == 0u ? -3.4028234663852886e38f : (float)k_raw * 0.0625f;
+      width = k_raw == 0u ? 0.0f : (k_raw == 16u ? __builtin_inff() : 0.0625f);
+    } else {
+      const SrInterval iv = kSrIntervals.e[k_raw];
+      lower = iv.lower;
+      width = iv.width;
+    }
+    const bool up = noise.x[j] * width < q - lower;
+    int c = (int)k_raw - 1 + (up ? 1 : 0);
+    c = c < 0 ? 0 : (c > 15 ? 15 : c);
+    word |= (uint32_t)c << (4 * j);
+  }
+  return word;
+}
+
+// (x & mask) | base as one v_and_or_b32: the mask travels in a scalar register (the
+// compiler splits the operation when the mask is a literal, which a VOP3 encoding
+// cannot hold).
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t base) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(base));
+  return r;
+}
+
+// Byte BYTE of x, times 8 (the byte offset of an 8-byte table entry), as one SDWA
+// shift; `three` is the shift amount in a register.
+template <int BYTE>
+__device__ __forceinline__ uint32_t byte_times8(uint32_t x, uint32_t three) {
+  static_assert(BYTE >= 0 && BYTE <= 3, "");
+  uint32_t r;
+#define Q4_SDWA_SHIFT(SEL)                                                                          \
+  asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:" SEL \
+      : "=v"(r) : "v"(three), "v"(x))
+  if (BYTE == 0) Q4_SDWA_SHIFT("BYTE_0");
+  else if (BYTE == 1) Q4_SDWA_SHIFT("BYTE_1");
+  else if (BYTE == 2) Q4_SDWA_SHIFT("BYTE_2");
+  else Q4_SDWA_SHIFT("BYTE_3");
+#undef Q4_SDWA_SHIFT
+  return r;
+}
+
+// byte_times8 with the byte chosen by a loop index of an unrolled loop
+__device__ __forceinline__ uint32_t entry_offset(uint32_t x, int byte, uint32_t three) {
+  switch (byte) {
+    case 0: return byte_times8<0>(x, three);
+    case 1: return byte_times8<1>(x, three);
+    case 2: return byte_times8<2>(x, three);
+    default: return byte_times8<3>(x, three);
+  }
+}
+
+// 1/s to within half an ulp for s in [2^-100, 2^100]: hardware estimate plus one
+// Newton step
+__device__ __forceinline__ float refined_rcp(float s) {
+  const float r0 = __builtin_amdgcn_rcpf(s);
+  const float e = __builtin_fmaf(-s, r0, 1.0f);
+  return __builtin_fmaf(e, r0, r0);
+}
+
+constexpr float kScaleLo = 7.888609052210118e-31f;   // 2^-100
+constexpr float kScaleHi = 1.2676506002282294e+30f;  // 2^100
+constexpr float kVGuard = 7.62939453125e-06f;        // 2^-17, in units of 16*q
+
+// Uniform search of the launch's tensor list: the last tensor whose first chunk is
+// <= chunk.  first_chunk[0] is 0, so the result is never negative.  Chunk indices and
+// table entries are below 2^31, so bit 31 of (x - chunk - 1) says x <= chunk: plain
+// integer arithmetic that stays on the scalar unit.
+template <typename Args>
+__device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
+  uint32_t group = 0;
+#pragma unroll
+  for (int k = 1; k < Args::kPivots; ++k) group += (a.pivot[k] - chunk - 1u) >> 31;
+  uint32_t within = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) within += (a.first_chunk[group * 8 + k] - chunk - 1u) >> 31;
+  return (int)(group * 8 + within) - 1;
+}
+
+// LDS of a workgroup, one array of 8-byte entries:
+//   [0, 256)    the waves' private dequantization tables: per wave 64 entries, per
+//               quantization block 16 entries {code_book_m[i] * scale_m,
+//               code_book_v[i] * scale_v}, so that dequantizing an element is one read
+//               and an entry number fits a byte
+//   [256, 512)  bucket table of the first-moment quantizer, indexed by the high byte
+//               of the quotient as a half
+//   [512, 529)  stochastic rounding only: the first moment's interval table
+constexpr uint32_t kLdsBuckets = 64 * kWaves;
+constexpr uint32_t kLdsIntervals = kLdsBuckets + kHalfTableEntries;
+constexpr uint32_t kLdsEntries = kLdsIntervals + 32;
+static_assert(kLdsBuckets == 256, "dequantization entry numbers must fit a byte");
+static_assert(kThreads == (int)kHalfTableEntries, "one bucket table entry per thread");
+
+// What a thread fetches from the constant tables as the very first thing it does.
+struct TableSlot {
+  uint2 entry;     // bucket table entry number tid
+  float qm;        // first-moment code-book value number (lane & 15)
+  uint2 interval;  // stochastic rounding: interval table entry number tid (tid < 17)
+};
+
+template <bool SR>
+__device__ __forceinline__ TableSlot request_table_slot(int tid) {
+  TableSlot s;
+  if (SR) {
+    const SrEntry e = kSrHalfTable.e[tid];
+    s.entry = make_uint2(e.thr, e.base);
+    const SrInterval iv = kSrIntervals.e[tid < 17 ? tid : 0];
+    s.interval = make_uint2(f2bits(iv.lower), f2bits(iv.width));
+  } else {
+    const MtabEntry e = kHalfTable.e[tid];
+    s.entry = make_uint2(e.lo, e.hi);
+    s.interval = make_uint2(0u, 0u);
+  }
+  s.qm = bits2f(kQmapMDev[tid & 15]);
+  return s;
+}
+
+// Writes the slot into LDS and waits for the whole workgroup.  Called by every wave
+// exactly once, after it has issued its global loads, so that the latencies overlap.
+// The fences order LDS only: a full __syncthreads() would also drain the outstanding
+// global loads.
+template <bool SR>
+__device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlot &s) {
+  lds[kLdsBuckets + tid] = s.entry;
+  if (SR && tid < 17) lds[kLdsIntervals + tid] = s.interval;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// The launch's gradient multiplier; false if the launch is to do nothing.
+__device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale) {
+  if (go.skip && *as_global<const float>(go.skip) != 0.0f) return false;
+  gscale = go.scale;
+  if (go.scale_dev) gscale *= *as_global<const float>(go.scale_dev);
+  return true;
+}
+
+// Atomic maximum of non-negative floats through their bit patterns.
+__device__ __forceinline__ void atomic_max_nonneg(const float *addr, float x) {
+  // non-negative floats order like their bit patterns
+  atomicMax(reinterpret_cast<unsigned int *>(const_cast<float *>(addr)), f2bits(x));
+}
+
+}  // namespace q4

@@ -1,0 +1,500 @@
+// The fused 4-bit AdamW step: one tile of one tensor (process_tile) and the kernels built on
+// it -- block-scaled, stochastic rounding, rank-1 scaled second moment (statistics, update,
+// commit).
+#pragma once
+#include "q4adamw_device.h"
+
+namespace q4 {
+
+// Geometry of the fused kernel: a lane owns 16 bytes of the widest of the parameter and
+// gradient streams, so that no stream needs two accesses per lane.
+template <bool PBF, bool GBF>
+struct Geometry {
+  static constexpr int kEpl = (PBF && GBF) ? 8 : 4;      // elements per lane
+  static constexpr int kTile = 64 * kEpl;                // elements per wave
+  static constexpr int kChunk = kTile * kWaves;          // elements per workgroup
+  static constexpr int kLanesPerBlock = Q4ADAMW_BLOCK / kEpl;   // 32 or 16
+  static constexpr int kBlocksPerTile = kTile / Q4ADAMW_BLOCK;  // 2 or 4
+};
+
+// ---------------------------------------------------------------------------
+// one tile (256 or 512 elements) of one tensor
+// ---------------------------------------------------------------------------
+// EXT: gradients are multiplied by gscale (one rounded fp32 multiplication per
+// element, before anything else uses them) and, if zero_g, overwritten with zeros.
+// RANK1 (Desc = Rank1Desc): the second moment's scale is min(row maximum, column
+// maximum) per element instead of one value per block: old statistics dequantize, the
+// step's new statistics (complete before this kernel starts) quantize.
+// SR: both moments are rounded stochastically between the two neighbouring code-book
+// entries; the noise of element e is a hash of e and the tensor's salt of this step.
+template <bool PBF, bool GBF, bool FULL, bool EXT, bool RANK1, bool SR, typename Desc>
+__device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
+                                             const StepConsts &sc, uint2 *lds, const TableSlot &slot,
+                                             float gscale, bool zero_g, uint32_t salt) {
+  static_assert(!(SR && RANK1), "stochastic rounding is built for block scaling only");
+  using G = Geometry<PBF, GBF>;
+  constexpr int N = G::kEpl;
+  // Uniform (scalar) part of every address: the tile's first element, byte and
+  // block; the per-lane part is a small 32-bit offset.
+  const int64_t numel = T.numel;
+  const int64_t tb = tile * G::kTile;
+  const void *p_tile = static_cast<const char *>(T.p) + tb * (PBF ? 2 : 4);
+  const void *g_tile = static_cast<const char *>(T.g) + tb * (GBF ? 2 : 4);
+  const uint8_t *m_tile = T.m + (tb >> 1);
+  const uint8_t *v_tile = T.v + (tb >> 1);
+  const float *sm_tile = T.sm + tile * G::kBlocksPerTile;
+  const float *sv_tile = nullptr;
+  if constexpr (!RANK1) sv_tile = T.sv + tile * G::kBlocksPerTile;
+  const uint32_t e0 = (uint32_t)lane * N;                          // first element of this lane in the tile
+  const uint32_t blk = (uint32_t)lane / G::kLanesPerBlock;         // which of the tile's blocks
+  const uint32_t code_off = (uint32_t)lane * (N / 2);              // byte offset of this lane's codes
+  int nv = N;
+  bool blk_ok = true;
+  if (!FULL) {
+    const int64_t rem = numel - tb - (int64_t)e0;
+    nv = rem >= N ? N : (rem > 0 ? (int)rem : 0);
+    blk_ok = tb + (int64_t)blk * Q4ADAMW_BLOCK < numel;
+  }
+
+  // rank-1: this lane's row maxima (old, new) and its N column maxima (old, new)
+  float r_old = 0.0f, r_new = 0.0f;
+  Vals<N> c_old, c_new;
+  if constexpr (RANK1) {
+    // (row, column) of the tile's first element, in units of 8 elements so that the
+    // division is a 32-bit one.  A tile is shorter than a row, so a lane is in that
+    // row or in the next one.
+    const uint32_t tb8 = (uint32_t)(tb >> 3), cols8 = (uint32_t)(T.cols >> 3);  // numel < 2^35
+    const uint32_t row32 = fast_div(tb8, T.div_magic, T.div_shift);
+    const int64_t row = row32;
+    const uint32_t col0 = (tb8 - row32 * cols8) << 3;
+    uint32_t col = col0 + e0;
+    const bool wrapped = col >= (uint32_t)T.cols;
+    if (wrapped) col -= (uint32_t)T.cols;
+    const int64_t last = T.rows - 1;
+    const int64_t ra = row < last ? row : last, rb = row + 1 < last ? row + 1 : last;  // past-the-end lanes stay in bounds
+    const float r_old_a = as_global<const float>(T.rmax)[ra], r_old_b = as_global<const float>(T.rmax)[rb];
+    const float r_new_a = as_global<const float>(T.rmax_next)[ra], r_new_b = as_global<const float>(T.rmax_next)[rb];
+    r_old = wrapped ? r_old_b : r_old_a;
+    r_new = wrapped ? r_new_b : r_new_a;
+#pragma unroll
+    for (int k = 0; k < N; k += 4) {
+      const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax), (col + k) * 4u, 0, 0);
+      const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax_next), (col + k) * 4u, 0, 0);
+      c_old.x[k] = bits2f(a.x); c_old.x[k + 1] = bits2f(a.y); c_old.x[k + 2] = bits2f(a.z); c_old.x[k + 3] = bits2f(a.w);
+      c_new.x[k] = bits2f(b.x); c_new.x[k + 1] = bits2f(b.y); c_new.x[k + 2] = bits2f(b.z); c_new.x[k + 3] = bits2f(b.w);
+    }
+  }
+
+  float p[N], g[N];
+  load_elems<PBF, N, FULL>(p_tile, e0, nv, p);
+  load_elems<GBF, N, FULL>(g_tile, e0, nv, g);
+  if (EXT) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) g[j] *= gscale;
+    if (zero_g) zero_elems<GBF, N, FULL>(const_cast<void *>(g_tile), e0, nv);
+  }
+  uint32_t mw = 0, vw = 0;
+  if (FULL) {
+    if (N == 4) {
+      mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), code_off, 0, kNt);
+      vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), code_off, 0, kNt);
+    } else {
+      mw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(m_tile), code_off, 0, kNt);
+      vw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_tile), code_off, 0, kNt);
+    }
+  } else {
+    const gptr<const uint8_t> mb = as_global<const uint8_t>(m_tile) + code_off;
+    const gptr<const uint8_t> vb = as_global<const uint8_t>(v_tile) + code_off;
+    const int nb = (nv + 1) >> 1;
+#pragma unroll
+    for (int k = 0; k < N / 2; ++k) {
+      if (k < nb) {
+        mw |= (uint32_t)mb[k] << (8 * k);
+        vw |= (uint32_t)vb[k] << (8 * k);
+      }
+    }
+  }
+  float sm_old = 0.0f, sv_old = 0.0f;
+  if (FULL) {
+    // scales are 4 bytes per block: cached, so that neighbouring blocks share lines
+    sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0));
+    if (!RANK1) sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0));
+  } else if (blk_ok) {
+    sm_old = as_global<const float>(sm_tile)[blk];
+    if (!RANK1) sv_old = as_global<const float>(sv_tile)[blk];
+  }
+  if (RANK1) sv_old = 1.0f;  // the table holds the bare code book; the scale follows per element
+  // this block's dequantization table: entry i = {code_book_m[i] * scale_m,
+  // code_book_v[i] * scale_v} (cuda_adamw_kernels.cu:340,343), written by the block's
+  // lanes (lane & 15 = i) into the wave's private LDS region
+  char *lds_bytes = reinterpret_cast<char *>(lds);
+  const uint32_t cb_entry = (uint32_t)wave * 64u + blk * 16u;  // entry number of code 0
+  *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) =
+      make_float2(slot.qm * sm_old, qmap_v(lane & 15) * sv_old);
+  setup_tables<SR>(lds, tid, slot);
+
+  // entry numbers of the lane's codes, one per byte: even elements, odd elements
+  const uint32_t three = 3u;
+  const uint32_t cb_bytes = cb_entry * 0x01010101u;
+  const uint32_t m_even = and_or(mw, 0x0F0F0F0Fu, cb_bytes), m_odd = and_or(mw >> 4, 0x0F0F0F0Fu, cb_bytes);
+  const uint32_t v_even = and_or(vw, 0x0F0F0F0Fu, cb_bytes), v_odd = and_or(vw >> 4, 0x0F0F0F0Fu, cb_bytes);
+
+  // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
+  Vals<N> mn, vn;
+  float am = 0.0f, av = 0.0f;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const uint32_t mo = entry_offset(j & 1 ? m_odd : m_even, j >> 1, three);
+    const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, three);
+    const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
+    float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
+    if constexpr (RANK1) v_old *= __builtin_fminf(r_old, c_old.x[j]);  // adamw_fourbit_triton.py:520-527
+    const float gj = g[j];
+    float m = sc.b1 * m_old + sc.r1 * gj;
+    float v = sc.b2 * v_old + sc.r2 * (gj * gj);
+    if (!FULL && j >= nv) { m = 0.0f; v = 0.0f; }
+    // parameter: only this part may use the hardware's 1-ulp sqrt and reciprocal
+    const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
+    p[j] = __builtin_fmaf(-m, __builtin_amdgcn_rcpf(den), p[j] * sc.wdu);
+    mn.x[j] = m;
+    vn.x[j] = v;
+    am = __builtin_fmaxf(am, __builtin_fabsf(m));
+    av = __builtin_fmaxf(av, v);
+  }
+  store_elems<PBF, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
+
+  // block scales (exact: max is order independent)
+  const float v_lane_max = av;
+  if (G::kLanesPerBlock == 32) {
+    block_max32_pair(am, av);
+  } else {
+    am = row_max16(am);
+    if (!RANK1) av = row_max16(av);
+  }
+  if (blk_ok && (lane & (G::kLanesPerBlock - 1)) == 0) {
+    if (FULL) {
+      __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), blk * 4u, 0, 0);
+      if (!RANK1) __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), blk * 4u, 0, 0);
+    } else {
+      as_global<float>(sm_tile)[blk] = am;
+      if (!RANK1) as_global<float>(sv_tile)[blk] = av;
+    }
+  }
+
+  // fast quantization: multiply by a refined reciprocal, decide every code whose
+  // quotient is clear of all thresholds, flag the rest
+  const bool safe_m = am >= kScaleLo && am <= kScaleHi;
+  const bool safe_v = RANK1 || (av >= kScaleLo && av <= kScaleHi);
+  const float rm = safe_m ? refined_rcp(am) : 0.0f;
+  const float rv16 = (safe_v && !RANK1) ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
+  bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
+  float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
+  // rank-1: the new scale of every element and 16 / scale.  The hardware reciprocal's
+  // one ulp is well inside the second moment's guard band (2^-17 in units of 16 q), so
+  // it goes unrefined.  Scales below the safe range are clamped for the reciprocal: a
+  // zero value under a zero scale then still gets code 0; any other value under such a
+  // scale sends the lane to the exact path.
+  Vals<N> s_new, inv16;
+  if constexpr (RANK1) {
+    float c_min = c_new.x[0];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float sj = __builtin_fminf(r_new, c_new.x[j]);   // adamw_fourbit_triton.py:749-755
+      s_new.x[j] = sj;
+      c_min = __builtin_fminf(c_min, c_new.x[j]);
+      inv16.x[j] = __builtin_amdgcn_rcpf(__builtin_fmaxf(sj, kScaleLo)) * 16.0f;
+    }
+    // every scale is at most r_new and at least min(r_new, c_min)
+    redo |= r_new > kScaleHi || (__builtin_fminf(r_new, c_min) < kScaleLo && v_lane_max != 0.0f);
+  }
+  uint32_t mword = 0, vword = 0;
+  Vals<N> um, uv;  // stochastic rounding: the elements' noise
+  if constexpr (SR) {
+    // key = low half of the element index, xor the salt, xor the mixed high half
+    const uint32_t tile_salt = salt ^ ((uint32_t)((uint64_t)tb >> 32) * 0x9E3779B9u);
+    const uint32_t first = (uint32_t)tb + e0;   // a tile never straddles a multiple of 2^32
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const uint32_t h = lowbias32((first + (uint32_t)j) ^ tile_salt);
+      um.x[j] = sr_noise_value(h >> 16);
+      uv.x[j] = sr_noise_value(h & 0xffffu);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < N; j += 2) {
+    // first moment: the quotients' bucket entries, two quotients per conversion
+    const float q0 = mn.x[j] * rm, q1 = mn.x[j + 1] * rm;
+    const uint32_t halves = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(q0, q1));
+    const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<1>(halves, three));
+    const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<3>(halves, three));
+    if constexpr (SR) {
+      // interval among the code-book entries, then up iff noise * width < q - lower end;
+      // a comparison closer than the quotient's error goes to the exact path
+      const float qq[2] = {q0, q1};
+      const uint2 ent[2] = {ent0, ent1};
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t k_raw = ent[h].y + (qq[h] >= bits2f(ent[h].x) ? 1u : 0u);
+        const uint2 iv = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsIntervals * 8u + k_raw * 8u);
+        const float d = qq[h] - bits2f(iv.x), t = um.x[j + h] * bits2f(iv.y);
+        redo |= __builtin_fabsf(t - d) <= __builtin_fabsf(qq[h]) * 4.76837158203125e-07f;  // 2^-21: 4 ulps
+        mword = __builtin_amdgcn_alignbit(k_raw - 1u + (t < d ? 1u : 0u), mword, 4);
+      }
+    } else {
+      const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
+      redo |= (hi0 != (q0 > bits2f(ent0.x))) | (hi1 != (q1 > bits2f(ent1.x)));
+      // base code in the entry's low nibble, plus one above the threshold; every
+      // code enters the word at the top and moves down four bits per later element
+      mword = __builtin_amdgcn_alignbit(ent0.x + (hi0 ? 1u : 0u), mword, 4);
+      mword = __builtin_amdgcn_alignbit(ent1.x + (hi1 ? 1u : 0u), mword, 4);
+    }
+
+    // second moment: thresholds at 16q = k + 0.5, k = 1..15
+#pragma unroll
+    for (int k = j; k < j + 2; ++k) {
+      if constexpr (SR) {
+        // code-book entries at 16 q = 1..16: interval number floor(16 q), position in
+        // it fract(16 q), up iff noise < position; the ends clamp
+        const float q16 = vn.x[k] * rv16;
+        const float kf = __builtin_floorf(q16), d16 = q16 - kf;
+        redo |= __builtin_fabsf(uv.x[k] - d16) <= kVGuard;
+        const float cf = __builtin_amdgcn_fmed3f(kf + (uv.x[k] < d16 ? 0.0f : -1.0f), 0.0f, 15.0f);
+        vword = __builtin_amdgcn_alignbit((uint32_t)(int)cf, vword, 4);
+      } else {
+        const float t = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, kVGuard - 0.5f);
+        vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
+        // t > -1, so truncation gives 0 for t < 0
+        vword = __builtin_amdgcn_alignbit((uint32_t)(int)t, vword, 4);
+      }
+    }
+  }
+  if (N == 4) {
+    mword >>= 16;
+    vword >>= 16;
+  }
+  redo |= vfrac < 2.0f * kVGuard;
+  if (__builtin_expect(redo, 0)) {
+    if constexpr (SR) {
+      mword = quantize_exact_sr<false, N>(mn, am, um);
+      vword = quantize_exact_sr<true, N>(vn, av, uv);
+    } else {
+      mword = quantize_exact<false, N>(mn, am);
+      if constexpr (RANK1) vword = quantize_exact_scales<N>(vn, s_new);
+      else vword = quantize_exact<true, N>(vn, av);
+    }
+  }
+  if (am == 0.0f) mword = 0;  // 0/0: code 0 for the whole block
+  if (!FULL) {
+    const uint32_t keep = nv >= 8 ? 0xffffffffu : ((1u << (4 * nv)) - 1u);
+    mword &= keep;
+    vword &= keep;
+  }
+
+  if (FULL) {
+    if (N == 4) {
+      __builtin_amdgcn_raw_buffer_store_b16((uint16_t)mword, tile_rsrc(m_tile), code_off, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b16((uint16_t)vword, tile_rsrc(v_tile), code_off, 0, kNt);
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b32(mword, tile_rsrc(m_tile), code_off, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(vword, tile_rsrc(v_tile), code_off, 0, kNt);
+    }
+  } else {
+    const gptr<uint8_t> mb = as_global<uint8_t>(m_tile) + code_off;
+    const gptr<uint8_t> vb = as_global<uint8_t>(v_tile) + code_off;
+    const int nb = (nv + 1) >> 1;
+#pragma unroll
+    for (int k = 0; k < N / 2; ++k) {
+      if (k < nb) {
+        mb[k] = (uint8_t)(mword >> (8 * k));
+        vb[k] = (uint8_t)(vword >> (8 * k));
+      }
+    }
+  }
+}
+
+template <bool PBF, bool GBF, bool EXT, bool SR>
+__global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
+  using G = Geometry<PBF, GBF>;
+  __shared__ uint2 lds[kLdsEntries];
+  const int tid = threadIdx.x;
+  const TableSlot slot = request_table_slot<SR>(tid);
+  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  if (chunk >= args.nchunks) return;  // whole workgroup: the grid is padded to a multiple of 8
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;  // whole grid
+  const bool zero_g = EXT && args.go.zero != 0u;
+  const int t = find_tensor(args, chunk);
+  const TensorDesc &T = args.desc[t];
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
+  const int64_t begin = tile * G::kTile;
+  if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
+    setup_tables<SR>(lds, tid, slot);
+    return;
+  }
+  const uint32_t salt = SR ? args.sr_salt[t] : 0u;
+  if (begin + G::kTile <= T.numel)
+    process_tile<PBF, GBF, true, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+  else
+    process_tile<PBF, GBF, false, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+}
+
+// ---------------------------------------------------------------------------
+// rank-1 scaling of the second moment: statistics, update, commit
+// ---------------------------------------------------------------------------
+constexpr int kStatRows = 64;            // rows per workgroup of the statistics kernel
+constexpr int kStatColsPerWave = 512;    // 8 columns per lane
+constexpr int kStatCols = kStatColsPerWave * kWaves;
+
+// New second moments of a tile of kStatRows x kStatCols elements, reduced to row and
+// column maxima (get_variance_tensor_statistics, adamw_fourbit_triton.py:738-746).  The
+// arithmetic is the update kernel's, operation for operation, so the maxima are maxima
+// of exactly the values that kernel quantizes.  Every lane keeps 8 columns over the
+// tile's rows: one atomic per column per tile, one per row per wave.
+template <bool GBF, bool EXT>
+__global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
+  constexpr int kAhead = 4;  // rows whose loads are in flight together
+  // row maxima of each 16-lane quarter of each wave; reduced by the last phase
+  __shared__ uint32_t row_bits[kWaves * 4][kStatRows];
+  const uint32_t chunk = blockIdx.x;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const int t = find_tensor(args, chunk);
+  const auto &T = args.desc[t];
+  const uint32_t local = chunk - args.first_chunk[t];
+  const uint32_t groups = args.col_groups[t];
+  const uint32_t rg = local / groups, cg = local - rg * groups;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t col = (int64_t)cg * kStatCols + wave * kStatColsPerWave + lane * 8;
+  const bool active = col < T.cols;  // cols is a multiple of 8: all 8 columns or none
+  const int64_t row0 = (int64_t)rg * kStatRows;
+  const int nrows = (int)(row0 + kStatRows < T.rows ? kStatRows : T.rows - row0);
+  // lanes past the last column work on zeros: code 0 under a zero scale and a zero
+  // gradient give a zero second moment, which leaves every maximum alone
+  float c_old[8], c_max[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    c_old[k] = active ? as_global<const float>(T.cmax)[col + k] : 0.0f;
+    c_max[k] = 0.0f;
+  }
+  const uint32_t quarter = (uint32_t)wave * 4u + ((uint32_t)lane >> 4);
+  for (int r0 = 0; r0 < nrows; r0 += kAhead) {
+    // a group past the tile's last row repeats that row: maxima do not mind
+    u32x4 gw[kAhead][GBF ? 1 : 2];
+    uint32_t vw[kAhead];
+    float r_old[kAhead];
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      const int r = r0 + i < nrows ? r0 + i : nrows - 1;
+      const int64_t row = row0 + r;
+      r_old[i] = as_global<const float>(T.rmax)[row];
+      // row bases are uniform; the lane's column is a 32-bit offset
+      const int64_t row_first = row * T.cols + ((int64_t)cg * kStatCols + wave * kStatColsPerWave);
+      const uint32_t lane_elem = (uint32_t)lane * 8u;
+      const void *g_row = static_cast<const char *>(T.g) + row_first * (GBF ? 2 : 4);
+      const void *v_row = T.v + (row_first >> 1);
+      vw[i] = 0u;
+#pragma unroll
+      for (int h = 0; h < (GBF ? 1 : 2); ++h) gw[i][h] = u32x4{0u, 0u, 0u, 0u};
+      if (active) {
+        vw[i] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_row), lane_elem >> 1, 0, kNtReadOnly);
+        if (GBF) {
+          gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 2u, 0, kNtReadOnly);
+        } else {
+          gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u, 0, kNtReadOnly);
+          gw[i][GBF ? 0 : 1] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u + 16u, 0, kNtReadOnly);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      float g[8];
+      if (GBF) {
+        widen_bf16_pair(gw[i][0].x, g[0], g[1]);
+        widen_bf16_pair(gw[i][0].y, g[2], g[3]);
+        widen_bf16_pair(gw[i][0].z, g[4], g[5]);
+        widen_bf16_pair(gw[i][0].w, g[6], g[7]);
+      } else {
+        const u32x4 lo = gw[i][0], hi = gw[i][GBF ? 0 : 1];
+        g[0] = bits2f(lo.x); g[1] = bits2f(lo.y); g[2] = bits2f(lo.z); g[3] = bits2f(lo.w);
+        g[4] = bits2f(hi.x); g[5] = bits2f(hi.y); g[6] = bits2f(hi.z); g[7] = bits2f(hi.w);
+      }
+      const uint32_t even = vw[i] & 0x0F0F0F0Fu, odd = (vw[i] >> 4) & 0x0F0F0F0Fu;  // one code per byte
+      float r_max = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float gk = EXT ? g[k] * gscale : g[k];
+        const uint32_t code = ((k & 1 ? odd : even) >> (8 * (k >> 1))) & 0xffu;
+        const float code_value = __builtin_fmaf((float)code, 0.0625f, 0.0625f);  // (code + 1) / 16, exact
+        const float v_old = code_value * __builtin_fminf(r_old[i], c_old[k]);
+        const float v = args.b2 * v_old + args.r2 * (gk * gk);
+        c_max[k] = __builtin_fmaxf(c_max[k], v);
+        r_max = __builtin_fmaxf(r_max, v);
+      }
+      uint32_t u = f2bits(r_max);
+      u = dpp_umax<0xB1>(u);
+      u = dpp_umax<0x4E>(u);
+      u = dpp_umax<0x141>(u);
+      u = dpp_umax<0x140>(u);           // maximum of each 16-lane quarter, in all its lanes
+      if ((lane & 15) == 0) row_bits[quarter][r0 + i] = u;   // slots past nrows are not read
+    }
+  }
+  if (active) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
+  }
+  __syncthreads();
+  if (tid < nrows) {
+    uint32_t u = 0u;
+#pragma unroll
+    for (int qi = 0; qi < kWaves * 4; ++qi) u = u > row_bits[qi][tid] ? u : row_bits[qi][tid];
+    if (u != 0u) atomic_max_nonneg(T.rmax_next + row0 + tid, bits2f(u));
+  }
+}
+
+template <bool PBF, bool GBF, bool EXT>
+__global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
+  using G = Geometry<PBF, GBF>;
+  __shared__ uint2 lds[kLdsEntries];
+  const int tid = threadIdx.x;
+  const TableSlot slot = request_table_slot<false>(tid);
+  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  if (chunk >= args.nchunks) return;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const bool zero_g = EXT && args.go.zero != 0u;
+  const int t = find_tensor(args, chunk);
+  const Rank1Desc &T = args.desc[t];
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
+  const int64_t begin = tile * G::kTile;
+  if (begin >= T.numel) {
+    setup_tables<false>(lds, tid, slot);
+    return;
+  }
+  if (begin + G::kTile <= T.numel)
+    process_tile<PBF, GBF, true, EXT, true, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, 0u);
+  else
+    process_tile<PBF, GBF, false, EXT, true, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, 0u);
+}
+
+// After the update: the new statistics become the current ones and the buffers that
+// received them go back to zero for the next step's maxima.  One workgroup column per
+// tensor (blockIdx.y), grid-stride over rows + cols floats.
+__global__ __launch_bounds__(256) void rank1_commit_kernel(const Rank1Args args) {
+  float gscale;
+  if (!grad_ops_begin(args.go, gscale)) return;
+  const Rank1Desc &T = args.desc[blockIdx.y];
+  const int64_t total = T.rows + T.cols;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const bool is_row = i < T.rows;
+    const gptr<float> cur = as_global<float>(is_row ? T.rmax : T.cmax) + (is_row ? i : i - T.rows);
+    const gptr<float> next = as_global<float>(is_row ? T.rmax_next : T.cmax_next) + (is_row ? i : i - T.rows);
+    *cur = *next;
+    *next = 0.0f;
+  }
+}
+
+}  // namespace q4
