@@ -26,8 +26,9 @@
  * Pinning status (what nails each function down besides this file itself):
  *   tables              : fp32 bit patterns checked against a committed KAT and
  *                         against closed forms (k/16, (2k+1)/32, decade means)
- *   q4o_quantize_search : checked against q4o_quantize_count, numpy.searchsorted
- *                         and hand-placed tie / boundary cases
+ *   q4o_quantize_search : checked against q4o_quantize_count on every one of the 2^32
+ *                         fp32 bit patterns (q4o_exhaustive_search_vs_count),
+ *                         numpy.searchsorted and hand-placed tie / boundary cases
  *   q4o_derive_scalars  : KAT for (0.9, 0.999, 1e-3, 0.01) and double-precision
  *                         closed forms
  *   q4o_step_unquant    : torch.optim.AdamW (library routine) to fp32 round-off
@@ -103,6 +104,48 @@ int q4o_quantize_count(int which, float x) {
     int c = 0;
     for (int j = 0; j < 15; ++j) c += (qmid[j] < x);
     return c;
+}
+
+/*
+ * Exhaustive check of the closed form against the search over EVERY fp32 bit pattern
+ * (all 2^32, NaN and infinities included): returns the number of patterns on which
+ * q4o_quantize_search and q4o_quantize_count disagree, and stores in first_bad the
+ * lowest such pattern.  Also counts, in *steps, the patterns where the code differs
+ * from the code of the next pattern up the number line (must be 15 for finite values:
+ * the map is a non-decreasing staircase with 15 steps).
+ */
+int64_t q4o_exhaustive_search_vs_count(int which, uint32_t *first_bad, int64_t *steps) {
+    int64_t bad = 0, nsteps = 0;
+    uint32_t first = 0xffffffffu;
+#pragma omp parallel for schedule(static) reduction(+ : bad, nsteps) reduction(min : first)
+    for (int64_t b = 0; b < ((int64_t)1 << 32); ++b) {
+        const uint32_t u = (uint32_t)b;
+        float x;
+        memcpy(&x, &u, 4);
+        const int cs = q4o_quantize_search(which, x);
+        /* the search sends NaN to 0 explicitly; the count does so because no comparison
+         * with NaN is true */
+        const int cc = q4o_quantize_count(which, x);
+        if (cs != cc) {
+            ++bad;
+            if (u < first) first = u;
+        }
+        /* neighbour one ulp up in value: positive patterns b -> b + 1, negative
+         * patterns b -> b - 1; skip infinities, NaN and the step from -0 to +0 */
+        const uint32_t mag = u & 0x7fffffffu;
+        if (mag < 0x7f800000u - 1u || (mag == 0x7f800000u - 1u && (u >> 31))) {
+            uint32_t un = (u >> 31) ? (mag == 0 ? 0u : u - 1u) : u + 1u;
+            float y;
+            memcpy(&y, &un, 4);
+            if (y == y && q4o_quantize_count(which, y) != cc) {
+                if (q4o_quantize_count(which, y) != cc + 1) ++bad;   /* never jumps by more than one */
+                ++nsteps;
+            }
+        }
+    }
+    *first_bad = first;
+    *steps = nsteps;
+    return bad;
 }
 
 /*
