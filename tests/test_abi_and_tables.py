@@ -279,3 +279,20 @@ def test_fast_path_model_second_moment():
     q = rng.uniform(0, 1, 200000).astype(np.float32)
     t = _rn32(q.astype(np.float64) * 16 + np.float64(w - np.float32(0.5)))
     assert ((t - np.floor(t)) < 2 * w).mean() < 1e-3
+
+
+def test_tables_exhaustively_on_the_host(tmp_path):
+    """tests/native/check_tables.cpp walks every fp32 bit pattern in [-1, 1] (2.1e9 of them) through
+    the constexpr tables of csrc/q4adamw_tables.h: decided codes are exact for every value
+    within the quotient's error, and the stochastic-rounding interval numbers are exact"""
+    import shutil
+    import subprocess
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no g++")
+    exe = str(tmp_path / "check_tables")
+    subprocess.check_call([gxx, "-O2", "-std=c++17", "-fopenmp", "-o", exe,
+                           os.path.join(ROOT, "tests", "native", "check_tables.cpp")])
+    out = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=600)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout
+    assert "0 wrong" in out.stdout
