@@ -394,6 +394,19 @@ __device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale)
   return true;
 }
 
+// Minimum and maximum of non-negative, non-NaN floats (scales, maxima) through their bit
+// patterns: one integer instruction each, where fminf / fmaxf on loaded values would
+// first canonicalise both operands.
+__device__ __forceinline__ float min_nonneg(float a, float b) {
+  const uint32_t x = f2bits(a), y = f2bits(b);
+  return bits2f(x < y ? x : y);
+}
+
+__device__ __forceinline__ float max_nonneg(float a, float b) {
+  const uint32_t x = f2bits(a), y = f2bits(b);
+  return bits2f(x > y ? x : y);
+}
+
 // Atomic maximum of non-negative floats through their bit patterns.
 __device__ __forceinline__ void atomic_max_nonneg(const float *addr, float x) {
   // non-negative floats order like their bit patterns

@@ -148,7 +148,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, three);
     const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
     float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
-    if constexpr (RANK1) v_old *= __builtin_fminf(r_old, c_old.x[j]);  // adamw_fourbit_triton.py:520-527
+    if constexpr (RANK1) v_old *= min_nonneg(r_old, c_old.x[j]);  // adamw_fourbit_triton.py:520-527
     const float gj = g[j];
     float m = sc.b1 * m_old + sc.r1 * gj;
     float v = sc.b2 * v_old + sc.r2 * (gj * gj);
@@ -199,13 +199,13 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     float c_min = c_new.x[0];
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      const float sj = __builtin_fminf(r_new, c_new.x[j]);   // adamw_fourbit_triton.py:749-755
+      const float sj = min_nonneg(r_new, c_new.x[j]);        // adamw_fourbit_triton.py:749-755
       s_new.x[j] = sj;
-      c_min = __builtin_fminf(c_min, c_new.x[j]);
-      inv16.x[j] = __builtin_amdgcn_rcpf(__builtin_fmaxf(sj, kScaleLo)) * 16.0f;
+      c_min = min_nonneg(c_min, c_new.x[j]);
+      inv16.x[j] = __builtin_amdgcn_rcpf(max_nonneg(sj, kScaleLo)) * 16.0f;
     }
     // every scale is at most r_new and at least min(r_new, c_min)
-    redo |= r_new > kScaleHi || (__builtin_fminf(r_new, c_min) < kScaleLo && v_lane_max != 0.0f);
+    redo |= r_new > kScaleHi || (min_nonneg(r_new, c_min) < kScaleLo && v_lane_max != 0.0f);
   }
   uint32_t mword = 0, vword = 0;
   Vals<N> um, uv;  // stochastic rounding: the elements' noise
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
         const float gk = EXT ? g[k] * gscale : g[k];
         const uint32_t code = ((k & 1 ? odd : even) >> (8 * (k >> 1))) & 0xffu;
         const float code_value = __builtin_fmaf((float)code, 0.0625f, 0.0625f);  // (code + 1) / 16, exact
-        const float v_old = code_value * __builtin_fminf(r_old[i], c_old[k]);
+        const float v_old = code_value * min_nonneg(r_old[i], c_old[k]);
         const float v = args.b2 * v_old + args.r2 * (gk * gk);
         c_max[k] = __builtin_fmaxf(c_max[k], v);
         r_max = __builtin_fmaxf(r_max, v);
