@@ -1,0 +1,107 @@
+"""Seeded sweep over sizes, dtypes, hyper-parameters, step numbers and gradient magnitudes:
+the HIP step against the C oracle (block-scaled path) on configurations no hand-written test
+names.  Deterministic: every case derives from its index."""
+import numpy as np
+import pytest
+import torch
+
+import quantfour_adamw_cuda_amd as q4
+from tests.q4_testlib import DeviceTensor, OracleTensor, assert_state_equal
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [(torch.float32, torch.float32), (torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16),
+          (torch.bfloat16, torch.float32)]
+
+
+def _case(i):
+    rng = np.random.default_rng(1000 + i)
+    n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 5000), rng.integers(5000, 400000)]))
+    p_dt, g_dt = DTYPES[i % 4]
+    hp = dict(beta1=float(rng.choice([0.5, 0.8, 0.9, 0.95, 0.99])),
+              beta2=float(rng.choice([0.88, 0.95, 0.99, 0.999, 0.9999])),
+              lr=float(10.0 ** rng.uniform(-6, -1)), weight_decay=float(rng.choice([0.0, 1e-4, 0.01, 0.1, 0.5])),
+              eps=float(rng.choice([1e-12, 1e-8, 1e-6, 1e-3])))
+    first_step = int(rng.choice([1, 2, 10, 1000, 100000]))
+    g_scale = float(10.0 ** rng.uniform(-9, 3))
+    return rng, n, p_dt, g_dt, hp, first_step, g_scale
+
+
+@pytest.mark.parametrize("i", range(48))
+def test_random_configuration(cuda, i):
+    rng, n, p_dt, g_dt, hp, first_step, g_scale = _case(i)
+    print(f"[sweep {i}] n={n} p={p_dt} g={g_dt} hp={hp} step0={first_step} g_scale={g_scale:.3g}", flush=True)
+    p0 = torch.from_numpy((rng.standard_normal(n) * 10.0 ** rng.uniform(-4, 1)).astype(np.float32)).to(p_dt)
+    dev, ref = DeviceTensor(p0, cuda), OracleTensor(p0)
+    for k in range(3):
+        g = rng.standard_normal(n).astype(np.float32) * np.float32(g_scale)
+        u = rng.uniform(size=n)
+        g[u < 0.1] = 0.0
+        g[u > 0.999] *= np.float32(1e3)
+        if k == 1:
+            g[: n // 2] = 0.0                      # long runs of zero blocks
+        g = torch.from_numpy(g).to(g_dt)
+        step = first_step + k
+        q4.fused_4bit(dev.p, g.to(cuda), dev.m, dev.v, dev.sm, dev.sv, hp["beta1"], hp["beta2"], hp["lr"],
+                      hp["weight_decay"], hp["eps"], step)
+        prev = ref.step(g, step, hp)
+        assert_state_equal(dev, ref, prev, f"sweep {i} step {step}")
+        ref.resync(dev.p)
+
+
+@pytest.mark.parametrize("i", range(16))
+def test_random_configuration_stochastic_rounding(cuda, i):
+    from oracle import q4_oracle_torch as ot
+    from quantfour_adamw_cuda_amd import quantfour_hip as q
+    from tests.q4_testlib import p_close, to_np
+    rng, n, p_dt, g_dt, hp, first_step, g_scale = _case(100 + i)
+    seed, salt = int(rng.integers(0, 2 ** 63)), int(rng.integers(0, 2 ** 32))
+    print(f"[sweep sr {i}] n={n} p={p_dt} g={g_dt} hp={hp} step0={first_step} seed={seed} salt={salt}", flush=True)
+    p0 = torch.from_numpy((rng.standard_normal(n) * 0.05).astype(np.float32)).to(p_dt)
+    dev = DeviceTensor(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.sv.cpu())
+    for k in range(2):
+        g = torch.from_numpy(rng.standard_normal(n).astype(np.float32) * np.float32(g_scale)).to(g_dt)
+        step = first_step + k
+        prev = ref[0]
+        ref = ot.step_quant_sr(ref[0], g, *ref[1:], seed=seed, tensor_salt=salt, step=step, **hp)
+        q.fused_4bit_multi_sr([dev.p], [g.to(cuda)], [dev.m], [dev.v], [dev.sm], [dev.sv], hp["beta1"], hp["beta2"],
+                              hp["lr"], hp["weight_decay"], hp["eps"], step, seed, salts=[salt])
+        assert torch.equal(dev.m.cpu(), ref[1]) and torch.equal(dev.v.cpu(), ref[2]), f"sr sweep {i} step {step}: codes"
+        assert torch.equal(dev.sm.cpu().view(torch.int32), ref[3].view(torch.int32))
+        assert torch.equal(dev.sv.cpu().view(torch.int32), ref[4].view(torch.int32))
+        ok, worst = p_close(to_np(dev.p), to_np(ref[0]), to_np(prev), bf16=p_dt == torch.bfloat16)
+        assert ok, f"sr sweep {i} step {step}: parameters (worst {worst})"
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
+
+
+@pytest.mark.parametrize("i", range(16))
+def test_random_configuration_rank1(cuda, i):
+    from oracle import q4_oracle_torch as ot
+    from quantfour_adamw_cuda_amd import quantfour_hip as q
+    from tests.q4_testlib import p_close, to_np
+    rng, _, p_dt, g_dt, hp, first_step, g_scale = _case(200 + i)
+    rows, cols = int(rng.integers(1, 90)), 512 + 8 * int(rng.integers(0, 200))
+    print(f"[sweep rank1 {i}] {rows}x{cols} p={p_dt} g={g_dt} hp={hp} step0={first_step}", flush=True)
+    n = rows * cols
+    p0 = torch.from_numpy((rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)).to(p_dt)
+    z = lambda k, dt=torch.float32: torch.zeros(k, dtype=dt, device=cuda)
+    p, m, v, sm = p0.clone().to(cuda), z((n + 1) // 2, torch.uint8), z((n + 1) // 2, torch.uint8), z((n + 127) // 128)
+    r, c, rn, cn = z(rows), z(cols), z(rows), z(cols)
+    ref = (p0.clone(), m.cpu(), v.cpu(), sm.cpu(), r.cpu(), c.cpu())
+    for k in range(2):
+        g = rng.standard_normal((rows, cols)).astype(np.float32) * np.float32(g_scale)
+        g *= rng.uniform(0.01, 1.0, (rows, 1)).astype(np.float32) * rng.uniform(0.01, 1.0, (1, cols)).astype(np.float32)
+        g = torch.from_numpy(g).to(g_dt)
+        step = first_step + k
+        prev = ref[0]
+        ref = ot.step_quant_rank1(ref[0], g, *ref[1:], step=step, **hp)
+        q.fused_4bit_rank1_multi([p], [g.to(cuda)], [m], [v], [sm], [r], [c], [rn], [cn], hp["beta1"], hp["beta2"],
+                                 hp["lr"], hp["weight_decay"], hp["eps"], step)
+        for name, d, x in (("m", m, ref[1]), ("v", v, ref[2])):
+            assert torch.equal(d.cpu(), x), f"rank1 sweep {i} step {step}: {name} codes"
+        for name, d, x in (("sm", sm, ref[3]), ("r", r, ref[4]), ("c", c, ref[5])):
+            assert torch.equal(d.cpu().view(torch.int32), x.view(torch.int32)), f"rank1 sweep {i} step {step}: {name}"
+        ok, worst = p_close(to_np(p), to_np(ref[0]), to_np(prev), bf16=p_dt == torch.bfloat16)
+        assert ok, f"rank1 sweep {i} step {step}: parameters (worst {worst})"
+        ref = (p.cpu().clone(),) + tuple(ref[1:])
