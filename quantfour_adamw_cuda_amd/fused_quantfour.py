@@ -142,6 +142,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self.__dict__.setdefault("kernel_timing", None)
         self.__dict__.setdefault("last_grad_norm", None)
         self.__dict__.setdefault("variance_scale_type", "group")
+        self.__dict__.pop("_pending_skip", None)
+        self.__dict__.pop("_skip_flag_host", None)
         for group in self.param_groups:
             group.setdefault("fused", None)
             group.setdefault("round_type", "real-nearest")
@@ -399,7 +401,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                        the norm is left in `last_grad_norm` (a device scalar)
         found_inf      one-element float32 device tensor: a non-zero value makes the
                        step a no-op on the device, without synchronising; the step
-                       counters advance regardless
+                       counters of a skipped step are taken back when the next step
+                       (or state_dict()) looks at the flag's value, which by then has
+                       reached the host
         zero_grad      overwrite the gradients with zeros once the step has read them
         """
         loss = None
@@ -407,11 +411,13 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             with torch.enable_grad():
                 loss = closure()
 
+        self._settle_skipped_step()
         if found_inf is None:
             found_inf = getattr(self, "found_inf", None)    # set by GradScaler
         if found_inf is not None:
             found_inf = found_inf.detach().to(torch.float32).reshape(1)
         host_mult, dev_mult = self._grad_multiplier(grad_scale, max_grad_norm)
+        stepped = []   # step counters advanced by this call
 
         _lib.load()  # raises if the HIP library has not been built
 
@@ -448,6 +454,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             # update step (optim/fused_quantfour.py:178)
             torch._foreach_add_(state_steps, 1)
             steps = torch.stack(state_steps).tolist()
+            stepped.extend(state_steps)
 
             # one launch per (kind, device, dtypes, step)
             buckets: Dict[Any, list] = {}
@@ -525,4 +532,36 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                             "fused_4bit" if quantized else "fused_single_tensor")   # "sr" counts as fused_4bit
                     self.kernel_timing.append((kind, start, end))
 
+        if found_inf is not None and stepped:
+            self._watch_skip_flag(found_inf, stepped)
         return loss
+
+    # -- overflow flag: keeping the step counters right without a synchronisation -----
+    def _watch_skip_flag(self, found_inf, stepped):
+        """Starts an asynchronous copy of the flag to pinned host memory; an event marks its
+        arrival.  The next step() or state_dict() reads it."""
+        host = self.__dict__.get("_skip_flag_host")
+        if host is None:
+            host = torch.empty(1, dtype=torch.float32, pin_memory=True)
+            self._skip_flag_host = host
+        with torch.cuda.device(found_inf.device):
+            host.copy_(found_inf, non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+        self._pending_skip = (arrived, stepped)
+
+    def _settle_skipped_step(self):
+        """If the previous step ran under an overflow flag that turned out set, the device did
+        nothing: take its advance of the step counters back.  Waits for that step's flag
+        only (it has long arrived when the next step begins)."""
+        pending = self.__dict__.pop("_pending_skip", None)
+        if pending is None:
+            return
+        arrived, stepped = pending
+        arrived.synchronize()
+        if float(self._skip_flag_host[0]) != 0.0:
+            torch._foreach_sub_(stepped, 1)
+
+    def state_dict(self):
+        self._settle_skipped_step()
+        return super().state_dict()

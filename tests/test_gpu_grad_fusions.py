@@ -287,6 +287,19 @@ def test_grad_scaler_drives_the_fused_path(cuda):
     scaler.update()
     assert all(torch.equal(p, q0) for p, q0 in zip(m.parameters(), before))
     assert scaler.get_scale() == s0 * 0.5
+    # the skipped step does not count: state_dict() (and the next step) take its advance back
+    assert all(float(st["step"]) == 3.0 for st in opt.state_dict()["state"].values())
+    opt.zero_grad(set_to_none=True)
+    ref.zero_grad(set_to_none=True)
+    x = torch.randn(16, 96, device=cuda)
+    scaler.scale(m(x).square().mean()).backward()
+    scaler.step(opt)
+    scaler.update()
+    ref(x).square().mean().backward()
+    ropt.step()
+    assert all(float(st["step"]) == 4.0 for st in opt.state.values())
+    for pa, pb in zip(m.parameters(), ref.parameters()):
+        assert torch.equal(pa, pb)       # same bias corrections as the run that never overflowed
 
 
 def test_clip_pipeline_and_rank1_replay_under_graph_capture(cuda):
