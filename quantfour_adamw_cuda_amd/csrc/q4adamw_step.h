@@ -342,20 +342,23 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
 // ---------------------------------------------------------------------------
 // rank-1 scaling of the second moment: statistics, update, commit
 // ---------------------------------------------------------------------------
-constexpr int kStatRows = 64;            // rows per workgroup of the statistics kernel
-constexpr int kStatColsPerWave = 512;    // 8 columns per lane
-constexpr int kStatCols = kStatColsPerWave * kWaves;
+constexpr int kStatRowsPerWave = 64;     // rows a wave walks
+constexpr int kStatRows = kStatRowsPerWave * kWaves;   // rows per workgroup of the statistics kernel
+constexpr int kStatCols = 512;           // columns per workgroup: 8 per lane
 
 // New second moments of a tile of kStatRows x kStatCols elements, reduced to row and
 // column maxima (get_variance_tensor_statistics, adamw_fourbit_triton.py:738-746).  The
 // arithmetic is the update kernel's, operation for operation, so the maxima are maxima
-// of exactly the values that kernel quantizes.  Every lane keeps 8 columns over the
-// tile's rows: one atomic per column per tile, one per row per wave.
+// of exactly the values that kernel quantizes.  The four waves of a workgroup share the
+// columns and split the rows: every lane keeps 8 columns over its wave's rows, the waves'
+// column maxima meet in LDS, and the tile issues one atomic per column and one per row
+// (atomics on the column vector are what this kernel's time depends on most: a tile of
+// 64 rows with four times as many of them took 1.25 to 2 times as long).
 template <bool GBF, bool EXT>
 __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
   constexpr int kAhead = 4;  // rows whose loads are in flight together
-  // row maxima of each 16-lane quarter of each wave; reduced by the last phase
-  __shared__ uint32_t row_bits[kWaves * 4][kStatRows];
+  __shared__ uint32_t row_bits[4][kStatRows];       // row maxima of each 16-lane quarter of the row's wave
+  __shared__ uint32_t col_bits[kWaves][kStatCols];  // column maxima of each wave
   const uint32_t chunk = blockIdx.x;
   float gscale = 1.0f;
   if (EXT && !grad_ops_begin(args.go, gscale)) return;
@@ -366,10 +369,13 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   const uint32_t rg = local / groups, cg = local - rg * groups;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int64_t col = (int64_t)cg * kStatCols + wave * kStatColsPerWave + lane * 8;
+  const int64_t col = (int64_t)cg * kStatCols + lane * 8;
   const bool active = col < T.cols;  // cols is a multiple of 8: all 8 columns or none
-  const int64_t row0 = (int64_t)rg * kStatRows;
-  const int nrows = (int)(row0 + kStatRows < T.rows ? kStatRows : T.rows - row0);
+  const int64_t tile_row0 = (int64_t)rg * kStatRows;
+  const int tile_rows = (int)(tile_row0 + kStatRows < T.rows ? kStatRows : T.rows - tile_row0);
+  const int wave_row0 = wave * kStatRowsPerWave;                         // within the tile
+  int nrows = tile_rows - wave_row0;                                      // rows of this wave
+  nrows = nrows < 0 ? 0 : (nrows > kStatRowsPerWave ? kStatRowsPerWave : nrows);
   // lanes past the last column work on zeros: code 0 under a zero scale and a zero
   // gradient give a zero second moment, which leaves every maximum alone
   float c_old[8], c_max[8];
@@ -378,19 +384,19 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
     c_old[k] = active ? as_global<const float>(T.cmax)[col + k] : 0.0f;
     c_max[k] = 0.0f;
   }
-  const uint32_t quarter = (uint32_t)wave * 4u + ((uint32_t)lane >> 4);
+  const uint32_t quarter = (uint32_t)lane >> 4;
   for (int r0 = 0; r0 < nrows; r0 += kAhead) {
-    // a group past the tile's last row repeats that row: maxima do not mind
+    // a group past the wave's last row repeats that row: maxima do not mind
     u32x4 gw[kAhead][GBF ? 1 : 2];
     uint32_t vw[kAhead];
     float r_old[kAhead];
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) {
       const int r = r0 + i < nrows ? r0 + i : nrows - 1;
-      const int64_t row = row0 + r;
+      const int64_t row = tile_row0 + wave_row0 + r;
       r_old[i] = as_global<const float>(T.rmax)[row];
       // row bases are uniform; the lane's column is a 32-bit offset
-      const int64_t row_first = row * T.cols + ((int64_t)cg * kStatCols + wave * kStatColsPerWave);
+      const int64_t row_first = row * T.cols + (int64_t)cg * kStatCols;
       const uint32_t lane_elem = (uint32_t)lane * 8u;
       const void *g_row = static_cast<const char *>(T.g) + row_first * (GBF ? 2 : 4);
       const void *v_row = T.v + (row_first >> 1);
@@ -437,20 +443,31 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
       u = dpp_umax<0x4E>(u);
       u = dpp_umax<0x141>(u);
       u = dpp_umax<0x140>(u);           // maximum of each 16-lane quarter, in all its lanes
-      if ((lane & 15) == 0) row_bits[quarter][r0 + i] = u;   // slots past nrows are not read
+      if ((lane & 15) == 0) row_bits[quarter][wave_row0 + r0 + i] = u;   // slots past the last row are not read
     }
   }
-  if (active) {
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
-      if (c_max[k] != 0.0f) atomic_max_nonneg(T.cmax_next + col + k, c_max[k]);
-  }
+  for (int k = 0; k < 8; ++k) col_bits[wave][lane * 8 + k] = f2bits(c_max[k]);
   __syncthreads();
-  if (tid < nrows) {
-    uint32_t u = 0u;
+  // one atomic per column and per row of the tile
 #pragma unroll
-    for (int qi = 0; qi < kWaves * 4; ++qi) u = u > row_bits[qi][tid] ? u : row_bits[qi][tid];
-    if (u != 0u) atomic_max_nonneg(T.rmax_next + row0 + tid, bits2f(u));
+  for (int h = 0; h < kStatCols / kThreads; ++h) {
+    const int c = tid + h * kThreads;
+    uint32_t u = col_bits[0][c];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) u = u > col_bits[w][c] ? u : col_bits[w][c];
+    const int64_t cc = (int64_t)cg * kStatCols + c;
+    if (cc < T.cols && u != 0u) atomic_max_nonneg(T.cmax_next + cc, bits2f(u));
+  }
+#pragma unroll
+  for (int h = 0; h < kStatRows / kThreads; ++h) {
+    const int r = tid + h * kThreads;
+    if (r < tile_rows) {
+      uint32_t u = row_bits[0][r];
+#pragma unroll
+      for (int qi = 1; qi < 4; ++qi) u = u > row_bits[qi][r] ? u : row_bits[qi][r];
+      if (u != 0u) atomic_max_nonneg(T.rmax_next + tile_row0 + r, bits2f(u));
+    }
   }
 }
 
