@@ -87,9 +87,12 @@ typedef struct q4adamw_small_tensor {
  *                    1 / loss scale, a clip coefficient, q4adamw_grad_norm's
  *                    out3[2]) or NULL.
  *   skip_if_nonzero  device fp32 scalar or NULL: when it holds a non-zero value
- *                    (an overflow flag) the call changes nothing.
+ *                    (an overflow flag) the call leaves parameters and optimizer
+ *                    state as they are.
  *   zero_grad        non-zero: the gradients are overwritten with zeros once read
- *                    (the `g` pointers are written in that case).
+ *                    (the `g` pointers are written in that case), also by a call
+ *                    that skip_if_nonzero cancels: the overflowed gradients must
+ *                    not reach the next accumulation.
  * The device scalars are read when the kernels run, not when the call returns.
  */
 typedef struct q4adamw_grad_options {

@@ -306,7 +306,7 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
     if (!aligned(t.exp_avg, code_align) || !aligned(t.exp_avg_sq, code_align) ||
         !aligned(t.exp_avg_scale, 4) || !aligned(t.exp_avg_sq_scale, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "code and scale buffers must be 4-byte aligned");
-    if ((uint64_t)(t.numel + chunk_elems - 1) / chunk_elems > kMaxChunksPerLaunch)
+    if (((uint64_t)t.numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -316,7 +316,7 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   for (int i = 0; i < count; ++i) {
     const q4adamw_tensor &t = tensors[i];
     if (t.numel == 0) continue;
-    const uint64_t c = (uint64_t)(t.numel + chunk_elems - 1) / chunk_elems;
+    const uint64_t c = ((uint64_t)t.numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
     if (a.ntensors == kMaxTensors || chunks + c > kMaxChunksPerLaunch) {
       if (int rc = launch_fused_batch(a, chunks, kernel, s)) return rc;
       a.ntensors = 0;
@@ -410,7 +410,7 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
     const q4adamw_rank1_tensor &t = tensors[i];
     if (t.rows == 0 || t.cols == 0) continue;
     const int64_t numel = t.rows * t.cols;
-    const uint64_t c = (uint64_t)(numel + chunk_elems - 1) / chunk_elems;
+    const uint64_t c = ((uint64_t)numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
     const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
     const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
     if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
@@ -488,7 +488,7 @@ int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, in
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
     if (!aligned(t.p, pa) || !aligned(t.g, ga) || !aligned(t.exp_avg, 4) || !aligned(t.exp_avg_sq, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "tensor not aligned to its element size");
-    if ((uint64_t)(t.numel + kSmallChunk - 1) / kSmallChunk > kMaxChunksPerLaunch)
+    if (((uint64_t)t.numel + (uint64_t)kSmallChunk - 1) / (uint64_t)kSmallChunk > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -498,7 +498,7 @@ int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, in
   for (int i = 0; i < count; ++i) {
     const q4adamw_small_tensor &t = tensors[i];
     if (t.numel == 0) continue;
-    const uint64_t c = (uint64_t)(t.numel + kSmallChunk - 1) / kSmallChunk;
+    const uint64_t c = ((uint64_t)t.numel + (uint64_t)kSmallChunk - 1) / (uint64_t)kSmallChunk;
     if (a.ntensors == kMaxSmallTensors || chunks + c > kMaxChunksPerLaunch) {
       if (int rc = launch_small_batch(a, chunks, kernel, s)) return rc;
       a.ntensors = 0;
@@ -544,7 +544,7 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
     if (grads[i].numel == 0) continue;
     if (!grads[i].g) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
     if (!aligned(grads[i].g, 16)) return fail(Q4ADAMW_ERR_ALIGN, "gradients must be 16-byte aligned");
-    if ((uint64_t)(grads[i].numel + chunk_elems - 1) / chunk_elems > kMaxChunksPerLaunch)
+    if (((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -566,7 +566,7 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
   };
   for (int i = 0; i < count; ++i) {
     if (grads[i].numel == 0) continue;
-    const uint64_t c = (uint64_t)(grads[i].numel + chunk_elems - 1) / chunk_elems;
+    const uint64_t c = ((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
     if (a.ntensors == kMaxNormTensors || chunks + c > kMaxChunksPerLaunch) {
       if (int rc = launch()) return rc;
     }
@@ -592,7 +592,7 @@ int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, f
   if (numel == 0) return 0;
   if (!x || !codes || !scales) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(x, 4) || !aligned(scales, 4)) return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t blocks = (uint64_t)(numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
+  const uint64_t blocks = ((uint64_t)numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
   const uint64_t grid = (blocks + 3) / 4;
   if (grid > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -617,11 +617,11 @@ int q4adamw_quantize_rank1(const float *x, int64_t rows, int64_t cols, uint8_t *
   if (!x || !codes || !row_max || !col_max) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(x, 4) || !aligned(row_max, 4) || !aligned(col_max, 4))
     return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
+  const dim3 tiles((unsigned)((cols + 255) / 256), (unsigned)((rows + 63) / 64));
+  if (tiles.y > 65535u) return fail(Q4ADAMW_ERR_TOO_LARGE, "more than 4194240 rows");
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, row_max, rows);
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, col_max, cols);
-  const dim3 tiles((unsigned)((cols + 255) / 256), (unsigned)((rows + 63) / 64));
-  if (tiles.y > 65535u) return fail(Q4ADAMW_ERR_TOO_LARGE, "more than 4194240 rows");
   hipLaunchKernelGGL(rank1_absmax_kernel, tiles, dim3(256), 0, s, x, rows, cols, row_max, col_max);
   const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
   hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, rows, cols,
@@ -650,7 +650,7 @@ int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel,
   if (numel == 0) return 0;
   if (!out || !codes || !scales) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(out, 4) || !aligned(scales, 4)) return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t grid = ((uint64_t)(numel + 1) / 2 + 255) / 256;
+  const uint64_t grid = (((uint64_t)numel + 1) / 2 + 255) / 256;
   if (grid > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (which) hipLaunchKernelGGL(dequantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, codes, scales, numel, out);
@@ -663,6 +663,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1006; }
+int q4adamw_version(void) { return 1007; }
 
 }  // extern "C"

@@ -11,13 +11,21 @@ template <bool PBF, bool GBF, bool EXT>
 __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args) {
   const uint32_t chunk = blockIdx.x;
   float gscale = 1.0f;
-  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);
   const bool zero_g = EXT && args.go.zero != 0u;
+  if (cancelled && !zero_g) return;
   const int t = find_tensor(args, chunk);
   const SmallDesc &T = args.desc[t];
   const StepConsts &sc = args.sc;
   const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kSmallChunk;
   const int64_t end = base + kSmallChunk < T.numel ? base + kSmallChunk : T.numel;
+  if (cancelled) {  // a cancelled step still clears the gradients it was asked to clear
+    for (int64_t i = base + threadIdx.x; i < end; i += 256) {
+      if (GBF) as_global<uint16_t>(const_cast<void *>(T.g))[i] = 0;
+      else as_global<float>(const_cast<void *>(T.g))[i] = 0.0f;
+    }
+    return;
+  }
   for (int64_t i = base + threadIdx.x; i < end; i += 256) {
     float gi = GBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.g)[i])
                    : as_global<const float>(T.g)[i];

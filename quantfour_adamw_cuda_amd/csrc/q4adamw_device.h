@@ -184,6 +184,23 @@ __device__ __forceinline__ void zero_elems(void *base, uint32_t e0, int nv) {
   }
 }
 
+// Zeros over one tile of a gradient tensor: what is left of a step's work when an
+// overflow flag cancels it and the caller asked for the gradients to be cleared.
+template <bool BF, int N>
+__device__ __forceinline__ void zero_tile(const void *g, int64_t tile, int64_t numel, int lane) {
+  constexpr int64_t kTile = 64 * N;
+  const int64_t tb = tile * kTile;
+  if (tb >= numel) return;
+  void *g_tile = static_cast<char *>(const_cast<void *>(g)) + tb * (BF ? 2 : 4);
+  const uint32_t e0 = (uint32_t)lane * N;
+  if (tb + kTile <= numel) {
+    zero_elems<BF, N, true>(g_tile, e0, N);
+  } else {
+    const int64_t rem = numel - tb - (int64_t)e0;
+    zero_elems<BF, N, false>(g_tile, e0, rem >= N ? N : (rem > 0 ? (int)rem : 0));
+  }
+}
+
 template <int N>
 struct Vals {
   float x[N];

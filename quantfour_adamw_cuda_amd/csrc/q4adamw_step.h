@@ -321,12 +321,17 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;  // whole workgroup: the grid is padded to a multiple of 8
   float gscale = 1.0f;
-  if (EXT && !grad_ops_begin(args.go, gscale)) return;  // whole grid
+  const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);  // whole grid
   const bool zero_g = EXT && args.go.zero != 0u;
+  if (cancelled && !zero_g) return;
   const int t = find_tensor(args, chunk);
   const TensorDesc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
+  if (cancelled) {  // a cancelled step still clears the gradients it was asked to clear
+    zero_tile<GBF, G::kEpl>(T.g, tile, T.numel, lane);
+    return;
+  }
   const int64_t begin = tile * G::kTile;
   if (begin >= T.numel) {  // wave past the end of the tensor: only help with the tables
     setup_tables<SR>(lds, tid, slot);
@@ -480,12 +485,17 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;
   float gscale = 1.0f;
-  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);
   const bool zero_g = EXT && args.go.zero != 0u;
+  if (cancelled && !zero_g) return;
   const int t = find_tensor(args, chunk);
   const Rank1Desc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
+  if (cancelled) {
+    zero_tile<GBF, G::kEpl>(T.g, tile, T.numel, lane);
+    return;
+  }
   const int64_t begin = tile * G::kTile;
   if (begin >= T.numel) {
     setup_tables<false>(lds, tid, slot);

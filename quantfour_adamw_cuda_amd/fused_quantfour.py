@@ -400,11 +400,13 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                        torch.nn.utils.clip_grad_norm_ would, without rewriting them;
                        the norm is left in `last_grad_norm` (a device scalar)
         found_inf      one-element float32 device tensor: a non-zero value makes the
-                       step a no-op on the device, without synchronising; the step
+                       device leave parameters and state alone (gradients are still
+                       cleared if zero_grad asks for it), without synchronising; the step
                        counters of a skipped step are taken back when the next step
                        (or state_dict()) looks at the flag's value, which by then has
                        reached the host
-        zero_grad      overwrite the gradients with zeros once the step has read them
+        zero_grad      overwrite the gradients with zeros once the step has read them,
+                       or once an overflow flag has cancelled it
         """
         loss = None
         if closure:

@@ -151,8 +151,9 @@ def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr,
                      eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False):
     """One launch over many quantized tensors that share device, dtypes and step.  The
     gradients enter the step multiplied by grad_scale * grad_scale_dev (a device float32
-    scalar); found_inf (a device float32 scalar) turns the call into a no-op when it holds a
-    non-zero value; zero_grad overwrites the gradients with zeros once they are read."""
+    scalar); found_inf (a device float32 scalar) makes the call leave parameters and state
+    alone when it holds a non-zero value; zero_grad overwrites the gradients with zeros once
+    they are read, also in a call that found_inf cancels."""
     if not ps:
         return
     arr = make_table(ps, gs, exps, sqs, exp_scales, sq_scales)

@@ -99,13 +99,18 @@ def test_zero_grad_and_found_inf(cuda, g_dt):
         assert _same(_state_bits(a), _state_bits(b)), f"step {step}"
         assert torch.equal(ga, g)
         assert not gb.any(), "gradients must be zero after a zeroing step"
-    # overflow flag set: nothing changes, not even the gradients
+    # overflow flag set: parameters and state stay; the gradients stay too unless the call
+    # was to clear them (an overflowed gradient must not reach the next accumulation)
     before = _state_bits(b)
     flag.fill_(1.0)
     g = grads_config1(gen, n).to(DT[g_dt]).to(cuda)
+    g[::1000] = float("inf")
     g0 = g.clone()
-    _step(b, g, 3, zero_grad=True, found_inf=flag, grad_scale=0.5)
+    _step(b, g, 3, found_inf=flag, grad_scale=0.5)
     assert _same(before, _state_bits(b)) and torch.equal(g, g0)
+    _step(b, g, 3, zero_grad=True, found_inf=flag, grad_scale=0.5)
+    assert _same(before, _state_bits(b))
+    assert not g.any(), "a cancelled step still clears the gradients"
 
 
 def test_small_tensor_kernel_options(cuda):
@@ -137,8 +142,12 @@ def test_small_tensor_kernel_options(cuda):
     flag.fill_(3.0)
     before = [t.clone() for t in dp + dm + dv]
     dg = [grads_config1(gen, n).to(torch.bfloat16).to(cuda) for n in sizes]
+    dg0 = [g.clone() for g in dg]
     q.fused_single_tensor_multi(dp, dg, dm, dv, *HPA, 3, found_inf=flag)
+    assert all(torch.equal(x, y) for x, y in zip(before + dg0, dp + dm + dv + dg))
+    q.fused_single_tensor_multi(dp, dg, dm, dv, *HPA, 3, found_inf=flag, zero_grad=True)
     assert all(torch.equal(x, y) for x, y in zip(before, dp + dm + dv))
+    assert not any(bool(g.any()) for g in dg), "a cancelled step still clears the gradients"
 
 
 def test_option_argument_errors(cuda):
@@ -300,6 +309,37 @@ def test_grad_scaler_drives_the_fused_path(cuda):
     assert all(float(st["step"]) == 4.0 for st in opt.state.values())
     for pa, pb in zip(m.parameters(), ref.parameters()):
         assert torch.equal(pa, pb)       # same bias corrections as the run that never overflowed
+
+
+@pytest.mark.parametrize("variance", ["group", "rank1"])
+def test_optimizer_cancelled_step_clears_gradients(cuda, variance):
+    """an overflowed step changes neither parameters nor state nor step counters, and with
+    zero_grad=True the overflowed gradients are gone afterwards: the next backward
+    accumulates onto zeros and the run continues like one that never saw the overflow"""
+    torch.manual_seed(3)
+    mk = lambda: torch.nn.Sequential(torch.nn.Linear(512, 64), torch.nn.Tanh(), torch.nn.Linear(64, 8)).to(cuda)
+    a, b = mk(), mk()
+    b.load_state_dict(a.state_dict())
+    oa = AdamWFused_QuantFour(a.parameters(), lr=1e-3, variance_scale_type=variance)
+    ob = AdamWFused_QuantFour(b.parameters(), lr=1e-3, variance_scale_type=variance)
+    flag = torch.zeros(1, device=cuda)
+    for it in range(4):
+        x = torch.randn(16, 512, device=cuda)
+        if it == 2:    # a's extra, overflowed iteration
+            a(x).square().mean().backward()
+            next(a.parameters()).grad[0, :7] = float("nan")
+            flag.fill_(1.0)
+            oa.step(found_inf=flag, zero_grad=True)
+            assert all(not p.grad.any() for p in a.parameters())
+            flag.zero_()
+        a(x).square().mean().backward()
+        b(x).square().mean().backward()
+        oa.step(found_inf=flag, zero_grad=True)
+        ob.step(zero_grad=True)
+        for pa, pb in zip(a.parameters(), b.parameters()):
+            assert torch.equal(pa, pb), f"iteration {it}"
+    sa, sb = oa.state_dict()["state"], ob.state_dict()["state"]
+    assert all(float(sa[k]["step"]) == float(sb[k]["step"]) == 4.0 for k in sa)
 
 
 def test_clip_pipeline_and_rank1_replay_under_graph_capture(cuda):

@@ -114,9 +114,13 @@ def test_rank1_found_inf_leaves_everything(cuda):
     dev.step(g, 1)
     before = [t.clone() for t in dev.tensors()]
     flag = torch.ones(1, device=cuda)
+    g0 = g.clone()
     dev.step(g, 2, found_inf=flag)
     assert all(torch.equal(a, b) for a, b in zip(before, dev.tensors()))
-    assert not dev.rn.any() and not dev.cn.any()
+    assert not dev.rn.any() and not dev.cn.any() and torch.equal(g, g0)
+    dev.step(g, 2, found_inf=flag, zero_grad=True)   # cancelled, but the gradients are cleared
+    assert all(torch.equal(a, b) for a, b in zip(before, dev.tensors()))
+    assert not dev.rn.any() and not dev.cn.any() and not g.any()
 
 
 def test_rank1_full_size_matrix(cuda):
