@@ -115,6 +115,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         )
         super().__init__(params, defaults)
         self._launch_cache: Dict[Any, Any] = {}
+        self._step_buffers: Dict[Any, Any] = {}
         # global gradient norm of the last step(max_grad_norm=...), a device scalar
         self.last_grad_norm = None
         self._norm_buffers: Dict[Any, Any] = {}
@@ -138,6 +139,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         """optim/fused_quantfour.py:73-84"""
         super().__setstate__(state)
         self._launch_cache = {}
+        self._step_buffers = {}
         self._norm_buffers = {}
         self.__dict__.setdefault("kernel_timing", None)
         self.__dict__.setdefault("last_grad_norm", None)
@@ -454,8 +456,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             stochastic = group.get("round_type", "real-nearest") == "stochastic"
 
             # update step (optim/fused_quantfour.py:178)
-            torch._foreach_add_(state_steps, 1)
-            steps = torch.stack(state_steps).tolist()
+            steps = self._advance_steps(gi, params_with_grad, state_steps)
             stepped.extend(state_steps)
 
             # one launch per (kind, device, dtypes, step)
@@ -537,6 +538,27 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         if found_inf is not None and stepped:
             self._watch_skip_flag(found_inf, stepped)
         return loss
+
+    def _advance_steps(self, gi, params, state_steps):
+        """Adds 1 to every step counter and returns their new values as Python floats.  The
+        counters of a group's parameters are 0-dim views of one host buffer, so this is one
+        addition whatever the number of tensors; a counter that was replaced (lazy state,
+        load_state_dict, the user) is noticed by identity and the buffer is laid out again.
+        `state_steps` is updated in place to the tensors the state holds afterwards."""
+        cached = self._step_buffers.get(gi)
+        if (cached is None or len(cached[1]) != len(state_steps)
+                or any(a is not b for a, b in zip(cached[1], state_steps))):
+            buf = torch.stack([t.detach().to(device="cpu", dtype=torch.float32).reshape(())
+                               for t in state_steps])
+            views = list(buf.unbind(0))
+            for p, v in zip(params, views):
+                self.state[p]["step"] = v
+            cached = (buf, views)
+            self._step_buffers[gi] = cached
+            state_steps[:] = views
+        buf = cached[0]
+        buf.add_(1)
+        return buf.tolist()
 
     # -- overflow flag: keeping the step counters right without a synchronisation -----
     def _watch_skip_flag(self, found_inf, stepped):

@@ -151,6 +151,32 @@ def test_loaded_state_shares_nothing_with_its_source():
             != b["momentum_qstate"]["overhead"]["max1"].data_ptr())
 
 
+def test_step_counters_share_one_buffer_and_follow_replacements():
+    """the step counters of a group are views of one host buffer (one addition per step);
+    a counter replaced from outside is picked up by identity and keeps its own value"""
+    ps = [torch.nn.Parameter(torch.zeros(n)) for n in (5000, 3, 8192)]
+    opt = AdamWFused_QuantFour(ps)
+    for p in ps:
+        opt._init_state(p)
+    steps = [opt.state[p]["step"] for p in ps]
+    assert opt._advance_steps(0, ps, steps) == [1.0, 1.0, 1.0]
+    assert all(opt.state[p]["step"] is s for p, s in zip(ps, steps))
+    buf = opt._step_buffers[0][0]
+    assert all(s.dim() == 0 and s.dtype == torch.float32 and s.untyped_storage().data_ptr() ==
+               buf.untyped_storage().data_ptr() for s in steps)
+    assert opt._advance_steps(0, ps, steps) == [2.0, 2.0, 2.0] and opt._step_buffers[0][0] is buf
+    opt.state[ps[1]]["step"] = torch.tensor(7.0)
+    steps = [opt.state[p]["step"] for p in ps]
+    assert opt._advance_steps(0, ps, steps) == [3.0, 8.0, 3.0]
+    assert [float(opt.state[p]["step"]) for p in ps] == [3.0, 8.0, 3.0]
+    # a subset of the parameters (the others had no gradient this time)
+    steps = [opt.state[p]["step"] for p in ps[:2]]
+    assert opt._advance_steps(0, ps[:2], steps) == [4.0, 9.0]
+    assert [float(opt.state[p]["step"]) for p in ps] == [4.0, 9.0, 3.0]
+    sd = opt.state_dict()
+    assert [float(sd["state"][i]["step"]) for i in range(3)] == [4.0, 9.0, 3.0]
+
+
 def test_rank1_state_layout_and_round_trip():
     """variance_scale_type="rank1": matrices with cols % 8 == 0 and cols >= 512 keep row and
     column maxima (the draft's max_dims, keepdim shapes) instead of block scales; everything
