@@ -31,9 +31,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 # HBM bytes per optimizer step of the fused kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (each scaled by what the same counter reads for a 4 GiB device copy: 2.0 and 1.0);
-# summary in profiles/fused_4bit_kernel_llama3_8b_hbm_counters.txt.  Workloads that have not
-# been profiled report null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {"llama3-8b": 9.7374e10}
+# summaries in profiles/fused_4bit_kernel_llama3_8b_hbm_counters.txt and
+# profiles/fused_4bit_rank1_kernels_llama3_8b_hbm_counters.txt.  Keyed by (workload, rank-1
+# scaling); combinations that have not been profiled report null.
+MEASURED_TRAFFIC_BYTES_PER_STEP = {("llama3-8b", False): 9.7374e10, ("llama3-8b", True): 1.17325e11}
 HP = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 
 
@@ -304,8 +305,8 @@ def main():
             "frac": achieved / HBM_PEAK_GBS,
             # per launch, averaged over the step's launches (they differ in size): measured
             # HBM bytes, algorithmic bytes, duration; achieved = algorithmic bytes / duration
-            "traffic": (MEASURED_TRAFFIC_BYTES_PER_STEP[args.workload] / launches_per_step
-                        if args.workload in MEASURED_TRAFFIC_BYTES_PER_STEP and not rank1 else None),
+            "traffic": (MEASURED_TRAFFIC_BYTES_PER_STEP[(args.workload, bool(rank1))] / launches_per_step
+                        if (args.workload, bool(rank1)) in MEASURED_TRAFFIC_BYTES_PER_STEP else None),
             "algorithmic_bytes_per_launch": algo_bytes / launches_per_step,
             "kernel_ms_per_launch": avg_kernel_s * 1e3 / launches_per_step,
             "kernel_launches_per_step": launches_per_step,
