@@ -184,7 +184,7 @@ def main():
                     help="scaling of the second moment: per-128 block maxima (the fused CUDA path) or "
                          "rank-1 row/column maxima for matrices (a statistics pass precedes the update)")
     ap.add_argument("--round-type", choices=["real-nearest", "stochastic"], default="real-nearest",
-                    help="rounding of the quantizer (stochastic: hash noise per element, block scaling only)")
+                    help="rounding of the quantizer (stochastic: hash noise per element)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, run a plain 4 GiB device copy three times, so that "

@@ -195,6 +195,19 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
                                    const q4adamw_grad_options *opt, void *stream);
 
 /*
+ * q4adamw_fused_4bit_rank1_multi with stochastic rounding of both moments: the rule and
+ * the noise of q4adamw_fused_4bit_multi_sr (salts, seed as there), the second moment's
+ * quotient taken with its rank-1 scale min(row_max[i], col_max[j]).  The combination of
+ * the draft's settings scale_type "rank1" (optim/adamw_fourbit_triton.py:124) and
+ * round_type "stochastic" (:1050-1075).
+ */
+int q4adamw_fused_4bit_rank1_multi_sr(const q4adamw_rank1_tensor *tensors, int count,
+                                      const uint32_t *salts, uint64_t seed, int p_dtype, int g_dtype,
+                                      float beta1, float beta2, float lr, float weight_decay,
+                                      float eps, float step, const q4adamw_grad_options *opt,
+                                      void *stream);
+
+/*
  * Non-quantized AdamW step (fp32 moments) on one tensor.
  * Replaces fused_single_tensor (optim/cuda_fused_interface.cc:49-64) and
  * cuda_fused_single_tensor (optim/cuda_adamw_kernels.cu:136-164).

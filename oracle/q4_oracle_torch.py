@@ -245,6 +245,13 @@ def quantize_sr(x, which, u):
     max1 = np.fmax.reduce(np.abs(grouped), axis=1, initial=0.0, keepdims=True)   # a NaN never becomes the scale
     with np.errstate(invalid="ignore", divide="ignore"):
         q = (grouped / max1).reshape(-1)                     # 0/0 -> NaN -> code 0
+    code = sr_codes(q, which, noise)
+    return pack(torch.from_numpy(code.astype(np.int64))[:numel], numel), torch.from_numpy(max1.reshape(-1))
+
+
+def sr_codes(q, which, noise):
+    """Stochastic rounding of normalised values q (float32 numpy, NaN -> code 0) with one
+    noise value per element: numpy int codes."""
     Q = QMAP[which].numpy()
     # k_raw = number of code-book values <= q; the tables are extended so that both ends
     # need no special case: below Q[0] the "gap" is 0 (always up, from -1 to 0), at or
@@ -258,7 +265,34 @@ def quantize_sr(x, which, u):
         up = t < d
     code = np.clip(k_raw - 1 + up, 0, 15)
     code[np.isnan(q)] = 0
-    return pack(torch.from_numpy(code.astype(np.int64))[:numel], numel), torch.from_numpy(max1.reshape(-1))
+    return code
+
+
+def quantize_rank1_sr(x, u):
+    """quantize_rank1 with stochastic rounding: x fp32 matrix (CPU), u float32 numpy noise per
+    element (row-major).  Returns (packed codes, row maxima, column maxima)."""
+    ax = torch.nan_to_num(x.abs(), nan=0.0, posinf=float("inf"))   # statistics as in quantize_rank1
+    row_max = ax.amax(dim=1)
+    col_max = ax.amax(dim=0)
+    q = x.div(rank1_scale(row_max, col_max)).reshape(-1).numpy()   # 0/0 -> NaN -> code 0
+    code = sr_codes(q, 1, np.asarray(u, np.float32))
+    return pack(torch.from_numpy(code.astype(np.int64)), x.numel()), row_max, col_max
+
+
+def step_quant_rank1_sr(p, g, m_codes, v_codes, m_scale, row_max, col_max, *, seed, tensor_salt, beta1,
+                        beta2, lr, weight_decay, eps, step):
+    """step_quant_rank1 with stochastic rounding of both moments (CPU tensors): the first
+    moment as in step_quant_sr, the second moment's quotient taken with its rank-1 scale."""
+    rows, cols = p.shape
+    numel = p.numel()
+    sc = derive_scalars(beta1, beta2, lr, weight_decay, step)
+    m = dequantize(m_codes, m_scale, numel, 0)
+    v = dequantize_rank1(v_codes, row_max, col_max).reshape(-1)
+    p_new, m_new, v_new = adamw_update(p.reshape(-1).float(), g.reshape(-1).float(), m, v, sc, eps)
+    um, uv = sr_noise(numel, sr_tensor_salt(seed, step, tensor_salt))
+    mc, ms = quantize_sr(m_new, 0, um)
+    vc, rmax, cmax = quantize_rank1_sr(v_new.view(rows, cols), uv)
+    return p_new.to(p.dtype).view_as(p), mc, vc, ms, rmax, cmax
 
 
 def step_quant_sr(p, g, m_codes, v_codes, m_scale, v_scale, *, seed, tensor_salt, beta1, beta2, lr,

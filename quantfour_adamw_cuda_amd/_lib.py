@@ -81,6 +81,7 @@ EXPORTS = (
     "q4adamw_fused_4bit_multi_sr",
     "q4adamw_sr_tensor_salt",
     "q4adamw_fused_4bit_rank1_multi",
+    "q4adamw_fused_4bit_rank1_multi_sr",
     "q4adamw_fused_single_tensor",
     "q4adamw_fused_single_tensor_multi",
     "q4adamw_fused_single_tensor_multi_ex",
@@ -133,6 +134,10 @@ def load():
     L.q4adamw_sr_tensor_salt.restype = ctypes.c_uint32
     L.q4adamw_fused_4bit_rank1_multi.argtypes = [ctypes.POINTER(Q4Rank1Tensor), i, i, i] + hyper + [opt, vp]
     L.q4adamw_fused_4bit_rank1_multi.restype = i
+    L.q4adamw_fused_4bit_rank1_multi_sr.argtypes = ([ctypes.POINTER(Q4Rank1Tensor), i,
+                                                     ctypes.POINTER(ctypes.c_uint32), ctypes.c_uint64, i, i]
+                                                    + hyper + [opt, vp])
+    L.q4adamw_fused_4bit_rank1_multi_sr.restype = i
     L.q4adamw_grad_norm.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, ctypes.c_size_t, vp, vp]
     L.q4adamw_grad_norm.restype = i
     L.q4adamw_quantize.argtypes = [vp, i64, i, vp, vp, vp]

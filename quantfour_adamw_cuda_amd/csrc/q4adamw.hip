@@ -161,17 +161,18 @@ static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
 typedef void (*Rank1Kernel)(const Rank1Args);
 typedef void (*Rank1StatKernel)(const Rank1StatArgs);
 
-template <bool EXT>
+template <bool EXT, bool SR>
 static Rank1Kernel pick_rank1_ext(bool pb, bool gb) {
-  if (!pb && !gb) return fused_4bit_rank1_kernel<false, false, EXT>;
-  if (!pb && gb) return fused_4bit_rank1_kernel<false, true, EXT>;
-  if (pb && !gb) return fused_4bit_rank1_kernel<true, false, EXT>;
-  return fused_4bit_rank1_kernel<true, true, EXT>;
+  if (!pb && !gb) return fused_4bit_rank1_kernel<false, false, EXT, SR>;
+  if (!pb && gb) return fused_4bit_rank1_kernel<false, true, EXT, SR>;
+  if (pb && !gb) return fused_4bit_rank1_kernel<true, false, EXT, SR>;
+  return fused_4bit_rank1_kernel<true, true, EXT, SR>;
 }
 
-static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext) {
+static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr) {
   const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  return ext ? pick_rank1_ext<true>(pb, gb) : pick_rank1_ext<false>(pb, gb);
+  if (sr) return pick_rank1_ext<true, true>(pb, gb);
+  return ext ? pick_rank1_ext<true, false>(pb, gb) : pick_rank1_ext<false, false>(pb, gb);
 }
 
 static Rank1StatKernel pick_rank1_stats(int g_dtype, bool ext) {
@@ -210,6 +211,11 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
                                  float beta1, float beta2, float lr, float weight_decay, float eps,
                                  float step, const q4adamw_grad_options *opt, bool sr,
                                  const uint32_t *salts, uint64_t seed, void *stream);
+static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
+                                       int g_dtype, float beta1, float beta2, float lr,
+                                       float weight_decay, float eps, float step,
+                                       const q4adamw_grad_options *opt, bool sr, const uint32_t *salts,
+                                       uint64_t seed, void *stream);
 
 extern "C" {
 
@@ -339,12 +345,11 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   return 0;
 }
 
-extern "C" {
-
-int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
-                                   int g_dtype, float beta1, float beta2, float lr,
-                                   float weight_decay, float eps, float step,
-                                   const q4adamw_grad_options *opt, void *stream) {
+static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
+                                       int g_dtype, float beta1, float beta2, float lr,
+                                       float weight_decay, float eps, float step,
+                                       const q4adamw_grad_options *opt, bool sr, const uint32_t *salts,
+                                       uint64_t seed, void *stream) {
   if (count < 0 || (count > 0 && !tensors)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   Rank1Args a;
@@ -383,7 +388,7 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const Rank1Kernel kernel = pick_rank1(p_dtype, g_dtype, ext);
+  const Rank1Kernel kernel = pick_rank1(p_dtype, g_dtype, ext, sr);
   const Rank1StatKernel stat_kernel = pick_rank1_stats(g_dtype, ext);
   a.ntensors = 0;
   uint64_t chunks = 0, stat_chunks = 0;
@@ -433,6 +438,7 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
     const FastDiv fd = make_fast_div((uint32_t)(t.cols >> 3));
     d.div_magic = fd.magic;
     d.div_shift = fd.shift;
+    a.sr_salt[a.ntensors] = sr ? q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i) : 0u;
     a.first_chunk[a.ntensors] = (uint32_t)chunks;
     Rank1StatArgs::Desc &sd = sa.desc[a.ntensors];
     sd.g = t.g;
@@ -451,6 +457,25 @@ int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int coun
   }
   if (a.ntensors > 0) return launch();
   return 0;
+}
+
+extern "C" {
+
+int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
+                                   int g_dtype, float beta1, float beta2, float lr,
+                                   float weight_decay, float eps, float step,
+                                   const q4adamw_grad_options *opt, void *stream) {
+  return fused_4bit_rank1_multi_impl(tensors, count, p_dtype, g_dtype, beta1, beta2, lr, weight_decay,
+                                     eps, step, opt, false, nullptr, 0, stream);
+}
+
+int q4adamw_fused_4bit_rank1_multi_sr(const q4adamw_rank1_tensor *tensors, int count,
+                                      const uint32_t *salts, uint64_t seed, int p_dtype, int g_dtype,
+                                      float beta1, float beta2, float lr, float weight_decay,
+                                      float eps, float step, const q4adamw_grad_options *opt,
+                                      void *stream) {
+  return fused_4bit_rank1_multi_impl(tensors, count, p_dtype, g_dtype, beta1, beta2, lr, weight_decay,
+                                     eps, step, opt, true, salts, seed, stream);
 }
 
 int q4adamw_fused_4bit(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_avg_sq,
@@ -663,6 +688,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1007; }
+int q4adamw_version(void) { return 1008; }
 
 }  // extern "C"

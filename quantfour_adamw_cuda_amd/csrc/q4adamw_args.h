@@ -140,6 +140,7 @@ struct Rank1Args {
   uint32_t chunks_per_xcd;
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
+  uint32_t sr_salt[kMaxRank1Tensors];   // stochastic rounding: the tensors' salts of this step
   Rank1Desc desc[kMaxRank1Tensors];
 };
 

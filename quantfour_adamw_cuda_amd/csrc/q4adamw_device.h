@@ -260,32 +260,44 @@ __device__ __forceinline__ float sr_noise_value(uint32_t n16) {
 // optim/adamw_fourbit_triton.py:1050-1075, without its division): IEEE quotient, its
 // interval [Q[k], Q[k+1]) among the code-book entries, upper code iff
 // noise * (Q[k+1] - Q[k]) < q - Q[k].  0/0 is NaN and gets code 0.
+template <bool SECOND>
+__device__ __forceinline__ uint32_t sr_code_exact(float q, float noise) {
+  uint32_t k_raw = 0;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const float t = SECOND ? qmap_v(k) : bits2f(kQmapMBits[k]);
+    k_raw += (t <= q) ? 1u : 0u;
+  }
+  float lower, width;
+  if (SECOND) {
+    lower = k_raw == 0u ? -3.4028234663852886e38f : (float)k_raw * 0.0625f;
+    width = k_raw == 0u ? 0.0f : (k_raw == 16u ? __builtin_inff() : 0.0625f);
+  } else {
+    const SrInterval iv = kSrIntervals.e[k_raw];
+    lower = iv.lower;
+    width = iv.width;
+  }
+  const bool up = noise * width < q - lower;
+  int c = (int)k_raw - 1 + (up ? 1 : 0);
+  c = c < 0 ? 0 : (c > 15 ? 15 : c);
+  return (uint32_t)c;
+}
+
 template <bool SECOND, int N>
 __device__ __forceinline__ uint32_t quantize_exact_sr(const Vals<N> &v, float scale, const Vals<N> &noise) {
   uint32_t word = 0;
 #pragma unroll
-  for (int j = 0; j < N; ++j) {
-    const float q = v.x[j] / scale;
-    uint32_t k_raw = 0;
+  for (int j = 0; j < N; ++j) word |= sr_code_exact<SECOND>(v.x[j] / scale, noise.x[j]) << (4 * j);
+  return word;
+}
+
+// The same for the second moment with a scale per element (rank-1 scaling).
+template <int N>
+__device__ __forceinline__ uint32_t quantize_exact_sr_scales(const Vals<N> &v, const Vals<N> &scale,
+                                                             const Vals<N> &noise) {
+  uint32_t word = 0;
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const float t = SECOND ? qmap_v(k) : bits2f(kQmapMBits[k]);
-      k_raw += (t <= q) ? 1u : 0u;
-    }
-    float lower, width;
-    if (SECOND) {
-      lower = k_raw == 0u ? -3.4028234663852886e38f : (float)k_raw * 0.0625f;
-      width = k_raw == 0u ? 0.0f : (k_raw == 16u ? __builtin_inff() : 0.0625f);
-    } else {
-      const SrInterval iv = kSrIntervals.e[k_raw];
-      lower = iv.lower;
-      width = iv.width;
-    }
-    const bool up = noise.x[j] * width < q - lower;
-    int c = (int)k_raw - 1 + (up ? 1 : 0);
-    c = c < 0 ? 0 : (c > 15 ? 15 : c);
-    word |= (uint32_t)c << (4 * j);
-  }
+  for (int j = 0; j < N; ++j) word |= sr_code_exact<true>(v.x[j] / scale.x[j], noise.x[j]) << (4 * j);
   return word;
 }
 

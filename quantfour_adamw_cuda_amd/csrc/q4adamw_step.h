@@ -31,7 +31,6 @@ template <bool PBF, bool GBF, bool FULL, bool EXT, bool RANK1, bool SR, typename
 __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g, uint32_t salt) {
-  static_assert(!(SR && RANK1), "stochastic rounding is built for block scaling only");
   using G = Geometry<PBF, GBF>;
   constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
@@ -255,7 +254,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
       if constexpr (SR) {
         // code-book entries at 16 q = 1..16: interval number floor(16 q), position in
         // it fract(16 q), up iff noise < position; the ends clamp
-        const float q16 = vn.x[k] * rv16;
+        const float q16 = vn.x[k] * (RANK1 ? inv16.x[k] : rv16);
         const float kf = __builtin_floorf(q16), d16 = q16 - kf;
         redo |= __builtin_fabsf(uv.x[k] - d16) <= kVGuard;
         const float cf = __builtin_amdgcn_fmed3f(kf + (uv.x[k] < d16 ? 0.0f : -1.0f), 0.0f, 15.0f);
@@ -276,7 +275,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   if (__builtin_expect(redo, 0)) {
     if constexpr (SR) {
       mword = quantize_exact_sr<false, N>(mn, am, um);
-      vword = quantize_exact_sr<true, N>(vn, av, uv);
+      if constexpr (RANK1) vword = quantize_exact_sr_scales<N>(vn, s_new, uv);
+      else vword = quantize_exact_sr<true, N>(vn, av, uv);
     } else {
       mword = quantize_exact<false, N>(mn, am);
       if constexpr (RANK1) vword = quantize_exact_scales<N>(vn, s_new);
@@ -476,12 +476,12 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   }
 }
 
-template <bool PBF, bool GBF, bool EXT>
+template <bool PBF, bool GBF, bool EXT, bool SR>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
   using G = Geometry<PBF, GBF>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
-  const TableSlot slot = request_table_slot<false>(tid);
+  const TableSlot slot = request_table_slot<SR>(tid);
   const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;
   float gscale = 1.0f;
@@ -498,13 +498,14 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   }
   const int64_t begin = tile * G::kTile;
   if (begin >= T.numel) {
-    setup_tables<false>(lds, tid, slot);
+    setup_tables<SR>(lds, tid, slot);
     return;
   }
+  const uint32_t salt = SR ? args.sr_salt[t] : 0u;
   if (begin + G::kTile <= T.numel)
-    process_tile<PBF, GBF, true, EXT, true, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, 0u);
+    process_tile<PBF, GBF, true, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PBF, GBF, false, EXT, true, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, 0u);
+    process_tile<PBF, GBF, false, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
 }
 
 // After the update: the new statistics become the current ones and the buffers that

@@ -89,8 +89,6 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # param groups, so a resumed run continues the same noise sequence.
         if round_type not in ("real-nearest", "stochastic"):
             raise ValueError(f"Invalid round_type: {round_type=}")
-        if round_type == "stochastic" and variance_scale_type == "rank1":
-            raise ValueError("stochastic rounding is built for variance_scale_type='group' only")
         if round_type == "stochastic" and seed is None:
             seed_t = torch.randint(1 << 31, size=[1])
             if torch.distributed.is_available() and torch.distributed.is_initialized():
@@ -465,7 +463,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 assert param.is_cuda, "param must be on cuda"
                 kind = momentum_quant_enabled[i]
                 if kind and "max_dims" in variance_meta[i]:
-                    kind = "rank1"
+                    kind = "rank1_sr" if stochastic else "rank1"
                 elif kind and stochastic:
                     kind = "sr"
                 key = (kind, param.device, param.dtype, grads[i].dtype, steps[i])
@@ -476,7 +474,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 gs = [grads[i] for i in idx]
                 ms = [exp_avgs[i] for i in idx]
                 vs = [exp_avg_sqs[i] for i in idx]
-                if quantized == "rank1":
+                rank1 = quantized in ("rank1", "rank1_sr")
+                if rank1:
                     sms = [momentum_meta[i]["max1"] for i in idx]
                     stats = [[variance_meta[i][k][d] for i in idx]
                              for k in ("max_dims", "scratch_dims") for d in (0, 1)]
@@ -495,14 +494,14 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 cache_key = (gi, quantized, device, p_dtype, g_dtype)
                 cached = self._launch_cache.get(cache_key)
                 if cached is None or cached[0] != ptrs:
-                    if quantized == "rank1":
+                    if rank1:
                         arr = _q.make_rank1_table(ps, gs, ms, vs, sms, stats[0], stats[1], stats[2], stats[3])
                     elif quantized:
                         arr = _q.make_table(ps, gs, ms, vs, sms, svs)
                     else:
                         arr = _q.make_small_table(ps, gs, ms, vs)
                     tags = (_q._tag(ps[0], "param"), _q._tag(gs[0], "grad"))
-                    if quantized == "sr":   # noise salt of a tensor: its position among all parameters
+                    if quantized in ("sr", "rank1_sr"):   # noise salt of a tensor: its position among all parameters
                         tags += (_q.make_salts([self._param_position(p) for p in ps]),)
                     cached = (ptrs, arr, tags)
                     self._launch_cache[cache_key] = cached
@@ -515,11 +514,12 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                         assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
                         arr[i].g = g.data_ptr()
                 _, arr, (p_tag, g_tag, *extra) = cached
-                if quantized == "sr":
+                if quantized in ("sr", "rank1_sr"):
                     salts_arr, sr_seed = extra[0], group["seed"]
-                    launch = lambda *a: _q.launch_table_sr(a[0], salts_arr, sr_seed, *a[1:])
+                    launch_sr = _q.launch_rank1_table_sr if rank1 else _q.launch_table_sr
+                    launch = lambda *a: launch_sr(a[0], salts_arr, sr_seed, *a[1:])
                 else:
-                    launch = (_q.launch_rank1_table if quantized == "rank1" else
+                    launch = (_q.launch_rank1_table if rank1 else
                               _q.launch_table if quantized else _q.launch_small_table)
                 options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad)
                 if self.kernel_timing is None:
@@ -531,8 +531,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                         start.record()
                         launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                         end.record()
-                    kind = ("fused_4bit_rank1" if quantized == "rank1" else
-                            "fused_4bit" if quantized else "fused_single_tensor")   # "sr" counts as fused_4bit
+                    kind = ("fused_4bit_rank1" if rank1 else
+                            "fused_4bit" if quantized else "fused_single_tensor")   # stochastic rounding counts as its scaling's kind
                     self.kernel_timing.append((kind, start, end))
 
         if found_inf is not None and stepped:

@@ -267,12 +267,24 @@ def launch_rank1_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay
     _lib.check(rc, "fused_4bit_rank1_multi")
 
 
+def launch_rank1_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, beta2, lr, weight_decay,
+                          eps, step, options=None):
+    L = _lib.load()
+    assert salts_arr is None or len(salts_arr) == len(arr), "one salt per tensor"
+    with torch.cuda.device(device):
+        rc = L.q4adamw_fused_4bit_rank1_multi_sr(arr, len(arr), salts_arr, int(seed) & (2 ** 64 - 1), p_tag,
+                                                 g_tag, beta1, beta2, lr, weight_decay, eps, float(step),
+                                                 options, _stream(device))
+    _lib.check(rc, "fused_4bit_rank1_multi_sr")
+
+
 def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts,
                            beta1, beta2, lr, weight_decay, eps, step, grad_scale=1.0,
-                           grad_scale_dev=None, found_inf=None, zero_grad=False):
+                           grad_scale_dev=None, found_inf=None, zero_grad=False, seed=None, salts=None):
     """The fused step over matrices whose second moment is rank-1 scaled: scale of element
     (i, j) = min(row_maxes[i], col_maxes[j]).  row_nexts / col_nexts are state-owned scratch
-    that holds zeros between steps.  Gradient options as for fused_4bit_multi."""
+    that holds zeros between steps.  Gradient options as for fused_4bit_multi.  With a seed
+    both moments are rounded stochastically, noise and salts as for fused_4bit_multi_sr."""
     if not ps:
         return
     arr = make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts)
@@ -281,7 +293,11 @@ def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, 
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
     options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
-    launch_rank1_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
+    if seed is None:
+        launch_rank1_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
+    else:
+        launch_rank1_table_sr(arr, None if salts is None else make_salts(salts), seed, ps[0].device, p_tag,
+                              g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
 
 
 def make_grad_table(gs):

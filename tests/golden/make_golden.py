@@ -106,8 +106,10 @@ def make_sr(name, n, steps, hp, seed, sr_seed, tensor_salt, g_bf16=False):
     print(name, n, "elements,", steps, "steps")
 
 
-def make_rank1(name, rows, cols, steps, hp, seed, p_bf16=False, g_bf16=False):
-    """rank-1 scaled second moment (oracle/q4_oracle_torch.py step_quant_rank1)"""
+def make_rank1(name, rows, cols, steps, hp, seed, p_bf16=False, g_bf16=False, sr=None):
+    """rank-1 scaled second moment (oracle/q4_oracle_torch.py step_quant_rank1); with
+    sr = (noise seed, tensor salt) both moments are rounded stochastically
+    (step_quant_rank1_sr) and the pair travels in the fixture"""
     rng = np.random.default_rng(seed)
     n = rows * cols
     p = (rng.standard_normal(n) * 0.02).astype(np.float32)
@@ -121,8 +123,14 @@ def make_rank1(name, rows, cols, steps, hp, seed, p_bf16=False, g_bf16=False):
              torch.zeros(nk), torch.zeros(rows), torch.zeros(cols))
     out = dict(p0=p_in, shape=np.array([rows, cols], np.int64),
                hp=np.array([hp[k] for k in ("beta1", "beta2", "lr", "weight_decay", "eps")], np.float64))
+    if sr is not None:
+        out["sr"] = np.array(sr, np.uint64)
     for t, g in enumerate(gs, 1):
-        state = ot.step_quant_rank1(state[0], _to_torch(g).view(rows, cols), *state[1:], step=t, **hp)
+        if sr is None:
+            state = ot.step_quant_rank1(state[0], _to_torch(g).view(rows, cols), *state[1:], step=t, **hp)
+        else:
+            state = ot.step_quant_rank1_sr(state[0], _to_torch(g).view(rows, cols), *state[1:], seed=sr[0],
+                                           tensor_salt=sr[1], step=t, **hp)
         out[f"g{t}"] = g
         out[f"p{t}"] = _to_numpy(state[0].reshape(-1))
         out[f"m{t}"], out[f"v{t}"] = state[1].numpy().copy(), state[2].numpy().copy()
@@ -147,3 +155,4 @@ if __name__ == "__main__":
     make_sr("sr_fp32_fp32_n1100", 1100, 3, hp_driver, seed=6, sr_seed=42, tensor_salt=0)
     make_rank1("rank1_fp32_bf16_5x520", 5, 520, 3, hp, seed=7, g_bf16=True)
     make_rank1("rank1_bf16_bf16_3x1024", 3, 1024, 3, hp, seed=8, p_bf16=True, g_bf16=True)
+    make_rank1("rank1_sr_fp32_bf16_6x768", 6, 768, 3, hp, seed=9, g_bf16=True, sr=(0xFEDCBA9876543210, 11))

@@ -147,8 +147,12 @@ def test_oracle_replays_rank1_fixture(path):
     nb, nk = oc.state_sizes(rows * cols)
     st = (_t(z["p0"]).view(rows, cols), torch.zeros(nb, dtype=torch.uint8), torch.zeros(nb, dtype=torch.uint8),
           torch.zeros(nk), torch.zeros(rows), torch.zeros(cols))
+    sr = dict(seed=int(z["sr"][0]), tensor_salt=int(z["sr"][1])) if "sr" in z else None
     for t in range(1, steps + 1):
-        st = ot.step_quant_rank1(st[0], _t(z[f"g{t}"]).view(rows, cols), *st[1:], step=t, **hp)
+        if sr is None:
+            st = ot.step_quant_rank1(st[0], _t(z[f"g{t}"]).view(rows, cols), *st[1:], step=t, **hp)
+        else:
+            st = ot.step_quant_rank1_sr(st[0], _t(z[f"g{t}"]).view(rows, cols), *st[1:], step=t, **sr, **hp)
         for key, got in zip(("p", "m", "v", "sm", "r", "c"), st):
             assert np.array_equal(_bits(got), z[f"{key}{t}"].view(_bits(got).dtype)), (key, t)
 
@@ -166,8 +170,9 @@ def test_device_replays_rank1_fixture(path, cuda):
     r, c, rn, cn = (torch.zeros(k, device=cuda) for k in (rows, cols, rows, cols))
     prev = z["p0"]
     for t in range(1, steps + 1):
+        sr = dict(seed=int(z["sr"][0]), salts=[int(z["sr"][1])]) if "sr" in z else {}
         q.fused_4bit_rank1_multi([p], [_t(z[f"g{t}"]).view(rows, cols).to(cuda)], [m], [v], [sm], [r], [c], [rn], [cn],
-                                 hp["beta1"], hp["beta2"], hp["lr"], hp["weight_decay"], hp["eps"], t)
+                                 hp["beta1"], hp["beta2"], hp["lr"], hp["weight_decay"], hp["eps"], t, **sr)
         for key, got in (("m", m), ("v", v), ("sm", sm), ("r", r), ("c", c)):
             assert np.array_equal(_bits(got), z[f"{key}{t}"].view(_bits(got).dtype)), (key, t)
         ok, worst = p_close(_bits(p).view(z["p0"].dtype), z[f"p{t}"], prev, bf16=z["p0"].dtype == np.uint16)

@@ -75,14 +75,16 @@ def test_random_configuration_stochastic_rounding(cuda, i):
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
 
 
-@pytest.mark.parametrize("i", range(16))
+@pytest.mark.parametrize("i", range(24))
 def test_random_configuration_rank1(cuda, i):
+    """cases 16..23 add stochastic rounding (random seed and salt)"""
     from oracle import q4_oracle_torch as ot
     from quantfour_adamw_cuda_amd import quantfour_hip as q
     from tests.q4_testlib import p_close, to_np
     rng, _, p_dt, g_dt, hp, first_step, g_scale = _case(200 + i)
     rows, cols = int(rng.integers(1, 90)), 512 + 8 * int(rng.integers(0, 200))
-    print(f"[sweep rank1 {i}] {rows}x{cols} p={p_dt} g={g_dt} hp={hp} step0={first_step}", flush=True)
+    sr = dict(seed=int(rng.integers(0, 2 ** 63)), tensor_salt=int(rng.integers(0, 2 ** 32))) if i >= 16 else None
+    print(f"[sweep rank1 {i}] {rows}x{cols} p={p_dt} g={g_dt} hp={hp} step0={first_step} sr={sr}", flush=True)
     n = rows * cols
     p0 = torch.from_numpy((rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)).to(p_dt)
     z = lambda k, dt=torch.float32: torch.zeros(k, dtype=dt, device=cuda)
@@ -95,9 +97,14 @@ def test_random_configuration_rank1(cuda, i):
         g = torch.from_numpy(g).to(g_dt)
         step = first_step + k
         prev = ref[0]
-        ref = ot.step_quant_rank1(ref[0], g, *ref[1:], step=step, **hp)
+        if sr is None:
+            ref = ot.step_quant_rank1(ref[0], g, *ref[1:], step=step, **hp)
+            kw = {}
+        else:
+            ref = ot.step_quant_rank1_sr(ref[0], g, *ref[1:], step=step, **sr, **hp)
+            kw = dict(seed=sr["seed"], salts=[sr["tensor_salt"]])
         q.fused_4bit_rank1_multi([p], [g.to(cuda)], [m], [v], [sm], [r], [c], [rn], [cn], hp["beta1"], hp["beta2"],
-                                 hp["lr"], hp["weight_decay"], hp["eps"], step)
+                                 hp["lr"], hp["weight_decay"], hp["eps"], step, **kw)
         for name, d, x in (("m", m, ref[1]), ("v", v, ref[2])):
             assert torch.equal(d.cpu(), x), f"rank1 sweep {i} step {step}: {name} codes"
         for name, d, x in (("sm", sm, ref[3]), ("r", r, ref[4]), ("c", c, ref[5])):

@@ -83,6 +83,59 @@ def test_rank1_against_oracle(cuda, p_dt, g_dt, shape):
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])   # per-step parameter bound
 
 
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32")])
+@pytest.mark.parametrize("shape", [(64, 512), (100, 520), (130, 1032), (5, 8200)])
+def test_rank1_stochastic_rounding_against_oracle(cuda, p_dt, g_dt, shape):
+    """rank-1 scaling and stochastic rounding together: codes, scales and statistics bit for
+    bit against step_quant_rank1_sr; the noise follows seed, step and the tensor's salt"""
+    rows, cols = shape
+    gen = torch.Generator().manual_seed(rows * 137 + cols)
+    p0 = (torch.randn(rows, cols, generator=gen) * 0.05).to(DT[p_dt])
+    dev = Rank1State(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.r.cpu(), dev.c.cpu())
+    seed, salt = 0x1234_5678_9ABC_DEF0 + rows, cols % 13
+    make = (grads_config1, grads_config3, grads_config1, grads_config3)
+    for step in range(1, 5):
+        g = make[step - 1](gen, rows * cols).view(rows, cols)
+        if step == 2:
+            g[rows // 2] = 0.0
+            g[:, 8:16] = 0.0
+        g = g.to(DT[g_dt])
+        prev = ref[0]
+        ref = ot.step_quant_rank1_sr(ref[0], g, *ref[1:], seed=seed, tensor_salt=salt, step=step, **HP)
+        dev.step(g.to(cuda), step, seed=seed, salts=[salt])
+        _check(dev, ref, prev, f"sr {p_dt}/{g_dt} {shape} step {step}")
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
+
+
+def test_rank1_stochastic_rounding_many_tensors_and_options(cuda):
+    """40 matrices in one call (two launch batches): default salts are the positions in the
+    list, the call is reproducible, another seed changes codes; gradient multiplier on top"""
+    gen = torch.Generator().manual_seed(19)
+    shapes = [(6 + i % 4, 512 + 8 * (i % 5)) for i in range(40)]
+    ps = [(torch.randn(s, generator=gen) * 0.05) for s in shapes]
+    gs = [(grads_config1(gen, s[0] * s[1]) * 4).view(s).to(torch.bfloat16) for s in shapes]
+    dev_s = torch.tensor([0.25], device=cuda)
+
+    def run(seed):
+        devs = [Rank1State(p, cuda) for p in ps]
+        q.fused_4bit_rank1_multi([d.p for d in devs], [g.to(cuda) for g in gs], [d.m for d in devs],
+                                 [d.v for d in devs], [d.sm for d in devs], [d.r for d in devs],
+                                 [d.c for d in devs], [d.rn for d in devs], [d.cn for d in devs], *HPA, 1,
+                                 grad_scale_dev=dev_s, seed=seed)
+        return devs
+
+    a, b, c = run(5), run(5), run(6)
+    for i, (d, p, g) in enumerate(zip(a, ps, gs)):
+        z8, zs = torch.zeros_like(d.m).cpu(), torch.zeros_like(d.sm).cpu()
+        ref = ot.step_quant_rank1_sr(p, g.float() * np.float32(0.25), z8, z8.clone(), zs, torch.zeros(p.shape[0]),
+                                     torch.zeros(p.shape[1]), seed=5, tensor_salt=i, step=1, **HP)
+        _check(d, ref, p, f"tensor {i}")
+        assert all(torch.equal(x, y) for x, y in zip(d.tensors(), b[i].tensors()))
+    assert any(not torch.equal(x.v, y.v) for x, y in zip(a, c))
+    assert all(torch.equal(x.r, y.r) and torch.equal(x.c, y.c) for x, y in zip(a, c))   # statistics do not depend on the noise
+
+
 def test_rank1_multi_tensor_and_options(cuda):
     """several matrices in one call (more than one launch batch), with a multiplier"""
     gen = torch.Generator().manual_seed(9)
@@ -250,6 +303,49 @@ def test_optimizer_rank1_layout_tracking_and_resume(cuda):
     assert torch.equal(md[0].reshape(-1), v32.amax(1)) and torch.equal(md[1].reshape(-1), v32.amax(0))
     want_codes, _, _ = ot.quantize_rank1(v32.cpu())
     assert torch.equal(opt3.state[p3]["exp_avg_sq"].cpu(), want_codes)
+
+
+def test_optimizer_rank1_with_stochastic_rounding(cuda):
+    """variance_scale_type="rank1" with round_type="stochastic": same seed -> identical run,
+    another seed -> another run, resume continues the noise sequence, and the run tracks
+    torch.optim.AdamW within the draft's bar (tests/driver.py:70-71)"""
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+
+    def run(seed, steps, model=None, opt=None):
+        model = model or _mlp(cuda, 3)
+        opt = opt or (AdamWFused_QuantFour(model.parameters(), lr=1e-3, weight_decay=0.01,
+                                           variance_scale_type="rank1", round_type="stochastic", seed=seed)
+                      if seed is not None else torch.optim.AdamW(model.parameters(), lr=1e-3, weight_decay=0.01))
+        gen = torch.Generator(device=cuda).manual_seed(0)
+        for i in range(steps):
+            x = torch.randn(32, 512, generator=gen, device=cuda)
+            if i < int(getattr(opt, "_skip_first", 0)):
+                continue
+            opt.zero_grad(set_to_none=True)
+            model(x).square().mean().backward()
+            opt.step()
+        return model, opt
+
+    m1, o1 = run(7, 8)
+    m2, _ = run(7, 8)
+    m3, _ = run(8, 8)
+    assert all(torch.equal(a, b) for a, b in zip(m1.parameters(), m2.parameters()))
+    assert any(not torch.equal(a, b) for a, b in zip(m1.parameters(), m3.parameters()))
+    w0 = m1[0].weight
+    assert "max_dims" in o1.state[w0]["variance_qstate"]["overhead"]
+    ref, _ = run(None, 8)
+    for a, b in zip(m1.parameters(), ref.parameters()):
+        torch.testing.assert_close(a, b, atol=0.025, rtol=1e-5)
+    # resume after 5 steps == 8 steps straight through
+    m5, o5 = run(7, 5)
+    m_res = _mlp(cuda, 4)
+    m_res.load_state_dict(m5.state_dict())
+    o_res = AdamWFused_QuantFour(m_res.parameters(), variance_scale_type="rank1")
+    o_res.load_state_dict(o5.state_dict())
+    assert o_res.param_groups[0]["round_type"] == "stochastic" and o_res.param_groups[0]["seed"] == 7
+    o_res._skip_first = 5
+    run(7, 8, m_res, o_res)
+    assert all(torch.equal(a, b) for a, b in zip(m1.parameters(), m_res.parameters()))
 
 
 def test_rank1_more_than_2_to_32_elements(cuda):

@@ -214,8 +214,8 @@ def test_round_type_and_seed_travel_in_the_param_groups():
     (p,) = params((64, 130))
     with pytest.raises(ValueError, match="round_type"):
         AdamWFused_QuantFour([p], round_type="nearest-even")
-    with pytest.raises(ValueError, match="stochastic rounding"):
-        AdamWFused_QuantFour([p], round_type="stochastic", variance_scale_type="rank1")
+    both = AdamWFused_QuantFour([p], round_type="stochastic", variance_scale_type="rank1", seed=3)
+    assert both.variance_scale_type == "rank1" and both.param_groups[0]["round_type"] == "stochastic"
     assert AdamWFused_QuantFour([p]).param_groups[0]["round_type"] == "real-nearest"
     torch.manual_seed(5)
     a = AdamWFused_QuantFour([p], round_type="stochastic")

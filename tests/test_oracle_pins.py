@@ -423,6 +423,59 @@ def test_sr_quantizer_brute_force_and_exact_values():
         assert ot.unpack(codes, 128).tolist() == list(range(16)) * 8
 
 
+def test_rank1_sr_quantizer_brute_force_and_reductions():
+    """rank-1 scaling with stochastic rounding: scalar restatement on small matrices (zero
+    rows and columns included); a one-row matrix reduces to 'every non-zero element gets the
+    top code' whatever the noise; in the step, only the second moment's codes depend on how
+    the second moment is rounded"""
+    rng = np.random.default_rng(41)
+    f32 = np.float32
+    Q, _ = oc.tables(1)
+    for rows, cols in ((3, 8), (7, 16), (16, 24)):
+        x = np.abs(rng.standard_normal((rows, cols))).astype(np.float32) ** 2
+        x[1, :] = 0.0                                   # a zero row
+        x[:, 2] = 0.0                                   # a zero column
+        u = ((2 * rng.integers(0, 65536, rows * cols) + 1) / 2.0 ** 17).astype(np.float32)
+        codes, rmax, cmax = ot.quantize_rank1_sr(torch.from_numpy(x), u)
+        got = ot.unpack(codes, rows * cols).numpy().reshape(rows, cols)
+        assert np.array_equal(rmax.numpy(), x.max(1)) and np.array_equal(cmax.numpy(), x.max(0))
+        for i in range(rows):
+            for j in range(cols):
+                s = min(f32(x[i].max()), f32(x[:, j].max()))
+                if s == 0:
+                    want = 0
+                else:
+                    q = f32(x[i, j] / s)
+                    if q < Q[0]:
+                        want = 0          # below the first entry: code -1 + 1
+                    elif q >= Q[15]:
+                        want = 15
+                    else:
+                        k = max(t for t in range(16) if Q[t] <= q)
+                        want = k + (1 if f32(u[i * cols + j] * f32(Q[k + 1] - Q[k])) < f32(q - Q[k]) else 0)
+                assert got[i, j] == want, (rows, cols, i, j)
+    x = torch.tensor([[0.3, 0.0, 7.0, 1e-20]])
+    for noise in (2.0 ** -17, 0.5, 1 - 2.0 ** -17):
+        codes, _, _ = ot.quantize_rank1_sr(x, np.full(4, noise, np.float32))
+        assert ot.unpack(codes, 4).tolist() == [15, 0, 15, 15]
+    # the step: statistics, first moment and parameters do not depend on how the second
+    # moment is rounded; the first moment's codes are those of the block-scaled SR step
+    gen = torch.Generator().manual_seed(23)
+    rows, cols = 16, 128
+    g = torch.randn(rows, cols, generator=gen)
+    p = torch.randn(rows, cols, generator=gen) * 0.02
+    z8 = torch.zeros(rows * cols // 2, dtype=torch.uint8)
+    zs = torch.zeros(rows * cols // 128)
+    kw = dict(seed=77, tensor_salt=5, step=1, **HP)
+    out = ot.step_quant_rank1_sr(p, g, z8, z8.clone(), zs, torch.zeros(rows), torch.zeros(cols), **kw)
+    near = ot.step_quant_rank1(p, g, z8, z8.clone(), zs, torch.zeros(rows), torch.zeros(cols), step=1, **HP)
+    sr = ot.step_quant_sr(p.reshape(-1), g.reshape(-1), z8, z8.clone(), zs, zs.clone(), **kw)
+    assert torch.equal(out[0], near[0]) and torch.equal(out[4], near[4]) and torch.equal(out[5], near[5])
+    assert torch.equal(out[1], sr[1]) and torch.equal(out[3], sr[3])
+    a, b = ot.unpack(out[2], rows * cols), ot.unpack(near[2], rows * cols)
+    assert int((a - b).abs().max()) <= 1 and bool((a != b).any())     # a neighbouring code, not always the nearest
+
+
 def test_sr_is_unbiased_and_noise_is_uniform():
     um, uv = ot.sr_noise(1 << 20, ot.sr_tensor_salt(1234567890123, 7, 3))
     for u in (um, uv):
