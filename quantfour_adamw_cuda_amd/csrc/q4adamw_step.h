@@ -188,6 +188,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   const float rv16 = (safe_v && !RANK1) ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
+  float vfrac_hi = 0.0f;  // stochastic rounding: largest fractional part of 16 q - noise
   // rank-1: the new scale of every element and 16 / scale.  The hardware reciprocal's
   // one ulp is well inside the second moment's guard band (2^-17 in units of 16 q), so
   // it goes unrefined.  Scales below the safe range are clamped for the reciprocal: a
@@ -252,13 +253,17 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
 #pragma unroll
     for (int k = j; k < j + 2; ++k) {
       if constexpr (SR) {
-        // code-book entries at 16 q = 1..16: interval number floor(16 q), position in
-        // it fract(16 q), up iff noise < position; the ends clamp
-        const float q16 = vn.x[k] * (RANK1 ? inv16.x[k] : rv16);
-        const float kf = __builtin_floorf(q16), d16 = q16 - kf;
-        redo |= __builtin_fabsf(uv.x[k] - d16) <= kVGuard;
-        const float cf = __builtin_amdgcn_fmed3f(kf + (uv.x[k] < d16 ? 0.0f : -1.0f), 0.0f, 15.0f);
-        vword = __builtin_amdgcn_alignbit((uint32_t)(int)cf, vword, 4);
+        // code-book entries at 16 q = 1..16: interval number floor(16 q), position in it
+        // fract(16 q), up iff noise < position, i.e. code = floor(16 q - noise) wherever
+        // that difference is clear of an integer (the noise is never 0, so it is below
+        // 16); a difference within the guard band of an integer goes to the exact path.
+        // y > -1, so truncation gives 0 for y < 0
+        const float y = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, -uv.x[k]);
+        const float fr = __builtin_amdgcn_fractf(y);
+        vfrac = __builtin_fminf(vfrac, fr);
+        vfrac_hi = __builtin_fmaxf(vfrac_hi, fr);
+        const uint32_t c = (uint32_t)(int)y;
+        vword = __builtin_amdgcn_alignbit(c < 15u ? c : 15u, vword, 4);
       } else {
         const float t = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, kVGuard - 0.5f);
         vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
@@ -271,7 +276,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     mword >>= 16;
     vword >>= 16;
   }
-  redo |= vfrac < 2.0f * kVGuard;
+  if constexpr (SR) redo |= vfrac < kVGuard || vfrac_hi > 1.0f - kVGuard;
+  else redo |= vfrac < 2.0f * kVGuard;
   if (__builtin_expect(redo, 0)) {
     if constexpr (SR) {
       mword = quantize_exact_sr<false, N>(mn, am, um);
