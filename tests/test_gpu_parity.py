@@ -286,6 +286,61 @@ def test_replay_under_graph_capture(cuda):
             assert torch.equal(x.p.view(torch.int32), y.p.view(torch.int32))
 
 
+def test_concurrent_threads_and_streams(cuda):
+    """the library keeps no state between calls (descriptors travel in the kernel arguments,
+    the error text is per thread): four host threads, each on a stream of its own, step their
+    own tensors at the same time -- ctypes drops the interpreter lock during the calls -- and
+    every result equals the same steps made one after the other; a refusal in one thread
+    leaves its message in that thread only"""
+    import threading
+    from quantfour_adamw_cuda_amd import _lib
+    gen = torch.Generator().manual_seed(77)
+    nthreads, steps = 4, 12
+    sizes = [150_001 + 4096 * i for i in range(nthreads)]
+    p0s = [torch.randn(n, generator=gen) * 0.02 for n in sizes]
+    gs = [[grads_config1(gen, n).to(torch.bfloat16).to(cuda) for _ in range(steps)] for n in sizes]
+    seq = [DeviceTensor(p0, cuda) for p0 in p0s]
+    for d, g_list in zip(seq, gs):
+        for t, g in enumerate(g_list, 1):
+            q4.fused_4bit(d.p, g, d.m, d.v, d.sm, d.sv, *[HP[k] for k in ("beta1", "beta2", "lr", "weight_decay", "eps")], t)
+    torch.cuda.synchronize()
+    par = [DeviceTensor(p0, cuda) for p0 in p0s]
+    errors, messages = [], [None] * nthreads
+    barrier = threading.Barrier(nthreads)
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream(device=cuda)
+            L = _lib.load()
+            barrier.wait()
+            with torch.cuda.stream(stream):
+                d = par[i]
+                for t, g in enumerate(gs[i], 1):
+                    q4.fused_4bit(d.p, g, d.m, d.v, d.sm, d.sv,
+                                  *[HP[k] for k in ("beta1", "beta2", "lr", "weight_decay", "eps")], t)
+                    if i == 0 and t == 3:      # a refusal: nothing launched, message stays in this thread
+                        rc = L.q4adamw_fused_4bit(d.p.data_ptr() + 4, g.data_ptr(), d.m.data_ptr(), d.v.data_ptr(),
+                                                  d.sm.data_ptr(), d.sv.data_ptr(), 1000, 0, 1, 0.9, 0.999, 1e-3,
+                                                  0.01, 1e-8, 1.0, stream.cuda_stream)
+                        assert rc == -2
+                messages[i] = L.q4adamw_last_error().decode()
+            stream.synchronize()
+        except Exception as e:   # noqa: BLE001
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(nthreads)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=120)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for a, b in zip(seq, par):
+        for x, y in zip((a.p, a.m, a.v, a.sm, a.sv), (b.p, b.m, b.v, b.sm, b.sv)):
+            assert torch.equal(x, y)
+    assert "aligned" in messages[0] and all(m == "" for m in messages[1:]), messages
+
+
 @pytest.mark.parametrize("p_dtype,g_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
                                              (torch.bfloat16, torch.bfloat16)])
 def test_non_finite_gradients(cuda, p_dtype, g_dtype):
