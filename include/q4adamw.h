@@ -30,8 +30,14 @@
 extern "C" {
 #endif
 
+/* Element types of parameters and gradients (p_dtype, g_dtype), in any combination.
+ * The reference dispatches on the parameter's type over double, float and half
+ * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, optim/cuda_adamw_kernels.cu:443) and takes the
+ * gradient to have the same type; float and half are here, bfloat16 is added, and the
+ * arithmetic is fp32 whatever the storage type. */
 #define Q4ADAMW_FP32 0
 #define Q4ADAMW_BF16 1
+#define Q4ADAMW_FP16 2
 
 #define Q4ADAMW_BLOCK 128 /* elements per quantization block (one scale each) */
 
@@ -43,9 +49,9 @@ extern "C" {
 /*
  * One quantized tensor.  Field order follows the tensor arguments of
  * fused_4bit (optim/cuda_fused_interface.cc:19-21).
- *   p             numel elements, fp32 or bf16, 16-byte aligned
- *   g             numel elements, fp32 or bf16, 16-byte aligned (8 bytes suffice for a
- *                 bf16 gradient of an fp32 parameter)
+ *   p             numel elements, fp32, bf16 or fp16, 16-byte aligned
+ *   g             numel elements, fp32, bf16 or fp16, 16-byte aligned (8 bytes suffice for a
+ *                 16-bit gradient of an fp32 parameter)
  *   exp_avg       (numel+1)/2 bytes; byte i = code(2i) | code(2i+1) << 4
  *   exp_avg_sq    same layout
  *   exp_avg_scale ceil(numel/128) fp32 block scales of exp_avg

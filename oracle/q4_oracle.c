@@ -184,12 +184,54 @@ static inline uint16_t f32_to_bf16(float f) {
     return (uint16_t)(u >> 16);
 }
 
-/* dtype tags shared by every entry point here: 0 = fp32, 1 = bf16 */
+/* IEEE binary16 -> fp32, exact (subnormals are m * 2^-24) */
+static inline float f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 0x3ffu;
+    uint32_t u;
+    float f;
+    if (e == 0) {
+        f = (float)m * 5.9604644775390625e-08f;
+        memcpy(&u, &f, 4);
+        u |= sign;
+    } else if (e == 31) {
+        u = sign | 0x7f800000u | (m << 13);
+    } else {
+        u = sign | ((e + 112u) << 23) | (m << 13);
+    }
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* fp32 -> IEEE binary16, round to nearest even; overflow goes to infinity, NaN stays quiet */
+static inline uint16_t f32_to_f16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    u &= 0x7fffffffu;
+    if (u > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((u >> 13) & 0x3ffu));
+    if (u >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);           /* 65536 and above, infinity */
+    if (u < 0x38800000u) {                                             /* below 2^-14: subnormal or zero */
+        float a;
+        memcpy(&a, &u, 4);
+        return (uint16_t)(sign | (uint16_t)lrintf(a * 16777216.0f));    /* multiples of 2^-24, ties to even */
+    }
+    u += 0xfffu + ((u >> 13) & 1u);
+    return (uint16_t)(sign | (uint16_t)((u >> 13) - (112u << 10)));    /* 65520 and above round to infinity */
+}
+
+/* the two conversions, exported for their known-answer test */
+float q4o_f16_to_f32(uint16_t h) { return f16_to_f32(h); }
+uint16_t q4o_f32_to_f16(float f) { return f32_to_f16(f); }
+
+/* dtype tags shared by every entry point here: 0 = fp32, 1 = bf16, 2 = fp16 */
 static inline float load_elem(const void *base, int dtype, int64_t i) {
-    return dtype ? bf16_to_f32(((const uint16_t *)base)[i]) : ((const float *)base)[i];
+    if (dtype == 1) return bf16_to_f32(((const uint16_t *)base)[i]);
+    if (dtype == 2) return f16_to_f32(((const uint16_t *)base)[i]);
+    return ((const float *)base)[i];
 }
 static inline void store_elem(void *base, int dtype, int64_t i, float x) {
-    if (dtype) ((uint16_t *)base)[i] = f32_to_bf16(x);
+    if (dtype == 1) ((uint16_t *)base)[i] = f32_to_bf16(x);
+    else if (dtype == 2) ((uint16_t *)base)[i] = f32_to_f16(x);
     else ((float *)base)[i] = x;
 }
 

@@ -7,7 +7,7 @@ function restates (reference file:line) and for its pinning status.
 All tensors are numpy arrays (or anything exposing the buffer protocol through
 ``numpy.asarray``) that are updated IN PLACE, like the reference's kernels update
 their torch tensors in place (optim/cuda_fused_interface.cc:19-39).
-bf16 data is passed as uint16 bit patterns.
+bf16 data is passed as uint16 bit patterns, fp16 data as numpy float16.
 """
 import ctypes
 import os
@@ -19,7 +19,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libq4oracle.so")
 
 BLOCK = 128
-FP32, BF16 = 0, 1
+FP32, BF16, FP16 = 0, 1, 2
 
 
 def build(force=False):
@@ -51,6 +51,10 @@ def lib():
         L.q4o_step_unquant.argtypes = [vp, vp, vp, vp, i64, ci, ci, f, f, f, f, f, f]
         L.q4o_dequant.argtypes = [vp, vp, i64, ci, vp]
         L.q4o_quant.argtypes = [vp, i64, ci, vp, vp]
+        L.q4o_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.q4o_f16_to_f32.restype = f
+        L.q4o_f32_to_f16.argtypes = [f]
+        L.q4o_f32_to_f16.restype = ctypes.c_uint16
         _lib = L
     return _lib
 
@@ -62,9 +66,11 @@ def _ptr(a):
 def _dtype_tag(a):
     if a.dtype == np.float32:
         return FP32
+    if a.dtype == np.float16:
+        return FP16
     if a.dtype == np.uint16:
         return BF16
-    raise TypeError(f"expected float32 or uint16 (bf16 bits), got {a.dtype}")
+    raise TypeError(f"expected float32, float16 or uint16 (bf16 bits), got {a.dtype}")
 
 
 def tables(which):
@@ -159,7 +165,7 @@ def quant(x, which):
 # has no counterpart.
 # ---------------------------------------------------------------------------
 def as_f32(g):
-    """fp32 values of a gradient given as float32 or as bf16 bit patterns (uint16)."""
+    """fp32 values of a gradient given as float32, float16 or as bf16 bit patterns (uint16)."""
     g = np.asarray(g)
     if g.dtype == np.uint16:
         return (g.astype(np.uint32) << 16).view(np.float32)

@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libq4adamw.so")
 
-FP32, BF16 = 0, 1
+FP32, BF16, FP16 = 0, 1, 2
 BLOCK = 128
 
 

@@ -95,9 +95,8 @@ static int make_consts(float beta1, float beta2, float lr, float wd, float eps, 
 static bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 static int check_dtypes(int p_dtype, int g_dtype) {
-  if ((p_dtype != Q4ADAMW_FP32 && p_dtype != Q4ADAMW_BF16) ||
-      (g_dtype != Q4ADAMW_FP32 && g_dtype != Q4ADAMW_BF16))
-    return fail(Q4ADAMW_ERR_ARG, "dtype tag must be Q4ADAMW_FP32 or Q4ADAMW_BF16");
+  if (p_dtype < Q4ADAMW_FP32 || p_dtype > Q4ADAMW_FP16 || g_dtype < Q4ADAMW_FP32 || g_dtype > Q4ADAMW_FP16)
+    return fail(Q4ADAMW_ERR_ARG, "dtype tag must be Q4ADAMW_FP32, Q4ADAMW_BF16 or Q4ADAMW_FP16");
   return 0;
 }
 
@@ -130,54 +129,63 @@ static int launch_small_batch(SmallArgs &a, uint64_t chunks, void (*kernel)(cons
 typedef void (*FusedKernel)(const FusedArgs);
 typedef void (*SmallKernel)(const SmallArgs);
 
+// Kernel of a family for the (parameter, gradient) element types of a call: the tags
+// 0 = fp32, 1 = bf16, 2 = fp16 become template arguments.
+#define Q4_PICK_PG(KERNEL, ...)                                                   \
+  switch (p_dtype * 3 + g_dtype) {                                                \
+    case 0: return KERNEL<0, 0, __VA_ARGS__>;                                     \
+    case 1: return KERNEL<0, 1, __VA_ARGS__>;                                     \
+    case 2: return KERNEL<0, 2, __VA_ARGS__>;                                     \
+    case 3: return KERNEL<1, 0, __VA_ARGS__>;                                     \
+    case 4: return KERNEL<1, 1, __VA_ARGS__>;                                     \
+    case 5: return KERNEL<1, 2, __VA_ARGS__>;                                     \
+    case 6: return KERNEL<2, 0, __VA_ARGS__>;                                     \
+    case 7: return KERNEL<2, 1, __VA_ARGS__>;                                     \
+    default: return KERNEL<2, 2, __VA_ARGS__>;                                    \
+  }
+
 template <bool EXT, bool SR>
-static FusedKernel pick_fused_ext(bool pb, bool gb) {
-  if (!pb && !gb) return fused_4bit_kernel<false, false, EXT, SR>;
-  if (!pb && gb) return fused_4bit_kernel<false, true, EXT, SR>;
-  if (pb && !gb) return fused_4bit_kernel<true, false, EXT, SR>;
-  return fused_4bit_kernel<true, true, EXT, SR>;
+static FusedKernel pick_fused_ext(int p_dtype, int g_dtype) {
+  Q4_PICK_PG(fused_4bit_kernel, EXT, SR)
 }
 
 // stochastic rounding comes with the gradient options' kernels only
 static FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext, bool sr = false) {
-  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  if (sr) return pick_fused_ext<true, true>(pb, gb);
-  return ext ? pick_fused_ext<true, false>(pb, gb) : pick_fused_ext<false, false>(pb, gb);
+  if (sr) return pick_fused_ext<true, true>(p_dtype, g_dtype);
+  return ext ? pick_fused_ext<true, false>(p_dtype, g_dtype) : pick_fused_ext<false, false>(p_dtype, g_dtype);
 }
 
 template <bool EXT>
-static SmallKernel pick_small_ext(bool pb, bool gb) {
-  if (!pb && !gb) return single_tensor_kernel<false, false, EXT>;
-  if (!pb && gb) return single_tensor_kernel<false, true, EXT>;
-  if (pb && !gb) return single_tensor_kernel<true, false, EXT>;
-  return single_tensor_kernel<true, true, EXT>;
+static SmallKernel pick_small_ext(int p_dtype, int g_dtype) {
+  Q4_PICK_PG(single_tensor_kernel, EXT)
 }
 
 static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
-  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  return ext ? pick_small_ext<true>(pb, gb) : pick_small_ext<false>(pb, gb);
+  return ext ? pick_small_ext<true>(p_dtype, g_dtype) : pick_small_ext<false>(p_dtype, g_dtype);
 }
 
 typedef void (*Rank1Kernel)(const Rank1Args);
 typedef void (*Rank1StatKernel)(const Rank1StatArgs);
 
 template <bool EXT, bool SR>
-static Rank1Kernel pick_rank1_ext(bool pb, bool gb) {
-  if (!pb && !gb) return fused_4bit_rank1_kernel<false, false, EXT, SR>;
-  if (!pb && gb) return fused_4bit_rank1_kernel<false, true, EXT, SR>;
-  if (pb && !gb) return fused_4bit_rank1_kernel<true, false, EXT, SR>;
-  return fused_4bit_rank1_kernel<true, true, EXT, SR>;
+static Rank1Kernel pick_rank1_ext(int p_dtype, int g_dtype) {
+  Q4_PICK_PG(fused_4bit_rank1_kernel, EXT, SR)
 }
 
 static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr) {
-  const bool pb = p_dtype == Q4ADAMW_BF16, gb = g_dtype == Q4ADAMW_BF16;
-  if (sr) return pick_rank1_ext<true, true>(pb, gb);
-  return ext ? pick_rank1_ext<true, false>(pb, gb) : pick_rank1_ext<false, false>(pb, gb);
+  if (sr) return pick_rank1_ext<true, true>(p_dtype, g_dtype);
+  return ext ? pick_rank1_ext<true, false>(p_dtype, g_dtype) : pick_rank1_ext<false, false>(p_dtype, g_dtype);
+}
+
+template <bool EXT>
+static Rank1StatKernel pick_rank1_stats_ext(int g_dtype) {
+  if (g_dtype == Q4ADAMW_BF16) return rank1_stats_kernel<Q4ADAMW_BF16, EXT>;
+  if (g_dtype == Q4ADAMW_FP16) return rank1_stats_kernel<Q4ADAMW_FP16, EXT>;
+  return rank1_stats_kernel<Q4ADAMW_FP32, EXT>;
 }
 
 static Rank1StatKernel pick_rank1_stats(int g_dtype, bool ext) {
-  if (g_dtype == Q4ADAMW_BF16) return ext ? rank1_stats_kernel<true, true> : rank1_stats_kernel<true, false>;
-  return ext ? rank1_stats_kernel<false, true> : rank1_stats_kernel<false, false>;
+  return ext ? pick_rank1_stats_ext<true>(g_dtype) : pick_rank1_stats_ext<false>(g_dtype);
 }
 
 // Fills the kernels' view of the caller's gradient options; returns whether the
@@ -294,11 +302,11 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
-  // a lane reads 8 consecutive elements at once when parameters and gradients are bf16, else 4
-  const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
-  const bool wide = p_bf16 && g_dtype == Q4ADAMW_BF16;   // 8 elements per lane
-  const int64_t chunk_elems = wide ? Geometry<true, true>::kChunk : Geometry<false, false>::kChunk;
-  const uintptr_t p_align = 16, g_align = g_dtype == Q4ADAMW_BF16 ? (p_bf16 ? 16 : 8) : 16;
+  // a lane reads 8 consecutive elements at once when parameters and gradients are 16-bit types, else 4
+  const bool p_half = p_dtype != Q4ADAMW_FP32, g_half = g_dtype != Q4ADAMW_FP32;
+  const bool wide = p_half && g_half;   // 8 elements per lane
+  const int64_t chunk_elems = wide ? Geometry<1, 1>::kChunk : Geometry<0, 0>::kChunk;
+  const uintptr_t p_align = 16, g_align = g_half ? (p_half ? 16 : 8) : 16;
   const uintptr_t code_align = wide ? 4 : 2;
   // validate everything before the first launch
   for (int i = 0; i < count; ++i) {
@@ -360,9 +368,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   sa.go = a.go;
   sa.b2 = a.sc.b2;
   sa.r2 = a.sc.r2;
-  const bool p_bf16 = p_dtype == Q4ADAMW_BF16;
-  const bool wide = p_bf16 && g_dtype == Q4ADAMW_BF16;   // 8 elements per lane
-  const int64_t chunk_elems = wide ? Geometry<true, true>::kChunk : Geometry<false, false>::kChunk;
+  const bool wide = p_dtype != Q4ADAMW_FP32 && g_dtype != Q4ADAMW_FP32;   // 8 elements per lane
+  const int64_t chunk_elems = wide ? Geometry<1, 1>::kChunk : Geometry<0, 0>::kChunk;
   for (int i = 0; i < count; ++i) {
     const q4adamw_rank1_tensor &t = tensors[i];
     if (t.rows < 0 || t.cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
@@ -504,7 +511,7 @@ int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, in
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
-  const uintptr_t pa = p_dtype == Q4ADAMW_BF16 ? 2 : 4, ga = g_dtype == Q4ADAMW_BF16 ? 2 : 4;
+  const uintptr_t pa = p_dtype != Q4ADAMW_FP32 ? 2 : 4, ga = g_dtype != Q4ADAMW_FP32 ? 2 : 4;
   for (int i = 0; i < count; ++i) {
     const q4adamw_small_tensor &t = tensors[i];
     if (t.numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
@@ -562,8 +569,7 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
     return fail(Q4ADAMW_ERR_ARG, "workspace smaller than Q4ADAMW_NORM_WORKSPACE_BYTES");
   if (!aligned(workspace, 8) || !aligned(out3, 4) || (grad_scale_dev && !aligned(grad_scale_dev, 4)))
     return fail(Q4ADAMW_ERR_ALIGN, "workspace must be 8-byte, scalars 4-byte aligned");
-  const bool bf16 = g_dtype == Q4ADAMW_BF16;
-  const int64_t chunk_elems = kNormChunkBytes / (bf16 ? 2 : 4);
+  const int64_t chunk_elems = kNormChunkBytes / (g_dtype != Q4ADAMW_FP32 ? 2 : 4);
   for (int i = 0; i < count; ++i) {
     if (grads[i].numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
     if (grads[i].numel == 0) continue;
@@ -581,8 +587,9 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
   auto launch = [&]() -> int {
     finish_prefix(a);
     a.nchunks = (uint32_t)chunks;
-    if (bf16) hipLaunchKernelGGL(grad_sumsq_kernel<true>, dim3(kNormPartials), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(grad_sumsq_kernel<false>, dim3(kNormPartials), dim3(256), 0, s, a);
+    if (g_dtype == Q4ADAMW_BF16) hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_BF16>, dim3(kNormPartials), dim3(256), 0, s, a);
+    else if (g_dtype == Q4ADAMW_FP16) hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_FP16>, dim3(kNormPartials), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_FP32>, dim3(kNormPartials), dim3(256), 0, s, a);
     Q4_HIP(hipGetLastError());
     a.first = 0u;
     a.ntensors = 0;
@@ -688,6 +695,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1008; }
+int q4adamw_version(void) { return 1009; }
 
 }  // extern "C"

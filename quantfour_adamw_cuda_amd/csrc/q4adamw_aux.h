@@ -7,7 +7,7 @@ namespace q4 {
 
 // Non-quantized step for small tensors (cuda_adamw_kernels.cu:100-133): fp32
 // moments in place, same derived scalars and operation order as the fused path.
-template <bool PBF, bool GBF, bool EXT>
+template <int PT, int GT, bool EXT>
 __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args) {
   const uint32_t chunk = blockIdx.x;
   float gscale = 1.0f;
@@ -21,23 +21,19 @@ __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args
   const int64_t end = base + kSmallChunk < T.numel ? base + kSmallChunk : T.numel;
   if (cancelled) {  // a cancelled step still clears the gradients it was asked to clear
     for (int64_t i = base + threadIdx.x; i < end; i += 256) {
-      if (GBF) as_global<uint16_t>(const_cast<void *>(T.g))[i] = 0;
-      else as_global<float>(const_cast<void *>(T.g))[i] = 0.0f;
+      store_scalar<GT>(const_cast<void *>(T.g), i, 0.0f);
     }
     return;
   }
   for (int64_t i = base + threadIdx.x; i < end; i += 256) {
-    float gi = GBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.g)[i])
-                   : as_global<const float>(T.g)[i];
+    float gi = load_scalar<GT>(T.g, i);
     if (EXT) {
       gi *= gscale;
       if (zero_g) {
-        if (GBF) as_global<uint16_t>(const_cast<void *>(T.g))[i] = 0;
-        else as_global<float>(const_cast<void *>(T.g))[i] = 0.0f;
+        store_scalar<GT>(const_cast<void *>(T.g), i, 0.0f);
       }
     }
-    const float pi = PBF ? bf16_bits_to_f32(as_global<const uint16_t>(T.p)[i])
-                         : as_global<const float>(T.p)[i];
+    const float pi = load_scalar<PT>(T.p, i);
     const float m = sc.b1 * as_global<const float>(T.m)[i] + sc.r1 * gi;
     const float v = sc.b2 * as_global<const float>(T.v)[i] + sc.r2 * (gi * gi);
     as_global<float>(T.m)[i] = m;
@@ -45,8 +41,7 @@ __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args
     // exact form here: these tensors are tiny, so the divisions cost nothing
     const float den = __builtin_sqrtf(v) / sc.c2s + sc.eps;
     const float pn = pi * sc.wdu - sc.ss * (m / den);
-    if (PBF) as_global<uint16_t>(T.p)[i] = (uint16_t)f32_to_bf16_bits(pn);
-    else as_global<float>(T.p)[i] = pn;
+    store_scalar<PT>(T.p, i, pn);
   }
 }
 
@@ -65,9 +60,9 @@ __device__ __forceinline__ double workgroup_sum(double x, double *lds4) {
 
 // Squares are exact in fp64 and summed there: four accumulators per thread, chunks in
 // grid-stride order, so the sum depends on the tensor list only, not on scheduling.
-template <bool GBF>
+template <int GT>
 __global__ __launch_bounds__(256) void grad_sumsq_kernel(const NormArgs args) {
-  constexpr int kElemBytes = GBF ? 2 : 4;
+  constexpr int kElemBytes = GT ? 2 : 4;
   constexpr int64_t kChunkElems = kNormChunkBytes / kElemBytes;
   __shared__ double lds4[4];
   const int tid = threadIdx.x;
@@ -88,9 +83,9 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const NormArgs args) {
         const uint32_t u[4] = {w[k].x, w[k].y, w[k].z, w[k].w};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-          if (GBF) {
+          if constexpr (GT != 0) {
             float lo, hi;
-            widen_bf16_pair(u[c], lo, hi);
+            widen_pair<GT>(u[c], lo, hi);
             acc[c] = __builtin_fma((double)lo, (double)lo, acc[c]);
             acc[c] = __builtin_fma((double)hi, (double)hi, acc[c]);
           } else {
@@ -101,8 +96,7 @@ __global__ __launch_bounds__(256) void grad_sumsq_kernel(const NormArgs args) {
       }
     } else {
       for (int64_t i = tid; i < rem; i += 256) {
-        const double x = GBF ? (double)bf16_bits_to_f32(as_global<const uint16_t>(cb)[i])
-                             : (double)as_global<const float>(cb)[i];
+        const double x = (double)load_scalar<GT>(cb, i);
         acc[0] = __builtin_fma(x, x, acc[0]);
       }
     }

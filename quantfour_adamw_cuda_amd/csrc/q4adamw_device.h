@@ -1,5 +1,5 @@
 // Device helpers of the 4-bit AdamW kernels: address spaces and buffer resources, wave
-// reductions, bf16 conversion, element loads and stores, the exact quantizers, the rounding
+// reductions, 16-bit element conversion, element loads and stores, the exact quantizers, the rounding
 // noise, the tensor search.
 #pragma once
 #include "q4adamw_args.h"
@@ -73,39 +73,74 @@ __device__ __forceinline__ float row_max16(float x) {
   return bits2f(u);
 }
 
-__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return bits2f(h << 16); }
-
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nearest even
-  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
-}
-
+// Element types of parameters and gradients, by the tags of include/q4adamw.h:
+// 0 = fp32, 1 = bf16, 2 = fp16.  A non-zero tag is a 16-bit type.
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// two fp32 -> two bf16 (round to nearest even) in one 32-bit word, lo in the low half
-__device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+// one 16-bit pattern -> fp32 (exact)
+template <int DT>
+__device__ __forceinline__ float widen_bits(uint32_t h) {
+  static_assert(DT == Q4ADAMW_BF16 || DT == Q4ADAMW_FP16, "a 16-bit element type");
+  if (DT == Q4ADAMW_BF16) return bits2f(h << 16);
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
-__device__ __forceinline__ void widen_bf16_pair(uint32_t w, float &lo, float &hi) {
-  lo = bits2f(w << 16);
-  hi = bits2f(w & 0xffff0000u);
+// fp32 -> one 16-bit pattern, round to nearest even
+template <int DT>
+__device__ __forceinline__ uint32_t narrow_bits(float f) {
+  static_assert(DT == Q4ADAMW_BF16 || DT == Q4ADAMW_FP16, "a 16-bit element type");
+  if (DT == Q4ADAMW_BF16) return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// two fp32 -> two 16-bit values (round to nearest even) in one 32-bit word, lo in the low half
+template <int DT>
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  if (DT == Q4ADAMW_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
+}
+
+template <int DT>
+__device__ __forceinline__ void widen_pair(uint32_t w, float &lo, float &hi) {
+  if (DT == Q4ADAMW_BF16) {
+    lo = bits2f(w << 16);
+    hi = bits2f(w & 0xffff0000u);
+  } else {
+    const f32x2 f = __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+    lo = f.x;
+    hi = f.y;
+  }
+}
+
+// element i of an array of element type DT, as fp32
+template <int DT>
+__device__ __forceinline__ float load_scalar(const void *base, int64_t i) {
+  if constexpr (DT == Q4ADAMW_FP32) return as_global<const float>(base)[i];
+  else return widen_bits<DT>(as_global<const uint16_t>(base)[i]);
+}
+
+template <int DT>
+__device__ __forceinline__ void store_scalar(void *base, int64_t i, float x) {
+  if constexpr (DT == Q4ADAMW_FP32) as_global<float>(base)[i] = x;
+  else as_global<uint16_t>(base)[i] = (uint16_t)narrow_bits<DT>(x);
 }
 
 // N consecutive elements (N = 4 or 8) starting at element e0 of the tile at base
-template <bool BF, int N, bool FULL>
+template <int DT, int N, bool FULL>
 __device__ __forceinline__ void load_elems(const void *base, uint32_t e0, int nv, float (&x)[N]) {
   if (FULL) {
-    if (BF && N == 4) {
+    if constexpr (DT != 0 && N == 4) {
       const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(tile_rsrc(base), e0 * 2, 0, kNt);
-      widen_bf16_pair(w.x, x[0], x[1]);
-      widen_bf16_pair(w.y, x[2], x[3]);
-    } else if (BF) {
+      widen_pair<DT>(w.x, x[0], x[1]);
+      widen_pair<DT>(w.y, x[2], x[3]);
+    } else if constexpr (DT != 0) {
       const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(base), e0 * 2, 0, kNt);
-      widen_bf16_pair(w.x, x[0], x[1]);
-      widen_bf16_pair(w.y, x[2], x[3]);
-      widen_bf16_pair(w.z, x[N - 4], x[N - 3]);
-      widen_bf16_pair(w.w, x[N - 2], x[N - 1]);
+      widen_pair<DT>(w.x, x[0], x[1]);
+      widen_pair<DT>(w.y, x[2], x[3]);
+      widen_pair<DT>(w.z, x[N - 4], x[N - 3]);
+      widen_pair<DT>(w.w, x[N - 2], x[N - 1]);
     } else {
 #pragma unroll
       for (int k = 0; k < N; k += 4) {
@@ -118,27 +153,26 @@ __device__ __forceinline__ void load_elems(const void *base, uint32_t e0, int nv
     for (int j = 0; j < N; ++j) {
       x[j] = 0.0f;
       if (j < nv) {
-        x[j] = BF ? bf16_bits_to_f32(as_global<const uint16_t>(base)[e0 + j])
-                  : as_global<const float>(base)[e0 + j];
+        x[j] = load_scalar<DT>(base, e0 + j);
       }
     }
   }
 }
 
-template <bool BF, int N, bool FULL>
+template <int DT, int N, bool FULL>
 __device__ __forceinline__ void store_elems(void *base, uint32_t e0, int nv, const float (&x)[N]) {
   if (FULL) {
-    if (BF && N == 4) {
+    if constexpr (DT != 0 && N == 4) {
       u32x2 w;
-      w.x = pack_bf16_pair(x[0], x[1]);
-      w.y = pack_bf16_pair(x[2], x[3]);
+      w.x = pack_pair<DT>(x[0], x[1]);
+      w.y = pack_pair<DT>(x[2], x[3]);
       __builtin_amdgcn_raw_buffer_store_b64(w, tile_rsrc(base), e0 * 2, 0, kNt);
-    } else if (BF) {
+    } else if constexpr (DT != 0) {
       u32x4 w;
-      w.x = pack_bf16_pair(x[0], x[1]);
-      w.y = pack_bf16_pair(x[2], x[3]);
-      w.z = pack_bf16_pair(x[N - 4], x[N - 3]);
-      w.w = pack_bf16_pair(x[N - 2], x[N - 1]);
+      w.x = pack_pair<DT>(x[0], x[1]);
+      w.y = pack_pair<DT>(x[2], x[3]);
+      w.z = pack_pair<DT>(x[N - 4], x[N - 3]);
+      w.w = pack_pair<DT>(x[N - 2], x[N - 1]);
       __builtin_amdgcn_raw_buffer_store_b128(w, tile_rsrc(base), e0 * 2, 0, kNt);
     } else {
 #pragma unroll
@@ -151,22 +185,21 @@ __device__ __forceinline__ void store_elems(void *base, uint32_t e0, int nv, con
 #pragma unroll
     for (int j = 0; j < N; ++j) {
       if (j < nv) {
-        if (BF) as_global<uint16_t>(base)[e0 + j] = (uint16_t)f32_to_bf16_bits(x[j]);
-        else as_global<float>(base)[e0 + j] = x[j];
+        store_scalar<DT>(base, e0 + j, x[j]);
       }
     }
   }
 }
 
-// zeros over the N elements that load_elems<BF, N, FULL> read
-template <bool BF, int N, bool FULL>
+// zeros over the N elements that load_elems<DT, N, FULL> read
+template <int DT, int N, bool FULL>
 __device__ __forceinline__ void zero_elems(void *base, uint32_t e0, int nv) {
   if (FULL) {
     const u32x4 z4 = {0u, 0u, 0u, 0u};
-    if (BF && N == 4) {
+    if (DT && N == 4) {
       const u32x2 z2 = {0u, 0u};
       __builtin_amdgcn_raw_buffer_store_b64(z2, tile_rsrc(base), e0 * 2, 0, kNt);
-    } else if (BF) {
+    } else if (DT) {
       __builtin_amdgcn_raw_buffer_store_b128(z4, tile_rsrc(base), e0 * 2, 0, kNt);
     } else {
 #pragma unroll
@@ -177,7 +210,7 @@ __device__ __forceinline__ void zero_elems(void *base, uint32_t e0, int nv) {
 #pragma unroll
     for (int j = 0; j < N; ++j) {
       if (j < nv) {
-        if (BF) as_global<uint16_t>(base)[e0 + j] = 0;
+        if (DT) as_global<uint16_t>(base)[e0 + j] = 0;
         else as_global<float>(base)[e0 + j] = 0.0f;
       }
     }
@@ -186,18 +219,18 @@ __device__ __forceinline__ void zero_elems(void *base, uint32_t e0, int nv) {
 
 // Zeros over one tile of a gradient tensor: what is left of a step's work when an
 // overflow flag cancels it and the caller asked for the gradients to be cleared.
-template <bool BF, int N>
+template <int DT, int N>
 __device__ __forceinline__ void zero_tile(const void *g, int64_t tile, int64_t numel, int lane) {
   constexpr int64_t kTile = 64 * N;
   const int64_t tb = tile * kTile;
   if (tb >= numel) return;
-  void *g_tile = static_cast<char *>(const_cast<void *>(g)) + tb * (BF ? 2 : 4);
+  void *g_tile = static_cast<char *>(const_cast<void *>(g)) + tb * (DT ? 2 : 4);
   const uint32_t e0 = (uint32_t)lane * N;
   if (tb + kTile <= numel) {
-    zero_elems<BF, N, true>(g_tile, e0, N);
+    zero_elems<DT, N, true>(g_tile, e0, N);
   } else {
     const int64_t rem = numel - tb - (int64_t)e0;
-    zero_elems<BF, N, false>(g_tile, e0, rem >= N ? N : (rem > 0 ? (int)rem : 0));
+    zero_elems<DT, N, false>(g_tile, e0, rem >= N ? N : (rem > 0 ? (int)rem : 0));
   }
 }
 

@@ -8,9 +8,9 @@ namespace q4 {
 
 // Geometry of the fused kernel: a lane owns 16 bytes of the widest of the parameter and
 // gradient streams, so that no stream needs two accesses per lane.
-template <bool PBF, bool GBF>
+template <int PT, int GT>
 struct Geometry {
-  static constexpr int kEpl = (PBF && GBF) ? 8 : 4;      // elements per lane
+  static constexpr int kEpl = (PT && GT) ? 8 : 4;      // elements per lane
   static constexpr int kTile = 64 * kEpl;                // elements per wave
   static constexpr int kChunk = kTile * kWaves;          // elements per workgroup
   static constexpr int kLanesPerBlock = Q4ADAMW_BLOCK / kEpl;   // 32 or 16
@@ -27,18 +27,18 @@ struct Geometry {
 // step's new statistics (complete before this kernel starts) quantize.
 // SR: both moments are rounded stochastically between the two neighbouring code-book
 // entries; the noise of element e is a hash of e and the tensor's salt of this step.
-template <bool PBF, bool GBF, bool FULL, bool EXT, bool RANK1, bool SR, typename Desc>
+template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, typename Desc>
 __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g, uint32_t salt) {
-  using G = Geometry<PBF, GBF>;
+  using G = Geometry<PT, GT>;
   constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
   // block; the per-lane part is a small 32-bit offset.
   const int64_t numel = T.numel;
   const int64_t tb = tile * G::kTile;
-  const void *p_tile = static_cast<const char *>(T.p) + tb * (PBF ? 2 : 4);
-  const void *g_tile = static_cast<const char *>(T.g) + tb * (GBF ? 2 : 4);
+  const void *p_tile = static_cast<const char *>(T.p) + tb * (PT ? 2 : 4);
+  const void *g_tile = static_cast<const char *>(T.g) + tb * (GT ? 2 : 4);
   const uint8_t *m_tile = T.m + (tb >> 1);
   const uint8_t *v_tile = T.v + (tb >> 1);
   const float *sm_tile = T.sm + tile * G::kBlocksPerTile;
@@ -85,12 +85,12 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   }
 
   float p[N], g[N];
-  load_elems<PBF, N, FULL>(p_tile, e0, nv, p);
-  load_elems<GBF, N, FULL>(g_tile, e0, nv, g);
+  load_elems<PT, N, FULL>(p_tile, e0, nv, p);
+  load_elems<GT, N, FULL>(g_tile, e0, nv, g);
   if (EXT) {
 #pragma unroll
     for (int j = 0; j < N; ++j) g[j] *= gscale;
-    if (zero_g) zero_elems<GBF, N, FULL>(const_cast<void *>(g_tile), e0, nv);
+    if (zero_g) zero_elems<GT, N, FULL>(const_cast<void *>(g_tile), e0, nv);
   }
   uint32_t mw = 0, vw = 0;
   if (FULL) {
@@ -160,7 +160,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
     av = __builtin_fmaxf(av, v);
   }
-  store_elems<PBF, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
+  store_elems<PT, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
 
   // block scales (exact: max is order independent)
   const float v_lane_max = av;
@@ -318,9 +318,9 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   }
 }
 
-template <bool PBF, bool GBF, bool EXT, bool SR>
+template <int PT, int GT, bool EXT, bool SR>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
-  using G = Geometry<PBF, GBF>;
+  using G = Geometry<PT, GT>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
   if (cancelled) {  // a cancelled step still clears the gradients it was asked to clear
-    zero_tile<GBF, G::kEpl>(T.g, tile, T.numel, lane);
+    zero_tile<GT, G::kEpl>(T.g, tile, T.numel, lane);
     return;
   }
   const int64_t begin = tile * G::kTile;
@@ -345,9 +345,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   }
   const uint32_t salt = SR ? args.sr_salt[t] : 0u;
   if (begin + G::kTile <= T.numel)
-    process_tile<PBF, GBF, true, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PBF, GBF, false, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
@@ -365,7 +365,7 @@ constexpr int kStatCols = 512;           // columns per workgroup: 8 per lane
 // column maxima meet in LDS, and the tile issues one atomic per column and one per row
 // (atomics on the column vector are what this kernel's time depends on most: a tile of
 // 64 rows with four times as many of them took 1.25 to 2 times as long).
-template <bool GBF, bool EXT>
+template <int GT, bool EXT>
 __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
   constexpr int kAhead = 4;  // rows whose loads are in flight together
   __shared__ uint32_t row_bits[4][kStatRows];       // row maxima of each 16-lane quarter of the row's wave
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   const uint32_t quarter = (uint32_t)lane >> 4;
   for (int r0 = 0; r0 < nrows; r0 += kAhead) {
     // a group past the wave's last row repeats that row: maxima do not mind
-    u32x4 gw[kAhead][GBF ? 1 : 2];
+    u32x4 gw[kAhead][GT ? 1 : 2];
     uint32_t vw[kAhead];
     float r_old[kAhead];
 #pragma unroll
@@ -409,31 +409,31 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
       // row bases are uniform; the lane's column is a 32-bit offset
       const int64_t row_first = row * T.cols + (int64_t)cg * kStatCols;
       const uint32_t lane_elem = (uint32_t)lane * 8u;
-      const void *g_row = static_cast<const char *>(T.g) + row_first * (GBF ? 2 : 4);
+      const void *g_row = static_cast<const char *>(T.g) + row_first * (GT ? 2 : 4);
       const void *v_row = T.v + (row_first >> 1);
       vw[i] = 0u;
 #pragma unroll
-      for (int h = 0; h < (GBF ? 1 : 2); ++h) gw[i][h] = u32x4{0u, 0u, 0u, 0u};
+      for (int h = 0; h < (GT ? 1 : 2); ++h) gw[i][h] = u32x4{0u, 0u, 0u, 0u};
       if (active) {
         vw[i] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_row), lane_elem >> 1, 0, kNtReadOnly);
-        if (GBF) {
+        if (GT) {
           gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 2u, 0, kNtReadOnly);
         } else {
           gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u, 0, kNtReadOnly);
-          gw[i][GBF ? 0 : 1] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u + 16u, 0, kNtReadOnly);
+          gw[i][GT ? 0 : 1] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u + 16u, 0, kNtReadOnly);
         }
       }
     }
 #pragma unroll
     for (int i = 0; i < kAhead; ++i) {
       float g[8];
-      if (GBF) {
-        widen_bf16_pair(gw[i][0].x, g[0], g[1]);
-        widen_bf16_pair(gw[i][0].y, g[2], g[3]);
-        widen_bf16_pair(gw[i][0].z, g[4], g[5]);
-        widen_bf16_pair(gw[i][0].w, g[6], g[7]);
+      if constexpr (GT != 0) {
+        widen_pair<GT>(gw[i][0].x, g[0], g[1]);
+        widen_pair<GT>(gw[i][0].y, g[2], g[3]);
+        widen_pair<GT>(gw[i][0].z, g[4], g[5]);
+        widen_pair<GT>(gw[i][0].w, g[6], g[7]);
       } else {
-        const u32x4 lo = gw[i][0], hi = gw[i][GBF ? 0 : 1];
+        const u32x4 lo = gw[i][0], hi = gw[i][GT ? 0 : 1];
         g[0] = bits2f(lo.x); g[1] = bits2f(lo.y); g[2] = bits2f(lo.z); g[3] = bits2f(lo.w);
         g[4] = bits2f(hi.x); g[5] = bits2f(hi.y); g[6] = bits2f(hi.z); g[7] = bits2f(hi.w);
       }
@@ -482,9 +482,9 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   }
 }
 
-template <bool PBF, bool GBF, bool EXT, bool SR>
+template <int PT, int GT, bool EXT, bool SR>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
-  using G = Geometry<PBF, GBF>;
+  using G = Geometry<PT, GT>;
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
@@ -499,7 +499,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int64_t tile = (int64_t)(chunk - args.first_chunk[t]) * kWaves + wave;
   if (cancelled) {
-    zero_tile<GBF, G::kEpl>(T.g, tile, T.numel, lane);
+    zero_tile<GT, G::kEpl>(T.g, tile, T.numel, lane);
     return;
   }
   const int64_t begin = tile * G::kTile;
@@ -509,9 +509,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   }
   const uint32_t salt = SR ? args.sr_salt[t] : 0u;
   if (begin + G::kTile <= T.numel)
-    process_tile<PBF, GBF, true, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PBF, GBF, false, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
 }
 
 // After the update: the new statistics become the current ones and the buffers that

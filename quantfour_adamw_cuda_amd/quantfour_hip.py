@@ -12,7 +12,7 @@ import torch
 
 from . import _lib
 
-_DTYPE_TAG = {torch.float32: _lib.FP32, torch.bfloat16: _lib.BF16}
+_DTYPE_TAG = {torch.float32: _lib.FP32, torch.bfloat16: _lib.BF16, torch.float16: _lib.FP16}
 
 
 def state_sizes(numel):
@@ -24,7 +24,7 @@ def _tag(t, what):
     try:
         return _DTYPE_TAG[t.dtype]
     except KeyError:
-        raise TypeError(f"{what} must be float32 or bfloat16, got {t.dtype}") from None
+        raise TypeError(f"{what} must be float32, bfloat16 or float16, got {t.dtype}") from None
 
 
 def _check_common(p, g):

@@ -33,7 +33,8 @@ def bf16_round(x):
     return u.astype(np.uint16)
 
 
-def make(name, n, steps, hp, p_bf16=False, g_bf16=False, seed=0, special=None):
+def make(name, n, steps, hp, p_bf16=False, g_bf16=False, seed=0, special=None, p_f16=False, g_f16=False):
+    """bf16 tensors are stored as uint16 bit patterns, fp16 tensors as numpy float16"""
     rng = np.random.default_rng(seed)
     p = (rng.standard_normal(n) * 0.02).astype(np.float32)
     grads = []
@@ -46,8 +47,8 @@ def make(name, n, steps, hp, p_bf16=False, g_bf16=False, seed=0, special=None):
         if special is not None:
             special(g)
         grads.append(g)
-    p_in = bf16_round(p) if p_bf16 else p
-    g_in = [bf16_round(g) if g_bf16 else g for g in grads]
+    p_in = bf16_round(p) if p_bf16 else (p.astype(np.float16) if p_f16 else p)
+    g_in = [bf16_round(g) if g_bf16 else (g.astype(np.float16) if g_f16 else g) for g in grads]
     nb, nk = oc.state_sizes(n)
     m, v = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8)
     sm, sv = np.zeros(nk, np.float32), np.zeros(nk, np.float32)
@@ -151,6 +152,8 @@ if __name__ == "__main__":
     make("quant_fp32_bf16_n4099", 4099, 3, hp, g_bf16=True, seed=2)
     make("quant_bf16_bf16_n2050", 2050, 3, hp, p_bf16=True, g_bf16=True, seed=3)
     make("quant_driver_hp_n640", 640, 4, hp_driver, seed=4)
+    make("quant_fp16_fp16_n2309", 2309, 3, hp, p_f16=True, g_f16=True, seed=10)
+    make("quant_fp32_fp16_n1500", 1500, 3, hp, g_f16=True, seed=11)
     make_sr("sr_fp32_bf16_n3001", 3001, 3, hp, seed=5, sr_seed=0x0123456789ABCDEF, tensor_salt=7, g_bf16=True)
     make_sr("sr_fp32_fp32_n1100", 1100, 3, hp_driver, seed=6, sr_seed=42, tensor_salt=0)
     make_rank1("rank1_fp32_bf16_5x520", 5, 520, 3, hp, seed=7, g_bf16=True)

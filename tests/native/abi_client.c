@@ -5,7 +5,8 @@
  * not Python, and checks every result against the scalar C oracle (test
  * infrastructure, linked here as the checker only):
  *   - packed codes and block scales bit for bit, parameters within 1e-6 relative
- *     (fp32) or one bf16 ulp, over three steps on an odd-sized tensor, four dtype pairs
+ *     (fp32) or one ulp of bf16 / fp16, over three steps on an odd-sized tensor, all nine
+ *     pairs of parameter and gradient types
  *   - the multi-tensor entry point with an empty tensor in the list
  *   - the non-quantized entry point
  *   - quantize / dequantize against the oracle's
@@ -36,6 +37,8 @@ void q4o_step_unquant(void *p, const void *g, float *m, float *v, int64_t numel,
 void q4o_quant(const float *x, int64_t numel, int which, uint8_t *codes, float *scale);
 void q4o_dequant(const uint8_t *codes, const float *scale, int64_t numel, int which, float *out);
 void q4o_tables(int which, float *qmap16, float *qmid15);
+float q4o_f16_to_f32(uint16_t h);
+uint16_t q4o_f32_to_f16(float f);
 
 static const float B1 = 0.9f, B2 = 0.999f, LR = 1e-3f, WD = 0.01f, EPS = 1e-8f;
 
@@ -85,12 +88,13 @@ static uint16_t to_bf16(float f) {
   return (uint16_t)(u >> 16);
 }
 
-static size_t elem_size(int dtype) { return dtype == Q4ADAMW_BF16 ? 2 : 4; }
+static size_t elem_size(int dtype) { return dtype == Q4ADAMW_FP32 ? 4 : 2; }
 
 static void fill(void *dst, int dtype, int64_t n, float sigma) {
   for (int64_t i = 0; i < n; ++i) {
     const float x = normalish(sigma);
     if (dtype == Q4ADAMW_BF16) ((uint16_t *)dst)[i] = to_bf16(x);
+    else if (dtype == Q4ADAMW_FP16) ((uint16_t *)dst)[i] = q4o_f32_to_f16(x);
     else ((float *)dst)[i] = x;
   }
 }
@@ -102,17 +106,22 @@ static float from_bf16(uint16_t h) {
   return f;
 }
 
-/* parameters: 1e-6 relative to max(|p|, |step taken|) in fp32; in bf16 one ulp on that same
- * scale (a parameter that cancels against its update lands near zero, where its own ulp is tiny) */
+static float from_16(int dtype, uint16_t h) { return dtype == Q4ADAMW_BF16 ? from_bf16(h) : q4o_f16_to_f32(h); }
+
+/* parameters: 1e-6 relative to max(|p|, |step taken|) in fp32; in bf16 and fp16 one ulp of the
+ * type on that same scale (a parameter that cancels against its update lands near zero, where
+ * its own ulp is tiny) */
 static void check_params(const void *dev, const void *ref, const void *before, int dtype, int64_t n,
                          const char *what) {
   for (int64_t i = 0; i < n; ++i) {
-    if (dtype == Q4ADAMW_BF16) {
+    if (dtype != Q4ADAMW_FP32) {
       const uint16_t ab = ((const uint16_t *)dev)[i], bb = ((const uint16_t *)ref)[i];
-      const float a = from_bf16(ab), b = from_bf16(bb), p0 = from_bf16(((const uint16_t *)before)[i]);
+      const float a = from_16(dtype, ab), b = from_16(dtype, bb), p0 = from_16(dtype, ((const uint16_t *)before)[i]);
       const float scale = fmaxf(fmaxf(fabsf(b), fabsf(b - p0)), 1.17549435e-38f);
-      const float ulp = ldexpf(1.0f, (int)floorf(log2f(scale)) - 7);
-      CHECK(fabsf(a - b) <= ulp, "%s: bf16 parameter %lld differs by more than one ulp (%04x vs %04x)", what,
+      const int mant = dtype == Q4ADAMW_BF16 ? 7 : 10;
+      float ulp = ldexpf(1.0f, (int)floorf(log2f(scale)) - mant);
+      if (dtype == Q4ADAMW_FP16) ulp = fmaxf(ulp, 5.9604644775390625e-08f);   /* fp16 subnormal spacing */
+      CHECK(fabsf(a - b) <= ulp, "%s: 16-bit parameter %lld differs by more than one ulp (%04x vs %04x)", what,
             (long long)i, ab, bb);
     } else {
       const float a = ((const float *)dev)[i], b = ((const float *)ref)[i], p0 = ((const float *)before)[i];
@@ -315,8 +324,8 @@ int main(void) {
   CHECK(ndev > 0, "no GPU");
   HIP_OK(hipSetDevice(0));
   tables_and_errors();
-  for (int p_dtype = 0; p_dtype < 2; ++p_dtype)
-    for (int g_dtype = 0; g_dtype < 2; ++g_dtype) quantized_steps(p_dtype, g_dtype, 1000003);
+  for (int p_dtype = 0; p_dtype < 3; ++p_dtype)
+    for (int g_dtype = 0; g_dtype < 3; ++g_dtype) quantized_steps(p_dtype, g_dtype, 1000003);
   quantized_steps(Q4ADAMW_FP32, Q4ADAMW_FP32, 129);
   multi_and_small();
   interchange();

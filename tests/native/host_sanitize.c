@@ -84,7 +84,7 @@ static void refusals(void) {
   EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes + 2, codes + 2048, scales, scales + 64, 1000, H, H, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ALIGN);
   EXPECT(q4adamw_fused_4bit(buf, NULL, codes, codes + 2048, scales, scales + 64, 1000, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, -1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ARG);
-  EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, 1000, 2, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, 1000, 3, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, INT64_MAX, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_TOO_LARGE);
   const float bad_hyper[][6] = {{1.0f, B2, LR, WD, EPS, 1.0f}, {B1, 0.0f, LR, WD, EPS, 1.0f}, {B1, B2, 0.0f, WD, EPS, 1.0f},
                                 {B1, B2, LR, -1.0f, EPS, 1.0f}, {B1, B2, LR, WD, 0.0f, 1.0f}, {B1, B2, LR, WD, EPS, 0.5f},

@@ -95,16 +95,23 @@ def p_close(p_dev, p_ref, p_prev, bf16=False):
     fp32: |dev - ref| <= 1e-6 * max(|ref|, |ref - prev|): 1e-6 relative to the parameter
     or, for parameters near zero (where a relative bound on the parameter alone cannot
     hold for anything but bit-identical arithmetic), relative to the step it took.
-    bf16 parameters: at most one bf16 ulp, measured on the same scale.
+    bf16 parameters (uint16 bit patterns) and fp16 parameters (numpy float16): at most one
+    ulp of the storage type, measured on the same scale.
     Returns (ok, worst ratio or ulps)."""
-    if bf16:
-        # one bf16 ulp of the larger of the parameter and the step it took (a parameter
+    half = np.asarray(p_ref).dtype == np.float16
+    if bf16 or half:
+        # one ulp of the larger of the parameter and the step it took (a parameter
         # that cancels against its update lands near zero, where its own ulp is tiny)
-        f = lambda u: (u.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        if half:
+            f = lambda u: np.asarray(u).astype(np.float64)
+            mant, floor_ulp = 10, 2.0 ** -24          # below 2^-14 fp16 is spaced 2^-24 apart
+        else:
+            f = lambda u: (u.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+            mant, floor_ulp = 7, 0.0
         dev, ref, prev = f(p_dev), f(p_ref), f(p_prev)
         scale = np.maximum(np.maximum(np.abs(ref), np.abs(ref - prev)), np.finfo(np.float32).tiny)
-        ulp = 2.0 ** (np.floor(np.log2(scale)) - 7)
-        worst = float((np.abs(dev - ref) / ulp).max())
+        ulp = np.maximum(2.0 ** (np.floor(np.log2(scale)) - mant), floor_ulp)
+        worst = float((np.abs(dev - ref) / ulp).max()) if dev.size else 0.0
         return worst <= 1.0, worst
     ref = p_ref.astype(np.float64)
     diff = np.abs(p_dev.astype(np.float64) - ref)

@@ -39,12 +39,13 @@ def test_oracles_replay_fixture(path):
     m, v = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8)
     sm, sv = np.zeros(nk, np.float32), np.zeros(nk, np.float32)
     bf16_p = p.dtype == np.uint16
+    pbits = np.uint16 if p.dtype.itemsize == 2 else np.uint32      # bf16 bit patterns and fp16 are 2 bytes
     tp = torch.from_numpy(p.view(np.int16).copy()).view(torch.bfloat16) if bf16_p else torch.from_numpy(p.copy())
     tm, tv, tsm, tsv = (torch.from_numpy(x.copy()) for x in (m, v, sm, sv))
     for t in range(1, steps + 1):
         g = z[f"g{t}"]
         oc.step_quant(p, g, m, v, sm, sv, step=t, **hp)
-        assert np.array_equal(p.view(np.uint16 if bf16_p else np.uint32), z[f"p{t}"].view(np.uint16 if bf16_p else np.uint32))
+        assert np.array_equal(p.view(pbits), z[f"p{t}"].view(pbits))
         assert np.array_equal(m, z[f"m{t}"]) and np.array_equal(v, z[f"v{t}"])
         assert np.array_equal(sm.view(np.uint32), z[f"sm{t}"]) and np.array_equal(sv.view(np.uint32), z[f"sv{t}"])
         tg = torch.from_numpy(g.view(np.int16).copy()).view(torch.bfloat16) if g.dtype == np.uint16 else torch.from_numpy(g.copy())
@@ -52,7 +53,7 @@ def test_oracles_replay_fixture(path):
         assert np.array_equal(tm.numpy(), m) and np.array_equal(tv.numpy(), v)
         assert np.array_equal(tsm.numpy().view(np.uint32), z[f"sm{t}"])
         assert np.array_equal(tsv.numpy().view(np.uint32), z[f"sv{t}"])
-        got = tp.view(torch.int16).numpy().view(np.uint16) if bf16_p else tp.numpy().view(np.uint32)
+        got = tp.view(torch.int16).numpy().view(np.uint16) if bf16_p else tp.numpy().view(pbits)
         assert np.array_equal(got, z[f"p{t}"].view(got.dtype))
 
 

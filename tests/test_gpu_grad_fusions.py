@@ -19,7 +19,7 @@ from tests.q4_testlib import (HP, DeviceTensor, OracleTensor, assert_state_equal
 
 pytestmark = pytest.mark.gpu
 
-DT = {"fp32": torch.float32, "bf16": torch.bfloat16}
+DT = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}
 HPA = (HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"], HP["eps"])
 
 
@@ -35,7 +35,8 @@ def _same(a, b):
     return all(torch.equal(x.view(torch.uint8), y.view(torch.uint8)) for x, y in zip(a, b))
 
 
-@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32")])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
+                                       ("fp16", "fp16"), ("fp32", "fp16")])
 @pytest.mark.parametrize("n", [128 * 1024 + 77, 4097])
 def test_multiplier_against_oracle(cuda, p_dt, g_dt, n):
     """host multiplier, device multiplier and their product, three steps, ragged sizes"""

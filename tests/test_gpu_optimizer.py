@@ -223,6 +223,49 @@ def test_param_groups_missing_grads_and_bf16(cuda):
     assert float(opt.state[w1]["step"]) == 3.0 and float(opt.state[w2]["step"]) == 2.0
 
 
+def test_fp16_model_state_layout_resume_and_interchange(cuda):
+    """a model held in fp16 (the reference dispatches on half parameters,
+    optim/cuda_adamw_kernels.cu:443): packed states stay uint8 with fp32 scales, small tensors
+    keep fp32 moments, the run tracks torch.optim.AdamW on an fp32 twin within the draft's bar,
+    resume is bit-identical, and the exported AdamW state is fp32"""
+    torch.manual_seed(8)
+    mk = lambda: nn.Sequential(nn.Linear(256, 96), nn.Tanh(), nn.Linear(96, 32)).to(cuda)
+    model, twin = mk().half(), mk()
+    twin.load_state_dict({k: v.float() for k, v in model.state_dict().items()})
+    opt = AdamWFused_QuantFour(model.parameters(), lr=1e-3, weight_decay=0.01)
+    ref = torch.optim.AdamW(twin.parameters(), lr=1e-3, weight_decay=0.01)
+    for it in range(8):
+        x = torch.randn(32, 256, device=cuda)
+        opt.zero_grad(set_to_none=True)
+        model(x.half()).float().square().mean().backward()
+        opt.step()
+        ref.zero_grad(set_to_none=True)
+        twin(x).square().mean().backward()
+        ref.step()
+    w = model[0].weight
+    st = opt.state[w]
+    assert w.dtype == torch.float16 and w.grad.dtype == torch.float16
+    assert st["exp_avg"].dtype == torch.uint8 and st["momentum_qstate"]["overhead"]["max1"].dtype == torch.float32
+    assert opt.state[model[0].bias]["exp_avg"].dtype == torch.float32
+    for a, b in zip(model.parameters(), twin.parameters()):
+        torch.testing.assert_close(a.float(), b, atol=0.025, rtol=1e-5)
+    exported = opt.adamw_state_dict()["state"][0]
+    assert exported["exp_avg"].dtype == torch.float32 and exported["exp_avg"].shape == w.shape
+    model2 = mk().half()
+    model2.load_state_dict(model.state_dict())
+    opt2 = AdamWFused_QuantFour(model2.parameters(), lr=1e-3, weight_decay=0.01)
+    opt2.load_state_dict(opt.state_dict())
+    assert opt2.state[model2[0].weight]["exp_avg"].dtype == torch.uint8
+    assert opt2.state[model2[0].weight]["variance_qstate"]["overhead"]["max1"].dtype == torch.float32
+    x = torch.randn(32, 256, device=cuda).half()
+    for m_, o_ in ((model, opt), (model2, opt2)):
+        o_.zero_grad(set_to_none=True)
+        m_(x).float().square().mean().backward()
+        o_.step()
+    for a, b in zip(model.parameters(), model2.parameters()):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("shape", [(4096,), (1024, 4096), (4096, 4096), (14336, 4096), (4096, 14336)])
 def test_llama3_8b_tensor_shapes(cuda, shape):
     """Every distinct tensor shape of the headline configuration except the embedding, at its

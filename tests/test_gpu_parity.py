@@ -51,6 +51,19 @@ def test_ragged_lengths(cuda, n):
     run_steps(p0, lambda t: grads_config3(gen, n), 3, cuda, what=f"ragged n={n}")
 
 
+@pytest.mark.parametrize("n", [1, 3, 127, 129, 513, 4097, 100003])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_ragged_lengths_16_bit(cuda, n, dt):
+    """tail tiles of the 8-elements-per-lane geometry: element-wise conversions, half-filled
+    last byte, values that overflow fp16 (+-1e3 gradients stay finite; parameters near the top
+    of the fp16 range round to infinity in the oracle and on the device alike)"""
+    gen = torch.Generator().manual_seed(2000 + n)
+    p0 = (torch.randn(n, generator=gen) * 0.02).to(dt)
+    if dt == torch.float16 and n > 3:
+        p0[1], p0[2] = 65504.0, -65504.0
+    run_steps(p0, lambda t: grads_config3(gen, n), 3, cuda, g_dtype=dt, what=f"ragged {dt} n={n}")
+
+
 def test_all_zero_blocks_and_guard_bytes(cuda):
     """Blocks whose grads stay zero keep zero codes and zero scales; bytes past the
     packed length and scales past the last block are never written."""
@@ -173,9 +186,14 @@ def test_extreme_scales(cuda):
 
 @pytest.mark.parametrize("p_dtype,g_dtype", [(torch.float32, torch.bfloat16),
                                              (torch.bfloat16, torch.bfloat16),
-                                             (torch.bfloat16, torch.float32)])
+                                             (torch.bfloat16, torch.float32),
+                                             (torch.float16, torch.float16),
+                                             (torch.float32, torch.float16),
+                                             (torch.float16, torch.float32),
+                                             (torch.float16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float16)])
 def test_bf16_io(cuda, p_dtype, g_dtype):
-    """bf16 gradient and bf16 parameter variants (Llama-shaped distributions)."""
+    """16-bit gradient and parameter variants, bf16 and fp16 (Llama-shaped distributions)."""
     gen = torch.Generator().manual_seed(21)
     n = 1024 * 4096 + 777
     p0 = (torch.randn(n, generator=gen) * 0.02).to(p_dtype)
@@ -342,7 +360,7 @@ def test_concurrent_threads_and_streams(cuda):
 
 
 @pytest.mark.parametrize("p_dtype,g_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
-                                             (torch.bfloat16, torch.bfloat16)])
+                                             (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16)])
 def test_non_finite_gradients(cuda, p_dtype, g_dtype):
     """inf, -inf and NaN gradients in some blocks: codes and scales still match the oracle bit
     for bit (a block's scale is the maximum over its non-NaN magnitudes, an infinite scale sends
@@ -372,7 +390,8 @@ def test_non_finite_gradients(cuda, p_dtype, g_dtype):
         assert np.array_equal(dev.m.cpu().numpy(), ref.m), f"step {step}: m codes"
         assert np.array_equal(dev.v.cpu().numpy(), ref.v), f"step {step}: v codes"
         p_dev = dev.p.float().cpu().numpy()
-        p_ref = ref.p if ref.p.dtype == np.float32 else (ref.p.astype(np.uint32) << 16).view(np.float32)
+        p_ref = (ref.p.astype(np.float32) if ref.p.dtype != np.uint16
+                 else (ref.p.astype(np.uint32) << 16).view(np.float32))
         finite = np.isfinite(p_ref)
         assert np.array_equal(np.isfinite(p_dev), finite), f"step {step}: finiteness of the parameters"
         ok, worst = p_close(to_np(dev.p)[finite], ref.p[finite], prev[finite], bf16=p_dtype == torch.bfloat16)

@@ -15,7 +15,7 @@ from tests.q4_testlib import HP, grads_config1, grads_config3, p_close, to_np
 
 pytestmark = pytest.mark.gpu
 
-DT = {"fp32": torch.float32, "bf16": torch.bfloat16}
+DT = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}
 HPA = (HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"], HP["eps"])
 
 
@@ -61,7 +61,8 @@ def _check(dev, ref, prev, what):
 SHAPES = [(64, 512), (3, 4096), (100, 520), (257, 768), (130, 1032), (1, 512), (70, 2048 + 512), (5, 8200)]
 
 
-@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32")])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
+                                       ("fp16", "fp16"), ("fp32", "fp16"), ("fp16", "fp32")])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_rank1_against_oracle(cuda, p_dt, g_dt, shape):
     rows, cols = shape
@@ -83,7 +84,8 @@ def test_rank1_against_oracle(cuda, p_dt, g_dt, shape):
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])   # per-step parameter bound
 
 
-@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32")])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
+                                       ("fp16", "fp16")])
 @pytest.mark.parametrize("shape", [(64, 512), (100, 520), (130, 1032), (5, 8200)])
 def test_rank1_stochastic_rounding_against_oracle(cuda, p_dt, g_dt, shape):
     """rank-1 scaling and stochastic rounding together: codes, scales and statistics bit for

@@ -12,7 +12,7 @@ from tests.q4_testlib import HP, DeviceTensor, grads_config1, grads_config3, gra
 
 pytestmark = pytest.mark.gpu
 
-DT = {"fp32": torch.float32, "bf16": torch.bfloat16}
+DT = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}
 HPA = (HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"], HP["eps"])
 SEED = 0x1234_5678_9ABC_DEF0
 
@@ -34,7 +34,8 @@ def test_salt_function_matches_oracle():
         assert L.q4adamw_sr_tensor_salt(seed, float(step), salt) == ot.sr_tensor_salt(seed, step, salt)
 
 
-@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32")])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
+                                       ("fp16", "fp16"), ("fp32", "fp16")])
 @pytest.mark.parametrize("n", [128 * 300 + 77, 4097, 1 << 18])
 def test_sr_against_oracle(cuda, p_dt, g_dt, n):
     gen = torch.Generator().manual_seed(n % 1000)

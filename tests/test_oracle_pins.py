@@ -383,6 +383,54 @@ def test_rank1_closed_forms():
     assert torch.equal(out[0].reshape(-1), ref[0])
 
 
+def test_fp16_conversions_against_numpy():
+    """the C oracle's binary16 conversions against numpy's: every one of the 65536 patterns
+    widened; narrowing of every pattern's value, of the midpoints between neighbouring values
+    (ties go to even), of values one fp32 ulp either side of them, of the overflow boundary
+    (65520 rounds to infinity) and of random fp32 bit patterns"""
+    L = oc.lib()
+    h = np.arange(65536, dtype=np.uint16)
+    wide = h.view(np.float16).astype(np.float32)
+    got = np.array([L.q4o_f16_to_f32(int(x)) for x in h], np.float32)
+    nan = np.isnan(wide)
+    assert np.array_equal(got[~nan].view(np.uint32), wide[~nan].view(np.uint32)) and np.isnan(got[nan]).all()
+    finite = wide[np.isfinite(wide)]
+    srt = np.sort(finite.astype(np.float64))
+    mids = ((srt[:-1] + srt[1:]) / 2).astype(np.float32)       # exact in fp32
+    rng = np.random.default_rng(3)
+    rand = rng.integers(0, 2 ** 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    special = np.array([65504.0, 65519.99, 65520.0, 65536.0, 1e9, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                        np.nextafter(np.float32(2.0 ** -25), np.float32(1)), 2.0 ** -14, 0.0, -0.0], np.float32)
+    xs = np.concatenate([finite, mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+                         rand[~np.isnan(rand)], special, -special]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([L.q4o_f32_to_f16(float(x)) for x in xs], np.uint16)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, (xs[bad[:5]], got[bad[:5]], want[bad[:5]])
+    assert (L.q4o_f32_to_f16(float("nan")) & 0x7c00) == 0x7c00 and (L.q4o_f32_to_f16(float("nan")) & 0x3ff) != 0
+
+
+def test_c_and_torch_oracles_agree_on_fp16_tensors():
+    """fp16 parameters and gradients through both restatements, three steps on an odd size"""
+    gen = torch.Generator().manual_seed(44)
+    n = 128 * 5 + 77
+    p = (torch.randn(n, generator=gen) * 0.05).to(torch.float16)
+    nb, nk = oc.state_sizes(n)
+    pc = p.numpy().copy()
+    cm, cv, csm, csv = np.zeros(nb, np.uint8), np.zeros(nb, np.uint8), np.zeros(nk, np.float32), np.zeros(nk, np.float32)
+    ts = (p.clone(), torch.zeros(nb, dtype=torch.uint8), torch.zeros(nb, dtype=torch.uint8), torch.zeros(nk), torch.zeros(nk))
+    for step in (1, 2, 3):
+        g = (torch.randn(n, generator=gen) * 1e-3).to(torch.float16)
+        oc.step_quant(pc, g.numpy(), cm, cv, csm, csv, step=step, **HP)
+        ts = ot.step_quant(ts[0], g, *ts[1:], step=step, **HP)
+        assert np.array_equal(cm, ts[1].numpy()) and np.array_equal(cv, ts[2].numpy())
+        assert np.array_equal(csm.view(np.uint32), ts[3].numpy().view(np.uint32))
+        assert np.array_equal(csv.view(np.uint32), ts[4].numpy().view(np.uint32))
+        assert ts[0].dtype == torch.float16
+        assert np.array_equal(pc.view(np.uint16), ts[0].numpy().view(np.uint16)), f"step {step}"
+
+
 # ---------------------------------------------------------------------------
 # stochastic rounding
 # ---------------------------------------------------------------------------
