@@ -17,7 +17,7 @@
 //             and gradient streams: 4 consecutive elements (tile = 256 elements = 2
 //             quantization blocks, a block = 32 lanes, abs-max by one v_permlane16_swap
 //             plus four DPP row steps), or 8 when parameters and gradients are both
-//             bf16 (tile = 512 elements = 4 blocks, a block = one 16-lane DPP row).
+//             16-bit types (tile = 512 elements = 4 blocks, a block = one 16-lane DPP row).
 //             No LDS traffic and no barrier in the reduction.
 //   chunk   = 4 tiles of ONE tensor = one 256-thread workgroup.
 //   launch  = all chunks of up to kMaxTensors tensors.  The tensor descriptors and
