@@ -1,6 +1,9 @@
 """Seeded sweep over sizes, dtypes, hyper-parameters, step numbers and gradient magnitudes:
 the HIP step against the C oracle (block-scaled path) on configurations no hand-written test
-names.  Deterministic: every case derives from its index."""
+names.  Deterministic: every case derives from its index.  Q4ADAMW_SWEEP_EXTRA=N in the
+environment adds the indices 1000 .. 1000+N-1 to every sweep (a longer hunt, same rules)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -10,14 +13,24 @@ from tests.q4_testlib import DeviceTensor, OracleTensor, assert_state_equal
 
 pytestmark = pytest.mark.gpu
 
+EXTRA = list(range(1000, 1000 + int(os.environ.get("Q4ADAMW_SWEEP_EXTRA", "0"))))
+
 DTYPES = [(torch.float32, torch.float32), (torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16),
-          (torch.bfloat16, torch.float32)]
+          (torch.bfloat16, torch.float32), (torch.float16, torch.float16), (torch.float32, torch.float16)]
+
+
+def _as_grad(g, g_dt):
+    """numpy fp32 -> torch gradient of type g_dt; fp16 gradients are kept finite (the
+    non-finite cases have tests of their own)"""
+    if g_dt == torch.float16:
+        g = np.clip(g, -6.0e4, 6.0e4)
+    return torch.from_numpy(g).to(g_dt)
 
 
 def _case(i):
     rng = np.random.default_rng(1000 + i)
     n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 5000), rng.integers(5000, 400000)]))
-    p_dt, g_dt = DTYPES[i % 4]
+    p_dt, g_dt = DTYPES[i % len(DTYPES)]
     hp = dict(beta1=float(rng.choice([0.5, 0.8, 0.9, 0.95, 0.99])),
               beta2=float(rng.choice([0.88, 0.95, 0.99, 0.999, 0.9999])),
               lr=float(10.0 ** rng.uniform(-6, -1)), weight_decay=float(rng.choice([0.0, 1e-4, 0.01, 0.1, 0.5])),
@@ -27,7 +40,7 @@ def _case(i):
     return rng, n, p_dt, g_dt, hp, first_step, g_scale
 
 
-@pytest.mark.parametrize("i", range(48))
+@pytest.mark.parametrize("i", list(range(48)) + EXTRA)
 def test_random_configuration(cuda, i):
     rng, n, p_dt, g_dt, hp, first_step, g_scale = _case(i)
     print(f"[sweep {i}] n={n} p={p_dt} g={g_dt} hp={hp} step0={first_step} g_scale={g_scale:.3g}", flush=True)
@@ -40,7 +53,7 @@ def test_random_configuration(cuda, i):
         g[u > 0.999] *= np.float32(1e3)
         if k == 1:
             g[: n // 2] = 0.0                      # long runs of zero blocks
-        g = torch.from_numpy(g).to(g_dt)
+        g = _as_grad(g, g_dt)
         step = first_step + k
         q4.fused_4bit(dev.p, g.to(cuda), dev.m, dev.v, dev.sm, dev.sv, hp["beta1"], hp["beta2"], hp["lr"],
                       hp["weight_decay"], hp["eps"], step)
@@ -49,7 +62,7 @@ def test_random_configuration(cuda, i):
         ref.resync(dev.p)
 
 
-@pytest.mark.parametrize("i", range(16))
+@pytest.mark.parametrize("i", list(range(16)) + EXTRA)
 def test_random_configuration_stochastic_rounding(cuda, i):
     from oracle import q4_oracle_torch as ot
     from quantfour_adamw_cuda_amd import quantfour_hip as q
@@ -61,7 +74,7 @@ def test_random_configuration_stochastic_rounding(cuda, i):
     dev = DeviceTensor(p0, cuda)
     ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.sv.cpu())
     for k in range(2):
-        g = torch.from_numpy(rng.standard_normal(n).astype(np.float32) * np.float32(g_scale)).to(g_dt)
+        g = _as_grad(rng.standard_normal(n).astype(np.float32) * np.float32(g_scale), g_dt)
         step = first_step + k
         prev = ref[0]
         ref = ot.step_quant_sr(ref[0], g, *ref[1:], seed=seed, tensor_salt=salt, step=step, **hp)
@@ -75,15 +88,15 @@ def test_random_configuration_stochastic_rounding(cuda, i):
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
 
 
-@pytest.mark.parametrize("i", range(24))
+@pytest.mark.parametrize("i", list(range(24)) + EXTRA)
 def test_random_configuration_rank1(cuda, i):
-    """cases 16..23 add stochastic rounding (random seed and salt)"""
+    """every third case adds stochastic rounding (random seed and salt)"""
     from oracle import q4_oracle_torch as ot
     from quantfour_adamw_cuda_amd import quantfour_hip as q
     from tests.q4_testlib import p_close, to_np
     rng, _, p_dt, g_dt, hp, first_step, g_scale = _case(200 + i)
     rows, cols = int(rng.integers(1, 90)), 512 + 8 * int(rng.integers(0, 200))
-    sr = dict(seed=int(rng.integers(0, 2 ** 63)), tensor_salt=int(rng.integers(0, 2 ** 32))) if i >= 16 else None
+    sr = dict(seed=int(rng.integers(0, 2 ** 63)), tensor_salt=int(rng.integers(0, 2 ** 32))) if i % 3 == 2 else None
     print(f"[sweep rank1 {i}] {rows}x{cols} p={p_dt} g={g_dt} hp={hp} step0={first_step} sr={sr}", flush=True)
     n = rows * cols
     p0 = torch.from_numpy((rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)).to(p_dt)
@@ -94,7 +107,7 @@ def test_random_configuration_rank1(cuda, i):
     for k in range(2):
         g = rng.standard_normal((rows, cols)).astype(np.float32) * np.float32(g_scale)
         g *= rng.uniform(0.01, 1.0, (rows, 1)).astype(np.float32) * rng.uniform(0.01, 1.0, (1, cols)).astype(np.float32)
-        g = torch.from_numpy(g).to(g_dt)
+        g = _as_grad(g, g_dt)
         step = first_step + k
         prev = ref[0]
         if sr is None:
