@@ -169,7 +169,7 @@ uint32_t q4adamw_sr_tensor_salt(uint64_t seed, float step, uint32_t tensor_salt)
  * keeps its per-128 block scales.  row_max/col_max (rows and cols floats) are
  * updated by the call; row_max_next/col_max_next are state-owned scratch of the same
  * sizes that must hold zeros on entry and holds zeros again afterwards.
- * rows x cols, row-major, cols a multiple of 8 and at least 512; p, g, col_max and
+ * rows x cols, row-major, cols a multiple of 8 and at least 16; p, g, col_max and
  * col_max_next 16-byte aligned, the rest 4-byte aligned.
  */
 typedef struct q4adamw_rank1_tensor {

@@ -167,14 +167,19 @@ static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
 typedef void (*Rank1Kernel)(const Rank1Args);
 typedef void (*Rank1StatKernel)(const Rank1StatArgs);
 
-template <bool EXT, bool SR>
+template <bool EXT, bool SR, bool NARROW>
 static Rank1Kernel pick_rank1_ext(int p_dtype, int g_dtype) {
-  Q4_PICK_PG(fused_4bit_rank1_kernel, EXT, SR)
+  Q4_PICK_PG(fused_4bit_rank1_kernel, EXT, SR, NARROW)
 }
 
-static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr) {
-  if (sr) return pick_rank1_ext<true, true>(p_dtype, g_dtype);
-  return ext ? pick_rank1_ext<true, false>(p_dtype, g_dtype) : pick_rank1_ext<false, false>(p_dtype, g_dtype);
+// narrow: the kernel for matrices whose rows are shorter than a tile
+static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr, bool narrow) {
+  if (narrow) {
+    if (sr) return pick_rank1_ext<true, true, true>(p_dtype, g_dtype);
+    return ext ? pick_rank1_ext<true, false, true>(p_dtype, g_dtype) : pick_rank1_ext<false, false, true>(p_dtype, g_dtype);
+  }
+  if (sr) return pick_rank1_ext<true, true, false>(p_dtype, g_dtype);
+  return ext ? pick_rank1_ext<true, false, false>(p_dtype, g_dtype) : pick_rank1_ext<false, false, false>(p_dtype, g_dtype);
 }
 
 template <bool EXT>
@@ -374,8 +379,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     const q4adamw_rank1_tensor &t = tensors[i];
     if (t.rows < 0 || t.cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
     if (t.rows == 0 || t.cols == 0) continue;
-    if (t.cols % 8 != 0 || t.cols < 512)
-      return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8 and at least 512");
+    if (t.cols % 8 != 0 || t.cols < 16)
+      return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8 and at least 16");
     if (t.cols > 0x40000000ll || t.rows > 0x7ffffffffll / t.cols)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "rank-1 scaling handles matrices of up to 2^35 - 1 elements");
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.row_max || !t.col_max ||
@@ -395,7 +400,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const Rank1Kernel kernel = pick_rank1(p_dtype, g_dtype, ext, sr);
+  const int64_t tile_elems = chunk_elems / kWaves;
+  Rank1Kernel kernel = nullptr;
   const Rank1StatKernel stat_kernel = pick_rank1_stats(g_dtype, ext);
   a.ntensors = 0;
   uint64_t chunks = 0, stat_chunks = 0;
@@ -418,51 +424,58 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     stat_chunks = 0;
     return 0;
   };
-  for (int i = 0; i < count; ++i) {
-    const q4adamw_rank1_tensor &t = tensors[i];
-    if (t.rows == 0 || t.cols == 0) continue;
-    const int64_t numel = t.rows * t.cols;
-    const uint64_t c = ((uint64_t)numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
-    const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
-    const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
-    if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
-        stat_chunks + sc_ > kMaxChunksPerLaunch) {
+  // two passes: matrices whose rows are at least a tile long take the kernel that finds a
+  // tile's row on the scalar unit, narrower ones the kernel whose lanes find their own
+  for (int narrow = 0; narrow < 2; ++narrow) {
+    kernel = pick_rank1(p_dtype, g_dtype, ext, sr, narrow != 0);
+    for (int i = 0; i < count; ++i) {
+      const q4adamw_rank1_tensor &t = tensors[i];
+      if (t.rows == 0 || t.cols == 0 || (t.cols < tile_elems) != (narrow != 0)) continue;
+      const int64_t numel = t.rows * t.cols;
+      const uint64_t c = ((uint64_t)numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
+      const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
+      const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
+      if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
+          stat_chunks + sc_ > kMaxChunksPerLaunch) {
+        if (int rc = launch()) return rc;
+      }
+      Rank1Desc &d = a.desc[a.ntensors];
+      d.p = t.p;
+      d.g = t.g;
+      d.m = t.exp_avg;
+      d.v = t.exp_avg_sq;
+      d.sm = t.exp_avg_scale;
+      d.rmax = t.row_max;
+      d.cmax = t.col_max;
+      d.rmax_next = t.row_max_next;
+      d.cmax_next = t.col_max_next;
+      d.numel = numel;
+      d.rows = t.rows;
+      d.cols = t.cols;
+      const FastDiv fd = make_fast_div((uint32_t)(t.cols >> 3));
+      d.div_magic = fd.magic;
+      d.div_shift = fd.shift;
+      a.sr_salt[a.ntensors] = sr ? q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i) : 0u;
+      a.first_chunk[a.ntensors] = (uint32_t)chunks;
+      Rank1StatArgs::Desc &sd = sa.desc[a.ntensors];
+      sd.g = t.g;
+      sd.v = t.exp_avg_sq;
+      sd.rmax = t.row_max;
+      sd.cmax = t.col_max;
+      sd.rmax_next = t.row_max_next;
+      sd.cmax_next = t.col_max_next;
+      sd.rows = t.rows;
+      sd.cols = t.cols;
+      sa.first_chunk[a.ntensors] = (uint32_t)stat_chunks;
+      sa.col_groups[a.ntensors] = groups;
+      ++a.ntensors;
+      chunks += c;
+      stat_chunks += sc_;
+    }
+    if (a.ntensors > 0) {
       if (int rc = launch()) return rc;
     }
-    Rank1Desc &d = a.desc[a.ntensors];
-    d.p = t.p;
-    d.g = t.g;
-    d.m = t.exp_avg;
-    d.v = t.exp_avg_sq;
-    d.sm = t.exp_avg_scale;
-    d.rmax = t.row_max;
-    d.cmax = t.col_max;
-    d.rmax_next = t.row_max_next;
-    d.cmax_next = t.col_max_next;
-    d.numel = numel;
-    d.rows = t.rows;
-    d.cols = t.cols;
-    const FastDiv fd = make_fast_div((uint32_t)(t.cols >> 3));
-    d.div_magic = fd.magic;
-    d.div_shift = fd.shift;
-    a.sr_salt[a.ntensors] = sr ? q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i) : 0u;
-    a.first_chunk[a.ntensors] = (uint32_t)chunks;
-    Rank1StatArgs::Desc &sd = sa.desc[a.ntensors];
-    sd.g = t.g;
-    sd.v = t.exp_avg_sq;
-    sd.rmax = t.row_max;
-    sd.cmax = t.col_max;
-    sd.rmax_next = t.row_max_next;
-    sd.cmax_next = t.col_max_next;
-    sd.rows = t.rows;
-    sd.cols = t.cols;
-    sa.first_chunk[a.ntensors] = (uint32_t)stat_chunks;
-    sa.col_groups[a.ntensors] = groups;
-    ++a.ntensors;
-    chunks += c;
-    stat_chunks += sc_;
   }
-  if (a.ntensors > 0) return launch();
   return 0;
 }
 

@@ -27,7 +27,8 @@ struct Geometry {
 // step's new statistics (complete before this kernel starts) quantize.
 // SR: both moments are rounded stochastically between the two neighbouring code-book
 // entries; the noise of element e is a hash of e and the tensor's salt of this step.
-template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, typename Desc>
+// NARROW (with RANK1): rows may be shorter than a tile.
+template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, bool NARROW, typename Desc>
 __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g, uint32_t salt) {
@@ -60,21 +61,33 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   Vals<N> c_old, c_new;
   if constexpr (RANK1) {
     // (row, column) of the tile's first element, in units of 8 elements so that the
-    // division is a 32-bit one.  A tile is shorter than a row, so a lane is in that
-    // row or in the next one.
+    // division is a 32-bit one.  A lane's N elements (N = 4 or 8, first one a multiple of N)
+    // lie in one row, because rows are multiples of 8 elements long.
     const uint32_t tb8 = (uint32_t)(tb >> 3), cols8 = (uint32_t)(T.cols >> 3);  // numel < 2^35
-    const uint32_t row32 = fast_div(tb8, T.div_magic, T.div_shift);
-    const int64_t row = row32;
-    const uint32_t col0 = (tb8 - row32 * cols8) << 3;
-    uint32_t col = col0 + e0;
-    const bool wrapped = col >= (uint32_t)T.cols;
-    if (wrapped) col -= (uint32_t)T.cols;
     const int64_t last = T.rows - 1;
-    const int64_t ra = row < last ? row : last, rb = row + 1 < last ? row + 1 : last;  // past-the-end lanes stay in bounds
-    const float r_old_a = as_global<const float>(T.rmax)[ra], r_old_b = as_global<const float>(T.rmax)[rb];
-    const float r_new_a = as_global<const float>(T.rmax_next)[ra], r_new_b = as_global<const float>(T.rmax_next)[rb];
-    r_old = wrapped ? r_old_b : r_old_a;
-    r_new = wrapped ? r_new_b : r_new_a;
+    uint32_t col;
+    if constexpr (!NARROW) {
+      // a tile is no longer than a row, so a lane is in the tile's first row or in the next
+      const uint32_t row32 = fast_div(tb8, T.div_magic, T.div_shift);
+      const int64_t row = row32;
+      const uint32_t col0 = (tb8 - row32 * cols8) << 3;
+      col = col0 + e0;
+      const bool wrapped = col >= (uint32_t)T.cols;
+      if (wrapped) col -= (uint32_t)T.cols;
+      const int64_t ra = row < last ? row : last, rb = row + 1 < last ? row + 1 : last;  // past-the-end lanes stay in bounds
+      const float r_old_a = as_global<const float>(T.rmax)[ra], r_old_b = as_global<const float>(T.rmax)[rb];
+      const float r_new_a = as_global<const float>(T.rmax_next)[ra], r_new_b = as_global<const float>(T.rmax_next)[rb];
+      r_old = wrapped ? r_old_b : r_old_a;
+      r_new = wrapped ? r_new_b : r_new_a;
+    } else {
+      // a tile may span several rows (the matrix is narrower than a tile): every lane finds its own
+      const uint32_t u8 = tb8 + (e0 >> 3);
+      const uint32_t row32 = fast_div(u8, T.div_magic, T.div_shift);
+      col = ((u8 - row32 * cols8) << 3) + (e0 & 7u);
+      const int64_t row = (int64_t)row32 < last ? (int64_t)row32 : last;   // past-the-end lanes stay in bounds
+      r_old = as_global<const float>(T.rmax)[row];
+      r_new = as_global<const float>(T.rmax_next)[row];
+    }
 #pragma unroll
     for (int k = 0; k < N; k += 4) {
       const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax), (col + k) * 4u, 0, 0);
@@ -345,9 +358,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   }
   const uint32_t salt = SR ? args.sr_salt[t] : 0u;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, false, SR, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, false, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, false, SR, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
@@ -482,7 +495,7 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   }
 }
 
-template <int PT, int GT, bool EXT, bool SR>
+template <int PT, int GT, bool EXT, bool SR, bool NARROW>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
   using G = Geometry<PT, GT>;
   __shared__ uint2 lds[kLdsEntries];
@@ -509,9 +522,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   }
   const uint32_t salt = SR ? args.sr_salt[t] : 0u;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, true, SR>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
 }
 
 // After the update: the new statistics become the current ones and the buffers that

@@ -77,7 +77,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # 128 consecutive elements, what the fused CUDA path does (cuda_adamw_kernels.cu:353-383);
         # "rank1" = min(row maximum, column maximum) for matrices, the draft's SecondMoment
         # setting (adamw_fourbit_triton.py:124, :834-863); tensors that are not matrices with
-        # cols % 8 == 0 and cols >= 512 keep group scaling, as 1-D tensors do there (:841-846)
+        # cols % 8 == 0 and cols >= 16 keep group scaling, as 1-D tensors do there (:841-846)
         if variance_scale_type not in ("group", "rank1"):
             raise ValueError(f"Invalid variance_scale_type: {variance_scale_type=}")
         self.variance_scale_type = variance_scale_type

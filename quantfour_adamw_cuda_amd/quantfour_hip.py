@@ -217,19 +217,19 @@ def fused_4bit_multi_sr(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, 
                     beta1, beta2, lr, weight_decay, eps, step, options)
 
 
-RANK1_MIN_COLS = 512
+RANK1_MIN_COLS = 16
 
 
 def rank1_eligible(p):
     """Whether a parameter's second moment can take rank-1 scaling: a matrix whose rows hold a
-    multiple of 8 and at least 512 elements (other tensors keep per-128 block scales, as 1-D
+    multiple of 8 and at least 16 elements (other tensors keep per-128 block scales, as 1-D
     tensors do in the reference's draft, optim/adamw_fourbit_triton.py:841-846)."""
     return p.dim() == 2 and p.shape[1] % 8 == 0 and p.shape[1] >= RANK1_MIN_COLS
 
 
 def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next):
     _check_common(p, g)
-    assert rank1_eligible(p), "rank-1 scaling needs a matrix with cols % 8 == 0 and cols >= 512"
+    assert rank1_eligible(p), "rank-1 scaling needs a matrix with cols % 8 == 0 and cols >= 16"
     rows, cols = p.shape
     nbytes, nblk = state_sizes(p.numel())
     assert exp.dtype == torch.uint8 and sq.dtype == torch.uint8, "moments must be packed uint8"

@@ -125,8 +125,8 @@ static void refusals(void) {
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* null pointers */
   r[0].cols = 516;
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* cols % 8 */
-  r[0].cols = 256;
-  EXPECT(q4adamw_fused_4bit_rank1_multi_sr(r, 1, NULL, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* cols < 512 */
+  r[0].cols = 8;
+  EXPECT(q4adamw_fused_4bit_rank1_multi_sr(r, 1, NULL, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* cols < 16 */
   r[0].rows = -1;
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);
   r[0].rows = (int64_t)1 << 40; r[0].cols = 1024;

@@ -95,7 +95,7 @@ def test_random_configuration_rank1(cuda, i):
     from quantfour_adamw_cuda_amd import quantfour_hip as q
     from tests.q4_testlib import p_close, to_np
     rng, _, p_dt, g_dt, hp, first_step, g_scale = _case(200 + i)
-    rows, cols = int(rng.integers(1, 90)), 512 + 8 * int(rng.integers(0, 200))
+    rows, cols = int(rng.integers(1, 90)), 8 * int(rng.integers(2, 300))     # narrow matrices included
     sr = dict(seed=int(rng.integers(0, 2 ** 63)), tensor_salt=int(rng.integers(0, 2 ** 32))) if i % 3 == 2 else None
     print(f"[sweep rank1 {i}] {rows}x{cols} p={p_dt} g={g_dt} hp={hp} step0={first_step} sr={sr}", flush=True)
     n = rows * cols

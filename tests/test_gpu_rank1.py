@@ -58,7 +58,10 @@ def _check(dev, ref, prev, what):
     assert ok, f"{what}: parameters out of tolerance (worst {worst})"
 
 
-SHAPES = [(64, 512), (3, 4096), (100, 520), (257, 768), (130, 1032), (1, 512), (70, 2048 + 512), (5, 8200)]
+SHAPES = [(64, 512), (3, 4096), (100, 520), (257, 768), (130, 1032), (1, 512), (70, 2048 + 512), (5, 8200),
+          # narrow matrices: a tile spans several rows (fewer than 256 columns, or than 512 when
+          # parameters and gradients are 16-bit types)
+          (300, 16), (77, 64), (1000, 24), (513, 248), (40, 504), (9, 256), (2000, 136)]
 
 
 @pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
@@ -86,7 +89,7 @@ def test_rank1_against_oracle(cuda, p_dt, g_dt, shape):
 
 @pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
                                        ("fp16", "fp16")])
-@pytest.mark.parametrize("shape", [(64, 512), (100, 520), (130, 1032), (5, 8200)])
+@pytest.mark.parametrize("shape", [(64, 512), (100, 520), (130, 1032), (5, 8200), (333, 40), (50, 264)])
 def test_rank1_stochastic_rounding_against_oracle(cuda, p_dt, g_dt, shape):
     """rank-1 scaling and stochastic rounding together: codes, scales and statistics bit for
     bit against step_quant_rank1_sr; the noise follows seed, step and the tensor's salt"""
@@ -213,6 +216,8 @@ def test_rank1_argument_errors(cuda):
     call = lambda a: L.q4adamw_fused_4bit_rank1_multi(a, 1, 0, 0, *HPA, 1.0, None, None)
     arr[0].cols = 500
     assert call(arr) == -1 and b"cols" in L.q4adamw_last_error()
+    arr[0].cols = 8
+    assert call(arr) == -1 and b"cols" in L.q4adamw_last_error()
     arr[0].cols = 512
     arr[0].col_max = d.c.data_ptr() + 4
     assert call(arr) == -2
@@ -264,12 +269,12 @@ def test_optimizer_rank1_layout_tracking_and_resume(cuda):
             o_.zero_grad(set_to_none=True)
             m_(x).square().mean().backward()
             o_.step()
-    # layout: [96, 512] and [16, 1024] are rank-1 (cols >= 512), [1024, 96] keeps block scales
+    # layout: all three weight matrices are rank-1 scaled ([1024, 96] through the narrow path)
     w0, w1, w2 = model[0].weight, model[2].weight, model[4].weight
     ov = lambda p: opt.state[p]["variance_qstate"]["overhead"]
     assert [tuple(t.shape) for t in ov(w0)["max_dims"]] == [(96, 1), (1, 512)] and ov(w0)["max1"] is None
     assert [tuple(t.shape) for t in ov(w2)["max_dims"]] == [(16, 1), (1, 1024)]
-    assert "max_dims" not in ov(w1) and ov(w1)["max1"].numel() == 1024 * 96 // 128
+    assert [tuple(t.shape) for t in ov(w1)["max_dims"]] == [(1024, 1), (1, 96)] and ov(w1)["max1"] is None
     assert all(not t.any() for t in ov(w0)["scratch_dims"])
     assert opt.state[model[0].bias]["exp_avg_sq"].dtype == torch.float32      # below the threshold
     # the draft's own bar against AdamW (tests/driver.py:70-71)
