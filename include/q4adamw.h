@@ -95,6 +95,13 @@ typedef struct q4adamw_small_tensor {
  *   skip_if_nonzero  device fp32 scalar or NULL: when it holds a non-zero value
  *                    (an overflow flag) the call leaves parameters and optimizer
  *                    state as they are.
+ *   step_consts      device memory of Q4ADAMW_STEP_CONSTS_BYTES bytes that
+ *                    q4adamw_device_step has filled, or NULL.  Not NULL: the step's
+ *                    derived scalars (bias corrections, step size, weight-decay factor)
+ *                    are read from there and the call's own lr, weight_decay, eps and
+ *                    step only pass the range check -- for a step whose number the host
+ *                    does not know, e.g. inside a captured graph.  Not with the _sr
+ *                    entry points: their noise depends on the step number.
  *   zero_grad        non-zero: the gradients are overwritten with zeros once read
  *                    (the `g` pointers are written in that case), also by a call
  *                    that skip_if_nonzero cancels: the overflowed gradients must
@@ -106,6 +113,7 @@ typedef struct q4adamw_grad_options {
   int zero_grad;
   const float *grad_scale_dev;
   const float *skip_if_nonzero;
+  const void *step_consts;
 } q4adamw_grad_options;
 
 /* One gradient tensor for q4adamw_grad_norm: numel elements, 16-byte aligned. */
@@ -253,6 +261,28 @@ int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, in
 int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
                       const float *grad_scale_dev, float max_norm, void *workspace,
                       size_t workspace_bytes, float *out3, void *stream);
+
+/*
+ * A step whose number lives on the device.  The reference derives the scalars of a step on
+ * the host from the step number it is given (optim/cuda_adamw_kernels.cu:435-440); a host
+ * that replays a captured graph has no step number to give.  q4adamw_bias_table (host only)
+ * tabulates the two step-dependent values, 1 - beta1^t and sqrt(1 - beta2^t), for t =
+ * first_step .. first_step + count - 1, two floats per step, computed as the launcher
+ * computes them; the caller copies the table to the device.  q4adamw_device_step enqueues a
+ * one-thread kernel that adds 1 to the fp32 counter *step_dev (unless *skip_if_nonzero is
+ * non-zero: then it changes nothing), takes the table entry of the new step number (steps
+ * past the table take its last entry, so the table should reach the step at which both
+ * values have become 1), takes lr from *lr_dev if lr_dev is not NULL, and writes the derived
+ * scalars to consts_dev (Q4ADAMW_STEP_CONSTS_BYTES bytes, 16-byte aligned) with the host's
+ * own operations: a step made with them equals, bit for bit, the step made with that step
+ * number on the host.  Pass consts_dev as q4adamw_grad_options.step_consts.
+ */
+#define Q4ADAMW_STEP_CONSTS_BYTES 64
+int q4adamw_bias_table(float beta1, float beta2, int64_t first_step, int64_t count, float *out2);
+int q4adamw_device_step(float *step_dev, const float *bias_table_dev, int64_t table_first_step,
+                        int64_t table_steps, const float *lr_dev, float beta1, float beta2, float lr,
+                        float weight_decay, float eps, const float *skip_if_nonzero, void *consts_dev,
+                        void *stream);
 
 /*
  * Quantize one fp32 moment: per block of 128 consecutive elements the scale is the

@@ -61,6 +61,7 @@ class Q4GradOptions(ctypes.Structure):
         ("zero_grad", ctypes.c_int),
         ("grad_scale_dev", ctypes.c_void_p),
         ("skip_if_nonzero", ctypes.c_void_p),
+        ("step_consts", ctypes.c_void_p),
     ]
 
 
@@ -73,6 +74,7 @@ class Q4Grad(ctypes.Structure):
 
 
 NORM_WORKSPACE_BYTES = 16384
+STEP_CONSTS_BYTES = 64
 
 EXPORTS = (
     "q4adamw_fused_4bit",
@@ -86,6 +88,8 @@ EXPORTS = (
     "q4adamw_fused_single_tensor_multi",
     "q4adamw_fused_single_tensor_multi_ex",
     "q4adamw_grad_norm",
+    "q4adamw_bias_table",
+    "q4adamw_device_step",
     "q4adamw_quantize",
     "q4adamw_dequantize",
     "q4adamw_quantize_rank1",
@@ -140,6 +144,10 @@ def load():
     L.q4adamw_fused_4bit_rank1_multi_sr.restype = i
     L.q4adamw_grad_norm.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, ctypes.c_size_t, vp, vp]
     L.q4adamw_grad_norm.restype = i
+    L.q4adamw_bias_table.argtypes = [f, f, i64, i64, vp]
+    L.q4adamw_bias_table.restype = i
+    L.q4adamw_device_step.argtypes = [vp, vp, i64, i64, vp, f, f, f, f, f, vp, vp, vp]
+    L.q4adamw_device_step.restype = i
     L.q4adamw_quantize.argtypes = [vp, i64, i, vp, vp, vp]
     L.q4adamw_quantize.restype = i
     L.q4adamw_dequantize.argtypes = [vp, vp, i64, i, vp, vp]

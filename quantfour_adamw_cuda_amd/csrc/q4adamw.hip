@@ -200,8 +200,11 @@ static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext
   go->zero = 0u;
   go->scale_dev = nullptr;
   go->skip = nullptr;
+  go->sc_dev = nullptr;
   *ext = false;
   if (!opt) return 0;
+  if (opt->step_consts && (reinterpret_cast<uintptr_t>(opt->step_consts) & 15))
+    return fail(Q4ADAMW_ERR_ALIGN, "step_consts must be 16-byte aligned");
   if (opt->grad_scale_dev && (reinterpret_cast<uintptr_t>(opt->grad_scale_dev) & 3))
     return fail(Q4ADAMW_ERR_ALIGN, "grad_scale_dev must be 4-byte aligned");
   if (opt->skip_if_nonzero && (reinterpret_cast<uintptr_t>(opt->skip_if_nonzero) & 3))
@@ -210,7 +213,9 @@ static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext
   go->zero = opt->zero_grad ? 1u : 0u;
   go->scale_dev = opt->grad_scale_dev;
   go->skip = opt->skip_if_nonzero;
-  *ext = opt->grad_scale != 1.0f || opt->zero_grad || opt->grad_scale_dev || opt->skip_if_nonzero;
+  go->sc_dev = static_cast<const StepConsts *>(opt->step_consts);
+  *ext = opt->grad_scale != 1.0f || opt->zero_grad || opt->grad_scale_dev || opt->skip_if_nonzero ||
+         opt->step_consts;
   return 0;
 }
 
@@ -307,6 +312,8 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
+  if (sr && a.go.sc_dev)
+    return fail(Q4ADAMW_ERR_ARG, "stochastic rounding needs the step number on the host (its noise depends on it)");
   // a lane reads 8 consecutive elements at once when parameters and gradients are 16-bit types, else 4
   const bool p_half = p_dtype != Q4ADAMW_FP32, g_half = g_dtype != Q4ADAMW_FP32;
   const bool wide = p_half && g_half;   // 8 elements per lane
@@ -370,6 +377,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
+  if (sr && a.go.sc_dev)
+    return fail(Q4ADAMW_ERR_ARG, "stochastic rounding needs the step number on the host (its noise depends on it)");
   sa.go = a.go;
   sa.b2 = a.sc.b2;
   sa.r2 = a.sc.r2;
@@ -631,6 +640,37 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
   return 0;
 }
 
+int q4adamw_bias_table(float beta1, float beta2, int64_t first_step, int64_t count, float *out2) {
+  if (!(beta1 > 0.0f && beta1 < 1.0f) || !(beta2 > 0.0f && beta2 < 1.0f))
+    return fail(Q4ADAMW_ERR_HYPER, "hyper-parameter out of range (need 0<beta<1)");
+  if (first_step < 1 || count < 0 || (count > 0 && !out2)) return fail(Q4ADAMW_ERR_ARG, "bad step range or null output");
+  for (int64_t k = 0; k < count; ++k) {
+    float s[6];
+    q4adamw_derive_scalars(beta1, beta2, 1.0f, 0.0f, (float)(first_step + k), s);
+    out2[2 * k] = s[0];
+    out2[2 * k + 1] = s[1];
+  }
+  return 0;
+}
+
+int q4adamw_device_step(float *step_dev, const float *bias_table_dev, int64_t table_first_step,
+                        int64_t table_steps, const float *lr_dev, float beta1, float beta2, float lr,
+                        float weight_decay, float eps, const float *skip_if_nonzero, void *consts_dev,
+                        void *stream) {
+  StepConsts unused;
+  if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, 1.0f, &unused)) return rc;
+  if (!step_dev || !bias_table_dev || !consts_dev) return fail(Q4ADAMW_ERR_ARG, "null pointer");
+  if (table_first_step < 1 || table_steps < 1) return fail(Q4ADAMW_ERR_ARG, "empty bias table");
+  if (!aligned(step_dev, 4) || !aligned(bias_table_dev, 8) || (lr_dev && !aligned(lr_dev, 4)) ||
+      (skip_if_nonzero && !aligned(skip_if_nonzero, 4)) || !aligned(consts_dev, 16))
+    return fail(Q4ADAMW_ERR_ALIGN, "scalars must be 4-byte, the table 8-byte, the constants 16-byte aligned");
+  hipLaunchKernelGGL(device_step_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), step_dev,
+                     bias_table_dev, table_first_step, table_steps, lr_dev, beta1, beta2, lr, weight_decay, eps,
+                     skip_if_nonzero, static_cast<StepConsts *>(consts_dev));
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, float *scales,
                      void *stream) {
   if (numel < 0 || (which != 0 && which != 1)) return fail(Q4ADAMW_ERR_ARG, "bad numel or moment selector");
@@ -708,6 +748,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1009; }
+int q4adamw_version(void) { return 1010; }
 
 }  // extern "C"

@@ -33,6 +33,7 @@ struct GradOps {
   uint32_t zero;           // non-zero: overwrite the gradients with zeros once they are read
   const float *scale_dev;  // device part of the multiplier, or null
   const float *skip;       // device flag, or null: non-zero turns the launch into a no-op
+  const StepConsts *sc_dev;  // the step's derived scalars in device memory (device_step_kernel), or null
 };
 
 struct TensorDesc {  // 56 bytes
@@ -188,6 +189,7 @@ struct NormArgs {
   NormDesc desc[kMaxNormTensors];
 };
 
+static_assert(sizeof(StepConsts) <= Q4ADAMW_STEP_CONSTS_BYTES, "the device copy of a step's scalars");
 static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(NormArgs) <= 4096 &&
                   sizeof(Rank1Args) <= 4096 && sizeof(Rank1StatArgs) <= 4096,
               "kernel arguments are limited to 4 KiB");

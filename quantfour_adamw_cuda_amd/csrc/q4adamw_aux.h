@@ -16,7 +16,7 @@ __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args
   if (cancelled && !zero_g) return;
   const int t = find_tensor(args, chunk);
   const SmallDesc &T = args.desc[t];
-  const StepConsts &sc = args.sc;
+  const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   const int64_t base = (int64_t)(chunk - args.first_chunk[t]) * kSmallChunk;
   const int64_t end = base + kSmallChunk < T.numel ? base + kSmallChunk : T.numel;
   if (cancelled) {  // a cancelled step still clears the gradients it was asked to clear
@@ -45,6 +45,45 @@ __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// a step whose number lives on the device
+// ---------------------------------------------------------------------------
+// One thread: advances the step counter and derives the step's scalars exactly as the
+// host does for a step it knows (make_consts; optim/cuda_adamw_kernels.cu:435-440), from
+// the bias-correction pair the host tabulated for that step number: every operation
+// below is the IEEE operation the host performs, so the scalars agree bit for bit.  A
+// set overflow flag leaves counter and scalars alone (the step's launches do nothing then).
+__global__ void device_step_kernel(float *counter_, const float *table_, int64_t first_step, int64_t table_steps,
+                                   const float *lr_dev, float beta1, float beta2, float lr, float wd, float eps,
+                                   const float *skip, StepConsts *out_) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  if (skip && *as_global<const float>(skip) != 0.0f) return;
+  const gptr<float> counter = as_global<float>(counter_);
+  const float t = *counter + 1.0f;
+  *counter = t;
+  int64_t k = (int64_t)t - first_step;
+  k = k < 0 ? 0 : (k >= table_steps ? table_steps - 1 : k);   // past the table: its last, converged entry
+  const float c1 = as_global<const float>(table_)[2 * k], c2s = as_global<const float>(table_)[2 * k + 1];
+  const float lrv = lr_dev ? *as_global<const float>(lr_dev) : lr;
+  StepConsts sc;
+  sc.b1 = beta1;
+  sc.b2 = beta2;
+  sc.r1 = 1.0f - beta1;
+  sc.r2 = 1.0f - beta2;
+  const float lrwd = lrv * wd;
+  sc.wdu = 1.0f - lrwd;
+  sc.ss = lrv / c1;
+  sc.c2s = c2s;
+  sc.eps = eps;
+  const double den_scale = 1.0 / ((double)c2s * (double)sc.ss), den_eps = (double)eps / (double)sc.ss;
+  const bool fits = den_scale <= (double)FLT_MAX && den_eps <= (double)FLT_MAX;
+  sc.den_scale = fits ? (float)den_scale : 0.0f;
+  sc.den_eps = fits ? (float)den_eps : __builtin_inff();
+  const gptr<float> o = as_global<float>(out_);   // the order step_consts() reads
+  o[0] = sc.b1; o[1] = sc.b2; o[2] = sc.r1; o[3] = sc.r2; o[4] = sc.wdu;
+  o[5] = sc.ss; o[6] = sc.c2s; o[7] = sc.eps; o[8] = sc.den_scale; o[9] = sc.den_eps;
+}
 
 // ---------------------------------------------------------------------------
 // global gradient norm (what a caller computes before it clips)

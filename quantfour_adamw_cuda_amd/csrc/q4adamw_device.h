@@ -22,6 +22,15 @@ __device__ __forceinline__ gptr<T> as_global(const void *p) {
   return (gptr<T>)(uintptr_t)p;
 }
 
+// Memory that no kernel of the running launch writes, read through the scalar unit when
+// the address is uniform.
+template <typename T>
+using cptr = __attribute__((address_space(4))) T *;
+template <typename T>
+__device__ __forceinline__ cptr<T> as_constant(const void *p) {
+  return (cptr<T>)(uintptr_t)p;
+}
+
 // Full tiles go through buffer instructions: the tile's base address sits in a
 // scalar resource descriptor and each lane supplies a 32-bit byte offset, so no
 // vector ALU work goes into addresses.  Cache policy of the streamed tensors: the
@@ -449,6 +458,19 @@ __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlo
 }
 
 // The launch's gradient multiplier; false if the launch is to do nothing.
+// The step's derived scalars: the launch's arguments, or what device_step_kernel left in
+// device memory for a step whose number the host does not know (a captured graph).
+__device__ __forceinline__ StepConsts step_consts(const StepConsts &from_args, const GradOps &go) {
+  static_assert(sizeof(StepConsts) == 40, "ten floats, in the order read here and written by device_step_kernel");
+  StepConsts sc = from_args;
+  if (go.sc_dev) {
+    const cptr<const float> f = as_constant<const float>(go.sc_dev);
+    sc.b1 = f[0]; sc.b2 = f[1]; sc.r1 = f[2]; sc.r2 = f[3]; sc.wdu = f[4];
+    sc.ss = f[5]; sc.c2s = f[6]; sc.eps = f[7]; sc.den_scale = f[8]; sc.den_eps = f[9];
+  }
+  return sc;
+}
+
 __device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale) {
   if (go.skip && *as_global<const float>(go.skip) != 0.0f) return false;
   gscale = go.scale;

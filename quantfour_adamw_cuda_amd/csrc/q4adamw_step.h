@@ -357,10 +357,11 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
     return;
   }
   const uint32_t salt = SR ? args.sr_salt[t] : 0u;
+  const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, false, SR, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, false, SR, false>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, false, SR, false>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, false, SR, false>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
@@ -521,10 +522,11 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
     return;
   }
   const uint32_t salt = SR ? args.sr_salt[t] : 0u;
+  const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, args.sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // After the update: the new statistics become the current ones and the buffers that

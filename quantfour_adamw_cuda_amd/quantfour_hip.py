@@ -116,17 +116,67 @@ def _device_scalar(t, device, what):
     return t.data_ptr()
 
 
-def grad_options(device, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False):
+def grad_options(device, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False,
+                 step_consts=None):
     """struct q4adamw_grad_options, or None when the arguments change nothing.  The device
-    scalars are referenced, not copied: keep the tensors alive until the step has run."""
-    if grad_scale == 1.0 and grad_scale_dev is None and found_inf is None and not zero_grad:
+    scalars are referenced, not copied: keep the tensors alive until the step has run.
+    step_consts: the buffer device_step() filled, for a step whose number lives on the device."""
+    if (grad_scale == 1.0 and grad_scale_dev is None and found_inf is None and not zero_grad
+            and step_consts is None):
         return None
     o = _lib.Q4GradOptions()
     o.grad_scale = float(grad_scale)
     o.zero_grad = 1 if zero_grad else 0
     o.grad_scale_dev = None if grad_scale_dev is None else _device_scalar(grad_scale_dev, device, "grad_scale_dev")
     o.skip_if_nonzero = None if found_inf is None else _device_scalar(found_inf, device, "found_inf")
+    if step_consts is not None:
+        assert step_consts.is_cuda and step_consts.device == device and step_consts.is_contiguous()
+        assert step_consts.numel() * step_consts.element_size() >= _lib.STEP_CONSTS_BYTES, "step_consts too small"
+        o.step_consts = step_consts.data_ptr()
     return o
+
+
+def make_bias_table(beta1, beta2, device, max_steps=1 << 22):
+    """Device table of (1 - beta1^t, sqrt(1 - beta2^t)) for t = 1 .. T, two floats per step,
+    computed as the step's launcher computes them; T is the first power of two (from 1024)
+    at which both have become exactly 1, so that later steps may take the last entry."""
+    import ctypes
+    L = _lib.load()
+    steps = 1024
+    while True:
+        last = (ctypes.c_float * 2)()
+        _lib.check(L.q4adamw_bias_table(beta1, beta2, steps, 1, last), "bias_table")
+        if last[0] == 1.0 and last[1] == 1.0:
+            break
+        if steps >= max_steps:
+            raise ValueError(f"bias corrections of betas ({beta1}, {beta2}) have not reached 1 after {steps} steps")
+        steps *= 2
+    host = torch.empty(steps, 2, dtype=torch.float32)
+    _lib.check(L.q4adamw_bias_table(beta1, beta2, 1, steps, host.data_ptr()), "bias_table")
+    return host.to(device)
+
+
+def new_step_consts(device):
+    """Device buffer for device_step() to fill and grad_options(step_consts=...) to pass on."""
+    return torch.zeros(_lib.STEP_CONSTS_BYTES // 4, dtype=torch.float32, device=device)
+
+
+def device_step(step, table, consts, beta1, beta2, lr, weight_decay, eps, lr_dev=None, found_inf=None):
+    """Adds 1 to the device step counter `step` (one float32) unless found_inf holds a
+    non-zero value, and leaves the new step's derived scalars in `consts`; lr comes from the
+    device scalar lr_dev if given.  Asynchronous on the current stream; captures into a graph."""
+    L = _lib.load()
+    device = step.device
+    assert step.is_cuda and step.dtype == torch.float32 and step.numel() == 1, "step must be one device float32"
+    assert table.device == device and table.dtype == torch.float32 and table.dim() == 2 and table.shape[1] == 2 \
+        and table.is_contiguous(), "table must come from make_bias_table"
+    assert consts.device == device and consts.numel() * consts.element_size() >= _lib.STEP_CONSTS_BYTES
+    lr_ptr = None if lr_dev is None else _device_scalar(lr_dev, device, "lr_dev")
+    skip = None if found_inf is None else _device_scalar(found_inf, device, "found_inf")
+    with torch.cuda.device(device):
+        rc = L.q4adamw_device_step(step.data_ptr(), table.data_ptr(), 1, table.shape[0], lr_ptr, beta1, beta2,
+                                   float(lr), weight_decay, eps, skip, consts.data_ptr(), _stream(device))
+    _lib.check(rc, "device_step")
 
 
 def launch_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options=None):
@@ -148,12 +198,14 @@ def launch_small_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay
 
 
 def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr, weight_decay,
-                     eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False):
+                     eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False,
+                     step_consts=None):
     """One launch over many quantized tensors that share device, dtypes and step.  The
     gradients enter the step multiplied by grad_scale * grad_scale_dev (a device float32
     scalar); found_inf (a device float32 scalar) makes the call leave parameters and state
     alone when it holds a non-zero value; zero_grad overwrites the gradients with zeros once
-    they are read, also in a call that found_inf cancels."""
+    they are read, also in a call that found_inf cancels.  step_consts (filled by device_step)
+    replaces the scalars derived from lr, weight_decay, eps and step."""
     if not ps:
         return
     arr = make_table(ps, gs, exps, sqs, exp_scales, sq_scales)
@@ -161,13 +213,13 @@ def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr,
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts)
     launch_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
 
 
 def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, weight_decay,
                               eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None,
-                              zero_grad=False):
+                              zero_grad=False, step_consts=None):
     """One launch over many non-quantized tensors that share device, dtypes and step; gradient
     options as for fused_4bit_multi."""
     if not ps:
@@ -177,7 +229,7 @@ def fused_single_tensor_multi(ps, gs, exp_avgs, exp_avg_sqs, beta1, beta2, lr, w
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts)
     launch_small_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step,
                        options)
 
@@ -280,7 +332,8 @@ def launch_rank1_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, bet
 
 def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts,
                            beta1, beta2, lr, weight_decay, eps, step, grad_scale=1.0,
-                           grad_scale_dev=None, found_inf=None, zero_grad=False, seed=None, salts=None):
+                           grad_scale_dev=None, found_inf=None, zero_grad=False, seed=None, salts=None,
+                           step_consts=None):
     """The fused step over matrices whose second moment is rank-1 scaled: scale of element
     (i, j) = min(row_maxes[i], col_maxes[j]).  row_nexts / col_nexts are state-owned scratch
     that holds zeros between steps.  Gradient options as for fused_4bit_multi.  With a seed
@@ -292,7 +345,7 @@ def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, 
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts)
     if seed is None:
         launch_rank1_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
     else:
