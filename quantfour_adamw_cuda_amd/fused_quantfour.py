@@ -60,6 +60,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         variance_scale_type: str = "group",
         round_type: str = "real-nearest",
         seed: Optional[int] = None,
+        capturable: bool = False,
     ):
         # optim/fused_quantfour.py:38-47
         if not 0.0 < lr:
@@ -98,6 +99,15 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 seed_t = seed_t.cpu()
             seed = int(seed_t)
 
+        # capturable: the step number lives on the device (one counter per param group and
+        # device), so that step() can be captured in a graph and every replay is the next
+        # step; a tensor lr (one float32 on the parameters' device) is read by the kernels,
+        # a float lr, betas, eps and weight_decay are fixed when the graph is captured.  As
+        # for torch.optim.AdamW(capturable=True); the reference reads its step counter on the
+        # host (optim/fused_quantfour.py:178, :286-290) and cannot be captured.
+        if capturable and round_type == "stochastic":
+            raise ValueError("capturable=True is built for round_type='real-nearest' only")
+
         # tensors with numel <= threshold are not quantized
         # (FirstMoment.threshold / SecondMoment.threshold, adamw_fourbit_triton.py:118, :128)
         self.param_quant_threshold = 4096
@@ -110,10 +120,12 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             fused=fused,
             round_type=round_type,
             seed=seed,
+            capturable=capturable,
         )
         super().__init__(params, defaults)
         self._launch_cache: Dict[Any, Any] = {}
         self._step_buffers: Dict[Any, Any] = {}
+        self._device_steps: Dict[Any, Any] = {}
         # global gradient norm of the last step(max_grad_norm=...), a device scalar
         self.last_grad_norm = None
         self._norm_buffers: Dict[Any, Any] = {}
@@ -138,6 +150,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         super().__setstate__(state)
         self._launch_cache = {}
         self._step_buffers = {}
+        self._device_steps = {}
         self._norm_buffers = {}
         self.__dict__.setdefault("kernel_timing", None)
         self.__dict__.setdefault("last_grad_norm", None)
@@ -148,6 +161,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             group.setdefault("fused", None)
             group.setdefault("round_type", "real-nearest")
             group.setdefault("seed", None)
+            group.setdefault("capturable", False)
         state_values = list(self.state.values())
         step_is_tensor = len(state_values) != 0 and torch.is_tensor(state_values[0]["step"])
         if not step_is_tensor:
@@ -270,6 +284,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             if "momentum_qstate" not in src:
                 self._adopt_adamw_state(p, dst)
         self._launch_cache = {}
+        self._device_steps = {}      # device step counters restart from the loaded host numbers
 
     def _adopt_adamw_state(self, p, state):
         """Turns one parameter's torch.optim.AdamW state (step, exp_avg, exp_avg_sq in the
@@ -454,8 +469,22 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             stochastic = group.get("round_type", "real-nearest") == "stochastic"
 
             # update step (optim/fused_quantfour.py:178)
+            capturable = bool(group.get("capturable", False))
+            if capturable and len(params_with_grad) != sum(1 for p in group["params"] if p.numel() > 0):
+                raise ValueError("capturable=True needs a gradient for every parameter of the group: "
+                                 "the group's parameters share one step counter on the device")
+            before = [float(s) for s in state_steps] if capturable and not self._has_device_steps(gi) else None
             steps = self._advance_steps(gi, params_with_grad, state_steps)
-            stepped.extend(state_steps)
+            if not capturable:       # a capturable group's true counter is on the device
+                stepped.extend(state_steps)
+            step_consts = {}
+            if capturable:
+                if stochastic:
+                    raise ValueError("capturable=True is built for round_type='real-nearest' only")
+                # one counter per device: advance it and derive the step's scalars there
+                for device in {p.device for p in params_with_grad}:
+                    step_consts[device] = self._device_step(gi, device, group, before, found_inf)
+                steps = [0.0] * len(steps)      # the host's numbers play no part in the launches
 
             # one launch per (kind, device, dtypes, step)
             buckets: Dict[Any, list] = {}
@@ -521,7 +550,10 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 else:
                     launch = (_q.launch_rank1_table if rank1 else
                               _q.launch_table if quantized else _q.launch_small_table)
-                options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad)
+                options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad,
+                                          step_consts.get(device))
+                if capturable:   # lr and step enter through step_consts; these only pass the range check
+                    lr, t_step = 1.0, 1.0
                 if self.kernel_timing is None:
                     launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                 else:
@@ -538,6 +570,59 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         if found_inf is not None and stepped:
             self._watch_skip_flag(found_inf, stepped)
         return loss
+
+    # -- capturable: the step number on the device ------------------------------------
+    def _has_device_steps(self, gi):
+        return any(k[0] == gi for k in self._device_steps)
+
+    def _device_step(self, gi, device, group, steps_before, found_inf):
+        """Advances the device step counter of (param group, device) and returns the buffer
+        that holds the new step's derived scalars.  The counter starts from the host's
+        number of steps taken, which all parameters of the group must share."""
+        beta1, beta2 = group["betas"]
+        key = (gi, device)
+        st = self._device_steps.get(key)
+        if st is None:
+            if steps_before is None:     # another device of this group exists already: same number
+                other = next(v for k, v in self._device_steps.items() if k[0] == gi)
+                first = float(other["counter"])
+            else:
+                if len(set(steps_before)) != 1:
+                    raise ValueError("capturable=True needs all parameters of a group at the same step")
+                first = steps_before[0]
+            st = dict(counter=torch.full((1,), first, dtype=torch.float32, device=device),
+                      table=_q.make_bias_table(float(beta1), float(beta2), device),
+                      consts=_q.new_step_consts(device), betas=(float(beta1), float(beta2)),
+                      lr_dev=None, lr_host=None)
+            self._device_steps[key] = st
+        if st["betas"] != (float(beta1), float(beta2)):
+            st["table"] = _q.make_bias_table(float(beta1), float(beta2), device)
+            st["betas"] = (float(beta1), float(beta2))
+        lr = group["lr"]
+        if torch.is_tensor(lr):
+            assert lr.is_cuda and lr.device == device and lr.dtype == torch.float32 and lr.numel() == 1, \
+                "a tensor lr must be one float32 on the parameters' device"
+            lr_dev, lr_host = lr.reshape(1), 1.0
+        else:
+            if st["lr_dev"] is None:
+                st["lr_dev"] = torch.empty(1, dtype=torch.float32, device=device)
+            if st["lr_host"] != float(lr):      # refreshed only when the host's value changes
+                st["lr_dev"].fill_(float(lr))
+                st["lr_host"] = float(lr)
+            lr_dev, lr_host = st["lr_dev"], float(lr)
+        _q.device_step(st["counter"], st["table"], st["consts"], float(beta1), float(beta2), lr_host,
+                       group["weight_decay"], group["eps"], lr_dev=lr_dev, found_inf=found_inf)
+        return st["consts"]
+
+    def _sync_host_steps(self):
+        """capturable: the device counters are the truth (replays of a captured graph do not
+        pass through step()); copies them into the parameters' host step counters."""
+        for (gi, device), st in self._device_steps.items():
+            value = float(st["counter"])          # synchronises
+            for p in self.param_groups[gi]["params"]:
+                s = self.state.get(p)
+                if s and p.device == device and torch.is_tensor(s.get("step")):
+                    s["step"].fill_(value)
 
     def _advance_steps(self, gi, params, state_steps):
         """Adds 1 to every step counter and returns their new values as Python floats.  The
@@ -588,4 +673,5 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
 
     def state_dict(self):
         self._settle_skipped_step()
+        self._sync_host_steps()
         return super().state_dict()

@@ -176,3 +176,111 @@ def test_device_step_argument_errors(cuda):
     o.grad_scale, o.step_consts = 1.0, t.data_ptr() + 4
     arr = (_lib.Q4Tensor * 1)()
     assert L.q4adamw_fused_4bit_multi_ex(arr, 1, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, ctypes.byref(o), None) == -2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variance", ["group", "rank1"])
+def test_capturable_optimizer_replays_equal_the_eager_optimizer(cuda, variance):
+    """AdamWFused_QuantFour(capturable=True): one warm-up step, then step(zero_grad=True) is
+    captured once and replayed; every replay is the next step (device counter, tensor lr) and
+    equals, bit for bit, a second optimizer stepping eagerly with the step number on the host;
+    state_dict() reports the device's step count; a resumed optimizer continues identically"""
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+    gen = torch.Generator().manual_seed(12)
+    shapes = [(40, 1024), (300, 33), (64,), (5000,), (16, 520)]
+    init = [torch.randn(s, generator=gen) * 0.05 for s in shapes]
+    pc = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
+    pe = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
+    lr_t = torch.full((), 1e-3, device=cuda)
+    oc_ = AdamWFused_QuantFour(pc, lr=lr_t, weight_decay=0.01, variance_scale_type=variance, capturable=True)
+    oe = AdamWFused_QuantFour(pe, lr=1e-3, weight_decay=0.01, variance_scale_type=variance)
+    static = [torch.zeros_like(p) for p in pc]
+    for p, g in zip(pc, static):
+        p.grad = g
+
+    def fresh_grads(step):
+        gs = [(grads_config1(gen, p.numel()).view(p.shape)).to(cuda) for p in pc]
+        for buf, g, p in zip(static, gs, pe):
+            buf.copy_(g)
+            p.grad = g.clone()
+        lr = 1e-3 / step
+        lr_t.fill_(lr)
+        oe.param_groups[0]["lr"] = float(lr_t)
+
+    def check(step):
+        for i, (a, b) in enumerate(zip(pc, pe)):
+            assert torch.equal(a, b), f"step {step}: parameter {i}"
+            sa, sb = oc_.state[a], oe.state[b]
+            assert torch.equal(sa["exp_avg"], sb["exp_avg"]) and torch.equal(sa["exp_avg_sq"], sb["exp_avg_sq"]), (step, i)
+            assert not a.grad.any(), "zero_grad inside the captured step"
+
+    fresh_grads(1)
+    oc_.step(zero_grad=True)            # warm-up: state and descriptor tables exist before the capture
+    oe.step()
+    check(1)
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    graph = torch.cuda.CUDAGraph()
+    fresh_grads(2)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            oc_.step(zero_grad=True)
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    torch.cuda.synchronize()
+    for step in range(2, 8):
+        if step > 2:
+            fresh_grads(step)
+        graph.replay()
+        oe.step()
+        torch.cuda.synchronize()
+        check(step)
+    sd = oc_.state_dict()
+    assert all(float(s["step"]) == 7.0 for s in sd["state"].values())
+    assert all(float(s["step"]) == 7.0 for s in oe.state_dict()["state"].values())
+    # resume (eagerly) from the captured run's state: the counter restarts from the loaded number
+    p2 = [torch.nn.Parameter(p.detach().clone()) for p in pc]
+    o2 = AdamWFused_QuantFour(p2, lr=1e-3, weight_decay=0.01, variance_scale_type=variance, capturable=True)
+    o2.load_state_dict(sd)
+    assert torch.is_tensor(o2.param_groups[0]["lr"])      # a copy of the saved tensor
+    o2.param_groups[0]["lr"] = lr_t
+    fresh_grads(8)
+    for p, g in zip(p2, pe):
+        p.grad = g.grad.clone()
+    o2.step()
+    oe.step()
+    for a, b in zip(p2, pe):
+        assert torch.equal(a, b)
+    # a parameter without a gradient is refused: the group shares one counter
+    p2[0].grad = None
+    with pytest.raises(ValueError, match="every parameter"):
+        o2.step()
+
+
+@pytest.mark.gpu
+def test_capturable_optimizer_overflow_flag_and_float_lr(cuda):
+    """a set overflow flag leaves the device counter where it is (state_dict() reports it); a
+    float lr that changes between eager steps is picked up"""
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+    gen = torch.Generator().manual_seed(13)
+    init = [torch.randn(s, generator=gen) * 0.05 for s in ((70, 130), (33,))]
+    pc = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
+    pe = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
+    a = AdamWFused_QuantFour(pc, lr=1e-3, capturable=True)
+    b = AdamWFused_QuantFour(pe, lr=1e-3)
+    flag = torch.zeros(1, device=cuda)
+    for it in range(5):
+        gs = [grads_config1(gen, p.numel()).view(p.shape).to(cuda) for p in pc]
+        for opt, ps in ((a, pc), (b, pe)):
+            opt.param_groups[0]["lr"] = 1e-3 * (it + 1)
+            for p, g in zip(ps, gs):
+                p.grad = g.clone()
+        if it == 2:      # an overflowed iteration for the capturable optimizer only
+            flag.fill_(1.0)
+            a.step(found_inf=flag)
+            flag.zero_()
+            assert all(float(s["step"]) == 2.0 for s in a.state_dict()["state"].values())
+        a.step(found_inf=flag)
+        b.step()
+        for x, y in zip(pc, pe):
+            assert torch.equal(x, y), f"iteration {it}"
+    assert all(float(s["step"]) == 5.0 for s in a.state_dict()["state"].values())

@@ -233,6 +233,15 @@ def test_round_type_and_seed_travel_in_the_param_groups():
     assert d._param_position(q0) == 0 and d._param_position(q1) == 1
 
 
+def test_capturable_option():
+    (p,) = params((64, 130))
+    assert AdamWFused_QuantFour([p]).param_groups[0]["capturable"] is False
+    opt = AdamWFused_QuantFour([p], capturable=True)
+    assert opt.param_groups[0]["capturable"] is True and opt.state_dict()["param_groups"][0]["capturable"] is True
+    with pytest.raises(ValueError, match="capturable"):
+        AdamWFused_QuantFour([p], capturable=True, round_type="stochastic")
+
+
 def test_setstate_backfills():
     (p,) = params((4, 4))
     opt = AdamWFused_QuantFour([p])
