@@ -100,8 +100,8 @@ typedef struct q4adamw_small_tensor {
  *                    derived scalars (bias corrections, step size, weight-decay factor)
  *                    are read from there and the call's own lr, weight_decay, eps and
  *                    step only pass the range check -- for a step whose number the host
- *                    does not know, e.g. inside a captured graph.  Not with the _sr
- *                    entry points: their noise depends on the step number.
+ *                    does not know, e.g. inside a captured graph.  The _sr entry points
+ *                    then key their noise by the step number found there.
  *   zero_grad        non-zero: the gradients are overwritten with zeros once read
  *                    (the `g` pointers are written in that case), also by a call
  *                    that skip_if_nonzero cancels: the overflowed gradients must

@@ -312,8 +312,8 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
-  if (sr && a.go.sc_dev)
-    return fail(Q4ADAMW_ERR_ARG, "stochastic rounding needs the step number on the host (its noise depends on it)");
+  a.seed_lo = (uint32_t)seed;
+  a.seed_hi = (uint32_t)(seed >> 32);
   // a lane reads 8 consecutive elements at once when parameters and gradients are 16-bit types, else 4
   const bool p_half = p_dtype != Q4ADAMW_FP32, g_half = g_dtype != Q4ADAMW_FP32;
   const bool wide = p_half && g_half;   // 8 elements per lane
@@ -356,7 +356,8 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
     d.sm = t.exp_avg_scale;
     d.sv = t.exp_avg_sq_scale;
     d.numel = t.numel;
-    a.sr_salt[a.ntensors] = sr ? q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i) : 0u;
+    a.sr_salt[a.ntensors] = !sr ? 0u : a.go.sc_dev ? lowbias32(salts ? salts[i] : (uint32_t)i)
+                                                     : q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i);
     a.first_chunk[a.ntensors] = (uint32_t)chunks;
     ++a.ntensors;
     chunks += c;
@@ -377,8 +378,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   bool ext = false;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
   if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
-  if (sr && a.go.sc_dev)
-    return fail(Q4ADAMW_ERR_ARG, "stochastic rounding needs the step number on the host (its noise depends on it)");
+  a.seed_lo = (uint32_t)seed;
+  a.seed_hi = (uint32_t)(seed >> 32);
   sa.go = a.go;
   sa.b2 = a.sc.b2;
   sa.r2 = a.sc.r2;
@@ -464,7 +465,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       const FastDiv fd = make_fast_div((uint32_t)(t.cols >> 3));
       d.div_magic = fd.magic;
       d.div_shift = fd.shift;
-      a.sr_salt[a.ntensors] = sr ? q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i) : 0u;
+      a.sr_salt[a.ntensors] = !sr ? 0u : a.go.sc_dev ? lowbias32(salts ? salts[i] : (uint32_t)i)
+                                                     : q4adamw_sr_tensor_salt(seed, step, salts ? salts[i] : (uint32_t)i);
       a.first_chunk[a.ntensors] = (uint32_t)chunks;
       Rank1StatArgs::Desc &sd = sa.desc[a.ntensors];
       sd.g = t.g;
@@ -748,6 +750,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1010; }
+int q4adamw_version(void) { return 1011; }
 
 }  // extern "C"

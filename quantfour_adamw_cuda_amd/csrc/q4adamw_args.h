@@ -61,7 +61,11 @@ struct FusedArgs {
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
   TensorDesc desc[kMaxTensors];
-  uint32_t sr_salt[kMaxTensors];  // stochastic rounding: the tensors' noise salts of this step
+  // stochastic rounding: the tensors' noise salts of this step; with a step number on the
+  // device (go.sc_dev) the hash of each tensor's own salt, which the kernel carries on
+  // through step number and seed
+  uint32_t sr_salt[kMaxTensors];
+  uint32_t seed_lo, seed_hi;
 };
 
 struct SmallDesc {  // 40 bytes
@@ -141,7 +145,8 @@ struct Rank1Args {
   uint32_t chunks_per_xcd;
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
-  uint32_t sr_salt[kMaxRank1Tensors];   // stochastic rounding: the tensors' salts of this step
+  uint32_t sr_salt[kMaxRank1Tensors];   // stochastic rounding: as FusedArgs::sr_salt
+  uint32_t seed_lo, seed_hi;
   Rank1Desc desc[kMaxRank1Tensors];
 };
 

@@ -471,6 +471,17 @@ __device__ __forceinline__ StepConsts step_consts(const StepConsts &from_args, c
   return sc;
 }
 
+// The noise salt of a tensor in this step (q4adamw_sr_tensor_salt: the tensor's own salt,
+// the step number and the two halves of the seed, hashed in turn).  The host has finished the
+// chain when it knows the step number; otherwise it has hashed the tensor's salt and the
+// kernel goes on with the number device_step_kernel left behind its scalars.
+__device__ __forceinline__ uint32_t step_salt(uint32_t from_args, const GradOps &go, uint32_t seed_lo,
+                                              uint32_t seed_hi) {
+  if (!go.sc_dev) return from_args;
+  const uint32_t step = as_constant<const uint32_t>(go.sc_dev)[10];
+  return lowbias32(lowbias32(lowbias32(from_args ^ step) ^ seed_hi) ^ seed_lo);
+}
+
 __device__ __forceinline__ bool grad_ops_begin(const GradOps &go, float &gscale) {
   if (go.skip && *as_global<const float>(go.skip) != 0.0f) return false;
   gscale = go.scale;

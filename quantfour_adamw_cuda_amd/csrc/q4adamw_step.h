@@ -356,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
     setup_tables<SR>(lds, tid, slot);
     return;
   }
-  const uint32_t salt = SR ? args.sr_salt[t] : 0u;
+  const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
     process_tile<PT, GT, true, EXT, false, SR, false>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
@@ -521,7 +521,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
     setup_tables<SR>(lds, tid, slot);
     return;
   }
-  const uint32_t salt = SR ? args.sr_salt[t] : 0u;
+  const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
     process_tile<PT, GT, true, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);

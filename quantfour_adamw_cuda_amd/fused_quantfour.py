@@ -105,8 +105,6 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # a float lr, betas, eps and weight_decay are fixed when the graph is captured.  As
         # for torch.optim.AdamW(capturable=True); the reference reads its step counter on the
         # host (optim/fused_quantfour.py:178, :286-290) and cannot be captured.
-        if capturable and round_type == "stochastic":
-            raise ValueError("capturable=True is built for round_type='real-nearest' only")
 
         # tensors with numel <= threshold are not quantized
         # (FirstMoment.threshold / SecondMoment.threshold, adamw_fourbit_triton.py:118, :128)
@@ -479,8 +477,6 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 stepped.extend(state_steps)
             step_consts = {}
             if capturable:
-                if stochastic:
-                    raise ValueError("capturable=True is built for round_type='real-nearest' only")
                 # one counter per device: advance it and derive the step's scalars there
                 for device in {p.device for p in params_with_grad}:
                     step_consts[device] = self._device_step(gi, device, group, before, found_inf)

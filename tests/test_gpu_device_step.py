@@ -91,10 +91,15 @@ def test_device_step_equals_host_step(cuda, p_dt, g_dt):
     q.fused_4bit_multi([b.p], [g], [b.m], [b.v], [b.sm], [b.sv], *HPA, 1, step_consts=consts)
     q.fused_4bit_multi([a.p], [g], [a.m], [a.v], [a.sm], [a.sv], *HPA, far)
     assert _same(a, b)
+    # stochastic rounding: the noise's salt is finished on the device from the step number there
     arr = q.make_table([b.p], [g], [b.m], [b.v], [b.sm], [b.sv])
-    with pytest.raises(RuntimeError, match="stochastic"):   # its noise needs the step number on the host
-        q.launch_table_sr(arr, None, 5, cuda, q._tag(b.p, "param"), q._tag(g, "grad"), *HPA, 1,
+    salts = q.make_salts([77])
+    for k in (1, 2):
+        q.device_step(counter, table, consts, *HPA)
+        q.launch_table_sr(arr, salts, 0xABCDEF0123456789, cuda, q._tag(b.p, "param"), q._tag(g, "grad"), *HPA, 1,
                           q.grad_options(cuda, step_consts=consts))
+        q.fused_4bit_multi_sr([a.p], [g], [a.m], [a.v], [a.sm], [a.sv], *HPA, far + k, 0xABCDEF0123456789, salts=[77])
+        assert float(counter) == far + k and _same(a, b), f"stochastic rounding, step {far + k}"
 
 
 @pytest.mark.gpu
@@ -179,8 +184,9 @@ def test_device_step_argument_errors(cuda):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("variance", ["group", "rank1"])
-def test_capturable_optimizer_replays_equal_the_eager_optimizer(cuda, variance):
+@pytest.mark.parametrize("variance,rounding", [("group", "real-nearest"), ("rank1", "real-nearest"),
+                                               ("group", "stochastic"), ("rank1", "stochastic")])
+def test_capturable_optimizer_replays_equal_the_eager_optimizer(cuda, variance, rounding):
     """AdamWFused_QuantFour(capturable=True): one warm-up step, then step(zero_grad=True) is
     captured once and replayed; every replay is the next step (device counter, tensor lr) and
     equals, bit for bit, a second optimizer stepping eagerly with the step number on the host;
@@ -192,8 +198,9 @@ def test_capturable_optimizer_replays_equal_the_eager_optimizer(cuda, variance):
     pc = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
     pe = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
     lr_t = torch.full((), 1e-3, device=cuda)
-    oc_ = AdamWFused_QuantFour(pc, lr=lr_t, weight_decay=0.01, variance_scale_type=variance, capturable=True)
-    oe = AdamWFused_QuantFour(pe, lr=1e-3, weight_decay=0.01, variance_scale_type=variance)
+    kw = dict(weight_decay=0.01, variance_scale_type=variance, round_type=rounding, seed=31)
+    oc_ = AdamWFused_QuantFour(pc, lr=lr_t, capturable=True, **kw)
+    oe = AdamWFused_QuantFour(pe, lr=1e-3, **kw)
     static = [torch.zeros_like(p) for p in pc]
     for p, g in zip(pc, static):
         p.grad = g
@@ -239,7 +246,7 @@ def test_capturable_optimizer_replays_equal_the_eager_optimizer(cuda, variance):
     assert all(float(s["step"]) == 7.0 for s in oe.state_dict()["state"].values())
     # resume (eagerly) from the captured run's state: the counter restarts from the loaded number
     p2 = [torch.nn.Parameter(p.detach().clone()) for p in pc]
-    o2 = AdamWFused_QuantFour(p2, lr=1e-3, weight_decay=0.01, variance_scale_type=variance, capturable=True)
+    o2 = AdamWFused_QuantFour(p2, lr=1e-3, capturable=True, **kw)
     o2.load_state_dict(sd)
     assert torch.is_tensor(o2.param_groups[0]["lr"])      # a copy of the saved tensor
     o2.param_groups[0]["lr"] = lr_t
