@@ -135,14 +135,19 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     sm_old = as_global<const float>(sm_tile)[blk];
     if (!RANK1) sv_old = as_global<const float>(sv_tile)[blk];
   }
-  if (RANK1) sv_old = 1.0f;  // the table holds the bare code book; the scale follows per element
-  // this block's dequantization table: entry i = {code_book_m[i] * scale_m,
-  // code_book_v[i] * scale_v} (cuda_adamw_kernels.cu:340,343), written by the block's
-  // lanes (lane & 15 = i) into the wave's private LDS region
+  // this block's dequantization table: entry i = {beta1 * (code_book_m[i] * scale_m),
+  // beta2 * (code_book_v[i] * scale_v)}: the old moments (cuda_adamw_kernels.cu:340,343)
+  // with the first product of their updates (:341,344) already applied, each product
+  // rounded as the per-element form rounds it.  Written by the block's lanes (lane & 15 =
+  // i) into the wave's private LDS region.  Rank-1: the second entry is the bare code-book
+  // value; scale and beta2 follow per element.
   char *lds_bytes = reinterpret_cast<char *>(lds);
   const uint32_t cb_entry = (uint32_t)wave * 64u + blk * 16u;  // entry number of code 0
-  *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) =
-      make_float2(slot.qm * sm_old, qmap_v(lane & 15) * sv_old);
+  {
+    const float m_entry = sc.b1 * (slot.qm * sm_old);
+    const float v_entry = RANK1 ? qmap_v(lane & 15) : sc.b2 * (qmap_v(lane & 15) * sv_old);
+    *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) = make_float2(m_entry, v_entry);
+  }
   setup_tables<SR>(lds, tid, slot);
 
   // entry numbers of the lane's codes, one per byte: even elements, odd elements
@@ -160,10 +165,10 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, three);
     const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
     float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
-    if constexpr (RANK1) v_old *= min_nonneg(r_old, c_old.x[j]);  // adamw_fourbit_triton.py:520-527
+    if constexpr (RANK1) v_old = sc.b2 * (v_old * min_nonneg(r_old, c_old.x[j]));  // adamw_fourbit_triton.py:520-527
     const float gj = g[j];
-    float m = sc.b1 * m_old + sc.r1 * gj;
-    float v = sc.b2 * v_old + sc.r2 * (gj * gj);
+    float m = m_old + sc.r1 * gj;                 // m_old, v_old: beta times the old moment
+    float v = v_old + sc.r2 * (gj * gj);
     if (!FULL && j >= nv) { m = 0.0f; v = 0.0f; }
     // parameter: only this part may use the hardware's 1-ulp sqrt and reciprocal
     const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
