@@ -179,6 +179,66 @@ def step_quant_rank1(p, g, m_codes, v_codes, m_scale, row_max, col_max, *, beta1
     return p_new.to(p.dtype).view_as(p), mc, vc, ms, rmax, cmax
 
 
+# Tensors of more than two dimensions: one statistic per dimension, the maximum over all
+# other dimensions (get_variance_tensor_statistics loops over x.dim(),
+# optim/adamw_fourbit_triton.py:738-746), the scale of an element their broadcast minimum
+# (compute_variance_tensor_scale, :749-755).  max_dims: one tensor per dimension in keepdim
+# shape ([d0,1,1], [1,d1,1], [1,1,d2] for a 3-D tensor), as the draft's metadata holds them.
+def rank1_stats_nd(x):
+    ax = torch.nan_to_num(x.abs(), nan=0.0, posinf=float("inf"))   # a NaN never becomes a maximum
+    out = []
+    for i in range(x.dim()):
+        others = [d for d in range(x.dim()) if d != i]
+        out.append(ax.amax(dim=others, keepdim=True))
+    return out
+
+
+def rank1_scale_nd(max_dims):
+    scale = max_dims[0]
+    for m in max_dims[1:]:
+        scale = torch.minimum(scale, m)                      # broadcasting
+    return scale
+
+
+def dequantize_rank1_nd(codes, max_dims):
+    scale = rank1_scale_nd(max_dims)
+    idx = unpack(codes, scale.numel())
+    return QMAP[1].to(codes.device)[idx].view(scale.shape) * scale
+
+
+def quantize_rank1_nd(x, u=None):
+    """x: fp32 tensor of two or more dimensions (non-negative).  u: float32 numpy noise per
+    element for stochastic rounding, or None for the nearest code.  Returns (packed codes,
+    max_dims)."""
+    max_dims = rank1_stats_nd(x)
+    qx = x.div(rank1_scale_nd(max_dims))                     # 0/0 -> NaN -> code 0
+    if u is None:
+        q = torch.bucketize(torch.nan_to_num(qx, nan=-2.0), QMID[1].to(x.device), right=False).reshape(-1)
+    else:
+        q = torch.from_numpy(sr_codes(qx.reshape(-1).numpy(), 1, np.asarray(u, np.float32)).astype(np.int64))
+    return pack(q, x.numel()), max_dims
+
+
+def step_quant_rank1_nd(p, g, m_codes, v_codes, m_scale, max_dims, *, beta1, beta2, lr, weight_decay, eps,
+                        step, seed=None, tensor_salt=0):
+    """The fused step on a tensor of two or more dimensions with a rank-1-scaled second moment
+    (with a seed: stochastic rounding of both moments).  Returns new (p, m_codes, v_codes,
+    m_scale, max_dims)."""
+    numel = p.numel()
+    sc = derive_scalars(beta1, beta2, lr, weight_decay, step)
+    m = dequantize(m_codes, m_scale, numel, 0)
+    v = dequantize_rank1_nd(v_codes, max_dims).reshape(-1)
+    p_new, m_new, v_new = adamw_update(p.reshape(-1).float(), g.reshape(-1).float(), m, v, sc, eps)
+    if seed is None:
+        mc, ms = quantize(m_new, 0)
+        vc, new_dims = quantize_rank1_nd(v_new.view(p.shape))
+    else:
+        um, uv = sr_noise(numel, sr_tensor_salt(seed, step, tensor_salt))
+        mc, ms = quantize_sr(m_new, 0, um)
+        vc, new_dims = quantize_rank1_nd(v_new.view(p.shape), uv)
+    return p_new.to(p.dtype).view_as(p), mc, vc, ms, new_dims
+
+
 # ---------------------------------------------------------------------------
 # stochastic rounding in the quantizer
 #

@@ -431,6 +431,50 @@ def test_c_and_torch_oracles_agree_on_fp16_tensors():
         assert np.array_equal(pc.view(np.uint16), ts[0].numpy().view(np.uint16)), f"step {step}"
 
 
+def test_rank1_nd_brute_force_and_reduction_to_matrices():
+    """statistics per dimension and their broadcast minimum on small 3-D and 4-D tensors, by
+    plain loops; on a matrix the N-D functions, quantizer and step, are the 2-D ones"""
+    rng = np.random.default_rng(51)
+    f32 = np.float32
+    mid = [f32((2 * k + 1) / 32) for k in range(1, 16)]
+    for shape in ((3, 4, 8), (2, 3, 2, 8), (5, 1, 16)):
+        x = (np.abs(rng.standard_normal(shape)) ** 3).astype(np.float32)
+        x[1] = 0.0 if len(shape) == 3 else x[1]
+        x[..., 2] = 0.0
+        codes, dims = ot.quantize_rank1_nd(torch.from_numpy(x))
+        got = ot.unpack(codes, x.size).numpy().reshape(shape)
+        back = ot.dequantize_rank1_nd(codes, dims).numpy()
+        for d, st in enumerate(dims):
+            want = x.max(axis=tuple(k for k in range(len(shape)) if k != d))
+            assert st.shape == tuple(n if k == d else 1 for k, n in enumerate(shape))
+            assert np.array_equal(st.numpy().reshape(-1), want)
+        for idx in np.ndindex(*shape):
+            s = min(f32(np.take(x, idx[d], axis=d).max()) for d in range(len(shape)))
+            if s == 0:
+                want = 0
+            else:
+                q = f32(x[idx] / s)
+                want = sum(1 for t in mid if t < q)
+            assert got[idx] == want, (shape, idx)
+            assert back[idx] == f32(f32((want + 1) / 16) * s)
+    m = torch.from_numpy((np.abs(rng.standard_normal((6, 24))) ** 2).astype(np.float32))
+    c2, r, c = ot.quantize_rank1(m)
+    cn, dims = ot.quantize_rank1_nd(m)
+    assert torch.equal(c2, cn) and torch.equal(dims[0].reshape(-1), r) and torch.equal(dims[1].reshape(-1), c)
+    # the step: a matrix through the N-D step equals the 2-D step, nearest and stochastic
+    gen = torch.Generator().manual_seed(24)
+    p, g = torch.randn(8, 128, generator=gen) * 0.02, torch.randn(8, 128, generator=gen)
+    z8, zs = torch.zeros(512, dtype=torch.uint8), torch.zeros(8)
+    a = ot.step_quant_rank1(p, g, z8, z8.clone(), zs, torch.zeros(8), torch.zeros(128), step=1, **HP)
+    b = ot.step_quant_rank1_nd(p, g, z8, z8.clone(), zs, [torch.zeros(8, 1), torch.zeros(1, 128)], step=1, **HP)
+    assert all(torch.equal(x, y) for x, y in zip(a[:4], b[:4]))
+    assert torch.equal(a[4], b[4][0].reshape(-1)) and torch.equal(a[5], b[4][1].reshape(-1))
+    a = ot.step_quant_rank1_sr(p, g, z8, z8.clone(), zs, torch.zeros(8), torch.zeros(128), seed=9, tensor_salt=2, step=1, **HP)
+    b = ot.step_quant_rank1_nd(p, g, z8, z8.clone(), zs, [torch.zeros(8, 1), torch.zeros(1, 128)], seed=9,
+                               tensor_salt=2, step=1, **HP)
+    assert all(torch.equal(x, y) for x, y in zip(a[:4], b[:4]))
+
+
 # ---------------------------------------------------------------------------
 # stochastic rounding
 # ---------------------------------------------------------------------------
