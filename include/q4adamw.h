@@ -179,6 +179,16 @@ uint32_t q4adamw_sr_tensor_salt(uint64_t seed, float step, uint32_t tensor_salt)
  * sizes that must hold zeros on entry and holds zeros again afterwards.
  * rows x cols, row-major, cols a multiple of 8 and at least 16; p, g, col_max and
  * col_max_next 16-byte aligned, the rest 4-byte aligned.
+ *
+ * Tensors of three or four dimensions (lead_dims = 2 or 3): cols is the last dimension,
+ * lead_shape the others, rows their product.  Every leading dimension has its own
+ * statistic, the maximum over all other dimensions (the loop over x.dim() at
+ * optim/adamw_fourbit_triton.py:741-745): lead_max[j] (lead_shape[j] floats, updated by the
+ * call) with scratch lead_max_next[j] (zeros on entry and afterwards).  The scale of an
+ * element is the minimum over all its dimensions' statistics (:749-755); row_max then holds,
+ * for every flattened row, the minimum over its leading statistics -- derived state that the
+ * call keeps up to date and the caller recomputes after loading a checkpoint.  lead_dims = 0
+ * or 1: a matrix, the lead_* fields are not read.
  */
 typedef struct q4adamw_rank1_tensor {
   void *p;
@@ -192,6 +202,11 @@ typedef struct q4adamw_rank1_tensor {
   float *col_max_next;
   int64_t rows;
   int64_t cols;
+  int32_t lead_dims;
+  int32_t reserved;
+  int64_t lead_shape[3];
+  float *lead_max[3];
+  float *lead_max_next[3];
 } q4adamw_rank1_tensor;
 
 /*
@@ -303,6 +318,14 @@ int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, f
  */
 int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel, int which,
                        float *out, void *stream);
+
+/*
+ * q4adamw_quantize_rank1 with the scales given instead of computed: element (i, j) is divided
+ * by min(row_scale[i], col_max[j]).  For tensors of more than two dimensions, whose rows'
+ * scales are the minimum over the leading dimensions' statistics (q4adamw_rank1_tensor).
+ */
+int q4adamw_quantize_rank1_scaled(const float *x, int64_t rows, int64_t cols, const float *row_scale,
+                                  const float *col_max, uint8_t *codes, void *stream);
 
 /*
  * The same pair for a second moment with rank-1 scaling: x is a rows x cols fp32

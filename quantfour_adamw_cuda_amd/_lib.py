@@ -51,6 +51,11 @@ class Q4Rank1Tensor(ctypes.Structure):
         ("col_max_next", ctypes.c_void_p),
         ("rows", ctypes.c_int64),
         ("cols", ctypes.c_int64),
+        ("lead_dims", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("lead_shape", ctypes.c_int64 * 3),
+        ("lead_max", ctypes.c_void_p * 3),
+        ("lead_max_next", ctypes.c_void_p * 3),
     ]
 
 
@@ -93,6 +98,7 @@ EXPORTS = (
     "q4adamw_quantize",
     "q4adamw_dequantize",
     "q4adamw_quantize_rank1",
+    "q4adamw_quantize_rank1_scaled",
     "q4adamw_dequantize_rank1",
     "q4adamw_derive_scalars",
     "q4adamw_tables",
@@ -154,6 +160,8 @@ def load():
     L.q4adamw_dequantize.restype = i
     L.q4adamw_quantize_rank1.argtypes = [vp, i64, i64, vp, vp, vp, vp]
     L.q4adamw_quantize_rank1.restype = i
+    L.q4adamw_quantize_rank1_scaled.argtypes = [vp, i64, i64, vp, vp, vp, vp]
+    L.q4adamw_quantize_rank1_scaled.restype = i
     L.q4adamw_dequantize_rank1.argtypes = [vp, vp, vp, i64, i64, vp, vp]
     L.q4adamw_dequantize_rank1.restype = i
     L.q4adamw_derive_scalars.argtypes = [f, f, f, f, f, ctypes.POINTER(f)]

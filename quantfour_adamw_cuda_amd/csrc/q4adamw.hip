@@ -403,6 +403,18 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       return fail(Q4ADAMW_ERR_ALIGN, "code, scale and row buffers must be 4-byte aligned");
     if (!aligned(t.col_max, 16) || !aligned(t.col_max_next, 16))
       return fail(Q4ADAMW_ERR_ALIGN, "column buffers must be 16-byte aligned");
+    if (t.lead_dims < 0 || t.lead_dims > 3) return fail(Q4ADAMW_ERR_ARG, "lead_dims must be 0 to 3");
+    if (t.lead_dims >= 2) {
+      int64_t prod = 1;
+      for (int j = 0; j < t.lead_dims; ++j) {
+        if (t.lead_shape[j] < 1 || !t.lead_max[j] || !t.lead_max_next[j])
+          return fail(Q4ADAMW_ERR_ARG, "leading dimensions need a positive size and their statistics");
+        if (!aligned(t.lead_max[j], 4) || !aligned(t.lead_max_next[j], 4))
+          return fail(Q4ADAMW_ERR_ALIGN, "leading statistics must be 4-byte aligned");
+        prod *= t.lead_shape[j];
+      }
+      if (prod != t.rows) return fail(Q4ADAMW_ERR_ARG, "rows must be the product of the leading dimensions");
+    }
     const uint64_t numel = (uint64_t)t.rows * (uint64_t)t.cols;
     const uint64_t stat_chunks = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) *
                                  (uint64_t)((t.cols + kStatCols - 1) / kStatCols);
@@ -411,6 +423,9 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t tile_elems = chunk_elems / kWaves;
+  FoldArgs fa;   // the batch's tensors with several leading dimensions
+  fa.go = a.go;
+  fa.ntensors = 0;
   Rank1Kernel kernel = nullptr;
   const Rank1StatKernel stat_kernel = pick_rank1_stats(g_dtype, ext);
   a.ntensors = 0;
@@ -422,6 +437,11 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     sa.nchunks = (uint32_t)stat_chunks;
     hipLaunchKernelGGL(stat_kernel, dim3(sa.nchunks), dim3(kThreads), 0, s, sa);
     Q4_HIP(hipGetLastError());
+    if (fa.ntensors > 0) {   // rows' maxima -> leading statistics -> rows' scales
+      hipLaunchKernelGGL(rank1_fold_kernel<0>, dim3(64, (unsigned)fa.ntensors), dim3(256), 0, s, fa);
+      hipLaunchKernelGGL(rank1_fold_kernel<1>, dim3(64, (unsigned)fa.ntensors), dim3(256), 0, s, fa);
+      Q4_HIP(hipGetLastError());
+    }
     finish_prefix(a);
     a.nchunks = (uint32_t)chunks;
     a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
@@ -429,6 +449,11 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     Q4_HIP(hipGetLastError());
     hipLaunchKernelGGL(rank1_commit_kernel, dim3(64, (unsigned)a.ntensors), dim3(256), 0, s, a);
     Q4_HIP(hipGetLastError());
+    if (fa.ntensors > 0) {
+      hipLaunchKernelGGL(rank1_fold_kernel<2>, dim3(8, (unsigned)fa.ntensors), dim3(256), 0, s, fa);
+      Q4_HIP(hipGetLastError());
+      fa.ntensors = 0;
+    }
     a.ntensors = 0;
     chunks = 0;
     stat_chunks = 0;
@@ -446,8 +471,19 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
       const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
       if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
-          stat_chunks + sc_ > kMaxChunksPerLaunch) {
+          stat_chunks + sc_ > kMaxChunksPerLaunch || (t.lead_dims >= 2 && fa.ntensors == kMaxFoldTensors)) {
         if (int rc = launch()) return rc;
+      }
+      if (t.lead_dims >= 2) {
+        FoldDesc &f = fa.desc[fa.ntensors++];
+        f.row_next = t.row_max_next;
+        f.rows = t.rows;
+        f.dims = t.lead_dims;
+        for (int j = 0; j < 3; ++j) {
+          f.shape[j] = j < t.lead_dims ? t.lead_shape[j] : 1;
+          f.cur[j] = j < t.lead_dims ? t.lead_max[j] : nullptr;
+          f.next[j] = j < t.lead_dims ? t.lead_max_next[j] : nullptr;
+        }
       }
       Rank1Desc &d = a.desc[a.ntensors];
       d.p = t.p;
@@ -717,6 +753,20 @@ int q4adamw_quantize_rank1(const float *x, int64_t rows, int64_t cols, uint8_t *
   return 0;
 }
 
+int q4adamw_quantize_rank1_scaled(const float *x, int64_t rows, int64_t cols, const float *row_scale,
+                                  const float *col_max, uint8_t *codes, void *stream) {
+  if (int rc = check_rank1_shape(rows, cols)) return rc;
+  if (rows == 0 || cols == 0) return 0;
+  if (!x || !codes || !row_scale || !col_max) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+  if (!aligned(x, 4) || !aligned(row_scale, 4) || !aligned(col_max, 4))
+    return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
+  const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
+  hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0, static_cast<hipStream_t>(stream), x,
+                     rows, cols, row_scale, col_max, codes);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 int q4adamw_dequantize_rank1(const uint8_t *codes, const float *row_max, const float *col_max,
                              int64_t rows, int64_t cols, float *out, void *stream) {
   if (int rc = check_rank1_shape(rows, cols)) return rc;
@@ -750,6 +800,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1011; }
+int q4adamw_version(void) { return 1012; }
 
 }  // extern "C"

@@ -172,6 +172,28 @@ struct Rank1StatArgs {
   } desc[kMaxRank1Tensors];
 };
 
+// Rank-1 scaling of a tensor with two or three leading dimensions (its rows are their
+// product): the statistics kernel leaves every flattened row's own maximum, these kernels
+// reduce them to one statistic per leading dimension and hand the update kernel the rows'
+// scales, the minimum over a row's leading statistics.
+constexpr int kMaxFoldTensors = 16;
+
+struct FoldDesc {  // 104 bytes
+  float *row_next;   // in: the rows' own new maxima; out: the rows' new scales
+  int64_t rows;
+  int32_t dims;      // 2 or 3 leading dimensions
+  int32_t pad_;
+  int64_t shape[3];
+  float *cur[3];     // current statistic of each leading dimension
+  float *next[3];    // the step's new statistics (all zero between steps)
+};
+
+struct FoldArgs {
+  GradOps go;
+  int ntensors;
+  FoldDesc desc[kMaxFoldTensors];
+};
+
 // Gradient-norm launch: every workgroup walks chunks of 32 KiB with a grid stride.
 constexpr int kMaxNormTensors = 160;
 constexpr int kNormPartials = Q4ADAMW_NORM_WORKSPACE_BYTES / 8;  // workgroups = fp64 partial sums
@@ -196,7 +218,7 @@ struct NormArgs {
 
 static_assert(sizeof(StepConsts) <= Q4ADAMW_STEP_CONSTS_BYTES, "the device copy of a step's scalars");
 static_assert(sizeof(FusedArgs) <= 4096 && sizeof(SmallArgs) <= 4096 && sizeof(NormArgs) <= 4096 &&
-                  sizeof(Rank1Args) <= 4096 && sizeof(Rank1StatArgs) <= 4096,
+                  sizeof(Rank1Args) <= 4096 && sizeof(Rank1StatArgs) <= 4096 && sizeof(FoldArgs) <= 4096,
               "kernel arguments are limited to 4 KiB");
 
 // the first-moment bucket table (see q4adamw_tables.h), copied into LDS by every

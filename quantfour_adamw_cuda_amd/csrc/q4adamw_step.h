@@ -551,4 +551,45 @@ __global__ __launch_bounds__(256) void rank1_commit_kernel(const Rank1Args args)
   }
 }
 
+// Tensors with several leading dimensions, between statistics and update: row -> its
+// index in leading dimension j (row-major).
+__device__ __forceinline__ int64_t lead_index(const FoldDesc &T, int64_t row, int j) {
+  int64_t stride = 1;
+  for (int k = T.dims - 1; k > j; --k) stride *= T.shape[k];
+  return (row / stride) % T.shape[j];
+}
+
+// mode 0: every leading dimension's new statistic = maximum over the rows that share the index
+// mode 1: every row's new scale = minimum over its leading statistics (after mode 0 is complete)
+// mode 2: after the update, new statistics become current, their buffers return to zero
+// One workgroup column per tensor (blockIdx.y), grid-stride over its rows.
+template <int MODE>
+__global__ __launch_bounds__(256) void rank1_fold_kernel(const FoldArgs args) {
+  float gscale;
+  if (!grad_ops_begin(args.go, gscale)) return;
+  const FoldDesc &T = args.desc[blockIdx.y];
+  const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x, stride = (int64_t)gridDim.x * 256;
+  if (MODE == 2) {
+    for (int j = 0; j < T.dims; ++j) {
+      for (int64_t i = first; i < T.shape[j]; i += stride) {
+        as_global<float>(T.cur[j])[i] = as_global<float>(T.next[j])[i];
+        as_global<float>(T.next[j])[i] = 0.0f;
+      }
+    }
+    return;
+  }
+  for (int64_t row = first; row < T.rows; row += stride) {
+    if (MODE == 0) {
+      const float r = as_global<const float>(T.row_next)[row];
+      if (r != 0.0f) {
+        for (int j = 0; j < T.dims; ++j) atomic_max_nonneg(T.next[j] + lead_index(T, row, j), r);
+      }
+    } else {
+      float s = as_global<const float>(T.next[0])[lead_index(T, row, 0)];
+      for (int j = 1; j < T.dims; ++j) s = min_nonneg(s, as_global<const float>(T.next[j])[lead_index(T, row, j)]);
+      as_global<float>(T.row_next)[row] = s;
+    }
+  }
+}
+
 }  // namespace q4

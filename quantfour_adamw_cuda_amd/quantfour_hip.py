@@ -273,16 +273,39 @@ RANK1_MIN_COLS = 16
 
 
 def rank1_eligible(p):
-    """Whether a parameter's second moment can take rank-1 scaling: a matrix whose rows hold a
-    multiple of 8 and at least 16 elements (other tensors keep per-128 block scales, as 1-D
-    tensors do in the reference's draft, optim/adamw_fourbit_triton.py:841-846)."""
-    return p.dim() == 2 and p.shape[1] % 8 == 0 and p.shape[1] >= RANK1_MIN_COLS
+    """Whether a parameter's second moment can take rank-1 scaling: a tensor of two to four
+    dimensions whose last dimension is a multiple of 8 and at least 16 (other tensors keep
+    per-128 block scales, as 1-D tensors do in the reference's draft,
+    optim/adamw_fourbit_triton.py:841-846)."""
+    return 2 <= p.dim() <= 4 and p.shape[-1] % 8 == 0 and p.shape[-1] >= RANK1_MIN_COLS
 
 
-def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next):
+def rank1_row_scale(lead_maxes, lead_shape):
+    """Scale of every flattened row of a tensor with several leading dimensions: the minimum
+    over the row's leading statistics (compute_variance_tensor_scale without the last
+    dimension, optim/adamw_fourbit_triton.py:749-755).  lead_maxes: one float32 tensor per
+    leading dimension with lead_shape[j] elements.  Returns a flat float32 tensor."""
+    k = len(lead_shape)
+    scale = None
+    for j, m in enumerate(lead_maxes):
+        view = m.reshape([lead_shape[j] if d == j else 1 for d in range(k)])
+        scale = view if scale is None else torch.minimum(scale, view)
+    return scale.expand(list(lead_shape)).reshape(-1).contiguous()
+
+
+def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next, lead=None):
     _check_common(p, g)
-    assert rank1_eligible(p), "rank-1 scaling needs a matrix with cols % 8 == 0 and cols >= 16"
-    rows, cols = p.shape
+    assert rank1_eligible(p), "rank-1 scaling needs 2 to 4 dimensions, the last a multiple of 8 and at least 16"
+    cols = p.shape[-1]
+    rows = p.numel() // cols
+    assert (lead is None) == (p.dim() == 2), "tensors of more than two dimensions need their leading statistics"
+    if lead is not None:
+        lead_maxes, lead_nexts = lead
+        assert len(lead_maxes) == len(lead_nexts) == p.dim() - 1, "one statistic per leading dimension"
+        for j, (m, nx) in enumerate(zip(lead_maxes, lead_nexts)):
+            for t in (m, nx):
+                assert t.dtype == torch.float32 and t.numel() == p.shape[j] and t.device == p.device \
+                    and t.is_contiguous(), f"leading statistic {j} must be {p.shape[j]} float32 on the param's device"
     nbytes, nblk = state_sizes(p.numel())
     assert exp.dtype == torch.uint8 and sq.dtype == torch.uint8, "moments must be packed uint8"
     assert exp.numel() == nbytes and sq.numel() == nbytes, f"packed moments must hold {nbytes} bytes"
@@ -294,19 +317,30 @@ def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next):
         assert t.device == p.device and t.is_contiguous(), "state must be contiguous on the param's device"
 
 
-def make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts):
+def make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts, leads=None):
+    """leads: None, or per tensor None (a matrix) or (leading statistics, their scratch), two
+    lists with one float32 tensor per leading dimension; row_maxes[i] then holds the flattened
+    rows' scales (rank1_row_scale)."""
     n = len(ps)
     arr = (_lib.Q4Rank1Tensor * n)()
     for i in range(n):
+        lead = None if leads is None else leads[i]
         check_rank1(ps[i], gs[i], exps[i], sqs[i], exp_scales[i], row_maxes[i], col_maxes[i],
-                    row_nexts[i], col_nexts[i])
+                    row_nexts[i], col_nexts[i], lead)
         a = arr[i]
         a.p, a.g = ps[i].data_ptr(), gs[i].data_ptr()
         a.exp_avg, a.exp_avg_sq = exps[i].data_ptr(), sqs[i].data_ptr()
         a.exp_avg_scale = exp_scales[i].data_ptr()
         a.row_max, a.col_max = row_maxes[i].data_ptr(), col_maxes[i].data_ptr()
         a.row_max_next, a.col_max_next = row_nexts[i].data_ptr(), col_nexts[i].data_ptr()
-        a.rows, a.cols = ps[i].shape
+        a.cols = ps[i].shape[-1]
+        a.rows = ps[i].numel() // a.cols
+        if lead is not None:
+            a.lead_dims = ps[i].dim() - 1
+            for j in range(a.lead_dims):
+                a.lead_shape[j] = ps[i].shape[j]
+                a.lead_max[j] = lead[0][j].data_ptr()
+                a.lead_max_next[j] = lead[1][j].data_ptr()
     return arr
 
 
@@ -333,14 +367,14 @@ def launch_rank1_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, bet
 def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts,
                            beta1, beta2, lr, weight_decay, eps, step, grad_scale=1.0,
                            grad_scale_dev=None, found_inf=None, zero_grad=False, seed=None, salts=None,
-                           step_consts=None):
+                           step_consts=None, leads=None):
     """The fused step over matrices whose second moment is rank-1 scaled: scale of element
     (i, j) = min(row_maxes[i], col_maxes[j]).  row_nexts / col_nexts are state-owned scratch
     that holds zeros between steps.  Gradient options as for fused_4bit_multi.  With a seed
     both moments are rounded stochastically, noise and salts as for fused_4bit_multi_sr."""
     if not ps:
         return
-    arr = make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts)
+    arr = make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts, leads)
     p_tag, g_tag = _tag(ps[0], "param"), _tag(gs[0], "grad")
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
@@ -443,6 +477,24 @@ def quantize_state_rank1(x):
                                       col_max.data_ptr(), _stream(x.device))
     _lib.check(rc, "quantize_rank1")
     return codes, row_max, col_max
+
+
+def quantize_state_rank1_scaled(x, row_scale, col_max):
+    """fp32 second moment viewed as a matrix [rows, cols] -> packed codes, every element divided
+    by min(row_scale[i], col_max[j]): the quantizer for tensors of more than two dimensions,
+    whose rows' scales come from rank1_row_scale."""
+    L = _lib.load()
+    assert x.is_cuda and x.dim() == 2 and x.shape[1] % 8 == 0, "needs a cuda matrix with cols % 8 == 0"
+    x = x.detach().to(torch.float32).contiguous()
+    rows, cols = x.shape
+    for t, n in ((row_scale, rows), (col_max, cols)):
+        assert t.dtype == torch.float32 and t.numel() == n and t.device == x.device and t.is_contiguous()
+    codes = torch.empty((rows * cols + 1) // 2, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.q4adamw_quantize_rank1_scaled(x.data_ptr(), rows, cols, row_scale.data_ptr(), col_max.data_ptr(),
+                                             codes.data_ptr(), _stream(x.device))
+    _lib.check(rc, "quantize_rank1_scaled")
+    return codes
 
 
 def dequantize_state_rank1(codes, row_max, col_max):

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(_lib.Q4Tensor) == 56 and ctypes.sizeof(_lib.Q4SmallTensor) == 40
     assert _lib.Q4Tensor.numel.offset == 48 and _lib.Q4SmallTensor.numel.offset == 32
-    assert ctypes.sizeof(_lib.Q4Rank1Tensor) == 88 and _lib.Q4Rank1Tensor.rows.offset == 72
+    assert ctypes.sizeof(_lib.Q4Rank1Tensor) == 168 and _lib.Q4Rank1Tensor.rows.offset == 72
     assert ctypes.sizeof(_lib.Q4GradOptions) == 32 and _lib.Q4GradOptions.grad_scale_dev.offset == 8
     assert ctypes.sizeof(_lib.Q4Grad) == 16 and _lib.NORM_WORKSPACE_BYTES == 16384
     header = open(os.path.join(ROOT, "include", "q4adamw.h")).read()

@@ -141,6 +141,55 @@ def test_rank1_stochastic_rounding_many_tensors_and_options(cuda):
     assert all(torch.equal(x.r, y.r) and torch.equal(x.c, y.c) for x, y in zip(a, c))   # statistics do not depend on the noise
 
 
+ND_SHAPES = [(4, 6, 64), (3, 5, 520), (2, 3, 4, 32), (8, 16, 1024), (1, 7, 16), (5, 1, 2, 264)]
+
+
+@pytest.mark.parametrize("stochastic", [False, True])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32")])
+@pytest.mark.parametrize("shape", ND_SHAPES)
+def test_rank1_more_than_two_dimensions_against_oracle(cuda, shape, p_dt, g_dt, stochastic):
+    """tensors of three and four dimensions: one statistic per dimension (maximum over all
+    others), scale = their minimum; codes, first-moment scales, every dimension's statistic
+    and the derived row scales bit for bit against step_quant_rank1_nd over four steps"""
+    gen = torch.Generator().manual_seed(sum(shape) * 7 + len(shape))
+    n, cols, k = int(np.prod(shape)), shape[-1], len(shape) - 1
+    rows = n // cols
+    p0 = (torch.randn(shape, generator=gen) * 0.05).to(DT[p_dt])
+    z = lambda m, dt=torch.float32: torch.zeros(m, dtype=dt, device=cuda)
+    p, m, v, sm = p0.clone().to(cuda), z((n + 1) // 2, torch.uint8), z((n + 1) // 2, torch.uint8), z((n + 127) // 128)
+    lead, lead_next = [z(shape[j]) for j in range(k)], [z(shape[j]) for j in range(k)]
+    rs, rn, c, cn = z(rows), z(rows), z(cols), z(cols)
+    ref = (p0.clone(), m.cpu(), v.cpu(), sm.cpu(),
+           [torch.zeros([shape[j] if d == j else 1 for d in range(len(shape))]) for j in range(len(shape))])
+    sr = dict(seed=0x5151_0000_ABCD + n, tensor_salt=3) if stochastic else {}
+    make = (grads_config1, grads_config3, grads_config1, grads_config3)
+    for step in range(1, 5):
+        g = make[step - 1](gen, n).view(shape)
+        if step == 2:
+            g[shape[0] // 2] = 0.0          # a slice of the first dimension and some columns without gradient
+            g[..., 8:16] = 0.0
+        g = g.to(DT[g_dt])
+        prev = ref[0]
+        ref = ot.step_quant_rank1_nd(ref[0], g, *ref[1:], step=step, **sr, **HP)
+        kw = dict(seed=sr["seed"], salts=[sr["tensor_salt"]]) if stochastic else {}
+        q.fused_4bit_rank1_multi([p], [g.to(cuda)], [m], [v], [sm], [rs], [c], [rn], [cn], *HPA, step,
+                                 leads=[(lead, lead_next)], **kw)
+        what = f"{shape} {p_dt}/{g_dt} sr={stochastic} step {step}"
+        assert torch.equal(m.cpu(), ref[1]), f"{what}: m codes"
+        assert torch.equal(sm.cpu().view(torch.int32), ref[3].view(torch.int32)), f"{what}: m scales"
+        for j in range(k):
+            assert torch.equal(lead[j].cpu().view(torch.int32), ref[4][j].reshape(-1).view(torch.int32)), f"{what}: statistic {j}"
+            assert not lead_next[j].any()
+        assert torch.equal(c.cpu().view(torch.int32), ref[4][k].reshape(-1).view(torch.int32)), f"{what}: last statistic"
+        assert torch.equal(rs, q.rank1_row_scale(lead, shape[:-1])), f"{what}: row scales"
+        assert not rn.any() and not cn.any(), f"{what}: scratch"
+        bad = torch.nonzero(v.cpu() != ref[2]).reshape(-1)
+        assert bad.numel() == 0, f"{what}: v codes differ at bytes {bad[:5].tolist()} ({bad.numel()})"
+        ok, worst = p_close(to_np(p), to_np(ref[0]), to_np(prev), bf16=DT[p_dt] == torch.bfloat16)
+        assert ok, f"{what}: parameters (worst {worst})"
+        ref = (p.cpu().clone(),) + tuple(ref[1:])
+
+
 def test_rank1_multi_tensor_and_options(cuda):
     """several matrices in one call (more than one launch batch), with a multiplier"""
     gen = torch.Generator().manual_seed(9)
