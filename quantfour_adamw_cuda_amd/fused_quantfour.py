@@ -77,8 +77,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # how the second moment is scaled before it is quantized: "group" = one abs-max per
         # 128 consecutive elements, what the fused CUDA path does (cuda_adamw_kernels.cu:353-383);
         # "rank1" = min(row maximum, column maximum) for matrices, the draft's SecondMoment
-        # setting (adamw_fourbit_triton.py:124, :834-863); tensors that are not matrices with
-        # cols % 8 == 0 and cols >= 16 keep group scaling, as 1-D tensors do there (:841-846)
+        # setting (adamw_fourbit_triton.py:124, :834-863), one statistic per dimension for
+        # tensors of two to four dimensions; others, and tensors whose last dimension is not
+        # a multiple of 8 or below 16, keep group scaling, as 1-D tensors do there (:841-846)
         if variance_scale_type not in ("group", "rank1"):
             raise ValueError(f"Invalid variance_scale_type: {variance_scale_type=}")
         self.variance_scale_type = variance_scale_type
@@ -202,18 +203,36 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         return self.variance_scale_type == "rank1" and _q.rank1_eligible(p)
 
     @staticmethod
-    def _init_rank1_overhead(p, overhead, row_max=None, col_max=None):
+    def _init_rank1_overhead(p, overhead, stats=None):
         """Statistics of a rank-1-scaled second moment, keys as in the draft's metadata
-        (adamw_fourbit_triton.py:846-852): max_dims = [row maxima [rows, 1], column maxima
-        [1, cols]], max1 = None; scratch_dims are same-sized buffers the step accumulates
-        the new maxima in (zeros between steps)."""
-        rows, cols = p.shape
+        (adamw_fourbit_triton.py:846-852): max_dims = one statistic per dimension in keepdim
+        shape (for a matrix: row maxima [rows, 1], column maxima [1, cols]), max1 = None;
+        scratch_dims are same-sized buffers the step accumulates the new maxima in (zeros
+        between steps).  Tensors of more than two dimensions also keep the scale of every
+        flattened row, the minimum over its leading statistics (derived; row_scale), and a
+        scratch of that size.  stats: the statistics to start from, one per dimension."""
         z = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=p.device)
-        overhead["dim"] = 2
+        keep = [[p.shape[d] if d == j else 1 for d in range(p.dim())] for j in range(p.dim())]
+        overhead["dim"] = p.dim()
         overhead["max1"] = None
-        overhead["max_dims"] = [z(rows, 1) if row_max is None else row_max.reshape(rows, 1),
-                                z(1, cols) if col_max is None else col_max.reshape(1, cols)]
-        overhead["scratch_dims"] = [z(rows, 1), z(1, cols)]
+        overhead["max_dims"] = [z(*keep[j]) if stats is None else
+                                stats[j].detach().to(device=p.device, dtype=torch.float32, copy=True).reshape(keep[j])
+                                for j in range(p.dim())]
+        overhead["scratch_dims"] = [z(*keep[j]) for j in range(p.dim())]
+        if p.dim() > 2:
+            lead = [t.reshape(-1) for t in overhead["max_dims"][:-1]]
+            overhead["row_scale"] = _q.rank1_row_scale(lead, p.shape[:-1])
+            overhead["row_scratch"] = z(overhead["row_scale"].numel())
+
+    @staticmethod
+    def _rank1_buffers(p, overhead):
+        """(rows' statistic or scale, last dimension's statistic, their scratch buffers,
+        leading statistics or None) as the rank-1 entry points take them."""
+        dims, scratch = overhead["max_dims"], overhead["scratch_dims"]
+        if p.dim() == 2:
+            return dims[0], dims[1], scratch[0], scratch[1], None
+        return (overhead["row_scale"], dims[-1], overhead["row_scratch"], scratch[-1],
+                ([t.view(-1) for t in dims[:-1]], [t.view(-1) for t in scratch[:-1]]))
 
     def _init_group(
         self,
@@ -275,10 +294,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 if torch.is_tensor(max1):
                     dst[key]["overhead"]["max1"] = max1.detach().to(
                         device=p.device, dtype=torch.float32, copy=True)
-                if "max_dims" in overhead:      # rank-1 statistics; the scratch restarts from zero
-                    rmax, cmax = (t.detach().to(device=p.device, dtype=torch.float32, copy=True)
-                                  for t in overhead["max_dims"])
-                    self._init_rank1_overhead(p, dst[key]["overhead"], rmax, cmax)
+                if "max_dims" in overhead:      # rank-1 statistics; scratch and derived row scales are made anew
+                    self._init_rank1_overhead(p, dst[key]["overhead"], overhead["max_dims"])
             if "momentum_qstate" not in src:
                 self._adopt_adamw_state(p, dst)
         self._launch_cache = {}
@@ -301,10 +318,20 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self.init_qstate(p, "variance")
         if state["momentum_qstate"]["enable"]:
             state["exp_avg"], state["momentum_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg, 0)
-            if self._use_rank1(p):
+            if self._use_rank1(p) and p.dim() == 2:
                 codes, rmax, cmax = _q.quantize_state_rank1(exp_avg_sq.reshape(p.shape))
                 state["exp_avg_sq"] = codes
-                self._init_rank1_overhead(p, state["variance_qstate"]["overhead"], rmax, cmax)
+                self._init_rank1_overhead(p, state["variance_qstate"]["overhead"], [rmax, cmax])
+            elif self._use_rank1(p):
+                # one statistic per dimension (maximum over all others); the rows of the tensor
+                # flattened to [rows, last dimension] are scaled by the minimum over their
+                # leading statistics (adamw_fourbit_triton.py:738-755)
+                v = torch.nan_to_num(exp_avg_sq.reshape(p.shape).abs(), nan=0.0, posinf=float("inf"))
+                stats = [v.amax(dim=[d for d in range(p.dim()) if d != j]) for j in range(p.dim())]
+                overhead = state["variance_qstate"]["overhead"]
+                self._init_rank1_overhead(p, overhead, stats)
+                state["exp_avg_sq"] = _q.quantize_state_rank1_scaled(
+                    exp_avg_sq.reshape(-1, p.shape[-1]), overhead["row_scale"], overhead["max_dims"][-1].view(-1))
             else:
                 state["exp_avg_sq"], state["variance_qstate"]["overhead"]["max1"] = _q.quantize_state(exp_avg_sq, 1)
         else:
@@ -328,8 +355,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 m = _q.dequantize_state(st["exp_avg"], st["momentum_qstate"]["overhead"]["max1"], p.numel(), 0)
                 v_meta = st["variance_qstate"]["overhead"]
                 if "max_dims" in v_meta:
-                    v = _q.dequantize_state_rank1(st["exp_avg_sq"], v_meta["max_dims"][0].reshape(-1),
-                                                  v_meta["max_dims"][1].reshape(-1))
+                    rmax, cmax = self._rank1_buffers(p, v_meta)[:2]
+                    v = _q.dequantize_state_rank1(st["exp_avg_sq"], rmax.reshape(-1), cmax.reshape(-1))
                 else:
                     v = _q.dequantize_state(st["exp_avg_sq"], v_meta["max1"], p.numel(), 1)
             else:
@@ -502,9 +529,10 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 rank1 = quantized in ("rank1", "rank1_sr")
                 if rank1:
                     sms = [momentum_meta[i]["max1"] for i in idx]
-                    stats = [[variance_meta[i][k][d] for i in idx]
-                             for k in ("max_dims", "scratch_dims") for d in (0, 1)]
-                    fixed = (ps, ms, vs, sms, *stats)
+                    bufs = [self._rank1_buffers(params_with_grad[i], variance_meta[i]) for i in idx]
+                    stats = [[b[d] for b in bufs] for d in range(4)]   # rows, last dimension, their scratch
+                    leads = [b[4] for b in bufs]
+                    fixed = (ps, ms, vs, sms, *stats, [t for ld in leads if ld is not None for ts in ld for t in ts])
                 elif quantized:
                     sms = [momentum_meta[i]["max1"] for i in idx]
                     svs = [variance_meta[i]["max1"] for i in idx]
@@ -520,7 +548,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 cached = self._launch_cache.get(cache_key)
                 if cached is None or cached[0] != ptrs:
                     if rank1:
-                        arr = _q.make_rank1_table(ps, gs, ms, vs, sms, stats[0], stats[1], stats[2], stats[3])
+                        arr = _q.make_rank1_table(ps, gs, ms, vs, sms, stats[0], stats[1], stats[2], stats[3], leads)
                     elif quantized:
                         arr = _q.make_table(ps, gs, ms, vs, sms, svs)
                     else:

@@ -404,6 +404,77 @@ def test_optimizer_rank1_with_stochastic_rounding(cuda):
     assert all(torch.equal(a, b) for a, b in zip(m1.parameters(), m_res.parameters()))
 
 
+def test_optimizer_rank1_with_tensors_of_more_than_two_dimensions(cuda):
+    """a stack of expert matrices [experts, in, out] and a 4-D kernel in one model: layout,
+    tracking of torch.optim.AdamW within the draft's bar, bit-identical resume, adoption of
+    AdamW state (codes equal the oracle's N-D quantizer) and fp32 export"""
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+
+    class Net(torch.nn.Module):
+        def __init__(self, seed):
+            super().__init__()
+            g_ = torch.Generator().manual_seed(seed)
+            self.experts = torch.nn.Parameter(torch.randn(4, 96, 512, generator=g_) * 0.05)
+            self.kernel = torch.nn.Parameter(torch.randn(16, 8, 3, 32, generator=g_) * 0.05)
+            self.out = torch.nn.Linear(512, 16)
+
+        def forward(self, x):                                    # x: [batch, 96]
+            h = torch.einsum("bi,eio->beo", x, self.experts).mean(1)           # [batch, 512]
+            k = self.kernel.sum(dim=(1, 2))                                      # [16, 32]
+            return self.out(torch.tanh(h)) + torch.tanh(h[:, :32] @ k.t())
+
+    def make(seed):
+        return Net(seed).to(cuda)
+
+    model, twin = make(5), make(5)
+    twin.load_state_dict(model.state_dict())          # the Linear layer draws from the global generator
+    opt = AdamWFused_QuantFour(model.parameters(), lr=1e-3, weight_decay=0.01, variance_scale_type="rank1")
+    ref = torch.optim.AdamW(twin.parameters(), lr=1e-3, weight_decay=0.01)
+    gen = torch.Generator(device=cuda).manual_seed(1)
+    for it in range(10):
+        x = torch.randn(32, 96, generator=gen, device=cuda)
+        for m_, o_ in ((model, opt), (twin, ref)):
+            o_.zero_grad(set_to_none=True)
+            m_(x).square().mean().backward()
+            o_.step()
+    ov = lambda p: opt.state[p]["variance_qstate"]["overhead"]
+    assert [tuple(t.shape) for t in ov(model.experts)["max_dims"]] == [(4, 1, 1), (1, 96, 1), (1, 1, 512)]
+    assert [tuple(t.shape) for t in ov(model.kernel)["max_dims"]] == [(16, 1, 1, 1), (1, 8, 1, 1), (1, 1, 3, 1), (1, 1, 1, 32)]
+    assert ov(model.experts)["row_scale"].numel() == 4 * 96 and not ov(model.experts)["row_scratch"].any()
+    assert all(not t.any() for t in ov(model.kernel)["scratch_dims"])
+    for a, b in zip(model.parameters(), twin.parameters()):
+        torch.testing.assert_close(a, b, atol=0.025, rtol=1e-5)
+    # export: the dequantized second moment is AdamW's to the 4-bit resolution of its scale
+    v32 = ref.state[twin.experts]["exp_avg_sq"]
+    exported = opt.adamw_state_dict()["state"][0]["exp_avg_sq"]
+    assert exported.shape == v32.shape and exported.dtype == torch.float32
+    stats = [v32.amax(dim=[d for d in range(3) if d != j], keepdim=True) for j in range(3)]
+    scale = torch.minimum(torch.minimum(stats[0], stats[1]), stats[2])
+    assert float(((exported - v32).abs() / scale).max()) < 0.3        # ten requantizations at 1/16 resolution
+    # resume: bit-identical continuation
+    model2 = make(6)
+    model2.load_state_dict(model.state_dict())
+    opt2 = AdamWFused_QuantFour(model2.parameters(), lr=1e-3, weight_decay=0.01, variance_scale_type="rank1")
+    opt2.load_state_dict(opt.state_dict())
+    x = torch.randn(32, 96, generator=gen, device=cuda)
+    for m_, o_ in ((model, opt), (model2, opt2)):
+        o_.zero_grad(set_to_none=True)
+        m_(x).square().mean().backward()
+        o_.step()
+    for a, b in zip(model.parameters(), model2.parameters()):
+        assert torch.equal(a, b)
+    for pa, pb in zip(model.parameters(), model2.parameters()):
+        assert torch.equal(opt.state[pa]["exp_avg_sq"], opt2.state[pb]["exp_avg_sq"])
+    # adopting torch.optim.AdamW's state
+    opt3 = AdamWFused_QuantFour(make(5).parameters(), lr=1e-3, variance_scale_type="rank1")
+    opt3.load_state_dict(ref.state_dict())
+    p3 = opt3.param_groups[0]["params"][0]
+    want_codes, want_dims = ot.quantize_rank1_nd(v32.cpu())
+    assert torch.equal(opt3.state[p3]["exp_avg_sq"].cpu(), want_codes)
+    for a, b in zip(opt3.state[p3]["variance_qstate"]["overhead"]["max_dims"], want_dims):
+        assert torch.equal(a.cpu(), b)
+
+
 def test_rank1_more_than_2_to_32_elements(cuda):
     """a matrix of 2 x 33000 x 65536 elements (4.3e9) whose lower half repeats the upper half:
     row and column maxima of the whole equal those of a half, so the run on the whole matrix

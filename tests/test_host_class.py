@@ -210,6 +210,33 @@ def test_rank1_state_layout_and_round_trip():
         AdamWFused_QuantFour([wide], variance_scale_type="rank2")
 
 
+def test_rank1_state_layout_of_tensors_with_more_than_two_dimensions():
+    """one statistic per dimension in keepdim shape (the draft's max_dims), plus the derived
+    scale of every flattened row; a state_dict round trip restores statistics and recomputes
+    the row scales; five dimensions, or a last dimension that is not a multiple of 8, keep
+    block scales"""
+    t3, t4, t5, odd = [torch.nn.Parameter(torch.randn(s)) for s in ((4, 6, 256), (3, 2, 5, 160), (2, 2, 2, 2, 512), (8, 8, 100))]
+    opt = AdamWFused_QuantFour([t3, t4, t5, odd], variance_scale_type="rank1")
+    for p in (t3, t4, t5, odd):
+        opt._init_state(p)
+    o3, o4 = (opt.state[p]["variance_qstate"]["overhead"] for p in (t3, t4))
+    assert o3["dim"] == 3 and [tuple(t.shape) for t in o3["max_dims"]] == [(4, 1, 1), (1, 6, 1), (1, 1, 256)]
+    assert o4["dim"] == 4 and [tuple(t.shape) for t in o4["scratch_dims"]] == [(3, 1, 1, 1), (1, 2, 1, 1), (1, 1, 5, 1), (1, 1, 1, 160)]
+    assert o3["row_scale"].shape == (24,) and o4["row_scale"].shape == (30,) and o4["row_scratch"].shape == (30,)
+    for p in (t5, odd):
+        assert "max_dims" not in opt.state[p]["variance_qstate"]["overhead"]
+    o3["max_dims"][0].copy_(torch.tensor([4.0, 1.0, 3.0, 2.0]).view(4, 1, 1))
+    o3["max_dims"][1].fill_(2.5)
+    o3["max_dims"][2].fill_(9.0)
+    opt2 = AdamWFused_QuantFour([torch.nn.Parameter(p.detach().clone()) for p in (t3, t4, t5, odd)],
+                                variance_scale_type="rank1")
+    opt2.load_state_dict(opt.state_dict())
+    n3 = opt2.state[opt2.param_groups[0]["params"][0]]["variance_qstate"]["overhead"]
+    assert all(torch.equal(a, b) and a.data_ptr() != b.data_ptr() for a, b in zip(n3["max_dims"], o3["max_dims"]))
+    want = torch.tensor([2.5, 1.0, 2.5, 2.0]).repeat_interleave(6)      # min(statistic of dim 0, 2.5) per row
+    assert torch.equal(n3["row_scale"], want) and not n3["row_scratch"].any()
+
+
 def test_round_type_and_seed_travel_in_the_param_groups():
     (p,) = params((64, 130))
     with pytest.raises(ValueError, match="round_type"):
