@@ -131,6 +131,27 @@ static void refusals(void) {
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);
   r[0].rows = (int64_t)1 << 40; r[0].cols = 1024;
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_TOO_LARGE);
+  /* leading dimensions: their product must be rows, their statistics must be there */
+  r[0].rows = 6; r[0].cols = 16;
+  r[0].p = buf; r[0].g = buf + 1024; r[0].exp_avg = codes; r[0].exp_avg_sq = codes + 1024; r[0].exp_avg_scale = scales;
+  r[0].row_max = scales + 64; r[0].row_max_next = scales + 128; r[0].col_max = buf + 2048; r[0].col_max_next = buf + 3072;
+  r[0].lead_dims = 4;
+  EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);
+  r[0].lead_dims = 2; r[0].lead_shape[0] = 2; r[0].lead_shape[1] = 3;
+  EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* no statistics */
+  r[0].lead_max[0] = scales + 192; r[0].lead_max[1] = scales + 200; r[0].lead_max_next[0] = scales + 208;
+  r[0].lead_max_next[1] = (float *)((char *)(scales + 216) + 2);
+  EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ALIGN);
+  r[0].lead_max_next[1] = scales + 216; r[0].lead_shape[1] = 4;
+  EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* 2 x 4 != 6 */
+  EXPECT(q4adamw_quantize_rank1_scaled(buf, 4, 12, scales, scales + 64, codes, NULL), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_quantize_rank1_scaled(buf, 4, 16, NULL, scales + 64, codes, NULL), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_quantize_rank1_scaled(buf, 0, 16, scales, scales + 64, codes, NULL), 0);
+  EXPECT(q4adamw_bias_table(0.9f, 0.999f, 1, 4, buf), 0);
+  EXPECT(q4adamw_bias_table(0.9f, 0.999f, 0, 4, buf), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_device_step(NULL, buf, 1, 4, NULL, B1, B2, LR, WD, EPS, NULL, buf + 64, NULL), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_device_step(buf, buf + 16, 1, 4, NULL, B1, B2, LR, WD, EPS, NULL, (char *)(buf + 64) + 4, NULL), Q4ADAMW_ERR_ALIGN);
+  EXPECT(q4adamw_device_step(buf, buf + 16, 1, 0, NULL, B1, B2, LR, WD, EPS, NULL, buf + 64, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_quantize_rank1(buf, 4, 12, codes, scales, scales + 64, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_quantize_rank1(buf, 0, 16, codes, scales, scales + 64, NULL), 0);
   EXPECT(q4adamw_quantize_rank1(buf, (int64_t)1 << 23, 8, codes, scales, scales + 64, NULL), Q4ADAMW_ERR_TOO_LARGE);
