@@ -488,13 +488,14 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             if not params_with_grad:
                 continue
 
-            lr = group["lr"]
+            capturable = bool(group.get("capturable", False))
+            # a tensor lr is read on the device in capturable mode; otherwise its value is taken now
+            lr = 1.0 if capturable else float(group["lr"])
             weight_decay = group["weight_decay"]
             eps = group["eps"]
             stochastic = group.get("round_type", "real-nearest") == "stochastic"
 
             # update step (optim/fused_quantfour.py:178)
-            capturable = bool(group.get("capturable", False))
             if capturable and len(params_with_grad) != sum(1 for p in group["params"] if p.numel() > 0):
                 raise ValueError("capturable=True needs a gradient for every parameter of the group: "
                                  "the group's parameters share one step counter on the device")
@@ -522,50 +523,11 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 buckets.setdefault(key, []).append(i)
 
             for (quantized, device, p_dtype, g_dtype, t_step), idx in buckets.items():
-                ps = [params_with_grad[i] for i in idx]
-                gs = [grads[i] for i in idx]
-                ms = [exp_avgs[i] for i in idx]
-                vs = [exp_avg_sqs[i] for i in idx]
                 rank1 = quantized in ("rank1", "rank1_sr")
-                if rank1:
-                    sms = [momentum_meta[i]["max1"] for i in idx]
-                    bufs = [self._rank1_buffers(params_with_grad[i], variance_meta[i]) for i in idx]
-                    stats = [[b[d] for b in bufs] for d in range(4)]   # rows, last dimension, their scratch
-                    leads = [b[4] for b in bufs]
-                    fixed = (ps, ms, vs, sms, *stats, [t for ld in leads if ld is not None for ts in ld for t in ts])
-                elif quantized:
-                    sms = [momentum_meta[i]["max1"] for i in idx]
-                    svs = [variance_meta[i]["max1"] for i in idx]
-                    fixed = (ps, ms, vs, sms, svs)
-                else:
-                    fixed = (ps, ms, vs)
-                # parameters and state stay where they are from step to step; gradients
-                # usually do not: a descriptor table is rebuilt (and everything validated)
-                # only when a parameter or state pointer changed, otherwise the gradients'
-                # pointers are refreshed in place
-                ptrs = tuple(t.data_ptr() for ts in fixed for t in ts)
-                cache_key = (gi, quantized, device, p_dtype, g_dtype)
-                cached = self._launch_cache.get(cache_key)
-                if cached is None or cached[0] != ptrs:
-                    if rank1:
-                        arr = _q.make_rank1_table(ps, gs, ms, vs, sms, stats[0], stats[1], stats[2], stats[3], leads)
-                    elif quantized:
-                        arr = _q.make_table(ps, gs, ms, vs, sms, svs)
-                    else:
-                        arr = _q.make_small_table(ps, gs, ms, vs)
-                    tags = (_q._tag(ps[0], "param"), _q._tag(gs[0], "grad"))
-                    if quantized in ("sr", "rank1_sr"):   # noise salt of a tensor: its position among all parameters
-                        tags += (_q.make_salts([self._param_position(p) for p in ps]),)
-                    cached = (ptrs, arr, tags)
-                    self._launch_cache[cache_key] = cached
-                else:
-                    arr = cached[1]
-                    for i, (p, g) in enumerate(zip(ps, gs)):
-                        # dtype and device are part of the bucket key (optim/fused_quantfour.py:255-261)
-                        assert g.device == device, "grad must be on the param's device"
-                        assert g.is_contiguous(), "grad must be contiguous"
-                        assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
-                        arr[i].g = g.data_ptr()
+                cached = self._bucket_table(
+                    (gi, quantized, device, p_dtype, g_dtype),
+                    [params_with_grad[i] for i in idx], [grads[i] for i in idx], [exp_avgs[i] for i in idx],
+                    [exp_avg_sqs[i] for i in idx], [momentum_meta[i] for i in idx], [variance_meta[i] for i in idx])
                 _, arr, (p_tag, g_tag, *extra) = cached
                 if quantized in ("sr", "rank1_sr"):
                     salts_arr, sr_seed = extra[0], group["seed"]
@@ -576,8 +538,8 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                               _q.launch_table if quantized else _q.launch_small_table)
                 options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad,
                                           step_consts.get(device))
-                if capturable:   # lr and step enter through step_consts; these only pass the range check
-                    lr, t_step = 1.0, 1.0
+                if capturable:   # lr and step enter through step_consts; the arguments only pass the range check
+                    t_step = 1.0
                 if self.kernel_timing is None:
                     launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
                 else:
@@ -647,6 +609,49 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 s = self.state.get(p)
                 if s and p.device == device and torch.is_tensor(s.get("step")):
                     s["step"].fill_(value)
+
+    def _bucket_table(self, cache_key, ps, gs, ms, vs, m_meta, v_meta):
+        """(pointers, ctypes descriptor array, (param tag, grad tag[, salts])) of one launch
+        bucket.  Parameters and state stay where they are from step to step; gradients usually
+        do not: the array is rebuilt (and everything validated) only when a parameter or state
+        pointer changed, otherwise the gradients' pointers are refreshed in place."""
+        _, quantized, device, _, _ = cache_key
+        rank1 = quantized in ("rank1", "rank1_sr")
+        if rank1:
+            sms = [mm["max1"] for mm in m_meta]
+            bufs = [self._rank1_buffers(p, vm) for p, vm in zip(ps, v_meta)]
+            stats = [[b[d] for b in bufs] for d in range(4)]   # rows, last dimension, their scratch
+            leads = [b[4] for b in bufs]
+            fixed = (ps, ms, vs, sms, *stats, [t for ld in leads if ld is not None for ts in ld for t in ts])
+        elif quantized:
+            sms = [mm["max1"] for mm in m_meta]
+            svs = [vm["max1"] for vm in v_meta]
+            fixed = (ps, ms, vs, sms, svs)
+        else:
+            fixed = (ps, ms, vs)
+        ptrs = tuple(t.data_ptr() for ts in fixed for t in ts)
+        cached = self._launch_cache.get(cache_key)
+        if cached is None or cached[0] != ptrs:
+            if rank1:
+                arr = _q.make_rank1_table(ps, gs, ms, vs, sms, stats[0], stats[1], stats[2], stats[3], leads)
+            elif quantized:
+                arr = _q.make_table(ps, gs, ms, vs, sms, svs)
+            else:
+                arr = _q.make_small_table(ps, gs, ms, vs)
+            tags = (_q._tag(ps[0], "param"), _q._tag(gs[0], "grad"))
+            if quantized in ("sr", "rank1_sr"):   # noise salt of a tensor: its position among all parameters
+                tags += (_q.make_salts([self._param_position(p) for p in ps]),)
+            cached = (ptrs, arr, tags)
+            self._launch_cache[cache_key] = cached
+        else:
+            arr = cached[1]
+            for i, (p, g) in enumerate(zip(ps, gs)):
+                # dtype and device are part of the bucket key (optim/fused_quantfour.py:255-261)
+                assert g.device == device, "grad must be on the param's device"
+                assert g.is_contiguous(), "grad must be contiguous"
+                assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
+                arr[i].g = g.data_ptr()
+        return cached
 
     def _advance_steps(self, gi, params, state_steps):
         """Adds 1 to every step counter and returns their new values as Python floats.  The
