@@ -227,6 +227,7 @@ __device__ const HalfTable kHalfTable = make_half_table();
 // stochastic rounding: code-book entries per bucket and the 17 intervals between them
 __device__ const SrHalfTable kSrHalfTable = make_sr_half_table();
 __device__ const SrIntervalTable kSrIntervals = make_sr_interval_table();
+__device__ const SrAffineTable kSrAffine = make_sr_affine_table();
 // first-moment code book for kernels that index it per lane
 __device__ const uint32_t kQmapMDev[16] = {
     0xbf633333u, 0xbf29999au, 0xbee00000u, 0xbe59999au, 0xbd9eb852u, 0xbd051eb8u,

@@ -413,7 +413,7 @@ __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
 //               and an entry number fits a byte
 //   [256, 512)  bucket table of the first-moment quantizer, indexed by the high byte
 //               of the quotient as a half
-//   [512, 529)  stochastic rounding only: the first moment's interval table
+//   [512, 529)  stochastic rounding only: the first moment's intervals as affine maps
 constexpr uint32_t kLdsBuckets = 64 * kWaves;
 constexpr uint32_t kLdsIntervals = kLdsBuckets + kHalfTableEntries;
 constexpr uint32_t kLdsEntries = kLdsIntervals + 32;
@@ -424,7 +424,7 @@ static_assert(kThreads == (int)kHalfTableEntries, "one bucket table entry per th
 struct TableSlot {
   uint2 entry;     // bucket table entry number tid
   float qm;        // first-moment code-book value number (lane & 15)
-  uint2 interval;  // stochastic rounding: interval table entry number tid (tid < 17)
+  uint2 interval;  // stochastic rounding: affine table entry number tid (tid < 17)
 };
 
 template <bool SR>
@@ -433,8 +433,8 @@ __device__ __forceinline__ TableSlot request_table_slot(int tid) {
   if (SR) {
     const SrEntry e = kSrHalfTable.e[tid];
     s.entry = make_uint2(e.thr, e.base);
-    const SrInterval iv = kSrIntervals.e[tid < 17 ? tid : 0];
-    s.interval = make_uint2(f2bits(iv.lower), f2bits(iv.width));
+    const SrAffine af = kSrAffine.e[tid < 17 ? tid : 0];
+    s.interval = make_uint2(f2bits(af.a), f2bits(af.c));
   } else {
     const MtabEntry e = kHalfTable.e[tid];
     s.entry = make_uint2(e.lo, e.hi);

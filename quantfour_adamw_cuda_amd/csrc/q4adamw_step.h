@@ -206,7 +206,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   const float rv16 = (safe_v && !RANK1) ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
   float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
-  float vfrac_hi = 0.0f;  // stochastic rounding: largest fractional part of 16 q - noise
+  float vfrac_hi = 0.0f;  // stochastic rounding: with vfrac, the extreme fractional parts of
+                          // both moments' code coordinates minus noise
   // rank-1: the new scale of every element and 16 / scale.  The hardware reciprocal's
   // one ulp is well inside the second moment's guard band (2^-17 in units of 16 q), so
   // it goes unrefined.  Scales below the safe range are clamped for the reciprocal: a
@@ -246,17 +247,23 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<1>(halves, three));
     const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<3>(halves, three));
     if constexpr (SR) {
-      // interval among the code-book entries, then up iff noise * width < q - lower end;
-      // a comparison closer than the quotient's error goes to the exact path
+      // interval among the code-book entries; inside it the code is floor(k + position -
+      // noise), an affine function of the quotient; a value within the guard band of an
+      // integer goes to the exact path.  Error budget in units of one code: the quotient is
+      // within 2^-22 relative of the exact one and |q| / width < 9 (2.25 * 2^-20), the map's
+      // two roundings and the two operations here add 2^-21 each: 0.54 of the band.  The
+      // value is never negative, and below 16 outside the band.
       const float qq[2] = {q0, q1};
       const uint2 ent[2] = {ent0, ent1};
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const uint32_t k_raw = ent[h].y + (qq[h] >= bits2f(ent[h].x) ? 1u : 0u);
-        const uint2 iv = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsIntervals * 8u + k_raw * 8u);
-        const float d = qq[h] - bits2f(iv.x), t = um.x[j + h] * bits2f(iv.y);
-        redo |= __builtin_fabsf(t - d) <= __builtin_fabsf(qq[h]) * 4.76837158203125e-07f;  // 2^-21: 4 ulps
-        mword = __builtin_amdgcn_alignbit(k_raw - 1u + (t < d ? 1u : 0u), mword, 4);
+        const float2 af = *reinterpret_cast<const float2 *>(lds_bytes + kLdsIntervals * 8u + k_raw * 8u);
+        const float y = __builtin_fmaf(qq[h], af.x, af.y) - um.x[j + h];
+        const float fr = __builtin_amdgcn_fractf(y);
+        vfrac = __builtin_fminf(vfrac, fr);
+        vfrac_hi = __builtin_fmaxf(vfrac_hi, fr);
+        mword = __builtin_amdgcn_alignbit((uint32_t)(int)y, mword, 4);
       }
     } else {
       const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);

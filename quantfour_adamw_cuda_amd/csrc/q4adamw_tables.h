@@ -229,4 +229,43 @@ constexpr SrIntervalTable make_sr_interval_table() {
   return t;
 }
 
+// The fast path's form of the same decision: inside interval k_raw = 1..15 the code is
+// floor(k_raw + (q - lower) / width - noise), an affine function of q minus the noise, so
+// entry [k_raw] holds {1 / width, k_raw - lower / width} (from the exact interval in
+// double precision, rounded once).  Below the first entry {0, 1} gives floor(1 - noise) = 0,
+// at or above the last one {0, 16} gives floor(16 - noise) = 15.
+struct SrAffine {
+  float a, c;
+};
+
+Q4_HD constexpr SrAffine sr_affine_m(uint32_t k_raw) {  // k_raw 0..16
+  if (k_raw == 0u) return SrAffine{0.0f, 1.0f};
+  if (k_raw == 16u) return SrAffine{0.0f, 16.0f};
+  const double lower = (double)bits2f(kQmapMBits[k_raw - 1u]);
+  const double width = (double)bits2f(kQmapMBits[k_raw]) - lower;
+  return SrAffine{(float)(1.0 / width), (float)((double)k_raw - lower / width)};
+}
+
+struct SrAffineTable {
+  SrAffine e[17];
+};
+
+constexpr SrAffineTable make_sr_affine_table() {
+  SrAffineTable t{};
+  for (uint32_t k = 0; k < 17; ++k) t.e[k] = sr_affine_m(k);
+  return t;
+}
+
+// The error of the affine form, in units of one code, is the quotient's relative error
+// times |q| / width: the guard band of the fast path is sized for a ratio below 9.
+constexpr bool sr_affine_ratio_ok() {
+  for (uint32_t k = 1; k < 16; ++k) {
+    const double lo = (double)bits2f(kQmapMBits[k - 1u]), hi = (double)bits2f(kQmapMBits[k]);
+    const double big = (lo < 0 ? -lo : lo) > (hi < 0 ? -hi : hi) ? (lo < 0 ? -lo : lo) : (hi < 0 ? -hi : hi);
+    if (big / (hi - lo) >= 9.0) return false;
+  }
+  return true;
+}
+static_assert(sr_affine_ratio_ok(), "first-moment code book: an interval too narrow for the guard band");
+
 }  // namespace q4

@@ -53,6 +53,25 @@ def test_sr_against_oracle(cuda, p_dt, g_dt, n):
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
 
 
+def test_sr_against_oracle_at_scale(cuda):
+    """16.8M elements, three steps: about a thousand elements per step fall into the fast
+    path's guard bands (2^-16 of the elements per moment), so both the bands' width and the
+    exact path behind them are exercised; every code must still agree."""
+    n = (1 << 24) + 12345
+    gen = torch.Generator().manual_seed(77)
+    p0 = torch.randn(n, generator=gen) * 0.05
+    dev = DeviceTensor(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.sv.cpu())
+    for step, maker in enumerate((grads_config1, grads_student_t, grads_config3), start=1):
+        g = maker(gen, n).to(torch.bfloat16)
+        prev = ref[0]
+        ref = ot.step_quant_sr(ref[0], g, *ref[1:], seed=SEED + step, tensor_salt=3, step=step, **HP)
+        q.fused_4bit_multi_sr([dev.p], [g.to(cuda)], [dev.m], [dev.v], [dev.sm], [dev.sv], *HPA, step,
+                              SEED + step, salts=[3])
+        _check(dev, ref, prev, f"n={n} step {step}")
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
+
+
 def test_sr_multi_tensor_salts_reproducibility_and_options(cuda):
     gen = torch.Generator().manual_seed(5)
     sizes = [5000 + 131 * i for i in range(60)]          # more than one launch batch
