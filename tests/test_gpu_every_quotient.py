@@ -219,3 +219,69 @@ def test_every_square_under_rank1_scaling(cuda, pin, stochastic):
                 raise AssertionError(f"{what}: {name}-moment codes differ in {bad.numel()} bytes; first at element {e}: "
                                      f"g = {flat[e:e + 2].tolist()}, got byte {int(codes[bad[0]])}, want {int(want[bad[0]])}")
         del g, flat, m_new, q_m, q_v, want_m, want_v
+
+
+@pytest.mark.parametrize("which", [0, 1])
+def test_every_value_through_the_checkpoint_quantizer(cuda, which):
+    """q4adamw_quantize (checkpoint interchange: exact division, one wave per block) on every
+    fp32 value of magnitude up to a block scale of 1.5; the second moment's values are not
+    negative."""
+    scale = 1.5
+    mid = torch.tensor(oc.tables(which)[1], device=cuda)
+    per_sign = _bits(scale) + 1
+    total = per_sign if which else 2 * per_sign
+    chunk = BLOCKS_PER_CHUNK * 127
+    for start in range(0, total, chunk):
+        idx = torch.arange(start, start + chunk, device=cuda, dtype=torch.int64)
+        idx = torch.where(idx < total, idx, torch.zeros_like(idx))
+        pat = torch.where(idx < per_sign, idx, (idx - per_sign) | 0x80000000)
+        x = (pat - ((pat >> 31) << 32)).to(torch.int32).view(torch.float32)
+        x = torch.cat([x.view(-1, 127), torch.full((BLOCKS_PER_CHUNK, 1), scale, device=cuda)], dim=1).reshape(-1)
+        del idx, pat
+        codes, scales = qh.quantize_state(x, which)
+        assert bool((scales == scale).all()), f"moment {which} chunk {start}: scales"
+        want = _packed(torch.bucketize(x / torch.full((1,), scale, device=cuda), mid, right=False))
+        bad = torch.nonzero(codes != want).reshape(-1)
+        assert bad.numel() == 0, (f"moment {which} chunk {start}: codes differ in {bad.numel()} bytes; first at element "
+                                  f"{int(bad[0]) * 2}: got byte {int(codes[bad[0]])}, want {int(want[bad[0]])}")
+        del x, codes, scales, want, bad
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_every_16bit_gradient(cuda, dt):
+    """Parameters and gradients both in a 16-bit type take the kernel that owns eight elements
+    per lane (a block is sixteen lanes).  Its gradients have only 2^16 patterns: all of them up
+    to the pinned one, at 48 pinned values, with nearest and with stochastic rounding."""
+    mid_m = torch.tensor(oc.tables(0)[1], device=cuda)
+    mid_v = torch.tensor(oc.tables(1)[1], device=cuda)
+    gen = torch.Generator().manual_seed(8)
+    pins = (torch.rand(48, generator=gen) * 3.9 + 0.05).to(dt)
+    for launch, pin_t in enumerate(pins):
+        top = int(pin_t.view(torch.int16))                       # positive: the pattern as an integer
+        pat = torch.cat([torch.arange(0, top + 1), torch.arange(0, top + 1) - 32768]).to(torch.int16)
+        pad = (-pat.numel()) % 127
+        x = torch.cat([pat, torch.zeros(pad, dtype=torch.int16)]).view(dt).to(cuda)
+        blocks = x.numel() // 127
+        g = torch.cat([x.view(-1, 127), pin_t.to(cuda).expand(blocks, 1)], dim=1).reshape(-1).contiguous()
+        n = g.numel()
+        gf = g.float()
+        m_new, v_new = gf * 0.5, (gf * gf) * 0.5
+        am, av = m_new.abs().max().reshape(1), v_new.max().reshape(1)
+        for stochastic in (False, True):
+            p = torch.zeros(n, dtype=dt, device=cuda)
+            m = torch.zeros(n // 2, dtype=torch.uint8, device=cuda)
+            v = torch.zeros_like(m)
+            sm = torch.zeros(n // 128, device=cuda)
+            sv = torch.zeros_like(sm)
+            what = f"{dt} pin {float(pin_t)} stochastic {stochastic}"
+            if stochastic:
+                qh.fused_4bit_multi_sr([p], [g], [m], [v], [sm], [sv], 0.5, 0.5, 1e-3, 0.0, 1e-8, 1, 31, salts=[launch])
+                um, uv = _sr_noise(n, ot.sr_tensor_salt(31, 1, launch), cuda)
+                want_m, want_v = _sr_codes(m_new / am, 0, um), _sr_codes(v_new / av, 1, uv)
+            else:
+                q4.fused_4bit(p, g, m, v, sm, sv, 0.5, 0.5, 1e-3, 0.0, 1e-8, 1)
+                want_m = torch.bucketize(m_new / am, mid_m, right=False)
+                want_v = torch.bucketize(v_new / av, mid_v, right=False)
+            assert bool((sm == am).all()) and bool((sv == av).all()), f"{what}: scales"
+            assert torch.equal(m, _packed(want_m)), f"{what}: first-moment codes"
+            assert torch.equal(v, _packed(want_v)), f"{what}: second-moment codes"
