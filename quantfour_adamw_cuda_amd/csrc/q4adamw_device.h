@@ -283,6 +283,15 @@ __device__ __forceinline__ uint32_t quantize_exact_scales(const Vals<N> &v, cons
   return word;
 }
 
+// Adds element j's code to a lane's word of 4-bit codes.  Four elements per lane: the code
+// (0..15 and no other bits) goes to its place.  Eight: every code enters at the top and
+// moves down four bits per later element.
+template <int N>
+__device__ __forceinline__ uint32_t append_code(uint32_t word, uint32_t code, int j) {
+  if (N == 4) return j == 0 ? code : ((code << (4 * j)) | word);
+  return __builtin_amdgcn_alignbit(code, word, 4);
+}
+
 // A 32-bit integer mixer (two multiply-xorshift rounds) for the rounding noise.
 __host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
   x ^= x >> 16;
@@ -293,9 +302,10 @@ __host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
   return x;
 }
 
-// noise in (0, 1) from a 16-bit number: (2 n + 1) / 2^17, exact
-__device__ __forceinline__ float sr_noise_value(uint32_t n16) {
-  return __builtin_fmaf((float)n16, 1.52587890625e-05f, 7.62939453125e-06f);
+// noise in (0, 1) from a 16-bit number (as a float): (2 n + 1) / 2^17, exact
+constexpr float kNoiseStep = 1.52587890625e-05f;     // 2^-16
+__device__ __forceinline__ float sr_noise_value(float n16) {
+  return __builtin_fmaf(n16, kNoiseStep, 0.5f * kNoiseStep);
 }
 
 // Stochastic rounding, exact form (the closed form of quantize_bsearch<STOCHASTIC>,
@@ -390,6 +400,7 @@ __device__ __forceinline__ float refined_rcp(float s) {
 constexpr float kScaleLo = 7.888609052210118e-31f;   // 2^-100
 constexpr float kScaleHi = 1.2676506002282294e+30f;  // 2^100
 constexpr float kVGuard = 7.62939453125e-06f;        // 2^-17, in units of 16*q
+static_assert(kVGuard == 0.5f * kNoiseStep, "the fast path lets the noise's offset cancel the guard band");
 
 // Uniform search of the launch's tensor list: the last tensor whose first chunk is
 // <= chunk.  first_chunk[0] is 0, so the result is never negative.  Chunk indices and

@@ -205,9 +205,9 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   const float rm = safe_m ? refined_rcp(am) : 0.0f;
   const float rv16 = (safe_v && !RANK1) ? refined_rcp(av) * 16.0f : 0.0f;  // exact scaling
   bool redo = (!safe_m && am != 0.0f) || (!safe_v && av != 0.0f);
-  float vfrac = 1.0f;  // smallest distance of a scaled second moment above a threshold
-  float vfrac_hi = 0.0f;  // stochastic rounding: with vfrac, the extreme fractional parts of
-                          // both moments' code coordinates minus noise
+  // smallest fractional part of a code coordinate shifted up by the guard band: second
+  // moment 16 q - 1/2 (nearest), both moments' coordinate minus noise (stochastic)
+  float vfrac = 1.0f;
   // rank-1: the new scale of every element and 16 / scale.  The hardware reciprocal's
   // one ulp is well inside the second moment's guard band (2^-17 in units of 16 q), so
   // it goes unrefined.  Scales below the safe range are clamped for the reciprocal: a
@@ -227,16 +227,21 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     redo |= r_new > kScaleHi || (min_nonneg(r_new, c_min) < kScaleLo && v_lane_max != 0.0f);
   }
   uint32_t mword = 0, vword = 0;
-  Vals<N> um, uv;  // stochastic rounding: the elements' noise
+  // stochastic rounding: the elements' 16-bit noise numbers n as floats; the noise itself is
+  // (2 n + 1) / 2^17 = n * kNoiseStep + kVGuard, and the fast path works with code
+  // coordinates shifted up by the guard band, so the two halves of a step cancel there
+  Vals<N> um, uv;
   if constexpr (SR) {
     // key = low half of the element index, xor the salt, xor the mixed high half
     const uint32_t tile_salt = salt ^ ((uint32_t)((uint64_t)tb >> 32) * 0x9E3779B9u);
-    const uint32_t first = (uint32_t)tb + e0;   // a tile never straddles a multiple of 2^32
+    // a tile never straddles a multiple of 2^32; the lane's first element is a multiple
+    // of N, so element j's key is the first one's with j in its low bits
+    const uint32_t key0 = ((uint32_t)tb + e0) ^ tile_salt;
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      const uint32_t h = lowbias32((first + (uint32_t)j) ^ tile_salt);
-      um.x[j] = sr_noise_value(h >> 16);
-      uv.x[j] = sr_noise_value(h & 0xffffu);
+      const uint32_t h = lowbias32(key0 ^ (uint32_t)j);
+      um.x[j] = (float)(h >> 16);
+      uv.x[j] = (float)(h & 0xffffu);
     }
   }
 #pragma unroll
@@ -248,22 +253,22 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<3>(halves, three));
     if constexpr (SR) {
       // interval among the code-book entries; inside it the code is floor(k + position -
-      // noise), an affine function of the quotient; a value within the guard band of an
-      // integer goes to the exact path.  Error budget in units of one code: the quotient is
-      // within 2^-22 relative of the exact one and |q| / width < 9 (2.25 * 2^-20), the map's
-      // two roundings and the two operations here add 2^-21 each: 0.54 of the band.  The
-      // value is never negative, and below 16 outside the band.
+      // noise), an affine function of the quotient.  Computed shifted up by the guard band
+      // (coordinate - n * kNoiseStep): a fractional part below twice the band then marks a
+      // value within the band of an integer on either side, which goes to the exact path,
+      // and every other value truncates to its code.  Error budget in units of one code: the
+      // quotient is within 2^-22 relative of the exact one and |q| / width < 9 (2.25 *
+      // 2^-20), the map's two roundings and the two operations here add 2^-21 each: 0.54 of
+      // the band.  The value is never negative, and below 16 outside the band.
       const float qq[2] = {q0, q1};
       const uint2 ent[2] = {ent0, ent1};
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const uint32_t k_raw = ent[h].y + (qq[h] >= bits2f(ent[h].x) ? 1u : 0u);
         const float2 af = *reinterpret_cast<const float2 *>(lds_bytes + kLdsIntervals * 8u + k_raw * 8u);
-        const float y = __builtin_fmaf(qq[h], af.x, af.y) - um.x[j + h];
-        const float fr = __builtin_amdgcn_fractf(y);
-        vfrac = __builtin_fminf(vfrac, fr);
-        vfrac_hi = __builtin_fmaxf(vfrac_hi, fr);
-        mword = __builtin_amdgcn_alignbit((uint32_t)(int)y, mword, 4);
+        const float y = __builtin_fmaf(um.x[j + h], -kNoiseStep, __builtin_fmaf(qq[h], af.x, af.y));
+        vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(y));
+        mword = append_code<N>(mword, (uint32_t)(int)y, j + h);
       }
     } else {
       const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
@@ -280,31 +285,29 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
       if constexpr (SR) {
         // code-book entries at 16 q = 1..16: interval number floor(16 q), position in it
         // fract(16 q), up iff noise < position, i.e. code = floor(16 q - noise) wherever
-        // that difference is clear of an integer (the noise is never 0, so it is below
-        // 16); a difference within the guard band of an integer goes to the exact path.
-        // y > -1, so truncation gives 0 for y < 0
-        const float y = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, -uv.x[k]);
-        const float fr = __builtin_amdgcn_fractf(y);
-        vfrac = __builtin_fminf(vfrac, fr);
-        vfrac_hi = __builtin_fmaxf(vfrac_hi, fr);
-        const uint32_t c = (uint32_t)(int)y;
-        vword = __builtin_amdgcn_alignbit(c < 15u ? c : 15u, vword, 4);
+        // that difference is clear of an integer; shifted up by the guard band as for the
+        // first moment.  The shifted value is above -1 (truncation gives 0 below 0) and,
+        // outside the band, below 16.
+        const float y = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, uv.x[k] * -kNoiseStep);
+        vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(y));
+        vword = append_code<N>(vword, (uint32_t)(int)y, k);
       } else {
         const float t = __builtin_fmaf(vn.x[k], RANK1 ? inv16.x[k] : rv16, kVGuard - 0.5f);
         vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(t));
         // t > -1, so truncation gives 0 for t < 0
-        vword = __builtin_amdgcn_alignbit((uint32_t)(int)t, vword, 4);
+        vword = append_code<N>(vword, (uint32_t)(int)t, k);
       }
     }
   }
-  if (N == 4) {
-    mword >>= 16;
-    vword >>= 16;
-  }
-  if constexpr (SR) redo |= vfrac < kVGuard || vfrac_hi > 1.0f - kVGuard;
-  else redo |= vfrac < 2.0f * kVGuard;
+  if (N == 4 && !SR) mword >>= 16;   // four codes entered at the top
+  redo |= vfrac < 2.0f * kVGuard;
   if (__builtin_expect(redo, 0)) {
     if constexpr (SR) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        um.x[j] = sr_noise_value(um.x[j]);
+        uv.x[j] = sr_noise_value(uv.x[j]);
+      }
       mword = quantize_exact_sr<false, N>(mn, am, um);
       if constexpr (RANK1) vword = quantize_exact_sr_scales<N>(vn, s_new, uv);
       else vword = quantize_exact_sr<true, N>(vn, av, uv);
