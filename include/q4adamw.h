@@ -370,6 +370,20 @@ int q4adamw_mtable_entry(uint32_t index, uint32_t *out2);
  */
 int q4adamw_mtable_half_bucket(uint32_t half_index);
 
+/*
+ * Host-only: the two tables the first moment's stochastic rounding indexes in its fast
+ * path (no counterpart in the reference, which only quotes the rounding rule,
+ * optim/adamw_fourbit_triton.py:1050-1075).  q4adamw_sr_bucket_entry: entry `half_index`
+ * (0..255) of the table indexed like the one above: out2[0] = fp32 bits of the code-book
+ * value inside the bucket (0x7f000000 if none), out2[1] = number of code-book values below
+ * the whole bucket; k = out2[1] + (q >= value) is the number of code-book values <= q.
+ * q4adamw_sr_affine_entry: entry k (0..16) of the table that turns a normalised value
+ * into its code coordinate, out2 = {slope, offset}: floor(slope * q + offset - noise) is
+ * the code wherever that value is clear of an integer.  For tests.
+ */
+int q4adamw_sr_bucket_entry(uint32_t half_index, uint32_t *out2);
+int q4adamw_sr_affine_entry(uint32_t k, float *out2);
+
 /* Kept for callers that pair an init with a release: the library holds no device
  * memory, so this does nothing and returns 0. */
 int q4adamw_release(void);

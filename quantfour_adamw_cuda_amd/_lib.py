@@ -104,6 +104,8 @@ EXPORTS = (
     "q4adamw_tables",
     "q4adamw_mtable_entry",
     "q4adamw_mtable_half_bucket",
+    "q4adamw_sr_bucket_entry",
+    "q4adamw_sr_affine_entry",
     "q4adamw_release",
     "q4adamw_last_error",
     "q4adamw_version",
@@ -172,6 +174,10 @@ def load():
     L.q4adamw_mtable_entry.restype = i
     L.q4adamw_mtable_half_bucket.argtypes = [ctypes.c_uint32]
     L.q4adamw_mtable_half_bucket.restype = i
+    L.q4adamw_sr_bucket_entry.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]
+    L.q4adamw_sr_bucket_entry.restype = i
+    L.q4adamw_sr_affine_entry.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_float)]
+    L.q4adamw_sr_affine_entry.restype = i
     L.q4adamw_release.argtypes = []
     L.q4adamw_release.restype = i
     L.q4adamw_last_error.argtypes = []

@@ -271,6 +271,22 @@ int q4adamw_mtable_half_bucket(uint32_t half_index) {
   return (int)half_index_bucket(half_index);
 }
 
+int q4adamw_sr_bucket_entry(uint32_t half_index, uint32_t *out2) {
+  if (half_index >= kHalfTableEntries || !out2) return fail(Q4ADAMW_ERR_ARG, "index out of range");
+  const SrEntry e = sr_entry(half_index);
+  out2[0] = e.thr;
+  out2[1] = e.base;
+  return 0;
+}
+
+int q4adamw_sr_affine_entry(uint32_t k, float *out2) {
+  if (k > 16u || !out2) return fail(Q4ADAMW_ERR_ARG, "index out of range");
+  const SrAffine a = sr_affine_m(k);
+  out2[0] = a.a;
+  out2[1] = a.c;
+  return 0;
+}
+
 int q4adamw_fused_4bit_multi(const q4adamw_tensor *tensors, int count, int p_dtype, int g_dtype,
                              float beta1, float beta2, float lr, float weight_decay, float eps,
                              float step, void *stream) {

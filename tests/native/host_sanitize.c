@@ -66,6 +66,15 @@ static void host_only_entry_points(void) {
     }
   }
   EXPECT(q4adamw_mtable_half_bucket(256), Q4ADAMW_ERR_ARG);
+  for (uint32_t i = 0; i < 256; ++i) EXPECT(q4adamw_sr_bucket_entry(i, pair), 0);
+  EXPECT(q4adamw_sr_bucket_entry(256, pair), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_sr_bucket_entry(0, NULL), Q4ADAMW_ERR_ARG);
+  {
+    float affine[2];
+    for (uint32_t k = 0; k <= 16; ++k) EXPECT(q4adamw_sr_affine_entry(k, affine), 0);
+    EXPECT(q4adamw_sr_affine_entry(17, affine), Q4ADAMW_ERR_ARG);
+    EXPECT(q4adamw_sr_affine_entry(0, NULL), Q4ADAMW_ERR_ARG);
+  }
   uint32_t acc = 0;
   for (uint32_t s = 0; s < 1000; ++s) acc ^= q4adamw_sr_tensor_salt(0xFFFFFFFFFFFFFFFFull - s, (float)(s + 1), s * 2654435761u);
   if (acc == 0) printf("(salts xor to zero)\n");

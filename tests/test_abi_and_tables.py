@@ -249,6 +249,83 @@ def test_fast_path_model_first_moment(lib):
     assert 0 < undecided < 0.6 * total
 
 
+def _sr_tables(lib):
+    thr = np.zeros(256, np.uint32)
+    base = np.zeros(256, np.int64)
+    out = (ctypes.c_uint32 * 2)()
+    for h in range(256):
+        assert lib.q4adamw_sr_bucket_entry(h, out) == 0
+        thr[h], base[h] = out[0], out[1]
+    slope = np.zeros(17, np.float32)
+    offset = np.zeros(17, np.float32)
+    pair = (ctypes.c_float * 2)()
+    for k in range(17):
+        assert lib.q4adamw_sr_affine_entry(k, pair) == 0
+        slope[k], offset[k] = pair[0], pair[1]
+    return thr.view(np.float32), base, slope, offset
+
+
+def test_sr_affine_table_is_the_code_coordinate(lib):
+    """Entry k of the affine table maps interval k's ends to k and k + 1 (to within the
+    rounding of its two numbers), neighbouring entries meet at the code-book value between
+    them, and the ends are constant."""
+    _, _, slope, offset = _sr_tables(lib)
+    Q = oc.tables(0)[0].astype(np.float64)
+    assert (slope[0], offset[0]) == (0.0, 1.0) and (slope[16], offset[16]) == (0.0, 16.0)
+    for k in range(1, 16):
+        f = lambda q: float(slope[k]) * q + float(offset[k])
+        assert abs(f(Q[k - 1]) - k) < 2.0 ** -20 and abs(f(Q[k]) - (k + 1)) < 2.0 ** -20
+        assert max(abs(Q[k - 1]), abs(Q[k])) * float(slope[k]) < 9.0
+        if k < 15:
+            g = float(slope[k + 1]) * Q[k] + float(offset[k + 1])
+            assert abs(f(Q[k]) - g) < 2.0 ** -20
+
+
+def test_fast_path_model_first_moment_stochastic(lib):
+    """Model of the first moment's fast path under stochastic rounding: q^ = RN(x * r), r
+    within one ulp of 1/s; interval number from the half-indexed table; y = fma(n, -2^-16,
+    fma(q^, slope, offset)); near tie iff fract(y) < 2^-16, else code trunc(y).  Wherever the
+    model decides, its code must be the oracle's for the exact quotient RN(x / s) and the noise
+    (2 n + 1) / 2^17 -- for positions spread over every interval and for positions within a
+    few guard bands of the noise, where the decision flips."""
+    from oracle import q4_oracle_torch as ot
+    thr, base, slope, offset = _sr_tables(lib)
+    Q = oc.tables(0)[0].astype(np.float64)
+    rng = np.random.default_rng(11)
+    count = 40000
+    decided_total = undecided_total = 0
+    for near in (False, True):
+        s = (10.0 ** rng.uniform(-25, 25, count)).astype(np.float32)
+        n = rng.integers(0, 1 << 16, count)
+        n[:64] = 0
+        n[64:128] = 65535
+        u = ((2.0 * n + 1.0) / 2.0 ** 17).astype(np.float32)
+        k = rng.integers(1, 16, count)
+        lower, width = Q[k - 1], Q[k] - Q[k - 1]
+        pos = u.astype(np.float64) + rng.uniform(-4, 4, count) * 2.0 ** -17 if near else rng.uniform(0, 1, count)
+        target = np.clip(lower + np.clip(pos, 0, 1) * width, -1.0, 1.0)
+        x = _rn32(target * s.astype(np.float64))
+        x = np.clip(x, -s, s)                                             # |x| <= scale, as in a block
+        exact_q = _rn32(x.astype(np.float64) / s.astype(np.float64))
+        want = ot.sr_codes(exact_q, 0, u)
+        r0 = _rn32(1.0 / s.astype(np.float64))
+        for dr in (-1, 0, 1):
+            q = _rn32(x.astype(np.float64) * _nudge(r0, dr).astype(np.float64))
+            h = _half_index(q)
+            k_raw = base[h] + (q >= thr[h])
+            t = _rn32(q.astype(np.float64) * slope[k_raw].astype(np.float64) + offset[k_raw].astype(np.float64))
+            y = _rn32(t.astype(np.float64) - n * 2.0 ** -16)
+            decided = (y - np.floor(y)) >= np.float32(2.0 ** -16)
+            assert np.all(y[decided] >= 0) and np.all(y[decided] < 16)
+            code = np.trunc(y).astype(np.int64)
+            bad = np.flatnonzero(decided & (code != want))
+            assert bad.size == 0, (near, dr, bad[:5], q[bad[:5]], n[bad[:5]], code[bad[:5]], want[bad[:5]])
+            decided_total += int(decided.sum())
+            undecided_total += int((~decided).sum())
+    # positions within +-4 bands of the noise: about a quarter lands inside the band
+    assert 0 < undecided_total < 0.25 * (decided_total + undecided_total)
+
+
 def test_fast_path_model_second_moment():
     """Same for the second moment: t = fma(x, 16 r, w - 0.5) with w = 2^-17; code = trunc(t)
     unless fract(t) < 2w."""
