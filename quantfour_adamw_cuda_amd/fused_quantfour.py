@@ -144,6 +144,14 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         }
         state[field]["enable"] = enable_param_quantization(p, self.param_quant_threshold)
 
+    def __getstate__(self) -> Dict[str, Any]:
+        """The base class pickles defaults, state and param groups; the settings that live
+        on the object travel with them (launch caches and device counters do not)."""
+        state = super().__getstate__()
+        state["variance_scale_type"] = self.variance_scale_type
+        state["param_quant_threshold"] = self.param_quant_threshold
+        return state
+
     def __setstate__(self, state: Dict[str, Any]) -> None:
         """optim/fused_quantfour.py:73-84"""
         super().__setstate__(state)
@@ -154,6 +162,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self.__dict__.setdefault("kernel_timing", None)
         self.__dict__.setdefault("last_grad_norm", None)
         self.__dict__.setdefault("variance_scale_type", "group")
+        self.__dict__.setdefault("param_quant_threshold", 4096)
         self.__dict__.pop("_pending_skip", None)
         self.__dict__.pop("_skip_flag_host", None)
         for group in self.param_groups:

@@ -279,6 +279,24 @@ def test_setstate_backfills():
     assert torch.is_tensor(opt.state[p]["step"]) and float(opt.state[p]["step"]) == 3.0
 
 
+def test_pickle_and_deepcopy_keep_the_settings():
+    import copy
+    import pickle
+    ps = params((64, 136), (8,))
+    opt = AdamWFused_QuantFour(ps, lr=2e-3, variance_scale_type="rank1", round_type="stochastic", seed=5)
+    for p in ps:
+        opt._init_state(p)
+    opt._launch_cache["x"] = object()        # caches hold ctypes arrays: they must not travel
+    for twin in (pickle.loads(pickle.dumps(opt)), copy.deepcopy(opt)):
+        assert twin.variance_scale_type == "rank1" and twin.param_quant_threshold == 4096
+        g = twin.param_groups[0]
+        assert g["lr"] == 2e-3 and g["round_type"] == "stochastic" and g["seed"] == 5
+        assert twin._launch_cache == {} and twin._device_steps == {} and twin.kernel_timing is None
+        big = twin.param_groups[0]["params"][0]
+        assert "max_dims" in twin.state[big]["variance_qstate"]["overhead"]
+        assert twin.state[big]["exp_avg"].dtype == torch.uint8
+
+
 def test_functional_wrappers_validate():
     p = torch.zeros(300)
     with pytest.raises(AssertionError, match="param must be on cuda"):
