@@ -298,7 +298,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "fused_4bit_kernel" if not rank1 else "rank1_stats_kernel + fused_4bit_rank1_kernel",
+            "kernel": "fused_4bit_kernel" if not rank1 else "rank1_stats_kernel + fused_4bit_rank1_rows_kernel",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

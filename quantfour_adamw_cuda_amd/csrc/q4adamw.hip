@@ -182,6 +182,35 @@ static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr, bool 
   return ext ? pick_rank1_ext<true, false, false>(p_dtype, g_dtype) : pick_rank1_ext<false, false, false>(p_dtype, g_dtype);
 }
 
+template <bool EXT, bool SR>
+static Rank1Kernel pick_rank1_rows_ext(int p_dtype, int g_dtype) {
+  Q4_PICK_PG(fused_4bit_rank1_rows_kernel, EXT, SR)
+}
+
+// the kernel for matrices whose rows are a whole number of tiles long
+static Rank1Kernel pick_rank1_rows(int p_dtype, int g_dtype, bool ext, bool sr) {
+  if (sr) return pick_rank1_rows_ext<true, true>(p_dtype, g_dtype);
+  return ext ? pick_rank1_rows_ext<true, false>(p_dtype, g_dtype) : pick_rank1_rows_ext<false, false>(p_dtype, g_dtype);
+}
+
+// Which of the three update kernels a matrix takes, in the order of the launch passes.
+// Rows form: rows of a whole number of tiles (at least two), and enough rows that the
+// waves left idle in the last group of four do not matter.
+enum Rank1Shape { kShapeRows = 0, kShapeWide = 1, kShapeNarrow = 2 };
+
+static Rank1Shape rank1_shape(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
+  if (t.cols < tile_elems) return kShapeNarrow;
+  if (t.cols % tile_elems == 0 && t.cols >= 2 * tile_elems && t.rows >= 64) return kShapeRows;
+  return kShapeWide;
+}
+
+static uint64_t rank1_chunks(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
+  if (rank1_shape(t, tile_elems) == kShapeRows)
+    return (uint64_t)((t.rows + kWaves - 1) / kWaves) * (uint64_t)(t.cols / tile_elems);
+  const uint64_t chunk_elems = (uint64_t)tile_elems * kWaves;
+  return ((uint64_t)t.rows * (uint64_t)t.cols + chunk_elems - 1) / chunk_elems;
+}
+
 template <bool EXT>
 static Rank1StatKernel pick_rank1_stats_ext(int g_dtype) {
   if (g_dtype == Q4ADAMW_BF16) return rank1_stats_kernel<Q4ADAMW_BF16, EXT>;
@@ -431,10 +460,9 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       }
       if (prod != t.rows) return fail(Q4ADAMW_ERR_ARG, "rows must be the product of the leading dimensions");
     }
-    const uint64_t numel = (uint64_t)t.rows * (uint64_t)t.cols;
     const uint64_t stat_chunks = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) *
                                  (uint64_t)((t.cols + kStatCols - 1) / kStatCols);
-    if ((numel + chunk_elems - 1) / chunk_elems > kMaxChunksPerLaunch || stat_chunks > kMaxChunksPerLaunch)
+    if (rank1_chunks(t, chunk_elems / kWaves) > kMaxChunksPerLaunch || stat_chunks > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -475,15 +503,17 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     stat_chunks = 0;
     return 0;
   };
-  // two passes: matrices whose rows are at least a tile long take the kernel that finds a
-  // tile's row on the scalar unit, narrower ones the kernel whose lanes find their own
-  for (int narrow = 0; narrow < 2; ++narrow) {
-    kernel = pick_rank1(p_dtype, g_dtype, ext, sr, narrow != 0);
+  // three passes: matrices whose rows are whole tiles take the kernel whose workgroups share
+  // the columns' maxima of four rows; other matrices with rows of at least a tile the one
+  // that finds a tile's row on the scalar unit; narrower ones the one whose lanes find their own
+  for (int shape = kShapeRows; shape <= kShapeNarrow; ++shape) {
+    kernel = shape == kShapeRows ? pick_rank1_rows(p_dtype, g_dtype, ext, sr)
+                                 : pick_rank1(p_dtype, g_dtype, ext, sr, shape == kShapeNarrow);
     for (int i = 0; i < count; ++i) {
       const q4adamw_rank1_tensor &t = tensors[i];
-      if (t.rows == 0 || t.cols == 0 || (t.cols < tile_elems) != (narrow != 0)) continue;
+      if (t.rows == 0 || t.cols == 0 || rank1_shape(t, tile_elems) != shape) continue;
       const int64_t numel = t.rows * t.cols;
-      const uint64_t c = ((uint64_t)numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
+      const uint64_t c = rank1_chunks(t, tile_elems);
       const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
       const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
       if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
@@ -514,7 +544,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       d.numel = numel;
       d.rows = t.rows;
       d.cols = t.cols;
-      const FastDiv fd = make_fast_div((uint32_t)(t.cols >> 3));
+      // the divisor the tensor's kernel needs: tiles per row, or cols / 8
+      const FastDiv fd = make_fast_div(shape == kShapeRows ? (uint32_t)(t.cols / tile_elems) : (uint32_t)(t.cols >> 3));
       d.div_magic = fd.magic;
       d.div_shift = fd.shift;
       a.sr_salt[a.ntensors] = !sr ? 0u : a.go.sc_dev ? lowbias32(salts ? salts[i] : (uint32_t)i)

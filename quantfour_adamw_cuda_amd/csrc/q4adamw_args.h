@@ -101,7 +101,8 @@ struct Rank1Desc {  // 104 bytes
   int64_t numel;      // rows * cols
   int64_t rows;
   int64_t cols;
-  // division of a 32-bit number by cols / 8 as multiply-high, add and shifts
+  // division of a 32-bit number by cols / 8 (rows form of the update kernel: by the number
+  // of tiles in a row) as multiply-high, add and shifts
   // (round-up method: exact for every 32-bit dividend)
   uint32_t div_magic;
   uint32_t div_shift;

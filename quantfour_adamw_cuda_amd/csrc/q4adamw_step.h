@@ -27,11 +27,41 @@ struct Geometry {
 // step's new statistics (complete before this kernel starts) quantize.
 // SR: both moments are rounded stochastically between the two neighbouring code-book
 // entries; the noise of element e is a hash of e and the tensor's salt of this step.
-// NARROW (with RANK1): rows may be shorter than a tile.
-template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, bool NARROW, typename Desc>
+// SHAPE (with RANK1): how a tile lies in its matrix.  kTileWide: rows are at least a tile
+// long, so a tile touches one row or two.  kTileNarrow: rows may be shorter than a tile.
+// kTileRows: rows are a whole number of tiles long and the workgroup's four waves work on
+// the same columns of four consecutive rows, so they fetch the columns' maxima once,
+// together, and pass them through LDS (RowsTile).
+constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2;
+
+// What a wave of the kTileRows form knows beyond its tile number: its row, the tile's first
+// column, and this thread's share of the workgroup's fetch of the columns' maxima (old and
+// new; kTile / 256 consecutive columns per thread), which goes to `columns` in LDS:
+// [0, kTile) old, [kTile, 2 kTile) new.
+struct RowsTile {
+  int64_t row;
+  uint32_t col0;
+  float *columns;
+  float2 share_old, share_new;
+};
+
+// Writes a thread's share of the columns' maxima into LDS (before the workgroup's barrier).
+template <int N>
+__device__ __forceinline__ void stage_columns(const RowsTile &rt, int tid) {
+  if (N == 4) {
+    rt.columns[tid] = rt.share_old.x;
+    rt.columns[64 * N + tid] = rt.share_new.x;
+  } else {
+    *reinterpret_cast<float2 *>(rt.columns + 2 * tid) = rt.share_old;
+    *reinterpret_cast<float2 *>(rt.columns + 64 * N + 2 * tid) = rt.share_new;
+  }
+}
+
+template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, int SHAPE, typename Desc>
 __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
-                                             float gscale, bool zero_g, uint32_t salt) {
+                                             float gscale, bool zero_g, uint32_t salt,
+                                             const RowsTile *rt = nullptr) {
   using G = Geometry<PT, GT>;
   constexpr int N = G::kEpl;
   // Uniform (scalar) part of every address: the tile's first element, byte and
@@ -66,7 +96,12 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint32_t tb8 = (uint32_t)(tb >> 3), cols8 = (uint32_t)(T.cols >> 3);  // numel < 2^35
     const int64_t last = T.rows - 1;
     uint32_t col;
-    if constexpr (!NARROW) {
+    if constexpr (SHAPE == kTileRows) {
+      // the whole tile lies in one row; the columns' maxima come through LDS further down
+      col = rt->col0 + e0;
+      r_old = as_global<const float>(T.rmax)[rt->row];
+      r_new = as_global<const float>(T.rmax_next)[rt->row];
+    } else if constexpr (SHAPE == kTileWide) {
       // a tile is no longer than a row, so a lane is in the tile's first row or in the next
       const uint32_t row32 = fast_div(tb8, T.div_magic, T.div_shift);
       const int64_t row = row32;
@@ -88,12 +123,14 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
       r_old = as_global<const float>(T.rmax)[row];
       r_new = as_global<const float>(T.rmax_next)[row];
     }
+    if constexpr (SHAPE != kTileRows) {
 #pragma unroll
-    for (int k = 0; k < N; k += 4) {
-      const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax), (col + k) * 4u, 0, 0);
-      const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax_next), (col + k) * 4u, 0, 0);
-      c_old.x[k] = bits2f(a.x); c_old.x[k + 1] = bits2f(a.y); c_old.x[k + 2] = bits2f(a.z); c_old.x[k + 3] = bits2f(a.w);
-      c_new.x[k] = bits2f(b.x); c_new.x[k + 1] = bits2f(b.y); c_new.x[k + 2] = bits2f(b.z); c_new.x[k + 3] = bits2f(b.w);
+      for (int k = 0; k < N; k += 4) {
+        const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax), (col + k) * 4u, 0, 0);
+        const u32x4 b = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax_next), (col + k) * 4u, 0, 0);
+        c_old.x[k] = bits2f(a.x); c_old.x[k + 1] = bits2f(a.y); c_old.x[k + 2] = bits2f(a.z); c_old.x[k + 3] = bits2f(a.w);
+        c_new.x[k] = bits2f(b.x); c_new.x[k + 1] = bits2f(b.y); c_new.x[k + 2] = bits2f(b.z); c_new.x[k + 3] = bits2f(b.w);
+      }
     }
   }
 
@@ -148,7 +185,17 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const float v_entry = RANK1 ? qmap_v(lane & 15) : sc.b2 * (qmap_v(lane & 15) * sv_old);
     *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) = make_float2(m_entry, v_entry);
   }
+  if constexpr (RANK1 && SHAPE == kTileRows) stage_columns<N>(*rt, tid);
   setup_tables<SR>(lds, tid, slot);
+  if constexpr (RANK1 && SHAPE == kTileRows) {
+#pragma unroll
+    for (int k = 0; k < N; k += 4) {
+      const float4 a = *reinterpret_cast<const float4 *>(rt->columns + e0 + k);
+      const float4 b = *reinterpret_cast<const float4 *>(rt->columns + 64 * N + e0 + k);
+      c_old.x[k] = a.x; c_old.x[k + 1] = a.y; c_old.x[k + 2] = a.z; c_old.x[k + 3] = a.w;
+      c_new.x[k] = b.x; c_new.x[k + 1] = b.y; c_new.x[k + 2] = b.z; c_new.x[k + 3] = b.w;
+    }
+  }
 
   // entry numbers of the lane's codes, one per byte: even elements, odd elements
   const uint32_t three = 3u;
@@ -374,9 +421,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, false, SR, false>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, false, SR, kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, false, SR, false>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, false, SR, kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
@@ -539,9 +586,62 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, true, SR, NARROW>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+}
+
+// The same for matrices whose rows are a whole number of tiles (at least two) long: a chunk
+// is one tile's columns of four consecutive rows, one row per wave; T.div_magic / div_shift
+// divide by the number of tiles in a row.  Every tile is full.
+template <int PT, int GT, bool EXT, bool SR>
+__global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const Rank1Args args) {
+  using G = Geometry<PT, GT>;
+  constexpr int N = G::kEpl;
+  __shared__ uint2 lds[kLdsEntries];
+  __shared__ __attribute__((aligned(16))) float columns[2 * G::kTile];
+  const int tid = threadIdx.x;
+  const TableSlot slot = request_table_slot<SR>(tid);
+  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  if (chunk >= args.nchunks) return;
+  float gscale = 1.0f;
+  const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);
+  const bool zero_g = EXT && args.go.zero != 0u;
+  if (cancelled && !zero_g) return;
+  const int t = find_tensor(args, chunk);
+  const Rank1Desc &T = args.desc[t];
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const uint32_t local = chunk - args.first_chunk[t];
+  const uint32_t tiles_per_row = (uint32_t)(T.cols / G::kTile);
+  const uint32_t row_group = fast_div(local, T.div_magic, T.div_shift);
+  const uint32_t col_tile = local - row_group * tiles_per_row;
+  RowsTile rt;
+  rt.row = (int64_t)row_group * kWaves + wave;
+  rt.col0 = col_tile * (uint32_t)G::kTile;
+  rt.columns = columns;
+  const bool idle = rt.row >= T.rows;   // the last rows of a matrix whose row count is no multiple of four
+  const int64_t tile = rt.row * tiles_per_row + col_tile;
+  if (cancelled) {
+    if (!idle) zero_tile<GT, N>(T.g, tile, T.numel, lane);
+    return;
+  }
+  // this thread's share of the columns' maxima: N / 4 consecutive columns
+  const uint32_t share = rt.col0 + (uint32_t)tid * (N / 4);
+  if (N == 4) {
+    rt.share_old = make_float2(as_global<const float>(T.cmax)[share], 0.0f);
+    rt.share_new = make_float2(as_global<const float>(T.cmax_next)[share], 0.0f);
+  } else {
+    rt.share_old = make_float2(as_global<const float>(T.cmax)[share], as_global<const float>(T.cmax)[share + 1]);
+    rt.share_new = make_float2(as_global<const float>(T.cmax_next)[share], as_global<const float>(T.cmax_next)[share + 1]);
+  }
+  if (idle) {  // only help with the tables and the columns
+    stage_columns<N>(rt, tid);
+    setup_tables<SR>(lds, tid, slot);
+    return;
+  }
+  const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
+  const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
+  process_tile<PT, GT, true, EXT, true, SR, kTileRows>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
 }
 
 // After the update: the new statistics become the current ones and the buffers that

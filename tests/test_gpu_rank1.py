@@ -58,7 +58,7 @@ def _check(dev, ref, prev, what):
     assert ok, f"{what}: parameters out of tolerance (worst {worst})"
 
 
-SHAPES = [(64, 512), (3, 4096), (100, 520), (257, 768), (130, 1032), (1, 512), (70, 2048 + 512), (5, 8200),
+SHAPES = [(66, 1024), (128, 1536), (64, 4096), (64, 512), (3, 4096), (100, 520), (257, 768), (130, 1032), (1, 512), (70, 2048 + 512), (5, 8200),
           # narrow matrices: a tile spans several rows (fewer than 256 columns, or than 512 when
           # parameters and gradients are 16-bit types)
           (300, 16), (77, 64), (1000, 24), (513, 248), (40, 504), (9, 256), (2000, 136)]
@@ -89,7 +89,7 @@ def test_rank1_against_oracle(cuda, p_dt, g_dt, shape):
 
 @pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
                                        ("fp16", "fp16")])
-@pytest.mark.parametrize("shape", [(64, 512), (100, 520), (130, 1032), (5, 8200), (333, 40), (50, 264)])
+@pytest.mark.parametrize("shape", [(64, 512), (70, 2048 + 512), (100, 520), (130, 1032), (5, 8200), (333, 40), (50, 264)])
 def test_rank1_stochastic_rounding_against_oracle(cuda, p_dt, g_dt, shape):
     """rank-1 scaling and stochastic rounding together: codes, scales and statistics bit for
     bit against step_quant_rank1_sr; the noise follows seed, step and the tensor's salt"""
