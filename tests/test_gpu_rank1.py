@@ -194,6 +194,7 @@ def test_rank1_multi_tensor_and_options(cuda):
     """several matrices in one call (more than one launch batch), with a multiplier"""
     gen = torch.Generator().manual_seed(9)
     shapes = [(8 + i % 5, 512 + 8 * (i % 7)) for i in range(37)]
+    shapes += [(65, 512), (70, 768), (64, 1024)]      # rows of whole tiles: the kernel that shares column maxima
     ps = [(torch.randn(s, generator=gen) * 0.05) for s in shapes]
     devs = [Rank1State(p, cuda) for p in ps]
     refs = [(p.clone(), d.m.cpu(), d.v.cpu(), d.sm.cpu(), d.r.cpu(), d.c.cpu()) for p, d in zip(ps, devs)]
@@ -213,9 +214,10 @@ def test_rank1_multi_tensor_and_options(cuda):
             assert bool(dgs[i].any()) == (step == 1)
 
 
-def test_rank1_found_inf_leaves_everything(cuda):
+@pytest.mark.parametrize("rows", [40, 66])           # 66 rows of four tiles: the kernel that shares column maxima
+def test_rank1_found_inf_leaves_everything(cuda, rows):
     gen = torch.Generator().manual_seed(10)
-    p0 = torch.randn(40, 1024, generator=gen) * 0.05
+    p0 = torch.randn(rows, 1024, generator=gen) * 0.05
     dev = Rank1State(p0, cuda)
     g = grads_config1(gen, p0.numel()).view(p0.shape).to(torch.bfloat16).to(cuda)
     dev.step(g, 1)
