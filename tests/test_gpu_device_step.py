@@ -108,7 +108,7 @@ def test_training_steps_replayed_from_one_captured_graph(cuda):
     replay is the next training step (fresh gradients in the same buffers, a new learning rate
     in device memory) and equals the eager step with that step number on the host"""
     gen = torch.Generator().manual_seed(9)
-    n, rows, cols = 70_001, 24, 1024
+    n, rows, cols = 70_001, 70, 1024      # rows of whole tiles: the update kernel that shares column maxima
     p0, s0, m0 = (torch.randn(k, generator=gen) * 0.05 for k in (n, 777, rows * cols))
 
     class State:
@@ -193,7 +193,7 @@ def test_capturable_optimizer_replays_equal_the_eager_optimizer(cuda, variance, 
     state_dict() reports the device's step count; a resumed optimizer continues identically"""
     from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
     gen = torch.Generator().manual_seed(12)
-    shapes = [(40, 1024), (300, 33), (64,), (5000,), (16, 520)]
+    shapes = [(40, 1024), (68, 768), (300, 33), (64,), (5000,), (16, 520)]
     init = [torch.randn(s, generator=gen) * 0.05 for s in shapes]
     pc = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
     pe = [torch.nn.Parameter(t.clone().to(cuda)) for t in init]
