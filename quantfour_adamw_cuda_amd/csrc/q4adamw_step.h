@@ -164,18 +164,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     }
   }
   float sm_old = 0.0f, sv_old = 0.0f;
-  if (FULL && N == 4) {
-    // the tile's two blocks' scales through the scalar unit (two vector loads fewer per
-    // lane: 0.8 % on the whole kernel).  Nobody else writes these two entries during the
-    // launch, and this wave only after it has read them.
-    const float s0 = as_constant<const float>(sm_tile)[0], s1 = as_constant<const float>(sm_tile)[1];
-    sm_old = blk ? s1 : s0;
-    if (!RANK1) {
-      const float t0 = as_constant<const float>(sv_tile)[0], t1 = as_constant<const float>(sv_tile)[1];
-      sv_old = blk ? t1 : t0;
-    }
-  } else if (FULL) {
-    // four blocks per tile: a cached vector load (neighbouring blocks share lines)
+  if (FULL) {
+    // scales are 4 bytes per block: cached, so that neighbouring blocks share lines
     sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0));
     if (!RANK1) sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0));
   } else if (blk_ok) {
