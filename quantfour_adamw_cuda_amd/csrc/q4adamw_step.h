@@ -319,7 +319,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
       }
     } else {
       const bool hi0 = q0 > bits2f(ent0.y), hi1 = q1 > bits2f(ent1.y);
-      redo |= (hi0 != (q0 > bits2f(ent0.x))) | (hi1 != (q1 > bits2f(ent1.x)));
+      redo |= hi0 != (q0 > bits2f(ent0.x));
+      redo |= hi1 != (q1 > bits2f(ent1.x));
       // base code in the entry's low nibble, plus one above the threshold; every
       // code enters the word at the top and moves down four bits per later element
       mword = __builtin_amdgcn_alignbit(ent0.x + (hi0 ? 1u : 0u), mword, 4);
