@@ -10,7 +10,7 @@ import torch.nn as nn
 
 from oracle import q4_oracle as oc
 from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
-from tests.q4_testlib import HP, bits, grads_config1, grads_student_t, p_close, to_np
+from tests.q4_testlib import HP, bits, grads_config1, p_close, to_np
 
 pytestmark = pytest.mark.gpu
 

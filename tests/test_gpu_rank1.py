@@ -2,8 +2,6 @@
 against the torch restatement in oracle/q4_oracle_torch.py (itself pinned by brute force and
 closed forms in tests/test_oracle_pins.py): codes, block scales and row / column maxima bit
 for bit, parameters within the step's tolerance."""
-import ctypes
-
 import numpy as np
 import pytest
 import torch

@@ -3,7 +3,6 @@ forms, the quantizer against brute force and a library routine, the derived scal
 against known answers, the two independent restatements against each other, the
 non-quantized step against torch.optim.AdamW, and the quantized step against
 invariants of the format."""
-import math
 
 import numpy as np
 import pytest
