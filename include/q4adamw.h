@@ -278,6 +278,23 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
                       size_t workspace_bytes, float *out3, void *stream);
 
 /*
+ * q4adamw_grad_norm for callers that cannot allocate device memory and so have no workspace
+ * to pass: code under graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * No counterpart in the reference.  The partial sums live in a 16 KiB (2048 x fp64) array
+ * inside the library's device image, one copy per GPU, held until the process ends; the
+ * call allocates and frees nothing and gives the results of q4adamw_grad_norm bit for bit.
+ * That array's size does not depend on the input: the limits are q4adamw_grad_norm's own (a
+ * tensor of more than 2^31 - 16 chunks of 32 KiB is refused with Q4ADAMW_ERR_TOO_LARGE), and
+ * device ordinals of 64 and above are refused with Q4ADAMW_ERR_ARG.  Every partial sum is
+ * overwritten before it is read, so nothing of an earlier call survives.  All calls on one
+ * GPU share the one array: two calls that overlap there (different streams, different
+ * threads) race; calls on one stream, or otherwise ordered, do not.  The first call on a
+ * device asks the runtime for the array's address (no allocation); make it outside a capture.
+ */
+int q4adamw_grad_norm_static(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
+                             const float *grad_scale_dev, float max_norm, float *out3, void *stream);
+
+/*
  * A step whose number lives on the device.  The reference derives the scalars of a step on
  * the host from the step number it is given (optim/cuda_adamw_kernels.cu:435-440); a host
  * that replays a captured graph has no step number to give.  q4adamw_bias_table (host only)

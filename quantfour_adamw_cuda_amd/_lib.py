@@ -93,6 +93,7 @@ EXPORTS = (
     "q4adamw_fused_single_tensor_multi",
     "q4adamw_fused_single_tensor_multi_ex",
     "q4adamw_grad_norm",
+    "q4adamw_grad_norm_static",
     "q4adamw_bias_table",
     "q4adamw_device_step",
     "q4adamw_quantize",
@@ -152,6 +153,8 @@ def load():
     L.q4adamw_fused_4bit_rank1_multi_sr.restype = i
     L.q4adamw_grad_norm.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, ctypes.c_size_t, vp, vp]
     L.q4adamw_grad_norm.restype = i
+    L.q4adamw_grad_norm_static.argtypes = [ctypes.POINTER(Q4Grad), i, i, f, vp, f, vp, vp]
+    L.q4adamw_grad_norm_static.restype = i
     L.q4adamw_bias_table.argtypes = [f, f, i64, i64, vp]
     L.q4adamw_bias_table.restype = i
     L.q4adamw_device_step.argtypes = [vp, vp, i64, i64, vp, f, f, f, f, f, vp, vp, vp]

@@ -35,6 +35,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <atomic>
 #include <string>
 
 #include "../../include/q4adamw.h"
@@ -573,6 +574,93 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   return 0;
 }
 
+// ---------------------------------------------------------------------------
+// global gradient norm
+// ---------------------------------------------------------------------------
+// Partial sums of q4adamw_grad_norm_static: one fp64 value per workgroup of the sum-of-squares
+// launch, 16 KiB, held by every device the library runs on until the process ends.  In host
+// code this name is not a device address; norm_scratch() asks the runtime for the current
+// device's copy once and hands that pointer to the kernels.
+static __device__ __align__(256) double g_norm_scratch[kNormPartials];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<double *> g_norm_scratch_ptr[kMaxDevices];
+
+static int norm_scratch(double **out) {
+  int dev = -1;
+  Q4_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(Q4ADAMW_ERR_ARG, "device ordinal beyond the scratch table");
+  double *p = g_norm_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {   // first call on this device (two threads racing here find the same address)
+    void *sym = nullptr;
+    Q4_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(g_norm_scratch)));
+    if (!sym) return fail(Q4ADAMW_ERR_ARG, "the runtime returned no address for the scratch array");
+    p = static_cast<double *>(sym);
+    g_norm_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return 0;
+}
+
+// partials: kNormPartials doubles of device memory, 8-byte aligned; every one of them is
+// written by the first launch before anything reads it, so its previous contents do not matter
+static int grad_norm_impl(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
+                          const float *grad_scale_dev, float max_norm, double *partials, float *out3,
+                          void *stream) {
+  if (count < 0 || (count > 0 && !grads)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
+  if (int rc = check_dtypes(Q4ADAMW_FP32, g_dtype)) return rc;
+  if (!out3) return fail(Q4ADAMW_ERR_ARG, "null workspace or output");
+  if (!aligned(out3, 4) || (grad_scale_dev && !aligned(grad_scale_dev, 4)))
+    return fail(Q4ADAMW_ERR_ALIGN, "workspace must be 8-byte, scalars 4-byte aligned");
+  const int64_t chunk_elems = kNormChunkBytes / (g_dtype != Q4ADAMW_FP32 ? 2 : 4);
+  for (int i = 0; i < count; ++i) {
+    if (grads[i].numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
+    if (grads[i].numel == 0) continue;
+    if (!grads[i].g) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
+    if (!aligned(grads[i].g, 16)) return fail(Q4ADAMW_ERR_ALIGN, "gradients must be 16-byte aligned");
+    if (((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  NormArgs a;
+  a.partials = partials;
+  a.first = 1u;
+  a.ntensors = 0;
+  uint64_t chunks = 0;
+  auto launch = [&]() -> int {
+    finish_prefix(a);
+    a.nchunks = (uint32_t)chunks;
+    if (g_dtype == Q4ADAMW_BF16) hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_BF16>, dim3(kNormPartials), dim3(256), 0, s, a);
+    else if (g_dtype == Q4ADAMW_FP16) hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_FP16>, dim3(kNormPartials), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_FP32>, dim3(kNormPartials), dim3(256), 0, s, a);
+    Q4_HIP(hipGetLastError());
+    a.first = 0u;
+    a.ntensors = 0;
+    chunks = 0;
+    return 0;
+  };
+  for (int i = 0; i < count; ++i) {
+    if (grads[i].numel == 0) continue;
+    const uint64_t c = ((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
+    if (a.ntensors == kMaxNormTensors || chunks + c > kMaxChunksPerLaunch) {
+      if (int rc = launch()) return rc;
+    }
+    a.desc[a.ntensors].g = grads[i].g;
+    a.desc[a.ntensors].numel = grads[i].numel;
+    a.first_chunk[a.ntensors] = (uint32_t)chunks;
+    ++a.ntensors;
+    chunks += c;
+  }
+  // the first launch also defines every partial sum, so an empty list still takes one
+  if (a.ntensors > 0 || a.first) {
+    if (int rc = launch()) return rc;
+  }
+  hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(256), 0, s, static_cast<const double *>(partials),
+                     grad_scale, grad_scale_dev, max_norm, out3);
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 extern "C" {
 
 int q4adamw_fused_4bit_rank1_multi(const q4adamw_rank1_tensor *tensors, int count, int p_dtype,
@@ -669,60 +757,19 @@ int q4adamw_fused_single_tensor(void *p, const void *g, float *exp_avg, float *e
 int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
                       const float *grad_scale_dev, float max_norm, void *workspace,
                       size_t workspace_bytes, float *out3, void *stream) {
-  if (count < 0 || (count > 0 && !grads)) return fail(Q4ADAMW_ERR_ARG, "bad tensor list");
-  if (int rc = check_dtypes(Q4ADAMW_FP32, g_dtype)) return rc;
-  if (!workspace || !out3) return fail(Q4ADAMW_ERR_ARG, "null workspace or output");
+  if (!workspace) return fail(Q4ADAMW_ERR_ARG, "null workspace or output");
   if (workspace_bytes < Q4ADAMW_NORM_WORKSPACE_BYTES)
     return fail(Q4ADAMW_ERR_ARG, "workspace smaller than Q4ADAMW_NORM_WORKSPACE_BYTES");
-  if (!aligned(workspace, 8) || !aligned(out3, 4) || (grad_scale_dev && !aligned(grad_scale_dev, 4)))
-    return fail(Q4ADAMW_ERR_ALIGN, "workspace must be 8-byte, scalars 4-byte aligned");
-  const int64_t chunk_elems = kNormChunkBytes / (g_dtype != Q4ADAMW_FP32 ? 2 : 4);
-  for (int i = 0; i < count; ++i) {
-    if (grads[i].numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
-    if (grads[i].numel == 0) continue;
-    if (!grads[i].g) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
-    if (!aligned(grads[i].g, 16)) return fail(Q4ADAMW_ERR_ALIGN, "gradients must be 16-byte aligned");
-    if (((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
-      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
-  }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  NormArgs a;
-  a.partials = static_cast<double *>(workspace);
-  a.first = 1u;
-  a.ntensors = 0;
-  uint64_t chunks = 0;
-  auto launch = [&]() -> int {
-    finish_prefix(a);
-    a.nchunks = (uint32_t)chunks;
-    if (g_dtype == Q4ADAMW_BF16) hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_BF16>, dim3(kNormPartials), dim3(256), 0, s, a);
-    else if (g_dtype == Q4ADAMW_FP16) hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_FP16>, dim3(kNormPartials), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(grad_sumsq_kernel<Q4ADAMW_FP32>, dim3(kNormPartials), dim3(256), 0, s, a);
-    Q4_HIP(hipGetLastError());
-    a.first = 0u;
-    a.ntensors = 0;
-    chunks = 0;
-    return 0;
-  };
-  for (int i = 0; i < count; ++i) {
-    if (grads[i].numel == 0) continue;
-    const uint64_t c = ((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems;
-    if (a.ntensors == kMaxNormTensors || chunks + c > kMaxChunksPerLaunch) {
-      if (int rc = launch()) return rc;
-    }
-    a.desc[a.ntensors].g = grads[i].g;
-    a.desc[a.ntensors].numel = grads[i].numel;
-    a.first_chunk[a.ntensors] = (uint32_t)chunks;
-    ++a.ntensors;
-    chunks += c;
-  }
-  // the first launch also defines every partial sum, so an empty list still takes one
-  if (a.ntensors > 0 || a.first) {
-    if (int rc = launch()) return rc;
-  }
-  hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(256), 0, s,
-                     static_cast<const double *>(workspace), grad_scale, grad_scale_dev, max_norm, out3);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  if (!aligned(workspace, 8)) return fail(Q4ADAMW_ERR_ALIGN, "workspace must be 8-byte, scalars 4-byte aligned");
+  return grad_norm_impl(grads, count, g_dtype, grad_scale, grad_scale_dev, max_norm,
+                        static_cast<double *>(workspace), out3, stream);
+}
+
+int q4adamw_grad_norm_static(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
+                             const float *grad_scale_dev, float max_norm, float *out3, void *stream) {
+  double *partials = nullptr;
+  if (int rc = norm_scratch(&partials)) return rc;
+  return grad_norm_impl(grads, count, g_dtype, grad_scale, grad_scale_dev, max_norm, partials, out3, stream);
 }
 
 int q4adamw_bias_table(float beta1, float beta2, int64_t first_step, int64_t count, float *out2) {
@@ -847,6 +894,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1012; }
+int q4adamw_version(void) { return 1013; }
 
 }  // extern "C"
