@@ -217,9 +217,14 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     float m = m_old + sc.r1 * gj;                 // m_old, v_old: beta times the old moment
     float v = v_old + sc.r2 * (gj * gj);
     if (!FULL && j >= nv) { m = 0.0f; v = 0.0f; }
-    // parameter: only this part may use the hardware's 1-ulp sqrt and reciprocal
+    // parameter: only this part may use the hardware's 1-ulp square root and a reciprocal
+    // in place of the division
     const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
-    p[j] = __builtin_fmaf(-m, __builtin_amdgcn_rcpf(den), p[j] * sc.wdu);
+    // reciprocal: hardware estimate plus one Newton step.  An infinite denominator (estimate
+    // 0) makes the residual a NaN, which the minimum replaces, so that the reciprocal stays 0.
+    float rden = __builtin_amdgcn_rcpf(den);
+    rden = __builtin_fmaf(__builtin_fminf(__builtin_fmaf(-den, rden, 1.0f), 1e-6f), rden, rden);
+    p[j] = __builtin_fmaf(-m, rden, p[j] * sc.wdu);
     mn.x[j] = m;
     vn.x[j] = v;
     am = __builtin_fmaxf(am, __builtin_fabsf(m));

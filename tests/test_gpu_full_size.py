@@ -11,7 +11,7 @@ import torch.nn as nn
 from oracle import q4_oracle as oc
 from oracle import q4_oracle_torch as ot
 from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
-from tests.q4_testlib import HP, bits, to_np
+from tests.q4_testlib import HP, bits, strict_param_metrics, to_np
 
 pytestmark = pytest.mark.gpu
 KW = dict(lr=HP["lr"], betas=(HP["beta1"], HP["beta2"]), eps=HP["eps"], weight_decay=HP["weight_decay"])
@@ -98,6 +98,10 @@ def _check_tensor(p, st, before, g, step):
         d = (p.detach().reshape(-1).double() - rp.reshape(-1).double()).abs()
         scale = torch.maximum(rp.reshape(-1).abs(), (rp.reshape(-1) - p0.reshape(-1)).abs()).double()
         assert bool((d <= 1e-6 * scale.clamp_min(1e-30)).all()), f"params, shape {tuple(p.shape)}"
+        # the strict bound, 1e-6 relative to the parameter itself, wherever the parameter is at
+        # least as large as the step it took; the rest is reported in the session summary
+        strict = strict_param_metrics(p.detach(), rp, p0)
+        assert strict["dom"] <= 1e-6, f"params, shape {tuple(p.shape)}: {strict}"
 
 
 def _run_config(shapes, p_dtype, cuda, steps, label):
