@@ -4,20 +4,30 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b]
 
 One "step" is one `optimizer.step()` over the whole synthetic parameter set: one
-multi-tensor launch of the fused 4-bit kernel plus one launch of the non-quantized
-kernel for the tensors of at most 4096 elements.  Inputs are resident in HBM before
-the timed region starts.  Prints ONE JSON line:
+multi-tensor launch of the fused 4-bit kernel per batch of 48 tensors plus one launch of
+the non-quantized kernel for the tensors of at most 4096 elements.  Inputs are resident in
+HBM before the timed region starts.  Prints ONE JSON line:
 
   value         parameters updated per second over the timed region (wall clock
                 around K steps, synchronised on both sides)
   roofline      the fused kernel against HBM: algorithmic bytes per launch divided
                 by its average duration, measured with events on the launch stream
-                inside the same timed region
+                inside the same timed region; `traffic` = HBM bytes per launch from
+                hardware counters (profiles/hbm_traffic.json), null when the kernel
+                sources have changed since they were read
   cpu_baseline  the CPU oracle (vectorised torch restatement of the reference's
                 PyTorch path) timed on this machine's host cores on a bounded
                 sample of the same workload
+  configs       (default run only) the other benchmark configurations and the step's
+                variants, each timed the same way in this same process: step time,
+                kernel time, launches, fraction of peak, host time per step
+  ceiling       what this GPU's memory system gives kernels that move the step's bytes
+                in the step's access pattern without its arithmetic (libq4probe.so): a
+                plain copy, a read-only stream and the step's seven streams; the
+                roofline entries carry `frac_of_ceiling` against the last of these
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -29,12 +39,6 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per optimizer step of the fused kernel, measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (each scaled by what the same counter reads for a 4 GiB device copy: 2.0 and 1.0);
-# summaries in profiles/fused_4bit_kernel_llama3_8b_hbm_counters.txt and
-# profiles/fused_4bit_rank1_kernels_llama3_8b_hbm_counters.txt.  Keyed by (workload, rank-1
-# scaling); combinations that have not been profiled report null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {("llama3-8b", False): 9.7374e10, ("llama3-8b", True): 1.17325e11}
 HP = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
 
 
@@ -88,17 +92,22 @@ def gpt2_small_shapes():
 WORKLOADS = {
     # name: (shapes, param dtype, grad dtype, grad distribution, description)
     "llama3-8b": (llama3_8b_shapes, "float32", "bfloat16", "student_t",
-                  "Llama-3-8B parameter set (benchmark configuration 3): 291 tensors, fp32 master "
+                  "BASELINE.json configs[3]: Llama-3-8B parameter set, 291 tensors, fp32 master "
                   "params, bf16 grads, 4-bit m/v, block 128"),
     "llama2-13b": (llama2_13b_shapes, "bfloat16", "bfloat16", "student_t",
-                   "Llama-2-13B-shaped parameter set (benchmark configuration 4): 362 tensors, bf16 "
+                   "BASELINE.json configs[4]: Llama-2-13B-shaped parameter set, 362 tensors, bf16 "
                    "params, bf16 grads, 4-bit m/v, block 128"),
     "gpt2-small": (gpt2_small_shapes, "float32", "float32", "normal_outliers",
-                   "GPT-2-small parameter set (benchmark configuration 1): 148 tensors, fp32 params and "
+                   "BASELINE.json configs[1]: GPT-2-small parameter set, 148 tensors, fp32 params and "
                    "grads, 4-bit m/v, block 128"),
     "single-4096": (lambda: [("w", (4096, 4096))], "float32", "float32", "normal_outliers",
-                    "single fp32 4096x4096 tensor (benchmark configuration 0)"),
+                    "BASELINE.json configs[0]: single fp32 4096x4096 tensor"),
+    # one 2^30-element tensor: the kernel alone, free of the parameter sets' launch mix
+    # (--param-dtype / --grad-dtype choose the kernel variant)
+    "single-2p30": (lambda: [("w", (1 << 30,))], "float32", "bfloat16", "student_t",
+                    "one tensor of 2^30 elements (kernel-only workload, not a BASELINE.json configuration)"),
 }
+DTYPE_NAMES = ("float32", "bfloat16", "float16")
 
 
 def make_grad(torch, shape, dist, gen, device, dtype):
@@ -168,12 +177,207 @@ def cpu_baseline(torch, params, grads_set, hp, budget_s=20.0):
     }
 
 
+def build_inputs(torch, device, shapes, p_dtype, g_dtype, dist, grad_sets):
+    """Parameters and pre-generated gradient sets of one workload, resident on the device."""
+    gen = torch.Generator(device=device).manual_seed(0)
+    params = []
+    for _, shape in shapes:
+        p = (torch.randn(shape, generator=gen, device=device) * 0.02).to(p_dtype)
+        p = torch.nn.Parameter(p, requires_grad=True)
+        if g_dtype != p_dtype:
+            p.grad_dtype = g_dtype  # e.g. an fp32 master parameter with a bf16 gradient
+        params.append(p)
+    grads = [[make_grad(torch, shape, dist, gen, device, g_dtype) for _, shape in shapes]
+             for _ in range(max(1, grad_sets))]
+    return params, grads
+
+
+def run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, steps, warmup, variance_scale="group",
+               round_type="real-nearest", clip="none"):
+    """W warm-up steps, then exactly K timed steps between two synchronisations, with a fresh
+    optimizer over `params`.  Returns the measurements of the timed region."""
+    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
+    opt = AdamWFused_QuantFour(params, variance_scale_type=variance_scale, round_type=round_type, seed=0, **HP)
+    opt.kernel_timing = []  # (kind, start event, end event) per launch
+    host_s = [0.0]
+
+    def one_step(i):
+        gs = grad_sets[i % len(grad_sets)]
+        for p, g in zip(params, gs):
+            p.grad = g
+        h0 = time.perf_counter()
+        if clip == "fused":
+            opt.step(grad_scale=1.0 / 1024.0, max_grad_norm=1.0)
+        elif clip == "separate":
+            torch._foreach_mul_(gs, 1.0 / 1024.0)
+            torch.nn.utils.clip_grad_norm_(params, 1.0, foreach=True)
+            opt.step()
+        else:
+            opt.step()
+        host_s[0] += time.perf_counter() - h0
+
+    for i in range(warmup):
+        one_step(i)
+    torch.cuda.synchronize()
+    opt.kernel_timing.clear()
+    host_s[0] = 0.0
+
+    t0 = time.perf_counter()
+    for i in range(steps):
+        one_step(warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    # one entry per step: the step's fused launches (one kernel per batch of up to 48
+    # tensors, back to back on the stream) between two events
+    fused_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind.startswith("fused_4bit")]
+    avg_kernel_s = sum(fused_ms) / steps / 1e3
+    rank1 = [p for p in params if opt.state[p]["variance_qstate"]["overhead"].get("max_dims") is not None]
+    grouped = sum(1 for p in params if p.numel() > 4096) - len(rank1)
+    # kernels per step: one per batch of 48 block-scaled tensors; statistics + update +
+    # commit per batch of 32 rank-1 tensors
+    launches_per_step = -(-grouped // 48) + 3 * -(-len(rank1) // 32)
+    quant_params = sum(p.numel() for p in params if p.numel() > 4096)
+    algo_bytes = quant_params * bytes_per_param(p_dtype_s, g_dtype_s)
+    if rank1:
+        # the statistics pass reads g and the second moment's codes once more; no block scales
+        # for the second moment, row and column maxima instead (read twice, written twice)
+        gb = 4 if g_dtype_s == "float32" else 2
+        n1 = sum(p.numel() for p in rank1)
+        algo_bytes += n1 * (gb + 0.5 - 2 * 4 / 128.0) + sum(16 * (p.shape[0] + p.shape[1]) for p in rank1)
+    m = dict(elapsed=elapsed, steps=steps, ms_per_step=elapsed / steps * 1e3, kernel_s=avg_kernel_s,
+             launches_per_step=launches_per_step, algo_bytes=algo_bytes, rank1=len(rank1),
+             quant_params=quant_params, total_params=sum(p.numel() for p in params),
+             host_ms_per_step=host_s[0] / steps * 1e3)
+    norm_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "grad_norm"]
+    if norm_ms:
+        m["norm_s"] = sum(norm_ms) / steps / 1e3
+    return m
+
+
+def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None):
+    from quantfour_adamw_cuda_amd import hbm_traffic
+    achieved = m["algo_bytes"] / m["kernel_s"] / 1e9
+    n = m["launches_per_step"]
+    rec = hbm_traffic.lookup(workload, variance_scale, round_type)
+    r = {
+        "bound": "hbm",
+        "kernel": "fused_4bit_kernel" if not m["rank1"] else "rank1_stats_kernel + fused_4bit_rank1_rows_kernel",
+        "achieved": achieved,
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS,
+        # per launch, averaged over the step's launches (they differ in size): HBM bytes from
+        # hardware counters, algorithmic bytes, duration; achieved = algorithmic bytes / duration
+        "traffic": rec["bytes_per_step"] / n if rec else None,
+        "traffic_source": (f"profiles/hbm_traffic.json, kernel sources {rec['source_hash']}" if rec else
+                           "no counter record for these kernel sources"),
+        "algorithmic_bytes_per_launch": m["algo_bytes"] / n,
+        "kernel_ms_per_launch": m["kernel_s"] * 1e3 / n,
+        "kernel_launches_per_step": n,
+        "algorithmic_bytes_per_step": m["algo_bytes"],
+        "kernel_ms_per_step": m["kernel_s"] * 1e3,
+    }
+    if ceiling_gbs:
+        r["frac_of_ceiling"] = achieved / ceiling_gbs
+    return r
+
+
+def config_entry(name, desc, m, workload, variance_scale, round_type):
+    r = roofline_entry(m, workload, variance_scale, round_type)
+    return {
+        "name": name,
+        "workload": desc,
+        "steps": m["steps"],
+        "ms_per_step": m["ms_per_step"],
+        "params_per_s": m["total_params"] * m["steps"] / m["elapsed"],
+        "host_ms_per_step": m["host_ms_per_step"],
+        "kernel_ms_per_step": r["kernel_ms_per_step"],
+        "kernel_launches_per_step": r["kernel_launches_per_step"],
+        "algorithmic_bytes_per_step": r["algorithmic_bytes_per_step"],
+        "achieved": r["achieved"],
+        "frac": r["frac"],
+        "traffic": r["traffic"],
+    }
+
+
+def load_probe():
+    path = os.path.join(ROOT, "quantfour_adamw_cuda_amd", "csrc", "libq4probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python -m quantfour_adamw_cuda_amd.build`")
+    L = ctypes.CDLL(path)
+    vp, u64, i = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int
+    L.q4probe_copy.argtypes = [vp, vp, u64, vp]
+    L.q4probe_read.argtypes = [vp, u64, vp, vp]
+    L.q4probe_step_streams.argtypes = [vp, vp, vp, vp, vp, vp, u64, i, i, vp]
+    for f in (L.q4probe_copy, L.q4probe_read, L.q4probe_step_streams):
+        f.restype = i
+    return L
+
+
+def measure_ceiling(torch, device, reps=10):
+    """Median over `reps` launches (after 3 untimed ones) of each probe on 2^30 elements,
+    events on the launch stream around every launch."""
+    L = load_probe()
+    n = 1 << 30
+    stream = torch.cuda.current_stream(device).cuda_stream
+    tag = {"float32": 0, "bfloat16": 1}
+    a = torch.empty(n, dtype=torch.float32, device=device).normal_()
+    b = torch.empty(n, dtype=torch.float32, device=device).normal_()
+    m = torch.zeros(n // 2, dtype=torch.uint8, device=device)
+    v = torch.zeros(n // 2, dtype=torch.uint8, device=device)
+    sm = torch.zeros(n // 128, dtype=torch.float32, device=device)
+    sv = torch.zeros(n // 128, dtype=torch.float32, device=device)
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+
+    def timed(fn):
+        for _ in range(3):
+            assert fn() == 0, "probe launch failed"
+        torch.cuda.synchronize()
+        evs = []
+        for _ in range(reps):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            assert fn() == 0, "probe launch failed"
+            e.record()
+            evs.append((s, e))
+        torch.cuda.synchronize()
+        ms = sorted(s.elapsed_time(e) for s, e in evs)
+        return ms[len(ms) // 2] / 1e3
+
+    out = {"unit": "GB/s", "elements": n, "launches": reps, "statistic": "median",
+           "kernels": "libq4probe.so: probe_move_kernel (copy, read), probe_step_streams_kernel"}
+    t = timed(lambda: L.q4probe_copy(b.data_ptr(), a.data_ptr(), 4 * n, stream))
+    out["copy"] = 8.0 * n / t / 1e9
+    t = timed(lambda: L.q4probe_read(a.data_ptr(), 4 * n, sink.data_ptr(), stream))
+    out["read"] = 4.0 * n / t / 1e9
+    for p_s, g_s in (("float32", "bfloat16"), ("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")):
+        t = timed(lambda: L.q4probe_step_streams(a.data_ptr(), b.data_ptr(), m.data_ptr(), v.data_ptr(),
+                                                 sm.data_ptr(), sv.data_ptr(), n, tag[p_s], tag[g_s], stream))
+        out[f"step_streams_{p_s}_{g_s}"] = n * bytes_per_param(p_s, g_s) / t / 1e9
+    return out
+
+
+def calibrate_copy(torch, device):
+    """Three plain copies of 4 GiB (libq4probe.so), so that a counter profile of this command
+    also holds a kernel whose traffic is known."""
+    L = load_probe()
+    src = torch.empty(1 << 30, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    for _ in range(3):
+        assert L.q4probe_copy(dst.data_ptr(), src.data_ptr(), 4 << 30, stream) == 0
+    torch.cuda.synchronize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama3-8b", choices=sorted(WORKLOADS))
+    ap.add_argument("--param-dtype", choices=DTYPE_NAMES, default=None, help="override the workload's parameter dtype")
+    ap.add_argument("--grad-dtype", choices=DTYPE_NAMES, default=None, help="override the workload's gradient dtype")
     ap.add_argument("--grad-sets", type=int, default=2,
                     help="distinct pre-generated gradient sets rotated over the steps")
     ap.add_argument("--clip", choices=["none", "fused", "separate"], default="none",
@@ -185,10 +389,14 @@ def main():
                          "rank-1 row/column maxima for matrices (a statistics pass precedes the update)")
     ap.add_argument("--round-type", choices=["real-nearest", "stochastic"], default="real-nearest",
                     help="rounding of the quantizer (stochastic: hash noise per element)")
+    ap.add_argument("--configs", choices=["auto", "all", "none"], default="auto",
+                    help="also time the other benchmark configurations and the step's variants and report "
+                         "them in `configs` (auto: only for the default workload without variant options)")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the memory-system probes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="after the timed region, run a plain 4 GiB device copy three times, so that "
-                         "a counter profile of this command also holds a kernel of known traffic")
+                    help="after the timed region, run the probe library's plain 4 GiB copy three times, "
+                         "so that a counter profile of this command also holds a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the optimizer step on ONE GPU; the step needs "
@@ -196,90 +404,32 @@ def main():
                  "on its own shard. Run with --gpus 1.")
 
     import torch
-    from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     shapes_fn, p_dtype_s, g_dtype_s, dist, desc = WORKLOADS[args.workload]
-    p_dtype, g_dtype = getattr(torch, p_dtype_s), getattr(torch, g_dtype_s)
-    shapes = shapes_fn()
+    p_dtype_s, g_dtype_s = args.param_dtype or p_dtype_s, args.grad_dtype or g_dtype_s
+    plain = (args.variance_scale == "group" and args.round_type == "real-nearest" and args.clip == "none"
+             and not args.param_dtype and not args.grad_dtype)
+    all_configs = args.configs == "all" or (args.configs == "auto" and args.workload == "llama3-8b" and plain)
 
-    gen = torch.Generator(device=device).manual_seed(0)
-    params = []
-    for _, shape in shapes:
-        p = (torch.randn(shape, generator=gen, device=device) * 0.02).to(p_dtype)
-        p = torch.nn.Parameter(p, requires_grad=True)
-        if g_dtype != p_dtype:
-            p.grad_dtype = g_dtype  # fp32 master parameter with a bf16 gradient
-        params.append(p)
-    grad_sets = [[make_grad(torch, shape, dist, gen, device, g_dtype) for _, shape in shapes]
-                 for _ in range(max(1, args.grad_sets))]
-    total_params = sum(p.numel() for p in params)
-    quant_params = sum(p.numel() for p in params if p.numel() > 4096)
-
-    opt = AdamWFused_QuantFour(params, variance_scale_type=args.variance_scale,
-                               round_type=args.round_type, seed=0, **HP)
-    opt.kernel_timing = []  # (kind, start event, end event) per launch
-
-    def one_step(i):
-        gs = grad_sets[i % len(grad_sets)]
-        for p, g in zip(params, gs):
-            p.grad = g
-        if args.clip == "fused":
-            opt.step(grad_scale=1.0 / 1024.0, max_grad_norm=1.0)
-        elif args.clip == "separate":
-            torch._foreach_mul_(gs, 1.0 / 1024.0)
-            torch.nn.utils.clip_grad_norm_(params, 1.0, foreach=True)
-            opt.step()
-        else:
-            opt.step()
-
-    for i in range(args.warmup):
-        one_step(i)
-    torch.cuda.synchronize()
-    opt.kernel_timing.clear()
-
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        one_step(args.warmup + i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-
-    # one entry per step: the step's fused launches (one kernel per batch of up to 48
-    # tensors, back to back on the stream) between two events
-    fused_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind.startswith("fused_4bit")]
-    avg_kernel_s = sum(fused_ms) / args.steps / 1e3
-    rank1 = [p for p in params if opt.state[p]["variance_qstate"]["overhead"].get("max_dims") is not None]
-    grouped = sum(1 for p in params if p.numel() > 4096) - len(rank1)
-    # kernels per step: one per batch of 48 block-scaled tensors; statistics + update +
-    # commit per batch of 32 rank-1 tensors
-    launches_per_step = -(-grouped // 48) + 3 * -(-len(rank1) // 32)
-
+    params, grad_sets = build_inputs(torch, device, shapes_fn(), getattr(torch, p_dtype_s),
+                                     getattr(torch, g_dtype_s), dist, args.grad_sets)
+    m = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, args.steps, args.warmup,
+                   args.variance_scale, args.round_type, args.clip)
     if args.calibrate_copy:
-        src = torch.empty(1 << 30, dtype=torch.float32, device=device).normal_()
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-    algo_bytes = quant_params * bytes_per_param(p_dtype_s, g_dtype_s)
-    if rank1:
-        # the statistics pass reads g and the second moment's codes once more; no block scales
-        # for the second moment, row and column maxima instead (read twice, written twice)
-        gb = 4 if g_dtype_s == "float32" else 2
-        n1 = sum(p.numel() for p in rank1)
-        algo_bytes += n1 * (gb + 0.5 - 2 * 4 / 128.0) + sum(16 * (p.shape[0] + p.shape[1]) for p in rank1)
-    achieved = algo_bytes / avg_kernel_s / 1e9
+        calibrate_copy(torch, device)
 
     out = {
         "metric": "params_updated_per_sec_fused_4bit_adamw_step",
-        "value": total_params * args.steps / elapsed,
+        "value": m["total_params"] * args.steps / m["elapsed"],
         "unit": "params/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": elapsed / args.steps * 1e3,
+        "ms_per_step": m["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -288,47 +438,59 @@ def main():
         "config": {
             "workload": desc,
             "tensors": len(params),
-            "params": total_params,
-            "params_quantized": quant_params,
+            "params": m["total_params"],
+            "params_quantized": m["quant_params"],
             "param_dtype": p_dtype_s,
             "grad_dtype": g_dtype_s,
             "grad_sets": len(grad_sets),
             "hyper": {"lr": HP["lr"], "betas": list(HP["betas"]), "eps": HP["eps"],
                       "weight_decay": HP["weight_decay"]},
         },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "fused_4bit_kernel" if not rank1 else "rank1_stats_kernel + fused_4bit_rank1_rows_kernel",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            # per launch, averaged over the step's launches (they differ in size): measured
-            # HBM bytes, algorithmic bytes, duration; achieved = algorithmic bytes / duration
-            "traffic": (MEASURED_TRAFFIC_BYTES_PER_STEP[(args.workload, bool(rank1))] / launches_per_step
-                        if (args.workload, bool(rank1)) in MEASURED_TRAFFIC_BYTES_PER_STEP else None),
-            "algorithmic_bytes_per_launch": algo_bytes / launches_per_step,
-            "kernel_ms_per_launch": avg_kernel_s * 1e3 / launches_per_step,
-            "kernel_launches_per_step": launches_per_step,
-            "algorithmic_bytes_per_step": algo_bytes,
-            "kernel_ms_per_step": avg_kernel_s * 1e3,
-        },
+        "host_ms_per_step": m["host_ms_per_step"],
     }
     if args.round_type == "stochastic":
         out["config"]["workload"] += "; stochastic rounding"
-    if rank1:
-        out["config"]["workload"] += f"; rank-1 scaled second moment on {len(rank1)} matrices"
+    if m["rank1"]:
+        out["config"]["workload"] += f"; rank-1 scaled second moment on {m['rank1']} matrices"
     if args.clip != "none":
         out["config"]["workload"] += f"; gradients unscaled by 1/1024 and clipped to norm 1.0 ({args.clip})"
-        norm_ms = [s.elapsed_time(e) for kind, s, e in opt.kernel_timing if kind == "grad_norm"]
-        if norm_ms:
+        if "norm_s" in m:
             g_bytes = sum(g.numel() * g.element_size() for g in grad_sets[0])
-            norm_s = sum(norm_ms) / args.steps / 1e3
-            out["grad_norm"] = {"bound": "hbm", "kernel": "grad_sumsq_kernel", "ms_per_step": norm_s * 1e3,
-                                "algorithmic_bytes_per_step": g_bytes, "achieved": g_bytes / norm_s / 1e9,
-                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g_bytes / norm_s / 1e9 / HBM_PEAK_GBS}
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(torch, params, grad_sets[0], HP)
+            out["grad_norm"] = {"bound": "hbm", "kernel": "grad_sumsq_kernel", "ms_per_step": m["norm_s"] * 1e3,
+                                "algorithmic_bytes_per_step": g_bytes, "achieved": g_bytes / m["norm_s"] / 1e9,
+                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": g_bytes / m["norm_s"] / 1e9 / HBM_PEAK_GBS}
+    cpu = None if args.no_cpu_baseline else cpu_baseline(torch, params, grad_sets[0], HP)
+
+    configs = []
+    if all_configs:
+        # the step's variants on the headline workload's own tensors, then the other configurations
+        k, w = 10, 3
+        for vs, rt, name in (("group", "stochastic", "stochastic rounding"),
+                             ("rank1", "real-nearest", "rank-1 scaled second moment"),
+                             ("rank1", "stochastic", "rank-1 scaled second moment + stochastic rounding")):
+            mv = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, k, w, vs, rt)
+            configs.append(config_entry(f"{args.workload}, {name}", desc + "; " + name, mv, args.workload, vs, rt))
+    del params, grad_sets
+    torch.cuda.empty_cache()
+    if all_configs:
+        for wl, k, w in (("llama2-13b", 10, 3), ("gpt2-small", 200, 20), ("single-4096", 500, 50)):
+            fn, ps, gs_, dist_, desc_ = WORKLOADS[wl]
+            pr, gr = build_inputs(torch, device, fn(), getattr(torch, ps), getattr(torch, gs_), dist_, 2)
+            mv = run_config(torch, pr, gr, ps, gs_, k, w)
+            configs.append(config_entry(wl, desc_, mv, wl, "group", "real-nearest"))
+            del pr, gr
+            torch.cuda.empty_cache()
+
+    ceiling = None if args.no_ceiling else measure_ceiling(torch, device)
+    key = f"step_streams_{p_dtype_s}_{g_dtype_s}"
+    out["roofline"] = roofline_entry(m, args.workload, args.variance_scale, args.round_type,
+                                     ceiling.get(key) if ceiling else None)
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    if configs:
+        out["configs"] = configs
+    if ceiling is not None:
+        out["ceiling"] = ceiling
     print(json.dumps(out), flush=True)
 
 

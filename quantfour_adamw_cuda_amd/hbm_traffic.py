@@ -1,0 +1,144 @@
+"""HBM traffic of the step's kernels as hardware counters saw it, kept in
+profiles/hbm_traffic.json and read by bench.py for its `roofline.traffic` field.
+
+An entry is valid for the kernel sources it was measured on: every entry carries the hash of
+csrc/q4adamw.hip and csrc/q4adamw_*.h at that time, and `lookup` returns None for an entry
+whose hash differs from the sources in the tree, so a number never outlives the kernel it
+describes.
+
+Recording (rocprofv3 cannot split counters over passes, so one run per counter; on the GPU
+machine, from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd -`):
+
+    rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/pmc_fetch -o fetch -- \\
+        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy
+    rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o write -- \\
+        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy
+    python3 -m quantfour_adamw_cuda_amd.hbm_traffic --workload llama3-8b --steps 4 \\
+        --fetch-csv out/pmc_fetch/*/fetch_counter_collection.csv \\
+        --write-csv out/pmc_write/*/write_counter_collection.csv \\
+        --out profiles/hbm_traffic.json
+
+(add the bench's --workload / --variance-scale / --round-type options to all three).  Both
+counters are in KiB per dispatch; each is scaled by what the same counter reads for the
+probe library's plain copy of 4 GiB (--calibrate-copy), whose traffic is known.
+"""
+import argparse
+import csv
+import glob
+import hashlib
+import json
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(_HERE)
+DEFAULT_PATH = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+COPY_KERNEL = "probe_move_kernel<0>"
+COPY_BYTES = 4 << 30
+STEP_KERNELS = ("fused_4bit_kernel", "fused_4bit_rank1", "rank1_stats_kernel", "rank1_commit_kernel",
+                "rank1_fold_kernel", "single_tensor_kernel")
+
+
+def source_hash():
+    """sha256 over the sources libq4adamw.so is built from (names and contents)."""
+    h = hashlib.sha256()
+    csrc = os.path.join(_HERE, "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name == "q4adamw.hip" or (name.startswith("q4adamw_") and name.endswith(".h")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def key(workload, variance_scale="group", round_type="real-nearest"):
+    return f"{workload}|{variance_scale}|{round_type}"
+
+
+def lookup(workload, variance_scale="group", round_type="real-nearest", path=DEFAULT_PATH):
+    """The recorded entry (a dict with bytes_per_step ...) if one exists for these kernel
+    sources, else None."""
+    try:
+        with open(path) as f:
+            entries = json.load(f)["entries"]
+    except (OSError, ValueError, KeyError):
+        return None
+    e = entries.get(key(workload, variance_scale, round_type))
+    if not e or e.get("source_hash") != source_hash():
+        return None
+    return e
+
+
+def _sum_counter(csv_paths, counter):
+    """{kernel name: [sum of the counter over its dispatches, dispatches]} of one run"""
+    out = {}
+    for pattern in csv_paths:
+        for path in glob.glob(pattern):
+            with open(path, newline="") as f:
+                for row in csv.DictReader(f):
+                    if row["Counter_Name"] != counter:
+                        continue
+                    k = out.setdefault(row["Kernel_Name"], [0.0, 0])
+                    k[0] += float(row["Counter_Value"])
+                    k[1] += 1
+    return out
+
+
+def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, out_path, profile=None):
+    fetch, write = _sum_counter(fetch_csv, "FETCH_SIZE"), _sum_counter(write_csv, "WRITE_SIZE")
+
+    def pick(table, names):
+        return {k: v for k, v in table.items() if any(n in k for n in names)}
+
+    scales = {}
+    for what, table in (("fetch", fetch), ("write", write)):
+        copies = pick(table, (COPY_KERNEL,))
+        if not copies:
+            raise SystemExit(f"no {COPY_KERNEL} dispatch in the {what} run: profile bench.py with --calibrate-copy")
+        kib, n = map(sum, zip(*copies.values()))
+        scales[what] = (COPY_BYTES / 1024.0) / (kib / n)
+    fetch_b = sum(v[0] for v in pick(fetch, STEP_KERNELS).values()) * 1024.0 * scales["fetch"] / steps
+    write_b = sum(v[0] for v in pick(write, STEP_KERNELS).values()) * 1024.0 * scales["write"] / steps
+    dispatches = sum(v[1] for v in pick(fetch, STEP_KERNELS).values()) / steps
+    entry = {
+        "source_hash": source_hash(),
+        "bytes_per_step": fetch_b + write_b,
+        "fetch_bytes_per_step": fetch_b,
+        "write_bytes_per_step": write_b,
+        "fetch_scale": scales["fetch"],
+        "write_scale": scales["write"],
+        "dispatches_per_step": dispatches,
+        "steps_profiled": steps,
+        "kernels": sorted(pick(fetch, STEP_KERNELS)),
+    }
+    if profile:
+        entry["profile"] = profile
+    try:
+        with open(out_path) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        doc = {"entries": {}}
+    doc.setdefault("entries", {})[key(workload, variance_scale, round_type)] = entry
+    doc["unit"] = "bytes of HBM traffic per optimizer step (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)"
+    with open(out_path, "w") as f:
+        json.dump(doc, f, indent=1, sort_keys=True)
+        f.write("\n")
+    return entry
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--workload", required=True)
+    ap.add_argument("--variance-scale", default="group")
+    ap.add_argument("--round-type", default="real-nearest")
+    ap.add_argument("--fetch-csv", nargs="+", required=True)
+    ap.add_argument("--write-csv", nargs="+", required=True)
+    ap.add_argument("--steps", type=int, required=True, help="optimizer steps the profiled command ran (warm-up included)")
+    ap.add_argument("--out", default=DEFAULT_PATH)
+    ap.add_argument("--profile", default=None, help="the profiles/ summary that documents the run")
+    a = ap.parse_args()
+    print(json.dumps(record(a.workload, a.variance_scale, a.round_type, a.fetch_csv, a.write_csv, a.steps,
+                            a.out, a.profile), indent=1))
+
+
+if __name__ == "__main__":
+    main()
