@@ -150,9 +150,8 @@ static FusedKernel pick_fused_ext(int p_dtype, int g_dtype) {
   Q4_PICK_PG(fused_4bit_kernel, EXT, SR)
 }
 
-// stochastic rounding comes with the gradient options' kernels only
 static FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext, bool sr = false) {
-  if (sr) return pick_fused_ext<true, true>(p_dtype, g_dtype);
+  if (sr) return ext ? pick_fused_ext<true, true>(p_dtype, g_dtype) : pick_fused_ext<false, true>(p_dtype, g_dtype);
   return ext ? pick_fused_ext<true, false>(p_dtype, g_dtype) : pick_fused_ext<false, false>(p_dtype, g_dtype);
 }
 
@@ -176,10 +175,10 @@ static Rank1Kernel pick_rank1_ext(int p_dtype, int g_dtype) {
 // narrow: the kernel for matrices whose rows are shorter than a tile
 static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr, bool narrow) {
   if (narrow) {
-    if (sr) return pick_rank1_ext<true, true, true>(p_dtype, g_dtype);
+    if (sr) return ext ? pick_rank1_ext<true, true, true>(p_dtype, g_dtype) : pick_rank1_ext<false, true, true>(p_dtype, g_dtype);
     return ext ? pick_rank1_ext<true, false, true>(p_dtype, g_dtype) : pick_rank1_ext<false, false, true>(p_dtype, g_dtype);
   }
-  if (sr) return pick_rank1_ext<true, true, false>(p_dtype, g_dtype);
+  if (sr) return ext ? pick_rank1_ext<true, true, false>(p_dtype, g_dtype) : pick_rank1_ext<false, true, false>(p_dtype, g_dtype);
   return ext ? pick_rank1_ext<true, false, false>(p_dtype, g_dtype) : pick_rank1_ext<false, false, false>(p_dtype, g_dtype);
 }
 
@@ -190,7 +189,7 @@ static Rank1Kernel pick_rank1_rows_ext(int p_dtype, int g_dtype) {
 
 // the kernel for matrices whose rows are a whole number of tiles long
 static Rank1Kernel pick_rank1_rows(int p_dtype, int g_dtype, bool ext, bool sr) {
-  if (sr) return pick_rank1_rows_ext<true, true>(p_dtype, g_dtype);
+  if (sr) return ext ? pick_rank1_rows_ext<true, true>(p_dtype, g_dtype) : pick_rank1_rows_ext<false, true>(p_dtype, g_dtype);
   return ext ? pick_rank1_rows_ext<true, false>(p_dtype, g_dtype) : pick_rank1_rows_ext<false, false>(p_dtype, g_dtype);
 }
 

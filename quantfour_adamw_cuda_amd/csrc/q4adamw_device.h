@@ -362,15 +362,15 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t b
   return r;
 }
 
-// Byte BYTE of x, times 8 (the byte offset of an 8-byte table entry), as one SDWA
-// shift; `three` is the shift amount in a register.
+// Byte BYTE of x shifted left by `shift` (the byte offset of a table entry of 1 << shift
+// bytes), as one SDWA shift; the shift amount travels in a register.
 template <int BYTE>
-__device__ __forceinline__ uint32_t byte_times8(uint32_t x, uint32_t three) {
+__device__ __forceinline__ uint32_t byte_shifted(uint32_t x, uint32_t shift) {
   static_assert(BYTE >= 0 && BYTE <= 3, "");
   uint32_t r;
 #define Q4_SDWA_SHIFT(SEL)                                                                          \
   asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:" SEL \
-      : "=v"(r) : "v"(three), "v"(x))
+      : "=v"(r) : "v"(shift), "v"(x))
   if (BYTE == 0) Q4_SDWA_SHIFT("BYTE_0");
   else if (BYTE == 1) Q4_SDWA_SHIFT("BYTE_1");
   else if (BYTE == 2) Q4_SDWA_SHIFT("BYTE_2");
@@ -379,13 +379,13 @@ __device__ __forceinline__ uint32_t byte_times8(uint32_t x, uint32_t three) {
   return r;
 }
 
-// byte_times8 with the byte chosen by a loop index of an unrolled loop
-__device__ __forceinline__ uint32_t entry_offset(uint32_t x, int byte, uint32_t three) {
+// byte_shifted with the byte chosen by a loop index of an unrolled loop
+__device__ __forceinline__ uint32_t entry_offset(uint32_t x, int byte, uint32_t shift) {
   switch (byte) {
-    case 0: return byte_times8<0>(x, three);
-    case 1: return byte_times8<1>(x, three);
-    case 2: return byte_times8<2>(x, three);
-    default: return byte_times8<3>(x, three);
+    case 0: return byte_shifted<0>(x, shift);
+    case 1: return byte_shifted<1>(x, shift);
+    case 2: return byte_shifted<2>(x, shift);
+    default: return byte_shifted<3>(x, shift);
   }
 }
 
@@ -418,14 +418,16 @@ __device__ __forceinline__ int find_tensor(const Args &a, uint32_t chunk) {
 }
 
 // LDS of a workgroup, one array of 8-byte entries:
-//   [0, 256)    the waves' private dequantization tables: per wave 64 entries, per
-//               quantization block 16 entries {code_book_m[i] * scale_m,
-//               code_book_v[i] * scale_v}, so that dequantizing an element is one read
-//               and an entry number fits a byte
+//   [0, 256)    the waves' private dequantization tables, as two arrays of 256 floats: the
+//               first moment's at float 0, the second moment's at float kLdsSecondMoment;
+//               per wave 64 entries of each, per quantization block 16 (code book value *
+//               block scale * beta), so that dequantizing an element is one 4-byte read
+//               per moment and an entry number fits a byte
 //   [256, 512)  bucket table of the first-moment quantizer, indexed by the high byte
 //               of the quotient as a half
 //   [512, 529)  stochastic rounding only: the first moment's intervals as affine maps
 constexpr uint32_t kLdsBuckets = 64 * kWaves;
+constexpr uint32_t kLdsSecondMoment = 64 * kWaves;   // in floats: the second array of the dequantization tables
 constexpr uint32_t kLdsIntervals = kLdsBuckets + kHalfTableEntries;
 constexpr uint32_t kLdsEntries = kLdsIntervals + 32;
 static_assert(kLdsBuckets == 256, "dequantization entry numbers must fit a byte");

@@ -172,18 +172,24 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     sm_old = as_global<const float>(sm_tile)[blk];
     if (!RANK1) sv_old = as_global<const float>(sv_tile)[blk];
   }
-  // this block's dequantization table: entry i = {beta1 * (code_book_m[i] * scale_m),
-  // beta2 * (code_book_v[i] * scale_v)}: the old moments (cuda_adamw_kernels.cu:340,343)
-  // with the first product of their updates (:341,344) already applied, each product
-  // rounded as the per-element form rounds it.  Written by the block's lanes (lane & 15 =
-  // i) into the wave's private LDS region.  Rank-1: the second entry is the bare code-book
-  // value; scale and beta2 follow per element.
+  // this block's dequantization tables: entry i = beta1 * (code_book_m[i] * scale_m) of the
+  // first moment's, beta2 * (code_book_v[i] * scale_v) of the second moment's: the old
+  // moments (cuda_adamw_kernels.cu:340,343) with the first product of their updates
+  // (:341,344) already applied, each product rounded as the per-element form rounds it.
+  // Written by the block's lanes (lane & 15 = i) into the wave's private LDS regions.  Two
+  // tables of 4-byte entries, not one of pairs: a block's 16 entries then lie in 16
+  // different banks and neighbouring blocks in the other 16, so that a wave's reads, with
+  // every lane choosing its own entry, do not collide (pairs left half the banks idle in
+  // every read).  Rank-1: the second entry is the bare code-book value; scale and beta2
+  // follow per element.
   char *lds_bytes = reinterpret_cast<char *>(lds);
   const uint32_t cb_entry = (uint32_t)wave * 64u + blk * 16u;  // entry number of code 0
   {
     const float m_entry = sc.b1 * (slot.qm * sm_old);
     const float v_entry = RANK1 ? qmap_v(lane & 15) : sc.b2 * (qmap_v(lane & 15) * sv_old);
-    *reinterpret_cast<float2 *>(lds_bytes + (cb_entry + ((uint32_t)lane & 15u)) * 8u) = make_float2(m_entry, v_entry);
+    float *entry = reinterpret_cast<float *>(lds_bytes) + cb_entry + ((uint32_t)lane & 15u);
+    entry[0] = m_entry;
+    entry[kLdsSecondMoment] = v_entry;
   }
   if constexpr (RANK1 && SHAPE == kTileRows) stage_columns<N>(*rt, tid);
   setup_tables<SR>(lds, tid, slot);
@@ -198,7 +204,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   }
 
   // entry numbers of the lane's codes, one per byte: even elements, odd elements
-  const uint32_t three = 3u;
+  const uint32_t three = 3u, two = 2u;
   const uint32_t cb_bytes = cb_entry * 0x01010101u;
   const uint32_t m_even = and_or(mw, 0x0F0F0F0Fu, cb_bytes), m_odd = and_or(mw >> 4, 0x0F0F0F0Fu, cb_bytes);
   const uint32_t v_even = and_or(vw, 0x0F0F0F0Fu, cb_bytes), v_odd = and_or(vw >> 4, 0x0F0F0F0Fu, cb_bytes);
@@ -208,10 +214,10 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   float am = 0.0f, av = 0.0f;
 #pragma unroll
   for (int j = 0; j < N; ++j) {
-    const uint32_t mo = entry_offset(j & 1 ? m_odd : m_even, j >> 1, three);
-    const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, three);
+    const uint32_t mo = entry_offset(j & 1 ? m_odd : m_even, j >> 1, two);
+    const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, two);
     const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
-    float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + 4);
+    float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + kLdsSecondMoment * 4u);
     if constexpr (RANK1) v_old = sc.b2 * (v_old * min_nonneg(r_old, c_old.x[j]));  // adamw_fourbit_triton.py:520-527
     const float gj = g[j];
     float m = m_old + sc.r1 * gj;                 // m_old, v_old: beta times the old moment
@@ -220,11 +226,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     // parameter: only this part may use the hardware's 1-ulp square root and a reciprocal
     // in place of the division
     const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
-    // reciprocal: hardware estimate plus one Newton step.  An infinite denominator (estimate
-    // 0) makes the residual a NaN, which the minimum replaces, so that the reciprocal stays 0.
-    float rden = __builtin_amdgcn_rcpf(den);
-    rden = __builtin_fmaf(__builtin_fminf(__builtin_fmaf(-den, rden, 1.0f), 1e-6f), rden, rden);
-    p[j] = __builtin_fmaf(-m, rden, p[j] * sc.wdu);
+    p[j] = __builtin_fmaf(-m, __builtin_amdgcn_rcpf(den), p[j] * sc.wdu);
     mn.x[j] = m;
     vn.x[j] = v;
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
@@ -301,8 +303,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     // first moment: the quotients' bucket entries, two quotients per conversion
     const float q0 = mn.x[j] * rm, q1 = mn.x[j + 1] * rm;
     const uint32_t halves = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(q0, q1));
-    const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<1>(halves, three));
-    const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_times8<3>(halves, three));
+    const uint2 ent0 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_shifted<1>(halves, three));
+    const uint2 ent1 = *reinterpret_cast<const uint2 *>(lds_bytes + kLdsBuckets * 8u + byte_shifted<3>(halves, three));
     if constexpr (SR) {
       // interval among the code-book entries; inside it the code is floor(k + position -
       // noise), an affine function of the quotient.  Computed shifted up by the guard band
@@ -424,7 +426,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
     setup_tables<SR>(lds, tid, slot);
     return;
   }
-  const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
+  const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
     process_tile<PT, GT, true, EXT, false, SR, kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
@@ -589,7 +591,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
     setup_tables<SR>(lds, tid, slot);
     return;
   }
-  const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
+  const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
     process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
@@ -645,7 +647,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const R
     setup_tables<SR>(lds, tid, slot);
     return;
   }
-  const uint32_t salt = SR ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : 0u;
+  const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   process_tile<PT, GT, true, EXT, true, SR, kTileRows>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
 }
