@@ -26,9 +26,11 @@ the same path through the `grad_scale` / `found_inf` attributes it sets.
 The step itself runs only in the HIP library (csrc/libq4adamw.so); without it,
 or with parameters that are not on a GPU, `step()` raises.
 """
-from itertools import chain
+from itertools import chain, compress, repeat
+from operator import attrgetter, is_, methodcaller
 from typing import Any, Dict, Optional
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -43,6 +45,18 @@ def enable_param_quantization(p, threshold) -> bool:
     if threshold and p.numel() <= threshold:
         return False
     return True
+
+
+class _Bucket:
+    """One launch of a step: the tensors of one (kind, device, dtypes, step) and their
+    descriptor array."""
+    __slots__ = ("kind", "device", "idx", "arr", "p_tag", "g_tag", "salts", "g_dtypes", "g_mask", "g_column")
+
+
+class _Plan:
+    """A param group's launches and what they rest on (see _build_plan / _refresh_plan)."""
+    __slots__ = ("gi", "capturable", "stochastic", "state_obj", "params_obj", "param_ids", "all_params",
+                 "has_grad", "plannable", "params", "p_ptrs", "step_views", "grads", "buckets", "held")
 
 
 class AdamWFused_QuantFour(torch.optim.Optimizer):
@@ -125,6 +139,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self._launch_cache: Dict[Any, Any] = {}
         self._step_buffers: Dict[Any, Any] = {}
         self._device_steps: Dict[Any, Any] = {}
+        self._plans: Dict[Any, Any] = {}
         # global gradient norm of the last step(max_grad_norm=...), a device scalar
         self.last_grad_norm = None
         self._norm_buffers: Dict[Any, Any] = {}
@@ -158,6 +173,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self._launch_cache = {}
         self._step_buffers = {}
         self._device_steps = {}
+        self._plans = {}
         self._norm_buffers = {}
         self.__dict__.setdefault("kernel_timing", None)
         self.__dict__.setdefault("last_grad_norm", None)
@@ -308,6 +324,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             if "momentum_qstate" not in src:
                 self._adopt_adamw_state(p, dst)
         self._launch_cache = {}
+        self._plans = {}
         self._device_steps = {}      # device step counters restart from the loaded host numbers
 
     def _adopt_adamw_state(self, p, state):
@@ -472,99 +489,215 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
 
         _lib.load()  # raises if the HIP library has not been built
 
+        # everything is gathered and validated before the first launch and before any step
+        # counter moves, so that a refusal leaves parameters, state and counters as they were
+        ready = []
         for gi, group in enumerate(self.param_groups):
-            params_with_grad = []
-            grads = []
-            exp_avgs = []
-            exp_avg_sqs = []
-            state_steps = []
-            momentum_meta = []
-            variance_meta = []
-            momentum_quant_enabled = []
-            beta1, beta2 = group["betas"]
-
-            self._init_group(
-                group,
-                params_with_grad,
-                grads,
-                exp_avgs,
-                exp_avg_sqs,
-                state_steps,
-                momentum_meta,
-                variance_meta,
-                momentum_quant_enabled,
-            )
-            if not params_with_grad:
-                continue
-
-            capturable = bool(group.get("capturable", False))
-            # a tensor lr is read on the device in capturable mode; otherwise its value is taken now
-            lr = 1.0 if capturable else float(group["lr"])
-            weight_decay = group["weight_decay"]
-            eps = group["eps"]
-            stochastic = group.get("round_type", "real-nearest") == "stochastic"
-
-            # update step (optim/fused_quantfour.py:178)
-            if capturable and len(params_with_grad) != sum(1 for p in group["params"] if p.numel() > 0):
-                raise ValueError("capturable=True needs a gradient for every parameter of the group: "
-                                 "the group's parameters share one step counter on the device")
-            before = [float(s) for s in state_steps] if capturable and not self._has_device_steps(gi) else None
-            steps = self._advance_steps(gi, params_with_grad, state_steps)
-            if not capturable:       # a capturable group's true counter is on the device
-                stepped.extend(state_steps)
-            step_consts = {}
-            if capturable:
-                # one counter per device: advance it and derive the step's scalars there
-                for device in {p.device for p in params_with_grad}:
-                    step_consts[device] = self._device_step(gi, device, group, before, found_inf)
-                steps = [0.0] * len(steps)      # the host's numbers play no part in the launches
-
-            # one launch per (kind, device, dtypes, step)
-            buckets: Dict[Any, list] = {}
-            for i, param in enumerate(params_with_grad):
-                assert param.is_cuda, "param must be on cuda"
-                kind = momentum_quant_enabled[i]
-                if kind and "max_dims" in variance_meta[i]:
-                    kind = "rank1_sr" if stochastic else "rank1"
-                elif kind and stochastic:
-                    kind = "sr"
-                key = (kind, param.device, param.dtype, grads[i].dtype, steps[i])
-                buckets.setdefault(key, []).append(i)
-
-            for (quantized, device, p_dtype, g_dtype, t_step), idx in buckets.items():
-                rank1 = quantized in ("rank1", "rank1_sr")
-                cached = self._bucket_table(
-                    (gi, quantized, device, p_dtype, g_dtype),
-                    [params_with_grad[i] for i in idx], [grads[i] for i in idx], [exp_avgs[i] for i in idx],
-                    [exp_avg_sqs[i] for i in idx], [momentum_meta[i] for i in idx], [variance_meta[i] for i in idx])
-                _, arr, (p_tag, g_tag, *extra) = cached
-                if quantized in ("sr", "rank1_sr"):
-                    salts_arr, sr_seed = extra[0], group["seed"]
-                    launch_sr = _q.launch_rank1_table_sr if rank1 else _q.launch_table_sr
-                    launch = lambda *a: launch_sr(a[0], salts_arr, sr_seed, *a[1:])
-                else:
-                    launch = (_q.launch_rank1_table if rank1 else
-                              _q.launch_table if quantized else _q.launch_small_table)
-                options = _q.grad_options(device, host_mult, dev_mult, found_inf, zero_grad,
-                                          step_consts.get(device))
-                if capturable:   # lr and step enter through step_consts; the arguments only pass the range check
-                    t_step = 1.0
-                if self.kernel_timing is None:
-                    launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
-                else:
-                    with torch.cuda.device(device):
-                        start = torch.cuda.Event(enable_timing=True)
-                        end = torch.cuda.Event(enable_timing=True)
-                        start.record()
-                        launch(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
-                        end.record()
-                    kind = ("fused_4bit_rank1" if rank1 else
-                            "fused_4bit" if quantized else "fused_single_tensor")   # stochastic rounding counts as its scaling's kind
-                    self.kernel_timing.append((kind, start, end))
+            plan = self._plans.get(gi)
+            if plan is None or not self._refresh_plan(group, plan):
+                plan = self._build_plan(gi, group)
+            if plan is not None:
+                ready.append((group, plan))
+        for group, plan in ready:
+            self._run_plan(group, plan, host_mult, dev_mult, found_inf, zero_grad, stepped)
 
         if found_inf is not None and stepped:
             self._watch_skip_flag(found_inf, stepped)
         return loss
+
+    def _build_plan(self, gi, group):
+        """One param group's launches from scratch: gathers the parameters that have a gradient
+        and their state (created on first use), sorts them into launch buckets -- one per
+        (kind, device, dtypes, step) -- and validates everything.  The plan it returns (None:
+        no parameter has a gradient) is kept, so that the following steps only have to check
+        that nothing it rests on has changed (_refresh_plan).  Replaces the per-parameter
+        loop of optim/fused_quantfour.py:171-292."""
+        params_with_grad = []
+        grads = []
+        exp_avgs = []
+        exp_avg_sqs = []
+        state_steps = []
+        momentum_meta = []
+        variance_meta = []
+        momentum_quant_enabled = []
+
+        self._init_group(
+            group,
+            params_with_grad,
+            grads,
+            exp_avgs,
+            exp_avg_sqs,
+            state_steps,
+            momentum_meta,
+            variance_meta,
+            momentum_quant_enabled,
+        )
+        self._plans.pop(gi, None)
+        if not params_with_grad:
+            return None
+
+        capturable = bool(group.get("capturable", False))
+        stochastic = group.get("round_type", "real-nearest") == "stochastic"
+        if capturable and len(params_with_grad) != sum(1 for p in group["params"] if p.numel() > 0):
+            raise ValueError("capturable=True needs a gradient for every parameter of the group: "
+                             "the group's parameters share one step counter on the device")
+        self._layout_steps(gi, params_with_grad, state_steps)
+        steps_now = self._step_buffers[gi][0].tolist()
+
+        buckets: Dict[Any, list] = {}
+        for i, param in enumerate(params_with_grad):
+            assert param.is_cuda, "param must be on cuda"
+            kind = momentum_quant_enabled[i]
+            if kind and "max_dims" in variance_meta[i]:
+                kind = "rank1_sr" if stochastic else "rank1"
+            elif kind and stochastic:
+                kind = "sr"
+            key = (kind, param.device, param.dtype, grads[i].dtype, 0.0 if capturable else steps_now[i])
+            buckets.setdefault(key, []).append(i)
+
+        plan = _Plan()
+        plan.gi = gi
+        plan.capturable = capturable
+        plan.stochastic = stochastic
+        plan.state_obj = self.state
+        plan.params_obj = group["params"]
+        plan.param_ids = list(map(id, group["params"]))
+        plan.all_params = tuple(group["params"])          # keeps the ids above from being reused
+        plan.has_grad = [p.grad is not None for p in group["params"]]
+        plan.plannable = all(p.numel() > 0 for p in group["params"])
+        plan.params = params_with_grad
+        plan.p_ptrs = [t.data_ptr() for t in params_with_grad]
+        plan.step_views = state_steps
+        plan.grads = grads
+        plan.buckets = []
+        for (quantized, device, p_dtype, g_dtype, _), idx in buckets.items():
+            cached = self._bucket_table(
+                (gi, quantized, device, p_dtype, g_dtype),
+                [params_with_grad[i] for i in idx], [grads[i] for i in idx], [exp_avgs[i] for i in idx],
+                [exp_avg_sqs[i] for i in idx], [momentum_meta[i] for i in idx], [variance_meta[i] for i in idx])
+            _, arr, (p_tag, g_tag, *extra) = cached
+            b = _Bucket()
+            b.kind, b.device, b.idx, b.arr, b.p_tag, b.g_tag = quantized, device, idx, arr, p_tag, g_tag
+            b.salts = extra[0] if extra else None
+            b.g_dtypes = [g_dtype] * len(idx)
+            b.g_mask = 15 if quantized in ("rank1", "rank1_sr") else _q.grad_alignment(p_dtype, g_dtype, bool(quantized)) - 1
+            # the gradient pointers inside the descriptor array: the second 8-byte field of
+            # every descriptor type (include/q4adamw.h)
+            b.g_column = np.frombuffer(arr, dtype=np.uint64).reshape(len(idx), -1)[:, 1]
+            plan.buckets.append(b)
+        # what the plan rests on besides the parameters: the state tensors, by identity.
+        # core: (state dict, step, exp_avg, exp_avg_sq) per parameter; extra: (dict, key,
+        # tensor or list) for the scales and statistics of the quantized ones
+        core, extra = [], []
+        for i, param in enumerate(params_with_grad):
+            core.append((self.state[param], state_steps[i], exp_avgs[i], exp_avg_sqs[i]))
+            if momentum_quant_enabled[i]:
+                extra.append((momentum_meta[i], "max1", momentum_meta[i]["max1"]))
+                for key in ("max1", "max_dims", "scratch_dims", "row_scale", "row_scratch"):
+                    if key in variance_meta[i]:
+                        extra.append((variance_meta[i], key, variance_meta[i][key]))
+        held = (core, extra)
+        plan.held = held
+        if plan.plannable:
+            self._plans[gi] = plan
+        return plan
+
+    def _refresh_plan(self, group, plan):
+        """True if the plan of the last step still describes this group -- the same parameters
+        at the same addresses, the same ones with a gradient, the same state tensors, dense
+        contiguous gradients of the same dtypes -- after pointing its descriptors at this
+        step's gradients.  False sends the group through _build_plan, which also words the
+        refusals."""
+        params = group["params"]
+        if (params is not plan.params_obj or self.state is not plan.state_obj
+                or bool(group.get("capturable", False)) != plan.capturable
+                or (group.get("round_type", "real-nearest") == "stochastic") != plan.stochastic
+                or list(map(id, params)) != plan.param_ids):
+            return False
+        all_grads = list(map(attrgetter("grad"), params))
+        if [g is not None for g in all_grads] != plan.has_grad:
+            return False
+        grads = list(compress(all_grads, plan.has_grad))
+        if list(map(methodcaller("data_ptr"), plan.params)) != plan.p_ptrs:
+            return False
+        core, extra = plan.held
+        try:
+            for st, step, exp_avg, exp_avg_sq in core:
+                if st["step"] is not step or st["exp_avg"] is not exp_avg or st["exp_avg_sq"] is not exp_avg_sq:
+                    return False
+            for holder, key, held in extra:
+                if holder[key] is not held:
+                    return False
+        except KeyError:
+            return False
+        steps_now = self._step_buffers[plan.gi][0].tolist()
+        pointers = []
+        # a gradient object that was validated last step is still dense, contiguous and of its
+        # dtype; only its address is read again
+        seen = all(map(is_, grads, plan.grads))
+        for b in plan.buckets:
+            gs = [grads[i] for i in b.idx]
+            # is_contiguous() is False for a sparse tensor
+            if not seen and (list(map(attrgetter("dtype"), gs)) != b.g_dtypes
+                             or not all(map(methodcaller("is_contiguous"), gs))):
+                return False
+            ptrs = np.fromiter(map(methodcaller("data_ptr"), gs), dtype=np.uint64, count=len(gs))
+            if np.bitwise_and(ptrs, np.uint64(b.g_mask)).any():
+                return False
+            if not plan.capturable and len({steps_now[i] for i in b.idx}) != 1:
+                return False
+            pointers.append(ptrs)
+        for b, ptrs in zip(plan.buckets, pointers):
+            b.g_column[:] = ptrs
+        plan.grads = grads
+        return True
+
+    def _run_plan(self, group, plan, host_mult, dev_mult, found_inf, zero_grad, stepped):
+        """Advances the step counters of the plan's parameters (optim/fused_quantfour.py:178)
+        and makes one launch per bucket."""
+        gi, capturable = plan.gi, plan.capturable
+        beta1, beta2 = group["betas"]
+        # a tensor lr is read on the device in capturable mode; otherwise its value is taken now
+        lr = 1.0 if capturable else float(group["lr"])
+        weight_decay = group["weight_decay"]
+        eps = group["eps"]
+        before = ([float(s) for s in plan.step_views]
+                  if capturable and not self._has_device_steps(gi) else None)
+        steps = self._advance_steps(gi, plan.params, plan.step_views)
+        if not capturable:       # a capturable group's true counter is on the device
+            stepped.extend(plan.step_views)
+        step_consts = {}
+        if capturable:
+            # one counter per device: advance it and derive the step's scalars there
+            for device in {b.device for b in plan.buckets}:
+                step_consts[device] = self._device_step(gi, device, group, before, found_inf)
+        for b in plan.buckets:
+            rank1 = b.kind in ("rank1", "rank1_sr")
+            # lr and step of a capturable group enter through step_consts; the arguments only
+            # pass the range check
+            t_step = 1.0 if capturable else steps[b.idx[0]]
+            options = _q.grad_options(b.device, host_mult, dev_mult, found_inf, zero_grad,
+                                      step_consts.get(b.device))
+            hyper = (b.device, b.p_tag, b.g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
+            if b.kind in ("sr", "rank1_sr"):
+                launch = _q.launch_rank1_table_sr if rank1 else _q.launch_table_sr
+                args = (b.arr, b.salts, group["seed"]) + hyper
+            else:
+                launch = (_q.launch_rank1_table if rank1 else
+                          _q.launch_table if b.kind else _q.launch_small_table)
+                args = (b.arr,) + hyper
+            if self.kernel_timing is None:
+                launch(*args)
+            else:
+                with _q._on(b.device):
+                    start = torch.cuda.Event(enable_timing=True)
+                    end = torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    launch(*args)
+                    end.record()
+                kind = ("fused_4bit_rank1" if rank1 else
+                        "fused_4bit" if b.kind else "fused_single_tensor")   # stochastic rounding counts as its scaling's kind
+                self.kernel_timing.append((kind, start, end))
 
     # -- capturable: the step number on the device ------------------------------------
     def _has_device_steps(self, gi):
@@ -659,18 +792,17 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 assert g.device == device, "grad must be on the param's device"
                 assert g.is_contiguous(), "grad must be contiguous"
                 assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
+                assert g.data_ptr() % (16 if rank1 else _q.grad_alignment(p.dtype, g.dtype, bool(quantized))) == 0, \
+                    "grad must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
                 arr[i].g = g.data_ptr()
         return cached
 
-    def _advance_steps(self, gi, params, state_steps):
-        """Adds 1 to every step counter and returns their new values as Python floats.  The
-        counters of a group's parameters are 0-dim views of one host buffer, so this is one
-        addition whatever the number of tensors; a counter that was replaced (lazy state,
-        load_state_dict, the user) is noticed by identity and the buffer is laid out again.
-        `state_steps` is updated in place to the tensors the state holds afterwards."""
+    def _layout_steps(self, gi, params, state_steps):
+        """Makes the step counters of `params` 0-dim views of one host buffer (values kept)
+        and `state_steps` the list of those views, unless they are already."""
         cached = self._step_buffers.get(gi)
         if (cached is None or len(cached[1]) != len(state_steps)
-                or any(a is not b for a, b in zip(cached[1], state_steps))):
+                or not all(map(is_, cached[1], state_steps))):
             buf = torch.stack([t.detach().to(device="cpu", dtype=torch.float32).reshape(())
                                for t in state_steps])
             views = list(buf.unbind(0))
@@ -679,7 +811,15 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             cached = (buf, views)
             self._step_buffers[gi] = cached
             state_steps[:] = views
-        buf = cached[0]
+        return cached[0]
+
+    def _advance_steps(self, gi, params, state_steps):
+        """Adds 1 to every step counter and returns their new values as Python floats.  The
+        counters of a group's parameters are 0-dim views of one host buffer, so this is one
+        addition whatever the number of tensors; a counter that was replaced (lazy state,
+        load_state_dict, the user) is noticed by identity and the buffer is laid out again.
+        `state_steps` is updated in place to the tensors the state holds afterwards."""
+        buf = self._layout_steps(gi, params, state_steps)
         buf.add_(1)
         return buf.tolist()
 

@@ -36,8 +36,28 @@ def _check_common(p, g):
     assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
 
 
+def grad_alignment(p_dtype, g_dtype, quantized=True):
+    """Bytes a gradient's address must be a multiple of: the fused kernels read 16 bytes per
+    lane (8 of a 16-bit gradient next to fp32 parameters), the non-quantized one element by
+    element."""
+    g16 = g_dtype != torch.float32
+    if not quantized:
+        return 2 if g16 else 4
+    return 8 if (g16 and p_dtype == torch.float32) else 16
+
+
+def _check_aligned(p, g, quantized=True):
+    # refused by the library as well (Q4ADAMW_ERR_ALIGN); checked here so that a step refuses
+    # before its first launch
+    assert p.data_ptr() % (16 if quantized else p.element_size()) == 0, \
+        "param must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
+    assert g.data_ptr() % grad_alignment(p.dtype, g.dtype, quantized) == 0, \
+        "grad must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
+
+
 def check_quantized(p, g, exp, sq, exp_scale, sq_scale):
     _check_common(p, g)
+    _check_aligned(p, g)
     nbytes, nblk = state_sizes(p.numel())
     assert exp.dtype == torch.uint8 and sq.dtype == torch.uint8, "moments must be packed uint8"
     assert exp.numel() == nbytes, f"exp_avg numel {exp.numel()} != packed size {nbytes}"
@@ -58,6 +78,28 @@ def check_unquantized(p, g, exp_avg, exp_avg_sq):
 
 def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _OnDevice:
+    """`with _on(device):` -- torch.cuda.device(device) when another device is current, else
+    nothing (the step's launches run in a loop where the context switch would cost as much
+    as the launch)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        self.ctx = None if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
+
+
+_on = _OnDevice
 
 
 def fused_4bit(p, g, exp, sq, exp_scale, sq_scale, beta1, beta2, lr, weight_decay, eps, step):
@@ -181,7 +223,7 @@ def device_step(step, table, consts, beta1, beta2, lr, weight_decay, eps, lr_dev
 
 def launch_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options=None):
     L = _lib.load()
-    with torch.cuda.device(device):
+    with _on(device):
         rc = L.q4adamw_fused_4bit_multi_ex(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
                                            weight_decay, eps, float(step), options, _stream(device))
     _lib.check(rc, "fused_4bit_multi")
@@ -190,7 +232,7 @@ def launch_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps,
 def launch_small_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step,
                        options=None):
     L = _lib.load()
-    with torch.cuda.device(device):
+    with _on(device):
         rc = L.q4adamw_fused_single_tensor_multi_ex(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
                                                     weight_decay, eps, float(step), options,
                                                     _stream(device))
@@ -244,7 +286,7 @@ def launch_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, beta2, lr
                     step, options=None):
     L = _lib.load()
     assert salts_arr is None or len(salts_arr) == len(arr), "one salt per tensor"
-    with torch.cuda.device(device):
+    with _on(device):
         rc = L.q4adamw_fused_4bit_multi_sr(arr, len(arr), salts_arr, int(seed) & (2 ** 64 - 1), p_tag, g_tag,
                                            beta1, beta2, lr, weight_decay, eps, float(step), options,
                                            _stream(device))
@@ -295,6 +337,8 @@ def rank1_row_scale(lead_maxes, lead_shape):
 
 def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next, lead=None):
     _check_common(p, g)
+    assert p.data_ptr() % 16 == 0 and g.data_ptr() % 16 == 0, \
+        "param and grad must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
     assert rank1_eligible(p), "rank-1 scaling needs 2 to 4 dimensions, the last a multiple of 8 and at least 16"
     cols = p.shape[-1]
     rows = p.numel() // cols
@@ -347,7 +391,7 @@ def make_rank1_table(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_ne
 def launch_rank1_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step,
                        options=None):
     L = _lib.load()
-    with torch.cuda.device(device):
+    with _on(device):
         rc = L.q4adamw_fused_4bit_rank1_multi(arr, len(arr), p_tag, g_tag, beta1, beta2, lr,
                                               weight_decay, eps, float(step), options, _stream(device))
     _lib.check(rc, "fused_4bit_rank1_multi")
@@ -357,7 +401,7 @@ def launch_rank1_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, bet
                           eps, step, options=None):
     L = _lib.load()
     assert salts_arr is None or len(salts_arr) == len(arr), "one salt per tensor"
-    with torch.cuda.device(device):
+    with _on(device):
         rc = L.q4adamw_fused_4bit_rank1_multi_sr(arr, len(arr), salts_arr, int(seed) & (2 ** 64 - 1), p_tag,
                                                  g_tag, beta1, beta2, lr, weight_decay, eps, float(step),
                                                  options, _stream(device))

@@ -303,3 +303,141 @@ def test_llama3_8b_embedding_shape(cuda):
     opt.step()
     torch.cuda.synchronize()
     ref.step_and_check([p], [g.cpu()], opt, 1, "llama embedding")
+
+
+def _twin_optimizers(cuda, shapes, dtype=torch.float32, **kw):
+    """two optimizers over equal parameters: `a` keeps its plan from step to step, `b` is
+    rebuilt from its own state_dict before every step and so always gathers from scratch"""
+    gen = torch.Generator().manual_seed(77)
+    base = [(torch.randn(s, generator=gen) * 0.02).to(dtype) for s in shapes]
+    pa = [nn.Parameter(t.clone().to(cuda)) for t in base]
+    pb = [nn.Parameter(t.clone().to(cuda)) for t in base]
+    return pa, pb, AdamWFused_QuantFour(pa, **KW, **kw), AdamWFused_QuantFour(pb, **KW, **kw), gen
+
+
+def _same_everything(opt_a, pa, opt_b, pb):
+    for x, y in zip(pa, pb):
+        assert torch.equal(x.detach().view(torch.uint8), y.detach().view(torch.uint8))
+        sa, sb = opt_a.state.get(x, {}), opt_b.state.get(y, {})
+        assert set(sa) == set(sb)
+        if not sa:
+            continue
+        assert float(sa["step"]) == float(sb["step"])
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(sa[key].view(torch.uint8), sb[key].view(torch.uint8)), key
+        for q in ("momentum_qstate", "variance_qstate"):
+            ma, mb = sa[q]["overhead"].get("max1"), sb[q]["overhead"].get("max1")
+            assert (ma is None) == (mb is None) and (ma is None or torch.equal(ma.view(torch.int32), mb.view(torch.int32)))
+
+
+def test_kept_plan_follows_every_change_of_what_it_rests_on(cuda):
+    """The optimizer keeps a group's launch plan between steps and re-gathers only when
+    something under it changed.  Each step below changes one such thing -- which parameters
+    have a gradient, a gradient's dtype, a parameter's storage, a state tensor, a step counter,
+    the group's parameter list -- and the result must equal, bit for bit, that of a twin
+    whose plan is thrown away before every step."""
+    shapes = [(40, 300), (5000,), (17,), (64, 128), (4096,)]
+    pa, pb, oa, ob, gen = _twin_optimizers(cuda, shapes)
+
+    def grads(mask=None, dtypes=None):
+        out = []
+        for i, s in enumerate(shapes):
+            if mask is not None and not mask[i]:
+                out.append(None)
+                continue
+            g = torch.randn(s, generator=gen) * 1e-3
+            out.append(g.to(dtypes[i] if dtypes else torch.float32))
+        return out
+
+    def step_both(gs):
+        for ps in (pa, pb):
+            for p, g in zip(ps, gs):
+                p.grad = None
+                if g is not None and g.dtype != p.dtype:
+                    p.grad_dtype = g.dtype
+                p.grad = None if g is None else g.to(cuda)
+        ob._plans.clear()
+        ob._launch_cache.clear()
+        oa.step()
+        ob.step()
+        torch.cuda.synchronize()
+        _same_everything(oa, pa, ob, pb)
+
+    step_both(grads())
+    assert 0 in oa._plans
+    kept = oa._plans[0]
+    step_both(grads())
+    assert oa._plans[0] is kept, "nothing changed: the plan must have been reused"
+    step_both(grads(mask=[True, False, True, True, True]))          # one parameter without a gradient
+    assert oa._plans[0] is not kept
+    step_both(grads())                                               # and with one again (its step lags by one)
+    assert [float(oa.state[p]["step"]) for p in pa] == [4.0, 3.0, 4.0, 4.0, 4.0]
+    kept = oa._plans[0]
+    step_both(grads())
+    assert oa._plans[0] is kept
+    step_both(grads(dtypes=[torch.bfloat16, torch.float32, torch.float32, torch.float32, torch.float32]))
+    assert oa._plans[0] is not kept                                  # a gradient changed its dtype
+    kept = oa._plans[0]
+    for ps in (pa, pb):                                              # a parameter moved to other storage
+        ps[3].data = ps[3].data.clone()
+    step_both(grads(dtypes=[torch.bfloat16, torch.float32, torch.float32, torch.float32, torch.float32]))
+    assert oa._plans[0] is not kept
+    kept = oa._plans[0]
+    for o, ps in ((oa, pa), (ob, pb)):                               # a state tensor replaced from outside
+        o.state[ps[1]]["exp_avg"] = o.state[ps[1]]["exp_avg"].clone()
+        o.state[ps[0]]["step"] = torch.tensor(11.0)
+    step_both(grads(dtypes=[torch.bfloat16, torch.float32, torch.float32, torch.float32, torch.float32]))
+    assert oa._plans[0] is not kept and float(oa.state[pa[0]]["step"]) == 12.0
+    kept = oa._plans[0]
+    sd = oa.state_dict()                                             # a loaded state_dict replaces every state tensor
+    oa.load_state_dict(sd)
+    ob.load_state_dict(ob.state_dict())
+    step_both(grads(dtypes=[torch.bfloat16, torch.float32, torch.float32, torch.float32, torch.float32]))
+    assert oa._plans[0] is not kept
+
+
+def test_a_refused_gradient_leaves_everything_as_it_was(cuda):
+    """Everything is validated before the first launch and before any step counter moves: a
+    gradient the kernels cannot take (a view at a 4-byte offset into a flat buffer, a
+    transposed view) in the LAST bucket of the LAST group leaves parameters, state and
+    counters of every group untouched, on the first step and on a step that had a plan."""
+    gen = torch.Generator().manual_seed(5)
+    shapes = [(64, 100), (3000,), (8192,)]
+    ps = [nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(cuda)) for s in shapes]
+    opt = AdamWFused_QuantFour([{"params": ps[:2]}, {"params": ps[2:], "lr": 2e-3}], **KW)
+    flat = torch.zeros(8192 + 8, device=cuda)
+
+    def snapshot():
+        """parameters, and the state that exists (the first refused step creates it, all zeros)"""
+        out = {("p", i): p.detach().clone() for i, p in enumerate(ps)}
+        for i, p in enumerate(ps):
+            st = opt.state.get(p, {})
+            out.update({(k, i): st[k].clone() for k in ("step", "exp_avg", "exp_avg_sq") if k in st})
+        return out
+
+    def unchanged(before, after):
+        return all(torch.equal(t, after[k]) for k, t in before.items())
+
+    def set_grads(bad):
+        for p in ps[:2]:
+            p.grad = (torch.randn(p.shape, generator=gen) * 1e-3).to(cuda)
+        ps[2].grad = None
+        ps[2].grad = bad if bad is not None else (torch.randn(8192, generator=gen) * 1e-3).to(cuda)
+
+    for round_ in range(2):
+        before = snapshot()
+        set_grads(flat[1:8193])                       # 4 bytes past a 16-byte boundary
+        with pytest.raises(AssertionError, match="16-byte aligned"):
+            opt.step()
+        torch.cuda.synchronize()
+        assert unchanged(before, snapshot()), round_
+        assert all(float(opt.state[p]["step"]) == round_ for p in ps if opt.state.get(p))
+        set_grads(None)                               # a good step: the next round starts from a kept plan
+        opt.step()
+        assert [float(opt.state[p]["step"]) for p in ps] == [round_ + 1.0] * 3
+    before = snapshot()
+    ps[0].grad = None
+    ps[0].grad = torch.zeros(100, 64, device=cuda).t()     # not contiguous
+    with pytest.raises(AssertionError, match="contiguous"):
+        opt.step()
+    assert unchanged(before, snapshot())
