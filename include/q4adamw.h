@@ -34,7 +34,9 @@ extern "C" {
  * The reference dispatches on the parameter's type over double, float and half
  * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, optim/cuda_adamw_kernels.cu:443) and takes the
  * gradient to have the same type; float and half are here, bfloat16 is added, and the
- * arithmetic is fp32 whatever the storage type. */
+ * arithmetic is fp32 whatever the storage type.  double is not taken: there is no tag for
+ * it and any other tag is refused with Q4ADAMW_ERR_ARG (a double tensor's optimizer state
+ * in 4 bits has no use; callers keep fp32 master parameters instead). */
 #define Q4ADAMW_FP32 0
 #define Q4ADAMW_BF16 1
 #define Q4ADAMW_FP16 2

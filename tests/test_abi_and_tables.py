@@ -32,6 +32,25 @@ def test_library_exports_every_declared_symbol(lib):
     assert lib.q4adamw_last_error() is not None
 
 
+def test_probe_library_exports_every_declared_symbol():
+    """libq4probe.so (the bench's memory-system probes) against include/q4probe.h; its
+    argument checks answer before any GPU call"""
+    from quantfour_adamw_cuda_amd import build
+    header = open(os.path.join(ROOT, "include", "q4probe.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(q4probe_\w+)\s*\(", header))
+    assert declared == {"q4probe_copy", "q4probe_read", "q4probe_step_streams"}
+    P = ctypes.CDLL(build.PROBE_LIB)
+    for name in declared:
+        assert hasattr(P, name), name
+    vp, u64 = ctypes.c_void_p, ctypes.c_uint64
+    P.q4probe_copy.argtypes = [vp, vp, u64, vp]
+    P.q4probe_step_streams.argtypes = [vp, vp, vp, vp, vp, vp, u64, ctypes.c_int, ctypes.c_int, vp]
+    assert P.q4probe_copy(None, None, 16, None) == -1
+    assert P.q4probe_copy(16, 32, 8, None) == -1                 # bytes not a multiple of 16
+    assert P.q4probe_step_streams(16, 16, 4, 4, 4, 4, 2048, 0, 7, None) == -1
+
+
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(_lib.Q4Tensor) == 56 and ctypes.sizeof(_lib.Q4SmallTensor) == 40
     assert _lib.Q4Tensor.numel.offset == 48 and _lib.Q4SmallTensor.numel.offset == 32
@@ -373,3 +392,30 @@ def test_tables_exhaustively_on_the_host(tmp_path):
     out = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=600)
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout
     assert "0 wrong" in out.stdout
+
+
+def test_device_code_holds_no_packed_fp32_instructions(tmp_path):
+    """The build passes -packed-fp32-ops as a target feature.  hipcc's host pass does not
+    know it (and says so); the gfx950 pass obeys it: a kernel that the compiler would
+    otherwise turn into v_pk_fma_f32 compiles without packed fp32 instructions under the
+    build's flags, and with them when the feature flag is left out."""
+    import subprocess
+    from quantfour_adamw_cuda_amd import build
+    src = tmp_path / "pk.hip"
+    src.write_text("#include <hip/hip_runtime.h>\n"
+                   "__global__ void k(float2 *a, const float2 *b, const float2 *c) {\n"
+                   "  int i = threadIdx.x; float2 x = a[i], y = b[i], z = c[i];\n"
+                   "  x.x = x.x * y.x + z.x; x.y = x.y * y.y + z.y; a[i] = x; }\n")
+    flags = [f for f in build.HIPCC_FLAGS if f not in ("-shared", "-fPIC", "-ffp-contract=off")]
+    feature = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+    assert all(f in flags for f in feature)
+    bare = [f for f in flags if f not in feature]
+
+    def packed(fl, name):
+        out = tmp_path / name
+        subprocess.run([build.hipcc_path()] + fl + ["--cuda-device-only", "-S", "-o", str(out), str(src)],
+                       check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+        return sum(1 for ln in out.read_text().splitlines() if ln.strip().startswith(("v_pk_fma_f32", "v_pk_mul_f32", "v_pk_add_f32")))
+
+    assert packed(bare, "bare.s") > 0, "the probe kernel no longer provokes packed instructions: pick another"
+    assert packed(flags, "flagged.s") == 0

@@ -304,3 +304,15 @@ def test_functional_wrappers_validate():
                       torch.zeros(3), torch.zeros(3), 0.9, 0.999, 1e-3, 0.01, 1e-8, 1)
     q4.fused_4bit_multi([], [], [], [], [], [], 0.9, 0.999, 1e-3, 0.01, 1e-8, 1)       # nothing to do
     q4.fused_single_tensor_multi([], [], [], [], 0.9, 0.999, 1e-3, 0.01, 1e-8, 1)
+
+
+def test_fp64_parameters_and_gradients_are_refused():
+    """The reference's launchers dispatch on double as well (AT_DISPATCH_FLOATING_TYPES_AND_HALF,
+    optim/cuda_adamw_kernels.cu:147, :443); this build's kernels take fp32, bf16 and fp16
+    storage (the arithmetic is fp32 either way) and say so before anything is launched."""
+    from quantfour_adamw_cuda_amd import quantfour_hip as qh
+    with pytest.raises(TypeError, match="param must be float32, bfloat16 or float16, got torch.float64"):
+        qh._tag(torch.zeros(4, dtype=torch.float64), "param")
+    with pytest.raises(TypeError, match="grad must be float32, bfloat16 or float16, got torch.float64"):
+        qh._tag(torch.zeros(4, dtype=torch.float64), "grad")
+    assert [qh._tag(torch.zeros(1, dtype=d), "param") for d in (torch.float32, torch.bfloat16, torch.float16)] == [0, 1, 2]
