@@ -309,7 +309,7 @@ def load_probe():
     vp, u64, i = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int
     L.q4probe_copy.argtypes = [vp, vp, u64, vp]
     L.q4probe_read.argtypes = [vp, u64, vp, vp]
-    L.q4probe_step_streams.argtypes = [vp, vp, vp, vp, vp, vp, u64, i, i, vp]
+    L.q4probe_step_streams.argtypes = [vp, vp, vp, vp, vp, vp, u64, i, i, i, vp]
     for f in (L.q4probe_copy, L.q4probe_read, L.q4probe_step_streams):
         f.restype = i
     return L
@@ -351,10 +351,16 @@ def measure_ceiling(torch, device, reps=10):
     out["copy"] = 8.0 * n / t / 1e9
     t = timed(lambda: L.q4probe_read(a.data_ptr(), 4 * n, sink.data_ptr(), stream))
     out["read"] = 4.0 * n / t / 1e9
+    def streams(p_s, g_s, which):
+        return timed(lambda: L.q4probe_step_streams(a.data_ptr(), b.data_ptr(), m.data_ptr(), v.data_ptr(),
+                                                    sm.data_ptr(), sv.data_ptr(), n, tag[p_s], tag[g_s], which, stream))
+
     for p_s, g_s in (("float32", "bfloat16"), ("float32", "float32"), ("bfloat16", "bfloat16"), ("bfloat16", "float32")):
-        t = timed(lambda: L.q4probe_step_streams(a.data_ptr(), b.data_ptr(), m.data_ptr(), v.data_ptr(),
-                                                 sm.data_ptr(), sv.data_ptr(), n, tag[p_s], tag[g_s], stream))
-        out[f"step_streams_{p_s}_{g_s}"] = n * bytes_per_param(p_s, g_s) / t / 1e9
+        out[f"step_streams_{p_s}_{g_s}"] = n * bytes_per_param(p_s, g_s) / streams(p_s, g_s, 3) / 1e9
+    # the headline's dtypes without the small streams: parameters read and written plus the
+    # gradients read (10 bytes per element), and with the scales but not the codes (10.125)
+    out["step_streams_float32_bfloat16_without_codes_and_scales"] = n * 10.0 / streams("float32", "bfloat16", 0) / 1e9
+    out["step_streams_float32_bfloat16_without_codes"] = n * 10.125 / streams("float32", "bfloat16", 2) / 1e9
     return out
 
 

@@ -32,11 +32,14 @@ int q4probe_read(const void *src, uint64_t bytes, void *sink4, void *stream);
  * cache policy, without its arithmetic: reads p, g, both moments' packed codes and block
  * scales, writes p, the codes and the scales.  Arguments as q4adamw_fused_4bit; only whole
  * workgroups' worth of elements (1024, or 2048 when p and g are both 16-bit types) are
- * touched, so pass a multiple of 2048.
+ * touched, so pass a multiple of 2048.  streams: Q4PROBE_CODES | Q4PROBE_SCALES for all seven;
+ * without a bit the two moments' streams of that kind are neither read nor written.
  */
+#define Q4PROBE_CODES 1
+#define Q4PROBE_SCALES 2
 int q4probe_step_streams(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_avg_sq,
                          float *exp_avg_scale, float *exp_avg_sq_scale, uint64_t numel, int p_dtype,
-                         int g_dtype, void *stream);
+                         int g_dtype, int streams, void *stream);
 
 #ifdef __cplusplus
 }

@@ -8,7 +8,8 @@
 //                 p and of g (16 bytes of the wider one), 2 or 4 bytes of each moment's codes,
 //                 per 128 elements one fp32 scale of each moment; p, the codes and the scales
 //                 are written back.  fp32 p / bf16 g: 7.0625 bytes read and 5.0625 written per
-//                 element, the step's own ratio.
+//                 element, the step's own ratio.  The code and scale streams can be left out,
+//                 which shows what these small streams cost the large ones.
 //
 // All three use the step's launch shape (one tile per wave64, four waves per workgroup,
 // workgroups dealt to the XCDs so that each walks a contiguous eighth), its buffer
@@ -58,7 +59,9 @@ __global__ __launch_bounds__(kThreads) void probe_move_kernel(const ProbeArgs a)
 }
 
 // PB, GB: bytes per element of p and g (4 or 2).  Full tiles only (the host rounds down).
-template <int PB, int GB>
+// CODES, SCALES: with the moments' code streams / scale streams (without them the probe shows
+// what those small streams cost the large ones).
+template <int PB, int GB, bool CODES, bool SCALES>
 __global__ __launch_bounds__(kThreads) void probe_step_streams_kernel(const ProbeArgs a) {
   constexpr int N = (PB == 2 && GB == 2) ? 8 : 4;          // elements per lane, as Geometry<PT, GT>
   constexpr int kTile = 64 * N;
@@ -91,16 +94,20 @@ __global__ __launch_bounds__(kThreads) void probe_step_streams_kernel(const Prob
     const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(tile_rsrc(g_tile), e0 * GB, 0, kNt);
     gw.x = t.x; gw.y = t.y;
   }
-  uint32_t mw, vw;
-  if (N == 4) {
-    mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), code_off, 0, kNt);
-    vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), code_off, 0, kNt);
-  } else {
-    mw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(m_tile), code_off, 0, kNt);
-    vw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_tile), code_off, 0, kNt);
+  uint32_t mw = 0u, vw = 0u, s_m = 0u, s_v = 0u;
+  if (CODES) {
+    if (N == 4) {
+      mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), code_off, 0, kNt);
+      vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), code_off, 0, kNt);
+    } else {
+      mw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(m_tile), code_off, 0, kNt);
+      vw = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_tile), code_off, 0, kNt);
+    }
   }
-  const uint32_t s_m = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0);
-  const uint32_t s_v = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0);
+  if (SCALES) {
+    s_m = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0);
+    s_v = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0);
+  }
 
   // every stored value depends on every loaded one, at the price of a few integer operations
   const uint32_t mix = gw.x ^ gw.y ^ gw.z ^ gw.w ^ mw ^ vw ^ s_m ^ s_v;
@@ -111,14 +118,16 @@ __global__ __launch_bounds__(kThreads) void probe_step_streams_kernel(const Prob
     const u32x2 t = {pw.x, pw.y};
     __builtin_amdgcn_raw_buffer_store_b64(t, tile_rsrc(p_tile), e0 * PB, 0, kNt);
   }
-  if (N == 4) {
-    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(mw ^ pw.x), tile_rsrc(m_tile), code_off, 0, kNt);
-    __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(vw ^ pw.y), tile_rsrc(v_tile), code_off, 0, kNt);
-  } else {
-    __builtin_amdgcn_raw_buffer_store_b32(mw ^ pw.x, tile_rsrc(m_tile), code_off, 0, kNt);
-    __builtin_amdgcn_raw_buffer_store_b32(vw ^ pw.y, tile_rsrc(v_tile), code_off, 0, kNt);
+  if (CODES) {
+    if (N == 4) {
+      __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(mw ^ pw.x), tile_rsrc(m_tile), code_off, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b16((uint16_t)(vw ^ pw.y), tile_rsrc(v_tile), code_off, 0, kNt);
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b32(mw ^ pw.x, tile_rsrc(m_tile), code_off, 0, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(vw ^ pw.y, tile_rsrc(v_tile), code_off, 0, kNt);
+    }
   }
-  if ((lane & (kLanesPerBlock - 1)) == 0) {
+  if (SCALES && (lane & (kLanesPerBlock - 1)) == 0) {
     __builtin_amdgcn_raw_buffer_store_b32(s_m ^ pw.x, tile_rsrc(sm_tile), blk * 4u, 0, 0);
     __builtin_amdgcn_raw_buffer_store_b32(s_v ^ pw.y, tile_rsrc(sv_tile), blk * 4u, 0, 0);
   }
@@ -131,6 +140,14 @@ static int probe_launch(ProbeArgs &a, uint64_t chunks, void (*kernel)(const Prob
   a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
   hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, static_cast<hipStream_t>(stream), a);
   return (int)hipGetLastError();
+}
+
+typedef void (*ProbeKernel)(const ProbeArgs);
+
+template <bool CODES, bool SCALES>
+static ProbeKernel pick_streams(bool p16, bool g16) {
+  if (p16) return g16 ? probe_step_streams_kernel<2, 2, CODES, SCALES> : probe_step_streams_kernel<2, 4, CODES, SCALES>;
+  return g16 ? probe_step_streams_kernel<4, 2, CODES, SCALES> : probe_step_streams_kernel<4, 4, CODES, SCALES>;
 }
 
 }  // namespace q4
@@ -160,7 +177,8 @@ int q4probe_read(const void *src, uint64_t bytes, void *sink4, void *stream) {
 }
 
 int q4probe_step_streams(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_avg_sq, float *exp_avg_scale,
-                         float *exp_avg_sq_scale, uint64_t numel, int p_dtype, int g_dtype, void *stream) {
+                         float *exp_avg_sq_scale, uint64_t numel, int p_dtype, int g_dtype, int streams,
+                         void *stream) {
   if (!p || !g || !exp_avg || !exp_avg_sq || !exp_avg_scale || !exp_avg_sq_scale) return Q4PROBE_ERR_ARG;
   if (p_dtype < 0 || p_dtype > 2 || g_dtype < 0 || g_dtype > 2) return Q4PROBE_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(g)) & 15u) return Q4PROBE_ERR_ARG;
@@ -177,8 +195,10 @@ int q4probe_step_streams(void *p, const void *g, uint8_t *exp_avg, uint8_t *exp_
   a.sm = exp_avg_scale;
   a.sv = exp_avg_sq_scale;
   a.units = numel;
-  void (*kernel)(const ProbeArgs) = p16 ? (g16 ? probe_step_streams_kernel<2, 2> : probe_step_streams_kernel<2, 4>)
-                                        : (g16 ? probe_step_streams_kernel<4, 2> : probe_step_streams_kernel<4, 4>);
+  if (streams < 0 || streams > 3) return Q4PROBE_ERR_ARG;
+  const bool codes = streams & Q4PROBE_CODES, scales = streams & Q4PROBE_SCALES;
+  const ProbeKernel kernel = codes ? (scales ? pick_streams<true, true>(p16, g16) : pick_streams<true, false>(p16, g16))
+                                          : (scales ? pick_streams<false, true>(p16, g16) : pick_streams<false, false>(p16, g16));
   return probe_launch(a, numel / chunk_elems, kernel, stream);   // whole chunks only
 }
 

@@ -14,8 +14,8 @@ machine, from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd -`
     rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o write -- \\
         python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy
     python3 -m quantfour_adamw_cuda_amd.hbm_traffic --workload llama3-8b --steps 4 \\
-        --fetch-csv out/pmc_fetch/*/fetch_counter_collection.csv \\
-        --write-csv out/pmc_write/*/write_counter_collection.csv \\
+        --fetch-csv 'out/pmc_fetch/**/*counter_collection.csv' \\
+        --write-csv 'out/pmc_write/**/*counter_collection.csv' \\
         --out profiles/hbm_traffic.json
 
 (add the bench's --workload / --variance-scale / --round-type options to all three).  Both
@@ -72,7 +72,7 @@ def _sum_counter(csv_paths, counter):
     """{kernel name: [sum of the counter over its dispatches, dispatches]} of one run"""
     out = {}
     for pattern in csv_paths:
-        for path in glob.glob(pattern):
+        for path in glob.glob(pattern, recursive=True):
             with open(path, newline="") as f:
                 for row in csv.DictReader(f):
                     if row["Counter_Name"] != counter:

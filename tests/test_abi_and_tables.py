@@ -45,10 +45,11 @@ def test_probe_library_exports_every_declared_symbol():
         assert hasattr(P, name), name
     vp, u64 = ctypes.c_void_p, ctypes.c_uint64
     P.q4probe_copy.argtypes = [vp, vp, u64, vp]
-    P.q4probe_step_streams.argtypes = [vp, vp, vp, vp, vp, vp, u64, ctypes.c_int, ctypes.c_int, vp]
+    P.q4probe_step_streams.argtypes = [vp, vp, vp, vp, vp, vp, u64, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
     assert P.q4probe_copy(None, None, 16, None) == -1
     assert P.q4probe_copy(16, 32, 8, None) == -1                 # bytes not a multiple of 16
-    assert P.q4probe_step_streams(16, 16, 4, 4, 4, 4, 2048, 0, 7, None) == -1
+    assert P.q4probe_step_streams(16, 16, 4, 4, 4, 4, 2048, 0, 7, 3, None) == -1
+    assert P.q4probe_step_streams(16, 16, 4, 4, 4, 4, 2048, 0, 1, 4, None) == -1        # streams mask
 
 
 def test_struct_layouts_match_header():

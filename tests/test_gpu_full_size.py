@@ -11,7 +11,7 @@ import torch.nn as nn
 from oracle import q4_oracle as oc
 from oracle import q4_oracle_torch as ot
 from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
-from tests.q4_testlib import HP, bits, strict_param_metrics, to_np
+from tests.q4_testlib import BASELINE_ATOL, HP, bits, strict_param_metrics, to_np
 
 pytestmark = pytest.mark.gpu
 KW = dict(lr=HP["lr"], betas=(HP["beta1"], HP["beta2"]), eps=HP["eps"], weight_decay=HP["weight_decay"])
@@ -102,6 +102,7 @@ def _check_tensor(p, st, before, g, step):
         # least as large as the step it took; the rest is reported in the session summary
         strict = strict_param_metrics(p.detach(), rp, p0)
         assert strict["dom"] <= 1e-6, f"params, shape {tuple(p.shape)}: {strict}"
+        assert strict["atol"] <= BASELINE_ATOL, f"params, shape {tuple(p.shape)}: {strict}"   # with rtol 1e-6
 
 
 def _run_config(shapes, p_dtype, cuda, steps, label):

@@ -8,7 +8,8 @@ import torch
 import quantfour_adamw_cuda_amd as q4
 from oracle import q4_oracle as oc
 from tests.q4_testlib import (HP, HP_DRIVER, DeviceTensor, OracleTensor, assert_state_equal, bits,
-                              grads_config1, grads_config3, grads_student_t, p_close, to_np)
+                              grads_config1, grads_config3, grads_student_t, p_close, to_np,
+                              BASELINE_ATOL, STRICT_LOG, strict_atol_since)
 
 pytestmark = pytest.mark.gpu
 
@@ -39,8 +40,10 @@ def test_config1_single_tensor(cuda):
     gen = torch.Generator().manual_seed(0)
     n = 4096 * 4096
     p0 = torch.randn(n, generator=gen) * 0.02
+    mark = len(STRICT_LOG)
     worst = run_steps(p0, lambda t: grads_config1(gen, n), 10, cuda, what="config1")
     say(f"config1 worst relative parameter error {worst:.3e}")
+    assert strict_atol_since(mark) <= BASELINE_ATOL        # |dev - ref| <= 5e-10 + 1e-6 |ref| every step
 
 
 @pytest.mark.parametrize("n", [1, 2, 127, 128, 129, 511, 512, 513, 4095, 4097, 1000003, 3 * 1000003])
