@@ -44,22 +44,25 @@ extern "C" {
 #define Q4ADAMW_BLOCK 128 /* elements per quantization block (one scale each) */
 
 #define Q4ADAMW_ERR_ARG (-1)       /* null pointer, negative size, bad dtype tag */
-#define Q4ADAMW_ERR_ALIGN (-2)     /* pointer not aligned for vector access      */
+#define Q4ADAMW_ERR_ALIGN (-2)     /* pointer not aligned as its buffer requires */
 #define Q4ADAMW_ERR_HYPER (-3)     /* hyper-parameter outside its domain         */
 #define Q4ADAMW_ERR_TOO_LARGE (-4) /* launch would exceed the grid limit         */
 
 /*
  * One quantized tensor.  Field order follows the tensor arguments of
  * fused_4bit (optim/cuda_fused_interface.cc:19-21).
- *   p             numel elements, fp32, bf16 or fp16, 16-byte aligned
- *   g             numel elements, fp32, bf16 or fp16, 16-byte aligned (8 bytes suffice for a
- *                 16-bit gradient of an fp32 parameter)
+ *   p             numel elements, fp32, bf16 or fp16
+ *   g             numel elements, fp32, bf16 or fp16
  *   exp_avg       (numel+1)/2 bytes; byte i = code(2i) | code(2i+1) << 4
  *   exp_avg_sq    same layout
  *   exp_avg_scale ceil(numel/128) fp32 block scales of exp_avg
  *   exp_avg_sq_scale  same for exp_avg_sq
- * Code and scale buffers must be 4-byte aligned (2 bytes suffice for the codes of an
- * fp32 parameter).
+ * p and g need the alignment of their element type only, like the reference's element-wise
+ * accesses (optim/cuda_adamw_kernels.cu:334-351), so views at any offset into a flat buffer
+ * are taken.  16-byte aligned addresses are the fast case: a parameter tensor that is not
+ * takes about a third longer (its stores no longer cover whole lines), a gradient tensor
+ * costs nothing extra.  Code and scale buffers must be 4-byte aligned (2 bytes suffice for
+ * the codes of an fp32 parameter).
  */
 typedef struct q4adamw_tensor {
   void *p;
@@ -118,7 +121,7 @@ typedef struct q4adamw_grad_options {
   const void *step_consts;
 } q4adamw_grad_options;
 
-/* One gradient tensor for q4adamw_grad_norm: numel elements, 16-byte aligned. */
+/* One gradient tensor for q4adamw_grad_norm: numel elements, aligned to the element type. */
 typedef struct q4adamw_grad {
   const void *g;
   int64_t numel;
@@ -179,8 +182,9 @@ uint32_t q4adamw_sr_tensor_salt(uint64_t seed, float step, uint32_t tensor_salt)
  * keeps its per-128 block scales.  row_max/col_max (rows and cols floats) are
  * updated by the call; row_max_next/col_max_next are state-owned scratch of the same
  * sizes that must hold zeros on entry and holds zeros again afterwards.
- * rows x cols, row-major, cols a multiple of 8 and at least 16; p, g, col_max and
- * col_max_next 16-byte aligned, the rest 4-byte aligned.
+ * rows x cols, row-major, cols a multiple of 8 and at least 16; p and g aligned to their
+ * element type (see q4adamw_tensor), col_max and col_max_next 16-byte aligned, the rest
+ * 4-byte aligned.
  *
  * Tensors of three or four dimensions (lead_dims = 2 or 3): cols is the last dimension,
  * lead_shape the others, rows their product.  Every leading dimension has its own

@@ -363,7 +363,12 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   const bool p_half = p_dtype != Q4ADAMW_FP32, g_half = g_dtype != Q4ADAMW_FP32;
   const bool wide = p_half && g_half;   // 8 elements per lane
   const int64_t chunk_elems = wide ? Geometry<1, 1>::kChunk : Geometry<0, 0>::kChunk;
-  const uintptr_t p_align = 16, g_align = g_half ? (p_half ? 16 : 8) : 16;
+  // Parameters and gradients need the alignment of their element type only: the 16-byte
+  // accesses of the kernels are legal at any such address (the memory pipeline runs in its
+  // unaligned mode under ROCm; the compiler relies on the same for amdhsa targets).  A view at
+  // an odd offset into a flat buffer costs nothing on the gradient side and about a third
+  // more time on the parameter side (partial lines written).
+  const uintptr_t p_align = p_half ? 2 : 4, g_align = g_half ? 2 : 4;
   const uintptr_t code_align = wide ? 4 : 2;
   // validate everything before the first launch
   for (int i = 0; i < count; ++i) {
@@ -373,7 +378,7 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.exp_avg_sq_scale)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
     if (!aligned(t.p, p_align) || !aligned(t.g, g_align))
-      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be 16-byte aligned");
+      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be aligned to their element size");
     if (!aligned(t.exp_avg, code_align) || !aligned(t.exp_avg_sq, code_align) ||
         !aligned(t.exp_avg_scale, 4) || !aligned(t.exp_avg_sq_scale, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "code and scale buffers must be 4-byte aligned");
@@ -441,8 +446,8 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.row_max || !t.col_max ||
         !t.row_max_next || !t.col_max_next)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
-    if (!aligned(t.p, 16) || !aligned(t.g, 16))
-      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be 16-byte aligned");
+    if (!aligned(t.p, p_dtype != Q4ADAMW_FP32 ? 2 : 4) || !aligned(t.g, g_dtype != Q4ADAMW_FP32 ? 2 : 4))
+      return fail(Q4ADAMW_ERR_ALIGN, "param and grad must be aligned to their element size");
     if (!aligned(t.exp_avg, 4) || !aligned(t.exp_avg_sq, 4) || !aligned(t.exp_avg_scale, 4) ||
         !aligned(t.row_max, 4) || !aligned(t.row_max_next, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "code, scale and row buffers must be 4-byte aligned");
@@ -616,7 +621,8 @@ static int grad_norm_impl(const q4adamw_grad *grads, int count, int g_dtype, flo
     if (grads[i].numel < 0) return fail(Q4ADAMW_ERR_ARG, "negative numel");
     if (grads[i].numel == 0) continue;
     if (!grads[i].g) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
-    if (!aligned(grads[i].g, 16)) return fail(Q4ADAMW_ERR_ALIGN, "gradients must be 16-byte aligned");
+    if (!aligned(grads[i].g, g_dtype != Q4ADAMW_FP32 ? 2 : 4))
+      return fail(Q4ADAMW_ERR_ALIGN, "gradients must be aligned to their element size");
     if (((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
@@ -893,6 +899,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1013; }
+int q4adamw_version(void) { return 1014; }
 
 }  // extern "C"

@@ -50,7 +50,7 @@ def enable_param_quantization(p, threshold) -> bool:
 class _Bucket:
     """One launch of a step: the tensors of one (kind, device, dtypes, step) and their
     descriptor array."""
-    __slots__ = ("kind", "device", "idx", "arr", "p_tag", "g_tag", "salts", "g_dtypes", "g_mask", "g_column")
+    __slots__ = ("kind", "device", "idx", "arr", "p_tag", "g_tag", "salts", "g_dtypes", "g_column")
 
 
 class _Plan:
@@ -580,7 +580,6 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             b.kind, b.device, b.idx, b.arr, b.p_tag, b.g_tag = quantized, device, idx, arr, p_tag, g_tag
             b.salts = extra[0] if extra else None
             b.g_dtypes = [g_dtype] * len(idx)
-            b.g_mask = 15 if quantized in ("rank1", "rank1_sr") else _q.grad_alignment(p_dtype, g_dtype, bool(quantized)) - 1
             # the gradient pointers inside the descriptor array: the second 8-byte field of
             # every descriptor type (include/q4adamw.h)
             b.g_column = np.frombuffer(arr, dtype=np.uint64).reshape(len(idx), -1)[:, 1]
@@ -642,8 +641,6 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                              or not all(map(methodcaller("is_contiguous"), gs))):
                 return False
             ptrs = np.fromiter(map(methodcaller("data_ptr"), gs), dtype=np.uint64, count=len(gs))
-            if np.bitwise_and(ptrs, np.uint64(b.g_mask)).any():
-                return False
             if not plan.capturable and len({steps_now[i] for i in b.idx}) != 1:
                 return False
             pointers.append(ptrs)
@@ -792,8 +789,6 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
                 assert g.device == device, "grad must be on the param's device"
                 assert g.is_contiguous(), "grad must be contiguous"
                 assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
-                assert g.data_ptr() % (16 if rank1 else _q.grad_alignment(p.dtype, g.dtype, bool(quantized))) == 0, \
-                    "grad must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
                 arr[i].g = g.data_ptr()
         return cached
 

@@ -36,28 +36,8 @@ def _check_common(p, g):
     assert g.numel() == p.numel(), f"grad numel {g.numel()} != param numel {p.numel()}"
 
 
-def grad_alignment(p_dtype, g_dtype, quantized=True):
-    """Bytes a gradient's address must be a multiple of: the fused kernels read 16 bytes per
-    lane (8 of a 16-bit gradient next to fp32 parameters), the non-quantized one element by
-    element."""
-    g16 = g_dtype != torch.float32
-    if not quantized:
-        return 2 if g16 else 4
-    return 8 if (g16 and p_dtype == torch.float32) else 16
-
-
-def _check_aligned(p, g, quantized=True):
-    # refused by the library as well (Q4ADAMW_ERR_ALIGN); checked here so that a step refuses
-    # before its first launch
-    assert p.data_ptr() % (16 if quantized else p.element_size()) == 0, \
-        "param must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
-    assert g.data_ptr() % grad_alignment(p.dtype, g.dtype, quantized) == 0, \
-        "grad must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
-
-
 def check_quantized(p, g, exp, sq, exp_scale, sq_scale):
     _check_common(p, g)
-    _check_aligned(p, g)
     nbytes, nblk = state_sizes(p.numel())
     assert exp.dtype == torch.uint8 and sq.dtype == torch.uint8, "moments must be packed uint8"
     assert exp.numel() == nbytes, f"exp_avg numel {exp.numel()} != packed size {nbytes}"
@@ -337,8 +317,6 @@ def rank1_row_scale(lead_maxes, lead_shape):
 
 def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next, lead=None):
     _check_common(p, g)
-    assert p.data_ptr() % 16 == 0 and g.data_ptr() % 16 == 0, \
-        "param and grad must be 16-byte aligned (a view at an odd offset into a flat buffer is not)"
     assert rank1_eligible(p), "rank-1 scaling needs 2 to 4 dimensions, the last a multiple of 8 and at least 16"
     cols = p.shape[-1]
     rows = p.numel() // cols

@@ -299,7 +299,7 @@ static void tables_and_errors(void) {
   uint8_t *c = (uint8_t *)d + 32768;
   float *s = d + 12000;
   /* every refusal must come before anything is launched and must leave a message */
-  int rc = q4adamw_fused_4bit(d + 1, d + 2048, c, c + 2048, s, s + 64, 1000, 0, 0, B1, B2, LR, WD, EPS, 1.0f, NULL);
+  int rc = q4adamw_fused_4bit((float *)((char *)d + 2), d + 2048, c, c + 2048, s, s + 64, 1000, 0, 0, B1, B2, LR, WD, EPS, 1.0f, NULL);
   CHECK(rc == Q4ADAMW_ERR_ALIGN && strlen(q4adamw_last_error()) > 0, "misaligned p: rc %d", rc);
   rc = q4adamw_fused_4bit(d, d + 2048, c, c + 2048, s, s + 64, 1000, 7, 0, B1, B2, LR, WD, EPS, 1.0f, NULL);
   CHECK(rc == Q4ADAMW_ERR_ARG && strlen(q4adamw_last_error()) > 0, "bad dtype tag: rc %d", rc);

@@ -88,7 +88,7 @@ static void refusals(void) {
   float *scales = buf + 12000;
   const int F = Q4ADAMW_FP32, H = Q4ADAMW_BF16;
   EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, 0, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), 0);
-  EXPECT(q4adamw_fused_4bit(buf + 1, buf + 2048, codes, codes + 2048, scales, scales + 64, 1000, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ALIGN);
+  EXPECT(q4adamw_fused_4bit((float *)((char *)buf + 2), buf + 2048, codes, codes + 2048, scales, scales + 64, 1000, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ALIGN);
   EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes + 1, codes + 2048, scales, scales + 64, 1000, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ALIGN);
   EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes + 2, codes + 2048, scales, scales + 64, 1000, H, H, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ALIGN);
   EXPECT(q4adamw_fused_4bit(buf, NULL, codes, codes + 2048, scales, scales + 64, 1000, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_ARG);
@@ -171,7 +171,7 @@ static void refusals(void) {
   EXPECT(q4adamw_grad_norm(gr, 1, F, 1.0f, NULL, 1.0f, NULL, Q4ADAMW_NORM_WORKSPACE_BYTES, buf, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_grad_norm(gr, 1, F, 1.0f, NULL, 1.0f, buf + 1024, 100, buf, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_grad_norm(gr, 1, F, 1.0f, NULL, 1.0f, (char *)(buf + 1024) + 4, Q4ADAMW_NORM_WORKSPACE_BYTES, buf, NULL), Q4ADAMW_ERR_ALIGN);
-  gr[0].g = (char *)buf + 4;
+  gr[0].g = (char *)buf + 2;
   EXPECT(q4adamw_grad_norm(gr, 1, F, 1.0f, NULL, 1.0f, buf + 1024, Q4ADAMW_NORM_WORKSPACE_BYTES, buf, NULL), Q4ADAMW_ERR_ALIGN);
   gr[0].g = NULL;
   EXPECT(q4adamw_grad_norm(gr, 1, H, 1.0f, NULL, 1.0f, buf + 1024, Q4ADAMW_NORM_WORKSPACE_BYTES, buf, NULL), Q4ADAMW_ERR_ARG);

@@ -116,9 +116,13 @@ def test_argument_errors_need_no_gpu(lib):
     assert rc == -3
     rc = lib.q4adamw_fused_4bit(z, z, z, z, z, z, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 0.0, z)
     assert rc == -3                                           # step counts from 1
-    a = ctypes.c_void_p(0x1004)
-    rc = lib.q4adamw_fused_4bit(a, a, a, a, a, a, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
-    assert rc == -2 and b"aligned" in lib.q4adamw_last_error()
+    a, odd = ctypes.c_void_p(0x1004), ctypes.c_void_p(0x1002)   # fp32 tensors two bytes off
+    rc = lib.q4adamw_fused_4bit(odd, a, a, a, a, a, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -2 and b"element size" in lib.q4adamw_last_error()
+    rc = lib.q4adamw_fused_4bit(a, odd, a, a, a, a, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -2 and b"element size" in lib.q4adamw_last_error()
+    rc = lib.q4adamw_fused_4bit(a, a, a, a, odd, a, 128, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
+    assert rc == -2 and b"4-byte aligned" in lib.q4adamw_last_error()
     rc = lib.q4adamw_fused_single_tensor(z, z, z, z, 16, 0, 0, 0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0, z)
     assert rc == -1
     assert lib.q4adamw_mtable_entry(4096, (ctypes.c_uint32 * 2)()) == -1

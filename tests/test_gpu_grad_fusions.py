@@ -207,7 +207,13 @@ def test_grad_norm_closed_forms_and_determinism(cuda):
     assert torch.equal(a, b)
     want = torch.linalg.vector_norm(torch.cat(g).double()).float()
     assert abs(float(a[0]) - float(want)) <= float(np.spacing(_f32(float(want))))
-    # non-finite gradients: inf clips everything to zero, NaN poisons the coefficient
+    # views at odd element offsets into a flat buffer give the bits of tensors of their own
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        flat = torch.randn((1 << 20) + 77, generator=gen, device=cuda).to(dt)
+        views = [flat[1:300001], flat[300003:]]
+        assert any(v.data_ptr() % 16 for v in views)
+        a = q.grad_norm(views, max_norm=1.0).clone()
+        assert torch.equal(a, q.grad_norm([v.clone() for v in views], max_norm=1.0)) and float(a[0]) > 0
     bad = torch.tensor([1.0, float("inf")], device=cuda)
     out = q.grad_norm([bad], max_norm=1.0).cpu().numpy()
     assert np.isinf(out[0]) and out[1] == 0.0
@@ -231,6 +237,7 @@ def test_grad_norm_argument_errors(cuda):
     assert call(arr, 1, 7, ws.data_ptr(), 16384, out.data_ptr()) == -1
     assert call(arr, -1, 0, ws.data_ptr(), 16384, out.data_ptr()) == -1
     off = q.make_grad_table([g[1:]])
+    off[0].g += 2                                              # half an element
     assert call(off, 1, 0, ws.data_ptr(), 16384, out.data_ptr()) == -2
 
 

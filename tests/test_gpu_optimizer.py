@@ -398,14 +398,14 @@ def test_kept_plan_follows_every_change_of_what_it_rests_on(cuda):
 
 def test_a_refused_gradient_leaves_everything_as_it_was(cuda):
     """Everything is validated before the first launch and before any step counter moves: a
-    gradient the kernels cannot take (a view at a 4-byte offset into a flat buffer, a
-    transposed view) in the LAST bucket of the LAST group leaves parameters, state and
-    counters of every group untouched, on the first step and on a step that had a plan."""
+    gradient the kernels cannot take (every other element of a buffer, a transposed view) in
+    the LAST bucket of the LAST group leaves parameters, state and counters of every group
+    untouched, on the first step and on a step that had a plan."""
     gen = torch.Generator().manual_seed(5)
     shapes = [(64, 100), (3000,), (8192,)]
     ps = [nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(cuda)) for s in shapes]
     opt = AdamWFused_QuantFour([{"params": ps[:2]}, {"params": ps[2:], "lr": 2e-3}], **KW)
-    flat = torch.zeros(8192 + 8, device=cuda)
+    flat = torch.zeros(2 * 8192, device=cuda)
 
     def snapshot():
         """parameters, and the state that exists (the first refused step creates it, all zeros)"""
@@ -426,8 +426,8 @@ def test_a_refused_gradient_leaves_everything_as_it_was(cuda):
 
     for round_ in range(2):
         before = snapshot()
-        set_grads(flat[1:8193])                       # 4 bytes past a 16-byte boundary
-        with pytest.raises(AssertionError, match="16-byte aligned"):
+        set_grads(flat[::2])                          # strided
+        with pytest.raises(AssertionError, match="contiguous"):
             opt.step()
         torch.cuda.synchronize()
         assert unchanged(before, snapshot()), round_
@@ -441,3 +441,53 @@ def test_a_refused_gradient_leaves_everything_as_it_was(cuda):
     with pytest.raises(AssertionError, match="contiguous"):
         opt.step()
     assert unchanged(before, snapshot())
+
+
+@pytest.mark.parametrize("found_inf_at", [None, 2])
+@pytest.mark.parametrize("round_type", ["real-nearest", "stochastic"])
+@pytest.mark.parametrize("variance_scale", ["group", "rank1"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_views_at_odd_offsets_into_flat_buffers(cuda, dtype, variance_scale, round_type, found_inf_at):
+    """Parameters and gradients that are views into flat buffers at odd element offsets (2 or 4
+    bytes past a 16-byte boundary, as a flat-parameter wrapper or a gradient bucket makes them
+    once one tensor has an odd size) take the same path as tensors of their own and give the
+    same bits: block-scaled and rank-1 (rows, wide, narrow and 3-D forms), nearest and
+    stochastic, with the gradient norm taken, the gradients cleared by the step, and a step
+    that an overflow flag cancels.  Elements of the buffers between the views stay as they were."""
+    shapes = [(8, 1024), (6, 520), (300, 24), (4, 6, 64), (100,), (5000,), (33, 129)]
+    gen = torch.Generator().manual_seed(123)
+    base = [(torch.randn(s, generator=gen) * 0.02).to(dtype) for s in shapes]
+    offsets, total = [], 1
+    for t in base:
+        offsets.append(total)
+        total += t.numel() + (1 if len(offsets) % 2 else 2)
+    flat_p = torch.full((total,), 7.0, dtype=dtype, device=cuda)
+    flat_g = torch.full((total,), 7.0, dtype=dtype, device=cuda)
+    pa = [nn.Parameter(flat_p[o:o + t.numel()].view(t.shape)) for o, t in zip(offsets, base)]
+    for p, t in zip(pa, base):
+        p.data.copy_(t)
+    assert any(p.data_ptr() % 16 for p in pa) and all(p.is_contiguous() for p in pa)
+    pb = [nn.Parameter(t.clone().to(cuda)) for t in base]
+    kw = dict(KW, variance_scale_type=variance_scale, round_type=round_type)
+    if round_type == "stochastic":
+        kw["seed"] = 99
+    oa, ob = AdamWFused_QuantFour(pa, **kw), AdamWFused_QuantFour(pb, **kw)
+    covered = torch.zeros(total, dtype=torch.bool, device=cuda)
+    for o, t in zip(offsets, base):
+        covered[o:o + t.numel()] = True
+    for step in range(1, 5):
+        gs = [(torch.randn(t.shape, generator=gen) * 1e-3).to(dtype) for t in base]
+        for o, p, q, g in zip(offsets, pa, pb, gs):
+            view = flat_g[o:o + g.numel()].view(g.shape)
+            view.copy_(g)
+            p.grad = view
+            q.grad = g.clone().to(cuda)
+        flag = torch.full((1,), 1.0 if step == found_inf_at else 0.0, device=cuda)
+        say(f"[flat views] {dtype} {variance_scale} {round_type} step {step} cancelled {step == found_inf_at}")
+        for o in (oa, ob):
+            o.step(grad_scale=0.5, max_grad_norm=0.01, found_inf=flag, zero_grad=True)
+        torch.cuda.synchronize()
+        assert torch.equal(oa.last_grad_norm, ob.last_grad_norm)
+        _same_everything(oa, pa, ob, pb)
+        assert all(not bool(p.grad.any()) for p in pa)                    # cleared, cancelled or not
+        assert bool((flat_p[~covered] == 7.0).all()) and bool((flat_g[~covered] == 7.0).all())

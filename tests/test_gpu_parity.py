@@ -67,6 +67,40 @@ def test_ragged_lengths_16_bit(cuda, n, dt):
     run_steps(p0, lambda t: grads_config3(gen, n), 3, cuda, g_dtype=dt, what=f"ragged {dt} n={n}")
 
 
+@pytest.mark.parametrize("offsets", [(1, 0), (0, 1), (1, 1), (3, 5), (7, 2)])
+@pytest.mark.parametrize("p_dtype,g_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                             (torch.float16, torch.float16)])
+def test_views_at_odd_element_offsets(cuda, p_dtype, g_dtype, offsets):
+    """Parameters and gradients that start 2 to 28 bytes past a 16-byte boundary (views into a
+    flat buffer): the 16-byte accesses of the full tiles and the element-wise ones of the last
+    tile give the oracle's results, and nothing outside the views is written."""
+    po, go = offsets
+    for n in (1000003, 4096 * 33):
+        gen = torch.Generator().manual_seed(n + 17 * po + go)
+        p0 = (torch.randn(n, generator=gen) * 0.02).to(p_dtype)
+        p_big = torch.full((n + 64,), 3.0, dtype=p_dtype, device=cuda)
+        g_big = torch.full((n + 64,), 5.0, dtype=g_dtype, device=cuda)
+        dev = DeviceTensor(p0, cuda)
+        dev.p = p_big[po:po + n]
+        dev.p.copy_(p0)
+        assert dev.p.data_ptr() % 16 or not po
+        g_view = g_big[go:go + n]
+        ref = OracleTensor(p0)
+        for t in range(1, 4):
+            g = (torch.randn(n, generator=gen) * 1e-3).to(g_dtype)
+            g_view.copy_(g)
+            say(f"[odd offsets] p {p_dtype}+{po} g {g_dtype}+{go} n {n} step {t}")
+            q4.fused_4bit(dev.p, g_view, dev.m, dev.v, dev.sm, dev.sv, HP["beta1"], HP["beta2"], HP["lr"],
+                          HP["weight_decay"], HP["eps"], t)
+            torch.cuda.synchronize()
+            prev = ref.step(g, t)
+            assert_state_equal(dev, ref, prev, f"odd offsets step {t}")
+            ref.resync(dev.p)
+        assert (p_big[:po] == 3.0).all() and (p_big[po + n:] == 3.0).all()
+        assert (g_big[:go] == 5.0).all() and (g_big[go + n:] == 5.0).all() and torch.equal(g_view.cpu(), g)
+
+
 def test_all_zero_blocks_and_guard_bytes(cuda):
     """Blocks whose grads stay zero keep zero codes and zero scales; bytes past the
     packed length and scales past the last block are never written."""
@@ -340,7 +374,7 @@ def test_concurrent_threads_and_streams(cuda):
                     q4.fused_4bit(d.p, g, d.m, d.v, d.sm, d.sv,
                                   *[HP[k] for k in ("beta1", "beta2", "lr", "weight_decay", "eps")], t)
                     if i == 0 and t == 3:      # a refusal: nothing launched, message stays in this thread
-                        rc = L.q4adamw_fused_4bit(d.p.data_ptr() + 4, g.data_ptr(), d.m.data_ptr(), d.v.data_ptr(),
+                        rc = L.q4adamw_fused_4bit(d.p.data_ptr() + 2, g.data_ptr(), d.m.data_ptr(), d.v.data_ptr(),
                                                   d.sm.data_ptr(), d.sv.data_ptr(), 1000, 0, 1, 0.9, 0.999, 1e-3,
                                                   0.01, 1e-8, 1.0, stream.cuda_stream)
                         assert rc == -2

@@ -82,8 +82,8 @@ def test_static_scratch_refusals(cuda):
     assert call(arr, 1, _lib.FP32, None) == -1 and b"null" in L.q4adamw_last_error()
     assert call(arr, -1, _lib.FP32, out.data_ptr()) == -1
     assert call(arr, 1, 7, out.data_ptr()) == -1
-    arr[0].g = g.data_ptr() + 4
-    assert call(arr, 1, _lib.FP32, out.data_ptr()) == -2 and b"16-byte" in L.q4adamw_last_error()
+    arr[0].g = g.data_ptr() + 2
+    assert call(arr, 1, _lib.FP32, out.data_ptr()) == -2 and b"element size" in L.q4adamw_last_error()
     arr[0].g, arr[0].numel = g.data_ptr(), 1 << 62
     assert call(arr, 1, _lib.FP32, out.data_ptr()) == -4 and b"too large" in L.q4adamw_last_error()
     torch.cuda.synchronize(cuda)
