@@ -60,9 +60,9 @@ extern "C" {
  * p and g need the alignment of their element type only, like the reference's element-wise
  * accesses (optim/cuda_adamw_kernels.cu:334-351), so views at any offset into a flat buffer
  * are taken.  16-byte aligned addresses are the fast case: a parameter tensor that is not
- * takes about a third longer (its stores no longer cover whole lines), a gradient tensor
- * costs nothing extra.  Code and scale buffers must be 4-byte aligned (2 bytes suffice for
- * the codes of an fp32 parameter).
+ * takes 6 to 9 % longer (its waves' stores share lines), a gradient tensor costs nothing
+ * extra.  Code and scale buffers must be 4-byte aligned (2 bytes suffice for the codes of
+ * an fp32 parameter).
  */
 typedef struct q4adamw_tensor {
   void *p;

@@ -366,8 +366,8 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   // Parameters and gradients need the alignment of their element type only: the 16-byte
   // accesses of the kernels are legal at any such address (the memory pipeline runs in its
   // unaligned mode under ROCm; the compiler relies on the same for amdhsa targets).  A view at
-  // an odd offset into a flat buffer costs nothing on the gradient side and about a third
-  // more time on the parameter side (partial lines written).
+  // an odd offset into a flat buffer costs nothing on the gradient side and 6 to 9 % more
+  // time on the parameter side (lines shared between waves; see kNtSharedLines).
   const uintptr_t p_align = p_half ? 2 : 4, g_align = g_half ? 2 : 4;
   const uintptr_t code_align = wide ? 4 : 2;
   // validate everything before the first launch
