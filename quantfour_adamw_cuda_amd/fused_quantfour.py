@@ -26,7 +26,7 @@ the same path through the `grad_scale` / `found_inf` attributes it sets.
 The step itself runs only in the HIP library (csrc/libq4adamw.so); without it,
 or with parameters that are not on a GPU, `step()` raises.
 """
-from itertools import chain, compress, repeat
+from itertools import chain, compress
 from operator import attrgetter, is_, methodcaller
 from typing import Any, Dict, Optional
 

@@ -22,7 +22,6 @@ the scale s.  Second moment: old code 0 under an old scale 2 s gives an old valu
 new one is s / 16 + g^2 / 2; the pinned element holds old code 15 (old value 2 s) and g = 0,
 which makes it exactly s.
 """
-import numpy as np
 import pytest
 import torch
 

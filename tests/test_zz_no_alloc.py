@@ -7,7 +7,6 @@ Two calls in a row, the second on a smaller input: the array keeps the first cal
 sums, and the second call must not see them.  Collected last (the file's name sorts after
 the other test files), and it passes alone in a fresh process as well as after the others.
 """
-import ctypes
 
 import numpy as np
 import pytest
