@@ -194,19 +194,28 @@ static Rank1Kernel pick_rank1_rows(int p_dtype, int g_dtype, bool ext, bool sr) 
 }
 
 // Which of the three update kernels a matrix takes, in the order of the launch passes.
-// Rows form: rows of a whole number of tiles (at least two), and enough rows that the
-// waves left idle in the last group of four do not matter.
+// Rows form: rows of a whole number of quantization blocks and at least two tiles, and enough
+// rows that the waves left idle in the last group of four do not matter.  The last tile of a
+// row may be a partial one as long as its idle lanes are at most a sixteenth of the row (they
+// cost issue slots, which the 16-bit kernels have none to spare of; the wide form is 5 to 8 %
+// slower than the rows form).
 enum Rank1Shape { kShapeRows = 0, kShapeWide = 1, kShapeNarrow = 2 };
 
 static Rank1Shape rank1_shape(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
   if (t.cols < tile_elems) return kShapeNarrow;
-  if (t.cols % tile_elems == 0 && t.cols >= 2 * tile_elems && t.rows >= 64) return kShapeRows;
+  const int64_t padded = (t.cols + tile_elems - 1) / tile_elems * tile_elems;
+  if (t.cols % Q4ADAMW_BLOCK == 0 && t.cols >= 2 * tile_elems && t.rows >= 64 && (padded - t.cols) * 16 <= t.cols)
+    return kShapeRows;
   return kShapeWide;
+}
+
+static uint64_t rank1_tiles_per_row(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
+  return (uint64_t)((t.cols + tile_elems - 1) / tile_elems);
 }
 
 static uint64_t rank1_chunks(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
   if (rank1_shape(t, tile_elems) == kShapeRows)
-    return (uint64_t)((t.rows + kWaves - 1) / kWaves) * (uint64_t)(t.cols / tile_elems);
+    return (uint64_t)((t.rows + kWaves - 1) / kWaves) * rank1_tiles_per_row(t, tile_elems);
   const uint64_t chunk_elems = (uint64_t)tile_elems * kWaves;
   return ((uint64_t)t.rows * (uint64_t)t.cols + chunk_elems - 1) / chunk_elems;
 }
@@ -550,7 +559,7 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       d.rows = t.rows;
       d.cols = t.cols;
       // the divisor the tensor's kernel needs: tiles per row, or cols / 8
-      const FastDiv fd = make_fast_div(shape == kShapeRows ? (uint32_t)(t.cols / tile_elems) : (uint32_t)(t.cols >> 3));
+      const FastDiv fd = make_fast_div(shape == kShapeRows ? (uint32_t)rank1_tiles_per_row(t, tile_elems) : (uint32_t)(t.cols >> 3));
       d.div_magic = fd.magic;
       d.div_shift = fd.shift;
       a.sr_salt[a.ntensors] = !sr ? 0u : a.go.sc_dev ? lowbias32(salts ? salts[i] : (uint32_t)i)

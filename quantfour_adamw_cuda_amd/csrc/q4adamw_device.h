@@ -185,7 +185,7 @@ __device__ __forceinline__ void store_b128(u32x4 w, const void *base, uint32_t o
 // whether a tensor's lines are shared between neighbouring waves (uniform: the low bits of a
 // tile's address are those of its tensor's)
 __device__ __forceinline__ bool shares_lines(const void *base) {
-  return (reinterpret_cast<uintptr_t>(base) & 15u) != 0;
+  return __builtin_expect((reinterpret_cast<uintptr_t>(base) & 15u) != 0, 0);
 }
 
 template <int DT, int N, bool FULL>

@@ -29,10 +29,13 @@ struct Geometry {
 // entries; the noise of element e is a hash of e and the tensor's salt of this step.
 // SHAPE (with RANK1): how a tile lies in its matrix.  kTileWide: rows are at least a tile
 // long, so a tile touches one row or two.  kTileNarrow: rows may be shorter than a tile.
-// kTileRows: rows are a whole number of tiles long and the workgroup's four waves work on
-// the same columns of four consecutive rows, so they fetch the columns' maxima once,
-// together, and pass them through LDS (RowsTile).
-constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2;
+// kTileRows: rows are a whole number of quantization blocks long and tiles start at the
+// beginning of a row, so that the workgroup's four waves work on the same columns of four
+// consecutive rows: they fetch the columns' maxima once, together, and pass them through LDS
+// (RowsTile).  kTileRowsLast is the same for the last tile of a row that is not a whole
+// number of tiles long: its first RowsTile::width elements are there (whole blocks), the
+// lanes of the others load nothing, work on zeros and store nothing.
+constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2, kTileRowsLast = 3;
 
 // What a wave of the kTileRows form knows beyond its tile number: its row, the tile's first
 // column, and this thread's share of the workgroup's fetch of the columns' maxima (old and
@@ -41,6 +44,7 @@ constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2;
 struct RowsTile {
   int64_t row;
   uint32_t col0;
+  uint32_t width;     // elements of the tile that lie in the row: kTile, or less in a row's last tile
   float *columns;
   float2 share_old, share_new;
 };
@@ -58,24 +62,26 @@ __device__ __forceinline__ void stage_columns(const RowsTile &rt, int tid) {
 }
 
 template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, int SHAPE, typename Desc>
-__device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int lane, int wave, int tid,
+__device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g, uint32_t salt,
                                              const RowsTile *rt = nullptr) {
   using G = Geometry<PT, GT>;
   constexpr int N = G::kEpl;
-  // Uniform (scalar) part of every address: the tile's first element, byte and
-  // block; the per-lane part is a small 32-bit offset.
+  constexpr bool kRows = SHAPE == kTileRows || SHAPE == kTileRowsLast;
+  // Uniform (scalar) part of every address: the tile's first element tb (a multiple of the
+  // block size), its byte and block; the per-lane part is a small 32-bit offset.
   const int64_t numel = T.numel;
-  const int64_t tb = tile * G::kTile;
   const void *p_tile = static_cast<const char *>(T.p) + tb * (PT ? 2 : 4);
   const void *g_tile = static_cast<const char *>(T.g) + tb * (GT ? 2 : 4);
   const uint8_t *m_tile = T.m + (tb >> 1);
   const uint8_t *v_tile = T.v + (tb >> 1);
-  const float *sm_tile = T.sm + tile * G::kBlocksPerTile;
+  const float *sm_tile = T.sm + tb / Q4ADAMW_BLOCK;
   const float *sv_tile = nullptr;
-  if constexpr (!RANK1) sv_tile = T.sv + tile * G::kBlocksPerTile;
+  if constexpr (!RANK1) sv_tile = T.sv + tb / Q4ADAMW_BLOCK;
   const uint32_t e0 = (uint32_t)lane * N;                          // first element of this lane in the tile
+  bool lane_on = true;                                             // whether the lane's elements exist
+  if constexpr (SHAPE == kTileRowsLast) lane_on = e0 < rt->width;
   const uint32_t blk = (uint32_t)lane / G::kLanesPerBlock;         // which of the tile's blocks
   const uint32_t code_off = (uint32_t)lane * (N / 2);              // byte offset of this lane's codes
   int nv = N;
@@ -96,11 +102,12 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     const uint32_t tb8 = (uint32_t)(tb >> 3), cols8 = (uint32_t)(T.cols >> 3);  // numel < 2^35
     const int64_t last = T.rows - 1;
     uint32_t col;
-    if constexpr (SHAPE == kTileRows) {
+    if constexpr (kRows) {
       // the whole tile lies in one row; the columns' maxima come through LDS further down
       col = rt->col0 + e0;
-      r_old = as_global<const float>(T.rmax)[rt->row];
-      r_new = as_global<const float>(T.rmax_next)[rt->row];
+      // the statistics are complete before this kernel starts and change after it ends
+      r_old = as_constant<const float>(T.rmax)[rt->row];
+      r_new = as_constant<const float>(T.rmax_next)[rt->row];
     } else if constexpr (SHAPE == kTileWide) {
       // a tile is no longer than a row, so a lane is in the tile's first row or in the next
       const uint32_t row32 = fast_div(tb8, T.div_magic, T.div_shift);
@@ -123,7 +130,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
       r_old = as_global<const float>(T.rmax)[row];
       r_new = as_global<const float>(T.rmax_next)[row];
     }
-    if constexpr (SHAPE != kTileRows) {
+    if constexpr (!kRows) {
 #pragma unroll
       for (int k = 0; k < N; k += 4) {
         const u32x4 a = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(T.cmax), (col + k) * 4u, 0, 0);
@@ -135,15 +142,23 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
   }
 
   float p[N], g[N];
-  load_elems<PT, N, FULL>(p_tile, e0, nv, p);
-  load_elems<GT, N, FULL>(g_tile, e0, nv, g);
+  if constexpr (SHAPE == kTileRowsLast) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) p[j] = g[j] = 0.0f;
+  }
+  if (lane_on) {
+    load_elems<PT, N, FULL>(p_tile, e0, nv, p);
+    load_elems<GT, N, FULL>(g_tile, e0, nv, g);
+  }
   if (EXT) {
 #pragma unroll
     for (int j = 0; j < N; ++j) g[j] *= gscale;
-    if (zero_g) zero_elems<GT, N, FULL>(const_cast<void *>(g_tile), e0, nv);
+    if (zero_g && lane_on) zero_elems<GT, N, FULL>(const_cast<void *>(g_tile), e0, nv);
   }
   uint32_t mw = 0, vw = 0;
-  if (FULL) {
+  if (!lane_on) {
+    // nothing to read: zero codes under a zero scale
+  } else if (FULL) {
     if (N == 4) {
       mw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(m_tile), code_off, 0, kNt);
       vw = __builtin_amdgcn_raw_buffer_load_b16(tile_rsrc(v_tile), code_off, 0, kNt);
@@ -164,7 +179,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     }
   }
   float sm_old = 0.0f, sv_old = 0.0f;
-  if (FULL) {
+  if (!lane_on) {
+  } else if (FULL) {
     // scales are 4 bytes per block: cached, so that neighbouring blocks share lines
     sm_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sm_tile), blk * 4u, 0, 0));
     if (!RANK1) sv_old = bits2f(__builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(sv_tile), blk * 4u, 0, 0));
@@ -191,9 +207,9 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     entry[0] = m_entry;
     entry[kLdsSecondMoment] = v_entry;
   }
-  if constexpr (RANK1 && SHAPE == kTileRows) stage_columns<N>(*rt, tid);
+  if constexpr (RANK1 && kRows) stage_columns<N>(*rt, tid);
   setup_tables<SR>(lds, tid, slot);
-  if constexpr (RANK1 && SHAPE == kTileRows) {
+  if constexpr (RANK1 && kRows) {
 #pragma unroll
     for (int k = 0; k < N; k += 4) {
       const float4 a = *reinterpret_cast<const float4 *>(rt->columns + e0 + k);
@@ -232,7 +248,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
     av = __builtin_fmaxf(av, v);
   }
-  store_elems<PT, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
+  if (lane_on) store_elems<PT, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
 
   // block scales (exact: max is order independent)
   const float v_lane_max = av;
@@ -242,7 +258,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     am = row_max16(am);
     if (!RANK1) av = row_max16(av);
   }
-  if (blk_ok && (lane & (G::kLanesPerBlock - 1)) == 0) {
+  if (blk_ok && lane_on && (lane & (G::kLanesPerBlock - 1)) == 0) {
     if (FULL) {
       __builtin_amdgcn_raw_buffer_store_b32(f2bits(am), tile_rsrc(sm_tile), blk * 4u, 0, 0);
       if (!RANK1) __builtin_amdgcn_raw_buffer_store_b32(f2bits(av), tile_rsrc(sv_tile), blk * 4u, 0, 0);
@@ -379,7 +395,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tile, int la
     vword &= keep;
   }
 
-  if (FULL) {
+  if (!lane_on) {
+  } else if (FULL) {
     if (N == 4) {
       __builtin_amdgcn_raw_buffer_store_b16((uint16_t)mword, tile_rsrc(m_tile), code_off, 0, kNt);
       __builtin_amdgcn_raw_buffer_store_b16((uint16_t)vword, tile_rsrc(v_tile), code_off, 0, kNt);
@@ -429,9 +446,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, false, SR, kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, false, SR, kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, false, SR, kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, false, SR, kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
@@ -594,14 +611,16 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
-// The same for matrices whose rows are a whole number of tiles (at least two) long: a chunk
-// is one tile's columns of four consecutive rows, one row per wave; T.div_magic / div_shift
-// divide by the number of tiles in a row.  Every tile is full.
+// The same for matrices whose rows are a whole number of quantization blocks and at least
+// two tiles long: a chunk is one tile's columns of four consecutive rows, one row per wave,
+// and tiles start at the beginning of a row, so that the last tile of a row may be a partial
+// one (whole blocks; its other lanes are idle).  T.div_magic / div_shift divide by the number
+// of tiles in a row.
 template <int PT, int GT, bool EXT, bool SR>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const Rank1Args args) {
   using G = Geometry<PT, GT>;
@@ -620,27 +639,34 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const R
   const Rank1Desc &T = args.desc[t];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const uint32_t local = chunk - args.first_chunk[t];
-  const uint32_t tiles_per_row = (uint32_t)(T.cols / G::kTile);
+  const uint32_t cols = (uint32_t)T.cols;
+  const uint32_t tiles_per_row = (cols + (uint32_t)G::kTile - 1u) / (uint32_t)G::kTile;
   const uint32_t row_group = fast_div(local, T.div_magic, T.div_shift);
   const uint32_t col_tile = local - row_group * tiles_per_row;
   RowsTile rt;
   rt.row = (int64_t)row_group * kWaves + wave;
   rt.col0 = col_tile * (uint32_t)G::kTile;
+  rt.width = cols - rt.col0 < (uint32_t)G::kTile ? cols - rt.col0 : (uint32_t)G::kTile;
   rt.columns = columns;
   const bool idle = rt.row >= T.rows;   // the last rows of a matrix whose row count is no multiple of four
-  const int64_t tile = rt.row * tiles_per_row + col_tile;
+  const int64_t begin = rt.row * T.cols + rt.col0;   // the tile's first element
+  const bool whole = rt.width == (uint32_t)G::kTile;
   if (cancelled) {
-    if (!idle) zero_tile<GT, N>(T.g, tile, T.numel, lane);
+    if (!idle && (uint32_t)lane * N < rt.width)
+      zero_elems<GT, N, true>(static_cast<char *>(const_cast<void *>(T.g)) + begin * (GT ? 2 : 4), (uint32_t)lane * N, N);
     return;
   }
-  // this thread's share of the columns' maxima: N / 4 consecutive columns
+  // this thread's share of the columns' maxima: N / 4 consecutive columns (zeros past the row's end)
   const uint32_t share = rt.col0 + (uint32_t)tid * (N / 4);
-  if (N == 4) {
-    rt.share_old = make_float2(as_global<const float>(T.cmax)[share], 0.0f);
-    rt.share_new = make_float2(as_global<const float>(T.cmax_next)[share], 0.0f);
-  } else {
-    rt.share_old = make_float2(as_global<const float>(T.cmax)[share], as_global<const float>(T.cmax)[share + 1]);
-    rt.share_new = make_float2(as_global<const float>(T.cmax_next)[share], as_global<const float>(T.cmax_next)[share + 1]);
+  rt.share_old = rt.share_new = make_float2(0.0f, 0.0f);
+  if (whole || share < cols) {
+    if (N == 4) {
+      rt.share_old.x = as_global<const float>(T.cmax)[share];
+      rt.share_new.x = as_global<const float>(T.cmax_next)[share];
+    } else {
+      rt.share_old = make_float2(as_global<const float>(T.cmax)[share], as_global<const float>(T.cmax)[share + 1]);
+      rt.share_new = make_float2(as_global<const float>(T.cmax_next)[share], as_global<const float>(T.cmax_next)[share + 1]);
+    }
   }
   if (idle) {  // only help with the tables and the columns
     stage_columns<N>(rt, tid);
@@ -649,7 +675,10 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const R
   }
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
-  process_tile<PT, GT, true, EXT, true, SR, kTileRows>(T, tile, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
+  if (__builtin_expect(whole, 1))
+    process_tile<PT, GT, true, EXT, true, SR, kTileRows>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
+  else
+    process_tile<PT, GT, true, EXT, true, SR, kTileRowsLast>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
 }
 
 // After the update: the new statistics become the current ones and the buffers that

@@ -57,6 +57,9 @@ def _check(dev, ref, prev, what):
 
 
 SHAPES = [(66, 1024), (128, 1536), (64, 4096), (64, 512), (3, 4096), (100, 520), (257, 768), (130, 1032), (1, 512), (70, 2048 + 512), (5, 8200),
+          # rows of whole blocks whose last tile is a partial one (384, 256 and 128 of a 512-element
+          # tile, 128 of a 256-element one), row counts that are and are not multiples of four
+          (66, 2432), (64, 4352), (65, 6272), (67, 2176),
           # narrow matrices: a tile spans several rows (fewer than 256 columns, or than 512 when
           # parameters and gradients are 16-bit types)
           (300, 16), (77, 64), (1000, 24), (513, 248), (40, 504), (9, 256), (2000, 136)]
@@ -87,7 +90,8 @@ def test_rank1_against_oracle(cuda, p_dt, g_dt, shape):
 
 @pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
                                        ("fp16", "fp16")])
-@pytest.mark.parametrize("shape", [(64, 512), (70, 2048 + 512), (100, 520), (130, 1032), (5, 8200), (333, 40), (50, 264)])
+@pytest.mark.parametrize("shape", [(64, 512), (70, 2048 + 512), (100, 520), (130, 1032), (5, 8200), (333, 40), (50, 264),
+                                   (65, 2432), (66, 4352)])     # rows whose last tile is a partial one
 def test_rank1_stochastic_rounding_against_oracle(cuda, p_dt, g_dt, shape):
     """rank-1 scaling and stochastic rounding together: codes, scales and statistics bit for
     bit against step_quant_rank1_sr; the noise follows seed, step and the tensor's salt"""
@@ -193,6 +197,7 @@ def test_rank1_multi_tensor_and_options(cuda):
     gen = torch.Generator().manual_seed(9)
     shapes = [(8 + i % 5, 512 + 8 * (i % 7)) for i in range(37)]
     shapes += [(65, 512), (70, 768), (64, 1024)]      # rows of whole tiles: the kernel that shares column maxima
+    shapes += [(66, 2176), (65, 2432)]                # the same with a partial last tile in every row
     ps = [(torch.randn(s, generator=gen) * 0.05) for s in shapes]
     devs = [Rank1State(p, cuda) for p in ps]
     refs = [(p.clone(), d.m.cpu(), d.v.cpu(), d.sm.cpu(), d.r.cpu(), d.c.cpu()) for p, d in zip(ps, devs)]
@@ -212,10 +217,11 @@ def test_rank1_multi_tensor_and_options(cuda):
             assert bool(dgs[i].any()) == (step == 1)
 
 
-@pytest.mark.parametrize("rows", [40, 66])           # 66 rows of four tiles: the kernel that shares column maxima
-def test_rank1_found_inf_leaves_everything(cuda, rows):
+@pytest.mark.parametrize("rows,cols", [(40, 1024), (66, 1024),     # 66 rows of four tiles: the kernel that shares column maxima
+                                       (66, 2176)])                # and with a partial last tile in every row
+def test_rank1_found_inf_leaves_everything(cuda, rows, cols):
     gen = torch.Generator().manual_seed(10)
-    p0 = torch.randn(rows, 1024, generator=gen) * 0.05
+    p0 = torch.randn(rows, cols, generator=gen) * 0.05
     dev = Rank1State(p0, cuda)
     g = grads_config1(gen, p0.numel()).view(p0.shape).to(torch.bfloat16).to(cuda)
     dev.step(g, 1)
