@@ -128,3 +128,38 @@ def test_random_configuration_rank1(cuda, i):
         ok, worst = p_close(to_np(p), to_np(ref[0]), to_np(prev), bf16=p_dt == torch.bfloat16)
         assert ok, f"rank1 sweep {i} step {step}: parameters (worst {worst})"
         ref = (p.cpu().clone(),) + tuple(ref[1:])
+
+
+@pytest.mark.parametrize("p_dt,g_dt", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16)])
+def test_long_run_stays_bit_exact(cuda, p_dt, g_dt):
+    """120 consecutive steps of one tensor: the packed state feeds back into itself, so any
+    difference from the oracle would persist and grow.  The gradient regime changes every few
+    steps (decaying magnitude, sparse steps, spikes, all-zero steps, a sign flip), which walks
+    the block scales up and down; codes and scales are compared bit for bit after every step."""
+    rng = np.random.default_rng(4242)
+    n = 128 * 1500 + 77
+    p0 = torch.from_numpy((rng.standard_normal(n) * 0.05).astype(np.float32)).to(p_dt)
+    dev, ref = DeviceTensor(p0, cuda), OracleTensor(p0)
+    hp = dict(beta1=0.9, beta2=0.95, lr=3e-3, weight_decay=0.05, eps=1e-8)   # short memory: scales move fast
+    base = rng.standard_normal(n).astype(np.float32)
+    for step in range(1, 121):
+        regime = (step // 6) % 5
+        g = base * np.float32(0.7) + rng.standard_normal(n).astype(np.float32) * np.float32(0.3)
+        g *= np.float32(1e-2 * 0.97 ** step)
+        if regime == 1:
+            g[rng.uniform(size=n) < 0.9] = 0.0
+        elif regime == 2:
+            g[rng.uniform(size=n) > 0.9995] *= np.float32(300.0)
+        elif regime == 3 and step % 2:
+            g[:] = 0.0
+        elif regime == 4:
+            g = -g
+        g = _as_grad(g, g_dt)
+        if step % 20 == 1:
+            print(f"[long run {p_dt}/{g_dt}] step {step}", flush=True)
+        q4.fused_4bit(dev.p, g.to(cuda), dev.m, dev.v, dev.sm, dev.sv, hp["beta1"], hp["beta2"], hp["lr"],
+                      hp["weight_decay"], hp["eps"], step)
+        prev = ref.step(g, step, hp)
+        assert_state_equal(dev, ref, prev, f"long run step {step}")
+        ref.resync(dev.p)
+    assert ref.m.any() and ref.v.any() and len(np.unique(ref.sm)) > 100

@@ -115,6 +115,42 @@ def test_rank1_stochastic_rounding_against_oracle(cuda, p_dt, g_dt, shape):
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
 
 
+@pytest.mark.parametrize("stochastic", [False, True])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16")])
+def test_rank1_long_run_stays_bit_exact(cuda, p_dt, g_dt, stochastic):
+    """60 consecutive steps of one matrix (rows that end in a partial tile): codes, scales and
+    statistics feed back into themselves and are compared bit for bit after every step, while
+    the gradients' magnitude decays, rows and columns fall silent and come back, and spikes
+    move the row and column maxima"""
+    rows, cols = 96, 2432
+    gen = torch.Generator().manual_seed(777)
+    p0 = (torch.randn(rows, cols, generator=gen) * 0.05).to(DT[p_dt])
+    dev = Rank1State(p0, cuda)
+    ref = (p0.clone(), dev.m.cpu(), dev.v.cpu(), dev.sm.cpu(), dev.r.cpu(), dev.c.cpu())
+    seed, salt = 0x0BAD_CAFE_1234, 5
+    for step in range(1, 61):
+        g = torch.randn(rows, cols, generator=gen) * (1e-2 * 0.95 ** step)
+        regime = (step // 5) % 4
+        if regime == 1:
+            g[step % rows] = 0.0
+            g[:, (step * 8) % cols:(step * 8) % cols + 64] = 0.0
+        elif regime == 2:
+            g[torch.rand(rows, cols, generator=gen) > 0.9995] *= 200.0
+        elif regime == 3 and step % 2:
+            g.zero_()
+        g = g.to(DT[g_dt])
+        prev = ref[0]
+        if stochastic:
+            ref = ot.step_quant_rank1_sr(ref[0], g, *ref[1:], seed=seed, tensor_salt=salt, step=step, **HP)
+            dev.step(g.to(cuda), step, seed=seed, salts=[salt])
+        else:
+            ref = ot.step_quant_rank1(ref[0], g, *ref[1:], step=step, **HP)
+            dev.step(g.to(cuda), step)
+        _check(dev, ref, prev, f"long run {p_dt}/{g_dt} sr={stochastic} step {step}")
+        ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
+    assert ref[1].any() and ref[2].any() and ref[4].min() > 0 and ref[5].min() > 0
+
+
 def test_rank1_stochastic_rounding_many_tensors_and_options(cuda):
     """40 matrices in one call (two launch batches): default salts are the positions in the
     list, the call is reproducible, another seed changes codes; gradient multiplier on top"""
