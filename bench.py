@@ -20,7 +20,9 @@ HBM before the timed region starts.  Prints ONE JSON line:
                 sample of the same workload
   configs       (default run only) the other benchmark configurations and the step's
                 variants, each timed the same way in this same process: step time,
-                kernel time, launches, fraction of peak, host time per step
+                kernel time, launches, fraction of peak, host time per step, and for
+                the block-scaled ones the fraction of the `ceiling` probe with their
+                element types (measured on 2^30 elements, whatever the configuration's size)
   ceiling       what this GPU's memory system gives kernels that move the step's bytes
                 in the step's access pattern without its arithmetic (libq4probe.so): a
                 plain copy, a read-only stream and the step's seven streams; the
@@ -283,11 +285,14 @@ def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None):
     return r
 
 
-def config_entry(name, desc, m, workload, variance_scale, round_type):
+def config_entry(name, desc, m, workload, variance_scale, round_type, p_dtype_s, g_dtype_s):
     r = roofline_entry(m, workload, variance_scale, round_type)
     return {
         "name": name,
         "workload": desc,
+        "param_dtype": p_dtype_s,
+        "grad_dtype": g_dtype_s,
+        "variance_scale": variance_scale,
         "steps": m["steps"],
         "ms_per_step": m["ms_per_step"],
         "params_per_s": m["total_params"] * m["steps"] / m["elapsed"],
@@ -475,7 +480,8 @@ def main():
                              ("rank1", "real-nearest", "rank-1 scaled second moment"),
                              ("rank1", "stochastic", "rank-1 scaled second moment + stochastic rounding")):
             mv = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, k, w, vs, rt)
-            configs.append(config_entry(f"{args.workload}, {name}", desc + "; " + name, mv, args.workload, vs, rt))
+            configs.append(config_entry(f"{args.workload}, {name}", desc + "; " + name, mv, args.workload, vs, rt,
+                                        p_dtype_s, g_dtype_s))
     del params, grad_sets
     torch.cuda.empty_cache()
     if all_configs:
@@ -483,7 +489,7 @@ def main():
             fn, ps, gs_, dist_, desc_ = WORKLOADS[wl]
             pr, gr = build_inputs(torch, device, fn(), getattr(torch, ps), getattr(torch, gs_), dist_, 2)
             mv = run_config(torch, pr, gr, ps, gs_, k, w)
-            configs.append(config_entry(wl, desc_, mv, wl, "group", "real-nearest"))
+            configs.append(config_entry(wl, desc_, mv, wl, "group", "real-nearest", ps, gs_))
             del pr, gr
             torch.cuda.empty_cache()
 
@@ -491,6 +497,11 @@ def main():
     key = f"step_streams_{p_dtype_s}_{g_dtype_s}"
     out["roofline"] = roofline_entry(m, args.workload, args.variance_scale, args.round_type,
                                      ceiling.get(key) if ceiling else None)
+    for c in configs:
+        # block-scaled variants move the bytes of the probe with their element types; rank-1
+        # scaling adds a second pass and the statistics, which no probe moves
+        probe = ceiling.get(f"step_streams_{c['param_dtype']}_{c['grad_dtype']}") if ceiling else None
+        c["frac_of_ceiling"] = c["achieved"] / probe if probe and c["variance_scale"] == "group" else None
     if cpu is not None:
         out["cpu_baseline"] = cpu
     if configs:
