@@ -366,6 +366,13 @@ def measure_ceiling(torch, device, reps=10):
     # gradients read (10 bytes per element), and with the scales but not the codes (10.125)
     out["step_streams_float32_bfloat16_without_codes_and_scales"] = n * 10.0 / streams("float32", "bfloat16", 0) / 1e9
     out["step_streams_float32_bfloat16_without_codes"] = n * 10.125 / streams("float32", "bfloat16", 2) / 1e9
+    # the same streams on 2^24 elements, the size of BASELINE.json configs[0]: what a launch of
+    # that size can reach at all (ramp-up and drain are part of it)
+    small = 1 << 24
+    reps = 50
+    t = timed(lambda: L.q4probe_step_streams(a.data_ptr(), b.data_ptr(), m.data_ptr(), v.data_ptr(), sm.data_ptr(),
+                                             sv.data_ptr(), small, tag["float32"], tag["float32"], 3, stream))
+    out["step_streams_float32_float32_2p24_elements"] = small * bytes_per_param("float32", "float32") / t / 1e9
     return out
 
 
@@ -502,6 +509,8 @@ def main():
         # scaling adds a second pass and the statistics, which no probe moves
         probe = ceiling.get(f"step_streams_{c['param_dtype']}_{c['grad_dtype']}") if ceiling else None
         c["frac_of_ceiling"] = c["achieved"] / probe if probe and c["variance_scale"] == "group" else None
+        if ceiling and c["name"] == "single-4096":
+            c["frac_of_ceiling_at_size"] = c["achieved"] / ceiling["step_streams_float32_float32_2p24_elements"]
     if cpu is not None:
         out["cpu_baseline"] = cpu
     if configs:
