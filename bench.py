@@ -412,6 +412,9 @@ def main():
                          "them in `configs` (auto: only for the default workload without variant options)")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the memory-system probes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--progress", action="store_true",
+                    help="name every phase on stderr as it ends (stdout keeps its one JSON line), so that a "
+                         "run that stops under a profiler shows where")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region, run the probe library's plain 4 GiB copy three times, "
                          "so that a counter profile of this command also holds a kernel of known traffic")
@@ -422,6 +425,10 @@ def main():
                  "on its own shard. Run with --gpus 1.")
 
     import torch
+
+    def phase(what):
+        if args.progress:
+            print(f"[bench] {what}", file=sys.stderr, flush=True)
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
@@ -435,10 +442,13 @@ def main():
 
     params, grad_sets = build_inputs(torch, device, shapes_fn(), getattr(torch, p_dtype_s),
                                      getattr(torch, g_dtype_s), dist, args.grad_sets)
+    phase(f"inputs of {args.workload} built")
     m = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, args.steps, args.warmup,
                    args.variance_scale, args.round_type, args.clip)
+    phase("headline steps timed")
     if args.calibrate_copy:
         calibrate_copy(torch, device)
+        phase("calibration copies done")
 
     out = {
         "metric": "params_updated_per_sec_fused_4bit_adamw_step",
@@ -489,6 +499,7 @@ def main():
             mv = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, k, w, vs, rt)
             configs.append(config_entry(f"{args.workload}, {name}", desc + "; " + name, mv, args.workload, vs, rt,
                                         p_dtype_s, g_dtype_s))
+            phase(f"variant timed: {name}")
     del params, grad_sets
     torch.cuda.empty_cache()
     if all_configs:
@@ -497,10 +508,12 @@ def main():
             pr, gr = build_inputs(torch, device, fn(), getattr(torch, ps), getattr(torch, gs_), dist_, 2)
             mv = run_config(torch, pr, gr, ps, gs_, k, w)
             configs.append(config_entry(wl, desc_, mv, wl, "group", "real-nearest", ps, gs_))
+            phase(f"configuration timed: {wl}")
             del pr, gr
             torch.cuda.empty_cache()
 
     ceiling = None if args.no_ceiling else measure_ceiling(torch, device)
+    phase("probes done")
     key = f"step_streams_{p_dtype_s}_{g_dtype_s}"
     out["roofline"] = roofline_entry(m, args.workload, args.variance_scale, args.round_type,
                                      ceiling.get(key) if ceiling else None)
