@@ -42,6 +42,15 @@
  *                         drafts disagree in rounding, so the bit-level choice
  *                         (unfused mul/add, fp32 derived scalars) is this build's:
  *                         bit-level parity with the reference is UNPINNED.
+ *   q4o_step_quant_variants (rank-1 scaling of the second moment after
+ *                         optim/adamw_fourbit_triton.py:738-755, :520-527, :834-863;
+ *                         stochastic rounding after :969-997, :1050-1075): scalar loops,
+ *                         written apart from the vectorised restatement in
+ *                         q4_oracle_torch.py (step_quant_rank1, step_quant_sr,
+ *                         step_quant_rank1_sr), which must agree with it bit for bit;
+ *                         with neither option it must reproduce q4o_step_quant.  The
+ *                         draft never runs either against data: parity with the
+ *                         reference is UNPINNED for both.
  */
 #include <math.h>
 #include <stdint.h>
@@ -367,6 +376,156 @@ void q4o_quant(const float *x, int64_t numel, int which, uint8_t *codes, float *
                 q |= q4o_quantize_count(which, x1) << 4;
             }
             codes[(base + k) >> 1] = (uint8_t)q;
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------
+ * Rank-1 scaling of the second moment and stochastic rounding, as scalar loops.
+ * ------------------------------------------------------------------------- */
+
+/* the rounding noise's 32-bit mixer: two multiply-xorshift rounds */
+static inline uint32_t q4o_mix32(uint32_t x) {
+    x ^= x >> 16;
+    x *= 0x7FEB352Du;
+    x ^= x >> 15;
+    x *= 0x846CA68Bu;
+    x ^= x >> 16;
+    return x;
+}
+
+/* salt of one tensor in one step: the tensor's own salt, the step number and the two
+ * halves of the seed, mixed one after the other */
+uint32_t q4o_sr_tensor_salt(uint64_t seed, uint32_t step, uint32_t tensor_salt) {
+    uint32_t h = q4o_mix32(tensor_salt);
+    h = q4o_mix32(h ^ step);
+    h = q4o_mix32(h ^ (uint32_t)(seed >> 32));
+    return q4o_mix32(h ^ (uint32_t)seed);
+}
+
+/* noise of element e: (2 n + 1) / 2^17 with n the high (first moment) and low (second
+ * moment) half of the hash of the element's index and the salt */
+void q4o_sr_noise(int64_t e, uint32_t salt, float *u_first, float *u_second) {
+    const uint64_t ue = (uint64_t)e;
+    const uint32_t key = (uint32_t)ue ^ salt ^ ((uint32_t)(ue >> 32) * 0x9E3779B9u);
+    const uint32_t h = q4o_mix32(key);
+    *u_first = (float)(2 * (h >> 16) + 1) / 131072.0f;       /* exact: 17 bits over 2^17 */
+    *u_second = (float)(2 * (h & 0xFFFFu) + 1) / 131072.0f;
+}
+
+/*
+ * Stochastic code of one normalised value q with noise u in (0, 1): q lies between two
+ * neighbouring code-book values lo <= q < hi and goes up with probability
+ * (q - lo) / (hi - lo), decided as u * (hi - lo) < q - lo with both sides rounded to
+ * fp32.  Below the first value the code is 0, at or above the last it is 15, NaN gets 0.
+ */
+int q4o_quantize_sr(int which, float q, float u) {
+    const float *qmap = which ? Q4O_QMAP_V : Q4O_QMAP_M;
+    if (q != q) return 0;
+    int above = 0;                       /* code-book values at or below q */
+    while (above < 16 && qmap[above] <= q) ++above;
+    if (above == 0) return 0;
+    if (above == 16) return 15;
+    volatile float gap = qmap[above] - qmap[above - 1];
+    volatile float dist = q - qmap[above - 1];
+    volatile float need = u * gap;
+    return above - 1 + (need < dist ? 1 : 0);
+}
+
+/*
+ * The fused step with its options: rank1 != 0 scales the second moment of the matrix
+ * [rows, cols] by min(row maximum, column maximum) instead of per-128 block maxima
+ * (v_scale is then unused; row_max / col_max hold the old statistics and receive the new
+ * ones); stochastic != 0 rounds both moments stochastically with the noise of
+ * (seed, step, tensor_salt).  numel = rows * cols; a flat tensor is rows = 1.
+ * First pass: new moments and parameters; second pass: statistics and codes.
+ */
+void q4o_step_quant_variants(void *p, const void *g, uint8_t *m_codes, uint8_t *v_codes,
+                             float *m_scale, float *v_scale, float *row_max, float *col_max,
+                             int64_t rows, int64_t cols, int p_dtype, int g_dtype,
+                             float beta1, float beta2, float lr, float weight_decay, float eps,
+                             float step, int rank1, int stochastic, uint64_t seed,
+                             uint32_t tensor_salt, float *scratch /* 2 * numel floats */) {
+    float sc[6];
+    q4o_derive_scalars(beta1, beta2, lr, weight_decay, step, sc);
+    const float c2s = sc[1], ss = sc[2], wdu = sc[3], r1 = sc[4], r2 = sc[5];
+    const int64_t numel = rows * cols;
+    float *mn = scratch, *vn = scratch + numel;
+    const uint32_t salt = stochastic ? q4o_sr_tensor_salt(seed, (uint32_t)step, tensor_salt) : 0u;
+    for (int64_t i = 0; i < numel; ++i) {
+        const uint8_t mb = m_codes[i >> 1], vb = v_codes[i >> 1];
+        const int cm = (i & 1) ? (mb >> 4) : (mb & 15);
+        const int cv = (i & 1) ? (vb >> 4) : (vb & 15);
+        float v_old_scale;
+        if (rank1) {
+            const float r = row_max[i / cols], c = col_max[i % cols];
+            v_old_scale = r < c ? r : c;
+        } else {
+            v_old_scale = v_scale[i / Q4O_BLOCK];
+        }
+        const float gi = load_elem(g, g_dtype, i);
+        volatile float m = Q4O_QMAP_M[cm] * m_scale[i / Q4O_BLOCK];
+        volatile float v = Q4O_QMAP_V[cv] * v_old_scale;
+        volatile float t0 = beta1 * m;
+        volatile float t1 = r1 * gi;
+        m = t0 + t1;
+        volatile float gg = gi * gi;
+        volatile float t2 = beta2 * v;
+        volatile float t3 = r2 * gg;
+        v = t2 + t3;
+        const float pi = load_elem(p, p_dtype, i);
+        store_elem(p, p_dtype, i, adamw_param(pi, m, v, wdu, ss, c2s, eps));
+        mn[i] = m;
+        vn[i] = v;
+    }
+    /* new statistics: a NaN never becomes a maximum, an infinity does */
+    const int64_t nblocks = (numel + Q4O_BLOCK - 1) / Q4O_BLOCK;
+    for (int64_t b = 0; b < nblocks; ++b) {
+        float sm = 0.0f, sv = 0.0f;
+        for (int64_t i = b * Q4O_BLOCK; i < numel && i < (b + 1) * Q4O_BLOCK; ++i) {
+            const float am = fabsf(mn[i]), av = fabsf(vn[i]);
+            if (am > sm) sm = am;
+            if (av > sv) sv = av;
+        }
+        m_scale[b] = sm;
+        if (!rank1) v_scale[b] = sv;
+    }
+    if (rank1) {
+        for (int64_t r = 0; r < rows; ++r) row_max[r] = 0.0f;
+        for (int64_t c = 0; c < cols; ++c) col_max[c] = 0.0f;
+        for (int64_t i = 0; i < numel; ++i) {
+            const float av = fabsf(vn[i]);
+            if (av > row_max[i / cols]) row_max[i / cols] = av;
+            if (av > col_max[i % cols]) col_max[i % cols] = av;
+        }
+    }
+    /* codes */
+    for (int64_t i = 0; i < numel; ++i) {
+        float sv;
+        if (rank1) {
+            const float r = row_max[i / cols], c = col_max[i % cols];
+            sv = r < c ? r : c;
+        } else {
+            sv = v_scale[i / Q4O_BLOCK];
+        }
+        volatile float qm = mn[i] / m_scale[i / Q4O_BLOCK];
+        volatile float qv = vn[i] / sv;
+        int code_m, code_v;
+        if (stochastic) {
+            float um, uv;
+            q4o_sr_noise(i, salt, &um, &uv);
+            code_m = q4o_quantize_sr(0, qm, um);
+            code_v = q4o_quantize_sr(1, qv, uv);
+        } else {
+            code_m = q4o_quantize_count(0, qm);
+            code_v = q4o_quantize_count(1, qv);
+        }
+        if (i & 1) {
+            m_codes[i >> 1] |= (uint8_t)(code_m << 4);
+            v_codes[i >> 1] |= (uint8_t)(code_v << 4);
+        } else {
+            m_codes[i >> 1] = (uint8_t)code_m;
+            v_codes[i >> 1] = (uint8_t)code_v;
         }
     }
 }

@@ -51,6 +51,14 @@ def lib():
         L.q4o_step_unquant.argtypes = [vp, vp, vp, vp, i64, ci, ci, f, f, f, f, f, f]
         L.q4o_dequant.argtypes = [vp, vp, i64, ci, vp]
         L.q4o_quant.argtypes = [vp, i64, ci, vp, vp]
+        u32, u64 = ctypes.c_uint32, ctypes.c_uint64
+        L.q4o_step_quant_variants.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci, f, f, f, f, f, f,
+                                              ci, ci, u64, u32, vp]
+        L.q4o_sr_tensor_salt.argtypes = [u64, u32, u32]
+        L.q4o_sr_tensor_salt.restype = u32
+        L.q4o_sr_noise.argtypes = [i64, u32, vp, vp]
+        L.q4o_quantize_sr.argtypes = [ci, f, f]
+        L.q4o_quantize_sr.restype = ci
         L.q4o_f16_to_f32.argtypes = [ctypes.c_uint16]
         L.q4o_f16_to_f32.restype = f
         L.q4o_f32_to_f16.argtypes = [f]
@@ -125,6 +133,50 @@ def step_quant(p, g, m_codes, v_codes, m_scale, v_scale, *, beta1, beta2, lr,
     lib().q4o_step_quant(_ptr(p), _ptr(g), _ptr(m_codes), _ptr(v_codes), _ptr(m_scale),
                          _ptr(v_scale), n, _dtype_tag(p), _dtype_tag(g), beta1, beta2, lr,
                          weight_decay, eps, float(step))
+
+
+def step_quant_variants(p, g, m_codes, v_codes, m_scale, v_scale=None, row_max=None, col_max=None, *, beta1,
+                        beta2, lr, weight_decay, eps, step, seed=None, tensor_salt=0):
+    """The fused step with its options, in place: row_max / col_max given (p a [rows, cols]
+    matrix) = rank-1 scaled second moment, else v_scale = per-128 block scales; seed given =
+    stochastic rounding with the noise of (seed, step, tensor_salt)."""
+    rank1 = row_max is not None
+    rows, cols = p.shape if rank1 else (1, p.size)
+    n = rows * cols
+    nbytes, nblk = state_sizes(n)
+    assert g.size == n and m_codes.size == nbytes and v_codes.size == nbytes and m_scale.size == nblk
+    assert m_codes.dtype == np.uint8 and v_codes.dtype == np.uint8 and m_scale.dtype == np.float32
+    if rank1:
+        assert row_max.size == rows and col_max.size == cols
+        assert row_max.dtype == np.float32 and col_max.dtype == np.float32 and v_scale is None
+    else:
+        assert v_scale.size == nblk and v_scale.dtype == np.float32
+    for a in (p, g, m_codes, v_codes, m_scale, v_scale, row_max, col_max):
+        assert a is None or a.flags.c_contiguous
+    scratch = np.empty(2 * n, np.float32)
+    none = ctypes.c_void_p(0)
+    lib().q4o_step_quant_variants(_ptr(p), _ptr(g), _ptr(m_codes), _ptr(v_codes), _ptr(m_scale),
+                                  none if rank1 else _ptr(v_scale), _ptr(row_max) if rank1 else none,
+                                  _ptr(col_max) if rank1 else none, rows, cols, _dtype_tag(p), _dtype_tag(g),
+                                  beta1, beta2, lr, weight_decay, eps, float(step), int(rank1),
+                                  int(seed is not None), int(seed or 0) & (2 ** 64 - 1),
+                                  int(tensor_salt) & 0xFFFFFFFF, _ptr(scratch))
+
+
+def sr_tensor_salt(seed, step, tensor_salt):
+    return int(lib().q4o_sr_tensor_salt(int(seed) & (2 ** 64 - 1), int(step) & 0xFFFFFFFF,
+                                        int(tensor_salt) & 0xFFFFFFFF))
+
+
+def sr_noise(e, salt):
+    """(first-moment noise, second-moment noise) of element e"""
+    um, uv = ctypes.c_float(), ctypes.c_float()
+    lib().q4o_sr_noise(int(e), int(salt) & 0xFFFFFFFF, ctypes.byref(um), ctypes.byref(uv))
+    return um.value, uv.value
+
+
+def quantize_sr(which, q, u):
+    return int(lib().q4o_quantize_sr(which, q, u))
 
 
 def step_unquant(p, g, m, v, *, beta1, beta2, lr, weight_decay, eps, step):

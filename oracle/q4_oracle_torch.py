@@ -139,7 +139,9 @@ def step_unquant(p, g, m, v, *, beta1, beta2, lr, weight_decay, eps, step):
 # :537-545), quantize x.div(scale) (:834-863), dequantize x.mul(scale) (:520-527).
 # The code book stays the fused path's linear map.  The draft never runs this
 # against data, so parity with the reference is UNPINNED; the functions are pinned
-# by brute force on small matrices and by closed forms (tests/test_oracle_pins.py).
+# by brute force on small matrices, by closed forms and by the scalar C restatement of
+# the whole step (q4o_step_quant_variants in q4_oracle.c), which must give the same bits
+# (tests/test_oracle_pins.py).
 # ---------------------------------------------------------------------------
 def rank1_scale(row_max, col_max):
     """compute_variance_tensor_scale for a matrix: min(row_max[i], col_max[j])."""
@@ -253,7 +255,8 @@ def step_quant_rank1_nd(p, g, m_codes, v_codes, m_scale, max_dims, *, beta1, bet
 #     up  <=>  RN(u * w[k]) < RN(q - Q[k]),   w[k] = RN(Q[k+1] - Q[k]),
 #     u = (2 n + 1) / 2^17 with n a 16-bit hash value (never 0, never 1).
 # Parity with the reference is UNPINNED (it has no runnable counterpart); pinned by
-# brute force, by exactness on code-book values and by the rounding's mean
+# brute force, by the scalar C restatement (q4o_sr_noise, q4o_quantize_sr,
+# q4o_step_quant_variants), by exactness on code-book values and by the rounding's mean
 # (tests/test_oracle_pins.py).
 # ---------------------------------------------------------------------------
 _M32 = np.uint64(0xFFFFFFFF)

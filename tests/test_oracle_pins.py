@@ -600,3 +600,118 @@ def test_quantizer_search_equals_count_on_every_fp32(which):
     bad, first, steps = oc.exhaustive_search_vs_count(which)
     assert bad == 0, f"{bad} patterns disagree, first {first:#010x}"
     assert steps == 15
+
+
+# ---------------------------------------------------------------------------
+# rank-1 scaling and stochastic rounding: the scalar C restatement against the vectorised one
+# ---------------------------------------------------------------------------
+def _np_elem(t):
+    """torch tensor -> the numpy form the C oracle takes (bf16 as uint16 bit patterns)"""
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.int16).numpy().view(np.uint16).copy()
+    return t.numpy().copy()
+
+
+def _variant_inputs(rows, cols, p_dt, g_dt, seed):
+    gen = torch.Generator().manual_seed(seed)
+    n = rows * cols
+    p = (torch.randn(rows, cols, generator=gen) * 0.05).to(p_dt)
+    make = (grads_config1, grads_config3, grads_student_t)
+    grads = []
+    for k in range(3):
+        g = make[k](gen, n).view(rows, cols).clone()
+        if k == 1:
+            g[rows // 2] = 0.0                      # a silent row and silent columns
+            g[:, : max(1, cols // 7)] = 0.0
+        if k == 2 and n > 40:
+            g.view(-1)[5] = float("inf")            # non-finite gradients reach the statistics
+            g.view(-1)[37] = float("nan")
+        grads.append(g.to(g_dt))
+    return p, grads
+
+
+@pytest.mark.parametrize("stochastic", [False, True])
+@pytest.mark.parametrize("rank1", [False, True])
+@pytest.mark.parametrize("p_dt,g_dt", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                       (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16)])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 50), (7, 129), (40, 264), (130, 96), (5, 1031)])
+def test_c_and_torch_restatements_of_the_variants_agree(shape, p_dt, g_dt, rank1, stochastic):
+    """q4o_step_quant_variants (scalar loops) and step_quant / step_quant_sr / step_quant_rank1 /
+    step_quant_rank1_sr (vectorised) are written apart from each other and must give the same
+    bits -- codes, block scales, row and column maxima and parameters -- over three steps that
+    feed back into each other, with silent rows and columns and non-finite gradients."""
+    rows, cols = shape
+    n = rows * cols
+    p, grads = _variant_inputs(rows, cols, p_dt, g_dt, 31 * rows + cols)
+    nbytes, nblk = oc.state_sizes(n)
+    seed, salt = 0x1234_5678_9ABC_DEF0 ^ (rows << 40), cols % 11
+    # C side (in place)
+    cp = _np_elem(p)
+    cm, cv = np.zeros(nbytes, np.uint8), np.zeros(nbytes, np.uint8)
+    csm, csv = np.zeros(nblk, np.float32), np.zeros(nblk, np.float32)
+    cr, cc = np.zeros(rows, np.float32), np.zeros(cols, np.float32)
+    # torch side (functional)
+    if rank1:
+        ref = (p.clone(), torch.zeros(nbytes, dtype=torch.uint8), torch.zeros(nbytes, dtype=torch.uint8),
+               torch.zeros(nblk), torch.zeros(rows), torch.zeros(cols))
+    else:
+        ref = (p.clone().reshape(-1), torch.zeros(nbytes, dtype=torch.uint8), torch.zeros(nbytes, dtype=torch.uint8),
+               torch.zeros(nblk), torch.zeros(nblk))
+    hp = dict(HP)
+    for step, g in enumerate(grads, 1):
+        kw = dict(seed=seed, tensor_salt=salt) if stochastic else {}
+        if rank1:
+            oc.step_quant_variants(cp, _np_elem(g), cm, cv, csm, None, cr, cc, step=step, **kw, **hp)
+            fn = ot.step_quant_rank1_sr if stochastic else ot.step_quant_rank1
+            ref = fn(ref[0], g, *ref[1:], step=step, **kw, **hp)
+        else:
+            oc.step_quant_variants(cp.reshape(-1), _np_elem(g).reshape(-1), cm, cv, csm, csv, step=step, **kw, **hp)
+            fn = ot.step_quant_sr if stochastic else ot.step_quant
+            ref = fn(ref[0], g.reshape(-1), *ref[1:], step=step, **kw, **hp)
+        what = f"{shape} {p_dt}/{g_dt} rank1={rank1} sr={stochastic} step {step}"
+        assert np.array_equal(cm, ref[1].numpy()), f"{what}: first-moment codes"
+        assert np.array_equal(cv, ref[2].numpy()), f"{what}: second-moment codes"
+        assert np.array_equal(bits(csm), bits(ref[3].numpy())), f"{what}: first-moment scales"
+        if rank1:
+            assert np.array_equal(bits(cr), bits(ref[4].numpy())), f"{what}: row maxima"
+            assert np.array_equal(bits(cc), bits(ref[5].numpy())), f"{what}: column maxima"
+        else:
+            assert np.array_equal(bits(csv), bits(ref[4].numpy())), f"{what}: second-moment scales"
+        # parameters: the same arithmetic on both sides (numpy's correctly rounded sqrt, IEEE
+        # division), so the same bits; a NaN (from a non-finite gradient) is a NaN whatever its payload
+        got, want = cp.reshape(-1), _np_elem(ref[0]).reshape(-1)
+        as_f32 = lambda a: ((a.astype(np.uint32) << 16).view(np.float32) if a.dtype == np.uint16
+                            else a.astype(np.float32))
+        nan = np.isnan(as_f32(want))
+        assert np.array_equal(nan, np.isnan(as_f32(got))), f"{what}: NaN parameters"
+        assert np.array_equal(got[~nan].view(np.uint8), want[~nan].view(np.uint8)), f"{what}: parameters"
+
+
+def test_c_variants_without_options_is_the_fused_step():
+    """with neither option q4o_step_quant_variants must be q4o_step_quant, bit for bit"""
+    gen = torch.Generator().manual_seed(3)
+    n = 128 * 37 + 19
+    p0 = (torch.randn(n, generator=gen) * 0.02).numpy()
+    nbytes, nblk = oc.state_sizes(n)
+    a = [p0.copy(), np.zeros(nbytes, np.uint8), np.zeros(nbytes, np.uint8), np.zeros(nblk, np.float32), np.zeros(nblk, np.float32)]
+    b = [x.copy() for x in a]
+    for step in range(1, 5):
+        g = grads_config1(gen, n).numpy()
+        oc.step_quant(a[0], g, *a[1:], step=step, **HP)
+        oc.step_quant_variants(b[0], g, *b[1:], step=step, **HP)
+        for x, y in zip(a, b):
+            assert np.array_equal(x.view(np.uint8), y.view(np.uint8)), step
+
+
+def test_c_noise_and_salt_are_the_vectorised_ones():
+    for seed, step, salt in ((0, 1, 0), (2 ** 64 - 1, 123456, 2 ** 32 - 1), (0x1234_5678_9ABC_DEF0, 7, 3)):
+        s = ot.sr_tensor_salt(seed, step, salt)
+        assert oc.sr_tensor_salt(seed, step, salt) == s
+        um, uv = ot.sr_noise(300, s)
+        for e in (0, 1, 2, 17, 255, 299):
+            assert oc.sr_noise(e, s) == (float(um[e]), float(uv[e]))
+    # beyond 2^32 elements the high half of the index enters the hash
+    e = (1 << 32) + 12345
+    key = (np.uint64(e) & ot._M32) ^ np.uint64(77) ^ ((np.uint64(e >> 32) * np.uint64(0x9E3779B9)) & ot._M32)
+    h = int(ot.lowbias32(key))
+    assert oc.sr_noise(e, 77) == ((2 * (h >> 16) + 1) / 2 ** 17, (2 * (h & 0xFFFF) + 1) / 2 ** 17)
