@@ -210,3 +210,54 @@ def test_sr_non_finite_gradients(cuda):
         for name, d, r in (("m scales", dev.sm, ref[3]), ("v scales", dev.sv, ref[4])):
             assert torch.equal(d.cpu().view(torch.int32), r.view(torch.int32)), f"step {step}: {name}"
         ref = (dev.p.cpu().clone(),) + tuple(ref[1:])
+
+
+@pytest.mark.parametrize("rank1", [False, True])
+@pytest.mark.parametrize("stochastic", [False, True])
+@pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16")])
+def test_variants_against_the_scalar_c_oracle(cuda, p_dt, g_dt, stochastic, rank1):
+    """the HIP step's variants against q4o_step_quant_variants, the scalar C loops, directly
+    (the other tests of this file and of test_gpu_rank1.py go through the vectorised torch
+    restatement): codes, scales and statistics bit for bit over four steps of a 96 x 2432 matrix"""
+    from oracle import q4_oracle as oc
+    rows, cols = 96, 2432
+    n = rows * cols
+    gen = torch.Generator().manual_seed(99)
+    p0 = (torch.randn(rows, cols, generator=gen) * 0.05).to(DT[p_dt])
+    as_np = lambda t: (t.view(torch.int16).numpy().view(np.uint16).copy() if t.dtype == torch.bfloat16
+                       else t.numpy().copy())
+    nbytes, nblk = oc.state_sizes(n)
+    cm, cv = np.zeros(nbytes, np.uint8), np.zeros(nbytes, np.uint8)
+    csm, csv = np.zeros(nblk, np.float32), np.zeros(nblk, np.float32)
+    cr, cc = np.zeros(rows, np.float32), np.zeros(cols, np.float32)
+    p = p0.clone().to(cuda)
+    m = torch.zeros(nbytes, dtype=torch.uint8, device=cuda)
+    v = torch.zeros_like(m)
+    sm, sv = torch.zeros(nblk, device=cuda), torch.zeros(nblk, device=cuda)
+    r, c, rn, cn = (torch.zeros(k, device=cuda) for k in (rows, cols, rows, cols))
+    kw = dict(seed=SEED, tensor_salt=4) if stochastic else {}
+    for step in range(1, 5):
+        g = (grads_config1 if step % 2 else grads_config3)(gen, n).view(rows, cols).to(DT[g_dt])
+        cp = as_np(p.cpu())                     # the oracle starts every step from the device's parameters
+        prev = cp.copy()
+        if rank1:
+            oc.step_quant_variants(cp, as_np(g), cm, cv, csm, None, cr, cc, step=step, **kw, **HP)
+            q.fused_4bit_rank1_multi([p], [g.to(cuda)], [m], [v], [sm], [r], [c], [rn], [cn], *HPA, step,
+                                     **(dict(seed=SEED, salts=[4]) if stochastic else {}))
+        else:
+            oc.step_quant_variants(cp.reshape(-1), as_np(g).reshape(-1), cm, cv, csm, csv, step=step, **kw, **HP)
+            if stochastic:
+                q.fused_4bit_multi_sr([p.view(-1)], [g.to(cuda).view(-1)], [m], [v], [sm], [sv], *HPA, step, SEED, salts=[4])
+            else:
+                q.fused_4bit(p.view(-1), g.to(cuda).view(-1), m, v, sm, sv, *HPA, step)
+        torch.cuda.synchronize()
+        what = f"{p_dt}/{g_dt} sr={stochastic} rank1={rank1} step {step}"
+        assert np.array_equal(m.cpu().numpy(), cm) and np.array_equal(v.cpu().numpy(), cv), f"{what}: codes"
+        assert np.array_equal(sm.cpu().numpy().view(np.uint32), csm.view(np.uint32)), f"{what}: first-moment scales"
+        if rank1:
+            assert np.array_equal(r.cpu().numpy().view(np.uint32), cr.view(np.uint32)), f"{what}: row maxima"
+            assert np.array_equal(c.cpu().numpy().view(np.uint32), cc.view(np.uint32)), f"{what}: column maxima"
+        else:
+            assert np.array_equal(sv.cpu().numpy().view(np.uint32), csv.view(np.uint32)), f"{what}: second-moment scales"
+        ok, worst = p_close(to_np(p), cp.reshape(-1), prev.reshape(-1), bf16=p_dt == "bf16")
+        assert ok, f"{what}: parameters out of tolerance (worst {worst})"
