@@ -42,12 +42,14 @@
  *                         drafts disagree in rounding, so the bit-level choice
  *                         (unfused mul/add, fp32 derived scalars) is this build's:
  *                         bit-level parity with the reference is UNPINNED.
- *   q4o_step_quant_variants (rank-1 scaling of the second moment after
+ *   q4o_step_quant_variants (rank-1 scaling of the second moment of tensors of two and
+ *                         more dimensions after
  *                         optim/adamw_fourbit_triton.py:738-755, :520-527, :834-863;
  *                         stochastic rounding after :969-997, :1050-1075): scalar loops,
  *                         written apart from the vectorised restatement in
- *                         q4_oracle_torch.py (step_quant_rank1, step_quant_sr,
- *                         step_quant_rank1_sr), which must agree with it bit for bit;
+ *                         q4_oracle_torch.py (step_quant_rank1, step_quant_rank1_nd,
+ *                         step_quant_sr, step_quant_rank1_sr), which must agree with it
+ *                         bit for bit;
  *                         with neither option it must reproduce q4o_step_quant.  The
  *                         draft never runs either against data: parity with the
  *                         reference is UNPINNED for both.
@@ -432,37 +434,49 @@ int q4o_quantize_sr(int which, float q, float u) {
     return above - 1 + (need < dist ? 1 : 0);
 }
 
+/* scale of element i of a tensor of shape[0..ndim) under rank-1 scaling: the minimum over
+ * its dimensions' statistics (compute_variance_tensor_scale,
+ * optim/adamw_fourbit_triton.py:749-755); index[k] receives the element's index in dimension k */
+static inline float q4o_rank1_scale(int64_t i, int ndim, const int64_t *shape, float *const *stats,
+                                    int64_t *index) {
+    float s = INFINITY;
+    for (int k = ndim - 1; k >= 0; --k) {
+        index[k] = i % shape[k];
+        i /= shape[k];
+        const float t = stats[k][index[k]];
+        if (t < s) s = t;
+    }
+    return s;
+}
+
 /*
- * The fused step with its options: rank1 != 0 scales the second moment of the matrix
- * [rows, cols] by min(row maximum, column maximum) instead of per-128 block maxima
- * (v_scale is then unused; row_max / col_max hold the old statistics and receive the new
- * ones); stochastic != 0 rounds both moments stochastically with the noise of
- * (seed, step, tensor_salt).  numel = rows * cols; a flat tensor is rows = 1.
- * First pass: new moments and parameters; second pass: statistics and codes.
+ * The fused step with its options.  ndim >= 2 scales the second moment of the tensor of
+ * shape[0..ndim) by the minimum over its dimensions' statistics instead of per-128 block
+ * maxima: stats[k] holds shape[k] floats, the maximum of the second moment over all other
+ * dimensions (get_variance_tensor_statistics, optim/adamw_fourbit_triton.py:738-746); the old
+ * ones dequantize, the new ones are left in their place; v_scale is then unused.  A matrix is
+ * ndim = 2 with stats = {row maxima, column maxima}; ndim = 0 is the block-scaled step.
+ * stochastic != 0 rounds both moments stochastically with the noise of (seed, step,
+ * tensor_salt).  First pass: new moments and parameters; second pass: statistics and codes.
  */
 void q4o_step_quant_variants(void *p, const void *g, uint8_t *m_codes, uint8_t *v_codes,
-                             float *m_scale, float *v_scale, float *row_max, float *col_max,
-                             int64_t rows, int64_t cols, int p_dtype, int g_dtype,
+                             float *m_scale, float *v_scale, float *const *stats,
+                             const int64_t *shape, int ndim, int64_t numel, int p_dtype, int g_dtype,
                              float beta1, float beta2, float lr, float weight_decay, float eps,
-                             float step, int rank1, int stochastic, uint64_t seed,
+                             float step, int stochastic, uint64_t seed,
                              uint32_t tensor_salt, float *scratch /* 2 * numel floats */) {
     float sc[6];
     q4o_derive_scalars(beta1, beta2, lr, weight_decay, step, sc);
     const float c2s = sc[1], ss = sc[2], wdu = sc[3], r1 = sc[4], r2 = sc[5];
-    const int64_t numel = rows * cols;
+    const int rank1 = ndim >= 2;
+    int64_t index[8];
     float *mn = scratch, *vn = scratch + numel;
     const uint32_t salt = stochastic ? q4o_sr_tensor_salt(seed, (uint32_t)step, tensor_salt) : 0u;
     for (int64_t i = 0; i < numel; ++i) {
         const uint8_t mb = m_codes[i >> 1], vb = v_codes[i >> 1];
         const int cm = (i & 1) ? (mb >> 4) : (mb & 15);
         const int cv = (i & 1) ? (vb >> 4) : (vb & 15);
-        float v_old_scale;
-        if (rank1) {
-            const float r = row_max[i / cols], c = col_max[i % cols];
-            v_old_scale = r < c ? r : c;
-        } else {
-            v_old_scale = v_scale[i / Q4O_BLOCK];
-        }
+        const float v_old_scale = rank1 ? q4o_rank1_scale(i, ndim, shape, stats, index) : v_scale[i / Q4O_BLOCK];
         const float gi = load_elem(g, g_dtype, i);
         volatile float m = Q4O_QMAP_M[cm] * m_scale[i / Q4O_BLOCK];
         volatile float v = Q4O_QMAP_V[cv] * v_old_scale;
@@ -491,23 +505,21 @@ void q4o_step_quant_variants(void *p, const void *g, uint8_t *m_codes, uint8_t *
         if (!rank1) v_scale[b] = sv;
     }
     if (rank1) {
-        for (int64_t r = 0; r < rows; ++r) row_max[r] = 0.0f;
-        for (int64_t c = 0; c < cols; ++c) col_max[c] = 0.0f;
+        for (int k = 0; k < ndim; ++k)
+            for (int64_t j = 0; j < shape[k]; ++j) stats[k][j] = 0.0f;
         for (int64_t i = 0; i < numel; ++i) {
             const float av = fabsf(vn[i]);
-            if (av > row_max[i / cols]) row_max[i / cols] = av;
-            if (av > col_max[i % cols]) col_max[i % cols] = av;
+            int64_t rem = i;
+            for (int k = ndim - 1; k >= 0; --k) {
+                const int64_t j = rem % shape[k];
+                rem /= shape[k];
+                if (av > stats[k][j]) stats[k][j] = av;
+            }
         }
     }
     /* codes */
     for (int64_t i = 0; i < numel; ++i) {
-        float sv;
-        if (rank1) {
-            const float r = row_max[i / cols], c = col_max[i % cols];
-            sv = r < c ? r : c;
-        } else {
-            sv = v_scale[i / Q4O_BLOCK];
-        }
+        const float sv = rank1 ? q4o_rank1_scale(i, ndim, shape, stats, index) : v_scale[i / Q4O_BLOCK];
         volatile float qm = mn[i] / m_scale[i / Q4O_BLOCK];
         volatile float qv = vn[i] / sv;
         int code_m, code_v;

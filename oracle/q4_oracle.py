@@ -52,8 +52,8 @@ def lib():
         L.q4o_dequant.argtypes = [vp, vp, i64, ci, vp]
         L.q4o_quant.argtypes = [vp, i64, ci, vp, vp]
         u32, u64 = ctypes.c_uint32, ctypes.c_uint64
-        L.q4o_step_quant_variants.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, ci, ci, f, f, f, f, f, f,
-                                              ci, ci, u64, u32, vp]
+        L.q4o_step_quant_variants.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, i64, ci, ci, f, f, f, f, f, f,
+                                              ci, u64, u32, vp]
         L.q4o_sr_tensor_salt.argtypes = [u64, u32, u32]
         L.q4o_sr_tensor_salt.restype = u32
         L.q4o_sr_noise.argtypes = [i64, u32, vp, vp]
@@ -136,29 +136,33 @@ def step_quant(p, g, m_codes, v_codes, m_scale, v_scale, *, beta1, beta2, lr,
 
 
 def step_quant_variants(p, g, m_codes, v_codes, m_scale, v_scale=None, row_max=None, col_max=None, *, beta1,
-                        beta2, lr, weight_decay, eps, step, seed=None, tensor_salt=0):
-    """The fused step with its options, in place: row_max / col_max given (p a [rows, cols]
-    matrix) = rank-1 scaled second moment, else v_scale = per-128 block scales; seed given =
-    stochastic rounding with the noise of (seed, step, tensor_salt)."""
-    rank1 = row_max is not None
-    rows, cols = p.shape if rank1 else (1, p.size)
-    n = rows * cols
+                        beta2, lr, weight_decay, eps, step, seed=None, tensor_salt=0, max_dims=None):
+    """The fused step with its options, in place.  row_max / col_max given (p a [rows, cols]
+    matrix), or max_dims = one float32 array per dimension of p: rank-1 scaled second moment;
+    else v_scale = per-128 block scales.  seed given = stochastic rounding with the noise of
+    (seed, step, tensor_salt)."""
+    if row_max is not None:
+        max_dims = [row_max, col_max]
+    rank1 = max_dims is not None
+    n = p.size
     nbytes, nblk = state_sizes(n)
     assert g.size == n and m_codes.size == nbytes and v_codes.size == nbytes and m_scale.size == nblk
     assert m_codes.dtype == np.uint8 and v_codes.dtype == np.uint8 and m_scale.dtype == np.float32
-    if rank1:
-        assert row_max.size == rows and col_max.size == cols
-        assert row_max.dtype == np.float32 and col_max.dtype == np.float32 and v_scale is None
-    else:
-        assert v_scale.size == nblk and v_scale.dtype == np.float32
-    for a in (p, g, m_codes, v_codes, m_scale, v_scale, row_max, col_max):
-        assert a is None or a.flags.c_contiguous
-    scratch = np.empty(2 * n, np.float32)
     none = ctypes.c_void_p(0)
+    if rank1:
+        assert v_scale is None and len(max_dims) == p.ndim >= 2
+        assert all(s.size == d and s.dtype == np.float32 and s.flags.c_contiguous for s, d in zip(max_dims, p.shape))
+        shape = (ctypes.c_int64 * p.ndim)(*p.shape)
+        stats = (ctypes.c_void_p * p.ndim)(*[s.ctypes.data for s in max_dims])
+    else:
+        assert v_scale.size == nblk and v_scale.dtype == np.float32 and v_scale.flags.c_contiguous
+        shape, stats = none, none
+    for a in (p, g, m_codes, v_codes, m_scale):
+        assert a.flags.c_contiguous
+    scratch = np.empty(2 * n, np.float32)
     lib().q4o_step_quant_variants(_ptr(p), _ptr(g), _ptr(m_codes), _ptr(v_codes), _ptr(m_scale),
-                                  none if rank1 else _ptr(v_scale), _ptr(row_max) if rank1 else none,
-                                  _ptr(col_max) if rank1 else none, rows, cols, _dtype_tag(p), _dtype_tag(g),
-                                  beta1, beta2, lr, weight_decay, eps, float(step), int(rank1),
+                                  none if rank1 else _ptr(v_scale), stats, shape, p.ndim if rank1 else 0, n,
+                                  _dtype_tag(p), _dtype_tag(g), beta1, beta2, lr, weight_decay, eps, float(step),
                                   int(seed is not None), int(seed or 0) & (2 ** 64 - 1),
                                   int(tensor_salt) & 0xFFFFFFFF, _ptr(scratch))
 

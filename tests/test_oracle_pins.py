@@ -715,3 +715,30 @@ def test_c_noise_and_salt_are_the_vectorised_ones():
     key = (np.uint64(e) & ot._M32) ^ np.uint64(77) ^ ((np.uint64(e >> 32) * np.uint64(0x9E3779B9)) & ot._M32)
     h = int(ot.lowbias32(key))
     assert oc.sr_noise(e, 77) == ((2 * (h >> 16) + 1) / 2 ** 17, (2 * (h & 0xFFFF) + 1) / 2 ** 17)
+
+
+@pytest.mark.parametrize("stochastic", [False, True])
+@pytest.mark.parametrize("p_dt,g_dt", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("shape", [(4, 6, 64), (3, 5, 24), (2, 3, 4, 32), (5, 1, 2, 40), (7, 33)])
+def test_c_and_torch_restatements_agree_on_more_than_two_dimensions(shape, p_dt, g_dt, stochastic):
+    """one statistic per dimension, scale = their minimum: q4o_step_quant_variants against
+    step_quant_rank1_nd, every dimension's statistic bit for bit over three steps"""
+    n = int(np.prod(shape))
+    p, grads = _variant_inputs(n // shape[-1], shape[-1], p_dt, g_dt, sum(shape))
+    p = p.view(shape)
+    nbytes, nblk = oc.state_sizes(n)
+    cp = _np_elem(p)
+    cm, cv, csm = np.zeros(nbytes, np.uint8), np.zeros(nbytes, np.uint8), np.zeros(nblk, np.float32)
+    cdims = [np.zeros(d, np.float32) for d in shape]
+    ref = (p.clone(), torch.zeros(nbytes, dtype=torch.uint8), torch.zeros(nbytes, dtype=torch.uint8), torch.zeros(nblk),
+           [torch.zeros([d if j == i else 1 for j, d in enumerate(shape)]) for i in range(len(shape))])
+    kw = dict(seed=0xFEED_FACE_0000_0001, tensor_salt=9) if stochastic else {}
+    for step, g in enumerate(grads, 1):
+        g = g.view(shape)
+        oc.step_quant_variants(cp, _np_elem(g), cm, cv, csm, max_dims=cdims, step=step, **kw, **HP)
+        ref = ot.step_quant_rank1_nd(ref[0], g, *ref[1:], step=step, **kw, **HP)
+        what = f"{shape} {p_dt}/{g_dt} sr={stochastic} step {step}"
+        assert np.array_equal(cm, ref[1].numpy()) and np.array_equal(cv, ref[2].numpy()), f"{what}: codes"
+        assert np.array_equal(bits(csm), bits(ref[3].numpy())), f"{what}: first-moment scales"
+        for k, (mine, theirs) in enumerate(zip(cdims, ref[4])):
+            assert np.array_equal(bits(mine), bits(theirs.reshape(-1).numpy())), f"{what}: statistic of dimension {k}"
