@@ -59,6 +59,35 @@ def test_driver_mlp_default_threshold(cuda):
         assert opt.state[p]["exp_avg"].dtype == torch.float32 and float(opt.state[p]["step"]) == 10.0
 
 
+def test_adam_equivalence_alternating_zero_grad(cuda):
+    """tests/test_4bit_AdamW.py:29-72 (_test_adam_equivalence, test_adam_equivalence_gpu) as it
+    was meant to run: three small Linear layers, betas (0.8, 0.88), weight decay 0.03, six
+    iterations that clear the gradients alternately in place and by dropping them, parameters
+    equal to torch.optim.AdamW's under assert_close's default tolerance after every step."""
+    torch.manual_seed(2020)
+    model = nn.Sequential(nn.Linear(5, 10), nn.Linear(10, 10), nn.Linear(10, 5)).cuda()
+    clone = deepcopy(model)
+    betas, weight_decay = (0.8, 0.88), 0.03
+    adam = torch.optim.AdamW(clone.parameters(), betas=betas, weight_decay=weight_decay)
+    opt = AdamWFused_QuantFour(model.parameters(), betas=betas, weight_decay=weight_decay)
+    orig = [p.clone() for p in model.parameters()]
+    for p1, p2 in zip(clone.parameters(), orig):
+        torch.testing.assert_close(p1, p2)
+    for i in range(6):
+        adam.zero_grad(set_to_none=bool(i % 2))
+        opt.zero_grad(set_to_none=bool(i % 2))
+        inp = torch.randn(5, 5, device="cuda")
+        model(inp).sum().backward()
+        clone(inp).sum().backward()
+        adam.step()
+        opt.step()
+        if i == 0:
+            for p1, p2 in zip(model.parameters(), orig):
+                assert not torch.equal(p1, p2)
+        for p1, p2 in zip(model.parameters(), clone.parameters()):
+            torch.testing.assert_close(p1, p2)
+
+
 def test_driver_mlp_forced_quantization(cuda):
     """Same loop with every tensor forced onto the 4-bit path (threshold 0), and a wider MLP
     whose weight matrices are quantized at the default threshold.  With betas (0.8, 0.88)
