@@ -91,7 +91,7 @@ def test_random_configuration_stochastic_rounding(cuda, i):
 @pytest.mark.parametrize("i", list(range(24)) + EXTRA)
 def test_random_configuration_rank1(cuda, i):
     """every third case adds stochastic rounding (random seed and salt), every fourth has rows
-    of whole tiles"""
+    of whole tiles, every eighth rows of whole blocks that end in a partial tile"""
     from oracle import q4_oracle_torch as ot
     from quantfour_adamw_cuda_amd import quantfour_hip as q
     from tests.q4_testlib import p_close, to_np
@@ -99,6 +99,8 @@ def test_random_configuration_rank1(cuda, i):
     rows, cols = int(rng.integers(1, 90)), 8 * int(rng.integers(2, 300))     # narrow matrices included
     if i % 4 == 1:      # rows of whole tiles, enough of them: the update kernel that shares column maxima
         rows, cols = rows + 63, 256 * (2 + cols % 7)
+    elif i % 8 == 3:    # the same kernel with a partial last tile: 17 to 63 blocks of 128 columns
+        rows, cols = 64 + rows % 8, 128 * (17 + cols % 47)
     sr = dict(seed=int(rng.integers(0, 2 ** 63)), tensor_salt=int(rng.integers(0, 2 ** 32))) if i % 3 == 2 else None
     print(f"[sweep rank1 {i}] {rows}x{cols} p={p_dt} g={g_dt} hp={hp} step0={first_step} sr={sr}", flush=True)
     n = rows * cols
