@@ -336,9 +336,10 @@ def load_probe():
     return L
 
 
-def measure_ceiling(torch, device, reps=10):
-    """Median over `reps` launches (after 3 untimed ones) of each probe on 2^30 elements,
-    events on the launch stream around every launch."""
+def measure_ceiling(torch, device, reps=20):
+    """Best of `reps` launches (after 3 untimed ones) of each probe on 2^30 elements, events on
+    the launch stream around every launch.  The best, not the median: the figure stands for
+    what the memory system can give such a kernel, and the step is compared with it."""
     L = load_probe()
     n = 1 << 30
     stream = torch.cuda.current_stream(device).cuda_stream
@@ -363,10 +364,14 @@ def measure_ceiling(torch, device, reps=10):
             e.record()
             evs.append((s, e))
         torch.cuda.synchronize()
-        ms = sorted(s.elapsed_time(e) for s, e in evs)
-        return ms[len(ms) // 2] / 1e3
+        return min(s.elapsed_time(e) for s, e in evs) / 1e3
 
-    out = {"unit": "GB/s", "elements": n, "launches": reps, "statistic": "median",
+    # the probes follow configurations of small kernels: bring the clocks back up first
+    for _ in range(40):
+        assert L.q4probe_copy(b.data_ptr(), a.data_ptr(), 4 * n, stream) == 0, "probe launch failed"
+    torch.cuda.synchronize()
+
+    out = {"unit": "GB/s", "elements": n, "launches": reps, "statistic": "best",
            "kernels": "libq4probe.so: probe_move_kernel (copy, read), probe_step_streams_kernel"}
     t = timed(lambda: L.q4probe_copy(b.data_ptr(), a.data_ptr(), 4 * n, stream))
     out["copy"] = 8.0 * n / t / 1e9
