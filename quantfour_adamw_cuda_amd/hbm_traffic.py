@@ -10,15 +10,16 @@ Recording (rocprofv3 cannot split counters over passes, so one run per counter; 
 machine, from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd -`):
 
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/pmc_fetch -o fetch -- \\
-        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy
+        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy --progress
     rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o write -- \\
-        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy
+        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy --progress
     python3 -m quantfour_adamw_cuda_amd.hbm_traffic --workload llama3-8b --steps 4 \\
         --fetch-csv 'out/pmc_fetch/**/*counter_collection.csv' \\
         --write-csv 'out/pmc_write/**/*counter_collection.csv' \\
         --out profiles/hbm_traffic.json
 
-(add the bench's --workload / --variance-scale / --round-type options to all three).  Both
+(add the bench's --workload / --variance-scale / --round-type options to all three; --progress
+names the bench's phases on stderr, so that a profiler run that stops shows where).  Both
 counters are in KiB per dispatch; each is scaled by what the same counter reads for the
 probe library's plain copy of 4 GiB (--calibrate-copy), whose traffic is known.
 """
