@@ -195,9 +195,11 @@ def build_inputs(torch, device, shapes, p_dtype, g_dtype, dist, grad_sets):
 
 
 def run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, steps, warmup, variance_scale="group",
-               round_type="real-nearest", clip="none"):
+               round_type="real-nearest", clip="none", host_burst=True):
     """W warm-up steps, then exactly K timed steps between two synchronisations, with a fresh
-    optimizer over `params`.  Returns the measurements of the timed region."""
+    optimizer over `params`.  Returns the measurements of the timed region.  host_burst=False
+    leaves out the extra steps that measure the host time of step() (host_ms_per_step is then
+    None): W + K steps run and no others, which a counter profile of the run relies on."""
     from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
     opt = AdamWFused_QuantFour(params, variance_scale_type=variance_scale, round_type=round_type, seed=0, **HP)
     opt.kernel_timing = []  # (kind, start event, end event) per launch
@@ -246,14 +248,16 @@ def run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, steps, warmup, va
     # period costs more).  Inside the timed region the device is the slower side, the launch
     # queue fills, and the time a launch call spends waiting for room would be counted as the
     # host's; the burst stays under 200 launches for the same reason.
-    small = sum(1 for p in params if p.numel() <= 4096)
-    burst = max(2, min(steps, 16, 192 // (launches_per_step + -(-small // 80)) - 2))
-    for i in range(2 + burst):
-        if i == 2:
-            host_s[0] = 0.0
-        one_step(warmup + steps + i)
-    host_ms_per_step = host_s[0] / burst * 1e3
-    torch.cuda.synchronize()
+    host_ms_per_step = None
+    if host_burst:
+        small = sum(1 for p in params if p.numel() <= 4096)
+        burst = max(2, min(steps, 16, 192 // (launches_per_step + -(-small // 80)) - 2))
+        for i in range(2 + burst):
+            if i == 2:
+                host_s[0] = 0.0
+            one_step(warmup + steps + i)
+        host_ms_per_step = host_s[0] / burst * 1e3
+        torch.cuda.synchronize()
 
     quant_params = sum(p.numel() for p in params if p.numel() > 4096)
     algo_bytes = quant_params * bytes_per_param(p_dtype_s, g_dtype_s)
@@ -437,8 +441,9 @@ def main():
                     help="name every phase on stderr as it ends (stdout keeps its one JSON line), so that a "
                          "run that stops under a profiler shows where")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="after the timed region, run the probe library's plain 4 GiB copy three times, "
-                         "so that a counter profile of this command also holds a kernel of known traffic")
+                    help="for counter profiles: after the timed region, run the probe library's plain 4 GiB "
+                         "copy three times, so that the profile also holds a kernel of known traffic, and run "
+                         "W + K steps and no others (no host-time burst)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the optimizer step on ONE GPU; the step needs "
@@ -465,7 +470,7 @@ def main():
                                      getattr(torch, g_dtype_s), dist, args.grad_sets)
     phase(f"inputs of {args.workload} built")
     m = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, args.steps, args.warmup,
-                   args.variance_scale, args.round_type, args.clip)
+                   args.variance_scale, args.round_type, args.clip, host_burst=not args.calibrate_copy)
     phase("headline steps timed")
     if args.calibrate_copy:
         calibrate_copy(torch, device)
