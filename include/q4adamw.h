@@ -111,14 +111,39 @@ typedef struct q4adamw_small_tensor {
  *                    (the `g` pointers are written in that case), also by a call
  *                    that skip_if_nonzero cancels: the overflowed gradients must
  *                    not reach the next accumulation.
+ *   update_form      how the quantized step computes the parameter
+ *                    (optim/cuda_adamw_kernels.cu:334,351:
+ *                    p * wdu - step_size * (m / (sqrtf(v) / correction2_sqrt + eps))):
+ *                    Q4ADAMW_UPDATE_EXACT   those seven operations, each rounded as IEEE 754
+ *                                           rounds it (nvcc's defaults for sqrtf and /): the
+ *                                           parameters come out bit for bit as that expression
+ *                                           gives them;
+ *                    Q4ADAMW_UPDATE_FOLDED  p * wdu - m * rcp(sqrt(v) * A + B), step size and
+ *                                           bias correction folded into A and B, hardware
+ *                                           square root and reciprocal (one ulp each): fp32
+ *                                           parameters within 1e-6 of max(|p|, |step taken|),
+ *                                           16-bit parameters within one ulp of their type;
+ *                    Q4ADAMW_UPDATE_AUTO    (0) exact for fp32 parameters in the block-scaled
+ *                                           step with nearest rounding, where it costs under
+ *                                           1 % of the step; folded for 16-bit parameters,
+ *                                           stochastic rounding and rank-1 scaling, where it
+ *                                           costs 5 to 10 %.
+ *                    Codes and scales do not depend on it.  The non-quantized step always
+ *                    computes the exact form.  Entry points without options take AUTO.
  * The device scalars are read when the kernels run, not when the call returns.
  */
+#define Q4ADAMW_UPDATE_AUTO 0
+#define Q4ADAMW_UPDATE_EXACT 1
+#define Q4ADAMW_UPDATE_FOLDED 2
+
 typedef struct q4adamw_grad_options {
   float grad_scale;
   int zero_grad;
   const float *grad_scale_dev;
   const float *skip_if_nonzero;
   const void *step_consts;
+  int update_form;
+  int reserved; /* 0 */
 } q4adamw_grad_options;
 
 /* One gradient tensor for q4adamw_grad_norm: numel elements, aligned to the element type. */

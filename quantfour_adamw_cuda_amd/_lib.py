@@ -67,6 +67,8 @@ class Q4GradOptions(ctypes.Structure):
         ("grad_scale_dev", ctypes.c_void_p),
         ("skip_if_nonzero", ctypes.c_void_p),
         ("step_consts", ctypes.c_void_p),
+        ("update_form", ctypes.c_int),
+        ("reserved", ctypes.c_int),
     ]
 
 
@@ -80,6 +82,9 @@ class Q4Grad(ctypes.Structure):
 
 NORM_WORKSPACE_BYTES = 16384
 STEP_CONSTS_BYTES = 64
+# q4adamw_grad_options.update_form (include/q4adamw.h)
+UPDATE_AUTO, UPDATE_EXACT, UPDATE_FOLDED = 0, 1, 2
+UPDATE_FORMS = {"auto": UPDATE_AUTO, "exact": UPDATE_EXACT, "folded": UPDATE_FOLDED}
 
 EXPORTS = (
     "q4adamw_fused_4bit",

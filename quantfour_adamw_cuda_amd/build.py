@@ -10,6 +10,7 @@ Usage:  python -m quantfour_adamw_cuda_amd.build
 import os
 import shutil
 import subprocess
+import tempfile
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libq4adamw.so")
@@ -28,8 +29,14 @@ HIPCC_FLAGS = [
     # same option, says that x86 does not know the feature and ignores it.  That message is
     # the only output of a clean build.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-shared", "-fPIC",
+    "-fPIC",
 ]
+
+# libq4adamw.so: the C ABI with its launchers and small kernels, and the step kernels'
+# instantiations in translation units of their own, compiled side by side
+STEP_SOURCES = ["q4adamw.hip", "q4adamw_pick_fused.hip", "q4adamw_pick_rank1_rows.hip",
+                "q4adamw_pick_rank1_wide.hip", "q4adamw_pick_rank1_narrow.hip"]
+PROBE_SOURCES = ["q4stream_probe.hip"]
 
 
 def hipcc_path():
@@ -39,25 +46,52 @@ def hipcc_path():
     raise RuntimeError("hipcc not found (set HIPCC or install ROCm)")
 
 
-def _compile(out, source, verbose):
-    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-o", out, os.path.join(CSRC, source)]
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+def _checked(proc, what, verbose):
     # anything besides the host pass's note about the device-only feature is a real diagnostic
     noise = [ln for ln in proc.stdout.splitlines() if ln.strip() and ln.strip() != HOST_PASS_NOTE]
     if verbose or proc.returncode != 0:
         print(proc.stdout)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + proc.stdout)
+        raise RuntimeError(f"hipcc failed for {what}:\n" + proc.stdout)
     if noise:
-        raise RuntimeError(f"hipcc printed diagnostics for {source}; the build is kept warning-free:\n"
+        raise RuntimeError(f"hipcc printed diagnostics for {what}; the build is kept warning-free:\n"
                            + "\n".join(noise))
+
+
+def compile_library(out, sources, flags=None, verbose=False, check_output=True):
+    """Compiles every source to an object file (all at once, one hipcc each) and links them
+    into the shared library `out`.  flags: hipcc options in place of HIPCC_FLAGS."""
+    flags = HIPCC_FLAGS if flags is None else flags
+    hipcc = hipcc_path()
+    with tempfile.TemporaryDirectory(prefix="q4adamw_build_") as tmp:
+        jobs = []
+        for src in sources:
+            obj = os.path.join(tmp, os.path.splitext(src)[0] + ".o")
+            cmd = [hipcc] + flags + ["-c", "-o", obj, os.path.join(CSRC, src)]
+            jobs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs = []
+        for src, obj, job in jobs:
+            job.stdout_text = job.communicate()[0]
+        for src, obj, job in jobs:
+            proc = subprocess.CompletedProcess(job.args, job.returncode, job.stdout_text)
+            if check_output:
+                _checked(proc, src, verbose)
+            elif proc.returncode != 0:
+                raise RuntimeError(f"hipcc failed for {src}:\n" + proc.stdout)
+            objs.append(obj)
+        link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs,
+                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if check_output:
+            _checked(link, os.path.basename(out), verbose)
+        elif link.returncode != 0:
+            raise RuntimeError("link failed:\n" + link.stdout)
     return out
 
 
 def build(verbose=False):
     """Compile unconditionally; returns the path of the step library."""
-    _compile(LIB, "q4adamw.hip", verbose)
-    _compile(PROBE_LIB, "q4stream_probe.hip", verbose)
+    compile_library(LIB, STEP_SOURCES, verbose=verbose)
+    compile_library(PROBE_LIB, PROBE_SOURCES, verbose=verbose)
     return LIB
 
 

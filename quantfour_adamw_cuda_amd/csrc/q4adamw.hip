@@ -3,7 +3,9 @@
 //   q4adamw_tables.h  code books, thresholds, bucket and interval tables (constexpr)
 //   q4adamw_args.h    kernel argument structs and the device copies of the tables
 //   q4adamw_device.h  device helpers
-//   q4adamw_step.h    the fused step (block-scaled, stochastic rounding, rank-1)
+//   q4adamw_step.h    the fused step (block-scaled, stochastic rounding, rank-1); its kernels are
+//                     instantiated in q4adamw_pick_*.hip (q4adamw_pick.h)
+//   q4adamw_rank1.h   rank-1 scaling: statistics, commit, folds
 //   q4adamw_aux.h     small-tensor step, gradient norm, quantize / dequantize
 //
 // Build: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off -shared -fPIC
@@ -42,6 +44,8 @@
 #include "q4adamw_args.h"
 #include "q4adamw_aux.h"
 #include "q4adamw_device.h"
+#include "q4adamw_pick.h"
+#include "q4adamw_rank1.h"
 #include "q4adamw_step.h"
 #include "q4adamw_tables.h"
 
@@ -90,6 +94,7 @@ static int make_consts(float beta1, float beta2, float lr, float wd, float eps, 
   const bool fits = den_scale <= (double)FLT_MAX && den_eps <= (double)FLT_MAX;
   out->den_scale = fits ? (float)den_scale : 0.0f;
   out->den_eps = fits ? (float)den_eps : INFINITY;
+  make_exact_consts(out);
   return 0;
 }
 
@@ -127,34 +132,6 @@ static int launch_small_batch(SmallArgs &a, uint64_t chunks, void (*kernel)(cons
   return 0;
 }
 
-typedef void (*FusedKernel)(const FusedArgs);
-typedef void (*SmallKernel)(const SmallArgs);
-
-// Kernel of a family for the (parameter, gradient) element types of a call: the tags
-// 0 = fp32, 1 = bf16, 2 = fp16 become template arguments.
-#define Q4_PICK_PG(KERNEL, ...)                                                   \
-  switch (p_dtype * 3 + g_dtype) {                                                \
-    case 0: return KERNEL<0, 0, __VA_ARGS__>;                                     \
-    case 1: return KERNEL<0, 1, __VA_ARGS__>;                                     \
-    case 2: return KERNEL<0, 2, __VA_ARGS__>;                                     \
-    case 3: return KERNEL<1, 0, __VA_ARGS__>;                                     \
-    case 4: return KERNEL<1, 1, __VA_ARGS__>;                                     \
-    case 5: return KERNEL<1, 2, __VA_ARGS__>;                                     \
-    case 6: return KERNEL<2, 0, __VA_ARGS__>;                                     \
-    case 7: return KERNEL<2, 1, __VA_ARGS__>;                                     \
-    default: return KERNEL<2, 2, __VA_ARGS__>;                                    \
-  }
-
-template <bool EXT, bool SR>
-static FusedKernel pick_fused_ext(int p_dtype, int g_dtype) {
-  Q4_PICK_PG(fused_4bit_kernel, EXT, SR)
-}
-
-static FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext, bool sr = false) {
-  if (sr) return ext ? pick_fused_ext<true, true>(p_dtype, g_dtype) : pick_fused_ext<false, true>(p_dtype, g_dtype);
-  return ext ? pick_fused_ext<true, false>(p_dtype, g_dtype) : pick_fused_ext<false, false>(p_dtype, g_dtype);
-}
-
 template <bool EXT>
 static SmallKernel pick_small_ext(int p_dtype, int g_dtype) {
   Q4_PICK_PG(single_tensor_kernel, EXT)
@@ -162,35 +139,6 @@ static SmallKernel pick_small_ext(int p_dtype, int g_dtype) {
 
 static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
   return ext ? pick_small_ext<true>(p_dtype, g_dtype) : pick_small_ext<false>(p_dtype, g_dtype);
-}
-
-typedef void (*Rank1Kernel)(const Rank1Args);
-typedef void (*Rank1StatKernel)(const Rank1StatArgs);
-
-template <bool EXT, bool SR, bool NARROW>
-static Rank1Kernel pick_rank1_ext(int p_dtype, int g_dtype) {
-  Q4_PICK_PG(fused_4bit_rank1_kernel, EXT, SR, NARROW)
-}
-
-// narrow: the kernel for matrices whose rows are shorter than a tile
-static Rank1Kernel pick_rank1(int p_dtype, int g_dtype, bool ext, bool sr, bool narrow) {
-  if (narrow) {
-    if (sr) return ext ? pick_rank1_ext<true, true, true>(p_dtype, g_dtype) : pick_rank1_ext<false, true, true>(p_dtype, g_dtype);
-    return ext ? pick_rank1_ext<true, false, true>(p_dtype, g_dtype) : pick_rank1_ext<false, false, true>(p_dtype, g_dtype);
-  }
-  if (sr) return ext ? pick_rank1_ext<true, true, false>(p_dtype, g_dtype) : pick_rank1_ext<false, true, false>(p_dtype, g_dtype);
-  return ext ? pick_rank1_ext<true, false, false>(p_dtype, g_dtype) : pick_rank1_ext<false, false, false>(p_dtype, g_dtype);
-}
-
-template <bool EXT, bool SR>
-static Rank1Kernel pick_rank1_rows_ext(int p_dtype, int g_dtype) {
-  Q4_PICK_PG(fused_4bit_rank1_rows_kernel, EXT, SR)
-}
-
-// the kernel for matrices whose rows are a whole number of tiles long
-static Rank1Kernel pick_rank1_rows(int p_dtype, int g_dtype, bool ext, bool sr) {
-  if (sr) return ext ? pick_rank1_rows_ext<true, true>(p_dtype, g_dtype) : pick_rank1_rows_ext<false, true>(p_dtype, g_dtype);
-  return ext ? pick_rank1_rows_ext<true, false>(p_dtype, g_dtype) : pick_rank1_rows_ext<false, false>(p_dtype, g_dtype);
 }
 
 // Which of the three update kernels a matrix takes, in the order of the launch passes.
@@ -233,14 +181,18 @@ static Rank1StatKernel pick_rank1_stats(int g_dtype, bool ext) {
 
 // Fills the kernels' view of the caller's gradient options; returns whether the
 // launch needs the EXT kernels (false: the options change nothing).
-static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext) {
+static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext, int *update_form) {
   go->scale = 1.0f;
   go->zero = 0u;
   go->scale_dev = nullptr;
   go->skip = nullptr;
   go->sc_dev = nullptr;
   *ext = false;
+  *update_form = Q4ADAMW_UPDATE_AUTO;
   if (!opt) return 0;
+  if (opt->update_form < Q4ADAMW_UPDATE_AUTO || opt->update_form > Q4ADAMW_UPDATE_FOLDED)
+    return fail(Q4ADAMW_ERR_ARG, "update_form must be Q4ADAMW_UPDATE_AUTO, Q4ADAMW_UPDATE_EXACT or Q4ADAMW_UPDATE_FOLDED");
+  *update_form = opt->update_form;
   if (opt->step_consts && (reinterpret_cast<uintptr_t>(opt->step_consts) & 15))
     return fail(Q4ADAMW_ERR_ALIGN, "step_consts must be 16-byte aligned");
   if (opt->grad_scale_dev && (reinterpret_cast<uintptr_t>(opt->grad_scale_dev) & 3))
@@ -255,6 +207,18 @@ static int make_grad_ops(const q4adamw_grad_options *opt, GradOps *go, bool *ext
   *ext = opt->grad_scale != 1.0f || opt->zero_grad || opt->grad_scale_dev || opt->skip_if_nonzero ||
          opt->step_consts;
   return 0;
+}
+
+// Whether a call takes the kernels whose parameter update rounds every operation as IEEE 754
+// does.  Left to the library (Q4ADAMW_UPDATE_AUTO) that is the case where it costs under one
+// per cent of the step: fp32 parameters in the block-scaled step with nearest rounding -- the
+// reference's fused path itself (optim/cuda_adamw_kernels.cu:266-419).  Elsewhere the folded
+// form runs unless the caller asks (16-bit parameters +9 %, stochastic rounding +10 %, rank-1
+// scaling +5 % of step time on the Llama parameter sets).
+static bool exact_update(int update_form, int p_dtype, bool sr, bool rank1) {
+  if (update_form == Q4ADAMW_UPDATE_EXACT) return true;
+  if (update_form == Q4ADAMW_UPDATE_FOLDED) return false;
+  return p_dtype == Q4ADAMW_FP32 && !sr && !rank1;
 }
 
 constexpr uint64_t kMaxChunksPerLaunch = 0x7ffffff0ull;  // grid.x limit, with room for padding to 8
@@ -364,8 +328,9 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   FusedArgs a;
   bool ext = false;
+  int update_form = Q4ADAMW_UPDATE_AUTO;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
-  if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
+  if (int rc = make_grad_ops(opt, &a.go, &ext, &update_form)) return rc;
   a.seed_lo = (uint32_t)seed;
   a.seed_hi = (uint32_t)(seed >> 32);
   // a lane reads 8 consecutive elements at once when parameters and gradients are 16-bit types, else 4
@@ -395,7 +360,7 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const FusedKernel kernel = pick_fused(p_dtype, g_dtype, ext, sr);
+  const FusedKernel kernel = pick_fused(p_dtype, g_dtype, ext, sr, exact_update(update_form, p_dtype, sr, false));
   a.ntensors = 0;
   uint64_t chunks = 0;
   for (int i = 0; i < count; ++i) {
@@ -435,8 +400,9 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   Rank1Args a;
   Rank1StatArgs sa;
   bool ext = false;
+  int update_form = Q4ADAMW_UPDATE_AUTO;
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
-  if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
+  if (int rc = make_grad_ops(opt, &a.go, &ext, &update_form)) return rc;
   a.seed_lo = (uint32_t)seed;
   a.seed_hi = (uint32_t)(seed >> 32);
   sa.go = a.go;
@@ -481,6 +447,7 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t tile_elems = chunk_elems / kWaves;
+  const bool exact = exact_update(update_form, p_dtype, sr, true);
   FoldArgs fa;   // the batch's tensors with several leading dimensions
   fa.go = a.go;
   fa.ntensors = 0;
@@ -521,8 +488,9 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   // the columns' maxima of four rows; other matrices with rows of at least a tile the one
   // that finds a tile's row on the scalar unit; narrower ones the one whose lanes find their own
   for (int shape = kShapeRows; shape <= kShapeNarrow; ++shape) {
-    kernel = shape == kShapeRows ? pick_rank1_rows(p_dtype, g_dtype, ext, sr)
-                                 : pick_rank1(p_dtype, g_dtype, ext, sr, shape == kShapeNarrow);
+    kernel = shape == kShapeRows   ? pick_rank1_rows(p_dtype, g_dtype, ext, sr, exact)
+             : shape == kShapeWide ? pick_rank1_wide(p_dtype, g_dtype, ext, sr, exact)
+                                   : pick_rank1_narrow(p_dtype, g_dtype, ext, sr, exact);
     for (int i = 0; i < count; ++i) {
       const q4adamw_rank1_tensor &t = tensors[i];
       if (t.rows == 0 || t.cols == 0 || rank1_shape(t, tile_elems) != shape) continue;
@@ -718,8 +686,9 @@ int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, in
   if (int rc = check_dtypes(p_dtype, g_dtype)) return rc;
   SmallArgs a;
   bool ext = false;
+  int update_form = Q4ADAMW_UPDATE_AUTO;   // this kernel's update is always the exact form
   if (int rc = make_consts(beta1, beta2, lr, weight_decay, eps, step, &a.sc)) return rc;
-  if (int rc = make_grad_ops(opt, &a.go, &ext)) return rc;
+  if (int rc = make_grad_ops(opt, &a.go, &ext, &update_form)) return rc;
   const uintptr_t pa = p_dtype != Q4ADAMW_FP32 ? 2 : 4, ga = g_dtype != Q4ADAMW_FP32 ? 2 : 4;
   for (int i = 0; i < count; ++i) {
     const q4adamw_small_tensor &t = tensors[i];
@@ -908,6 +877,6 @@ int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }
 
-int q4adamw_version(void) { return 1014; }
+int q4adamw_version(void) { return 1015; }
 
 }  // extern "C"

@@ -22,10 +22,24 @@ struct StepConsts {
   float wdu, ss;         // 1 - lr*wd, lr / (1 - beta1^t)
   float c2s;             // sqrt(1 - beta2^t)
   float eps;
-  // the fused kernel's parameter update p*wdu - m'/(sqrt(v')*den_scale + den_eps), the
-  // step size folded into the denominator: 1/(c2s*ss) and eps/ss
+  // the fused kernel's parameter update in its folded form, p*wdu - m'/(sqrt(v')*den_scale +
+  // den_eps), the step size folded into the denominator: 1/(c2s*ss) and eps/ss
   float den_scale, den_eps;
+  // For the correctly rounded form of the update: RN(1 / c2s), which sqrt(v') is divided by
+  // c2s with (div_by_reciprocal), and whether eps and c2s lie where that form's short
+  // sequences hold (non-zero: 2^-60 <= eps <= 2^60, 2^-13 <= c2s <= 1; otherwise every lane
+  // takes the general expansions).
+  float c2s_rcp;
+  uint32_t exact_short;
 };
+
+// (float)(1.0 / (double)c) is RN(1/c): rounding a quotient twice is harmless when the wide
+// format has at least 2 * 24 + 2 bits (host and device: fp64 division is IEEE on both).
+__host__ __device__ inline void make_exact_consts(StepConsts *sc) {
+  sc->c2s_rcp = (float)(1.0 / (double)sc->c2s);
+  sc->exact_short = (sc->eps >= 8.673617379884035e-19f && sc->eps <= 1.152921504606847e+18f &&
+                     sc->c2s >= 1.220703125e-4f && sc->c2s <= 1.0f) ? 1u : 0u;
+}
 
 // What a launch does to the gradients besides reading them (kernels with EXT only).
 struct GradOps {

@@ -84,6 +84,9 @@ __global__ void device_step_kernel(float *counter_, const float *table_, int64_t
   o[0] = sc.b1; o[1] = sc.b2; o[2] = sc.r1; o[3] = sc.r2; o[4] = sc.wdu;
   o[5] = sc.ss; o[6] = sc.c2s; o[7] = sc.eps; o[8] = sc.den_scale; o[9] = sc.den_eps;
   as_global<uint32_t>(out_)[10] = (uint32_t)t;   // the step number, for the rounding noise's salt
+  make_exact_consts(&sc);
+  o[11] = sc.c2s_rcp;
+  as_global<uint32_t>(out_)[12] = sc.exact_short;
 }
 
 // ---------------------------------------------------------------------------

@@ -426,6 +426,63 @@ __device__ __forceinline__ float refined_rcp(float s) {
   return __builtin_fmaf(e, r0, r0);
 }
 
+// ---------------------------------------------------------------------------
+// The parameter update with every operation rounded as IEEE 754 rounds it
+// (optim/cuda_adamw_kernels.cu:334,351: sqrtf, /, +, /, *, *, -), without the scaling and the
+// special-case instructions of the general expansions: the three functions below are exact
+// inside the ranges they name, the caller checks the ranges per lane and takes the general
+// expansions (`sqrtf`, `/`) outside them.
+// ---------------------------------------------------------------------------
+// RN(sqrt(v)) for 2^-96 <= v <= 2^100 (or NaN).  The hardware's estimate s is within one ulp,
+// so the answer is s or one of its neighbours s_dn, s_up, and the residuals against the two
+// midpoints decide: the root lies below the midpoint of s_dn and s iff v <= s_dn * s (the
+// midpoint's square exceeds that product by a quarter ulp squared, less than v's spacing),
+// above the midpoint of s and s_up iff v > s_up * s.  Each residual is one fma (only its
+// sign matters, so its rounding does not); written as s_dn * s - v >= 0 and s_up * s - v < 0
+// the two decisions are the residuals' sign bits (an fma never returns -0 for an exact zero),
+// and the answer's bit pattern is s_dn's plus one for each set sign bit.  Below 2^-96 the
+// residuals' operands leave the normal range.
+__device__ __forceinline__ float sqrt_rn(float v) {
+  const float s = __builtin_amdgcn_sqrtf(v);
+  const uint32_t s_dn = f2bits(s) - 1u, s_up = f2bits(s) + 1u;
+  const uint32_t above_dn = f2bits(__builtin_fmaf(bits2f(s_dn), s, -v)) >> 31;   // v >  s_dn * s
+  const uint32_t above_up = f2bits(__builtin_fmaf(bits2f(s_up), s, -v)) >> 31;   // v >  s_up * s
+  return bits2f(s_dn + above_dn + above_up);
+}
+
+// RN(x / c) given y = RN(1/c), for 2^-60 <= |x|, c <= 2^60: quotient, exact residual, one
+// correction.  The corrected value is t + r * (y - 1/c) with t the true quotient, within
+// 4.5 * 2^-24 ulp of t, so the result can differ from RN(t) only where t comes that close to
+// the midpoint of two floats; tests/native/check_division.c lists every such (x, c) -- for all
+// 2^23 divisor mantissas -- and shows that the sequence rounds each of them correctly.
+__device__ __forceinline__ float div_by_reciprocal(float x, float c, float y) {
+  const float q0 = x * y;
+  const float r = __builtin_fmaf(-c, q0, x);
+  return __builtin_fmaf(r, y, q0);
+}
+
+// RN(m / d) for 2^-60 <= |m|, d <= 2^60.  One Newton step takes the hardware's estimate of 1/d
+// (within one ulp) to RN(1/d): a property of this GPU's v_rcp_f32, established by walking every
+// divisor (tests/test_gpu_exact_update.py); arithmetic alone only promises it for divisors
+// whose mantissa is not all ones.
+__device__ __forceinline__ float div_rn(float m, float d) {
+  const float y0 = __builtin_amdgcn_rcpf(d);
+  const float y = __builtin_fmaf(__builtin_fmaf(-d, y0, 1.0f), y0, y0);
+  return div_by_reciprocal(m, d, y);
+}
+
+constexpr float kExactLo = 8.673617379884035e-19f;   // 2^-60
+constexpr float kExactHi = 1.152921504606847e+18f;   // 2^60
+constexpr float kExactVLo = 1.262177448353619e-29f;  // 2^-96
+constexpr float kExactVHi = 1.2379400392853803e+27f; // 2^90
+
+// The update as the reference writes it; `sqrtf` and `/` are the compiler's general
+// correctly rounded expansions, products and sums stay apart (-ffp-contract=off).
+__device__ __forceinline__ float param_update_ieee(float p, float m, float v, const StepConsts &sc) {
+  const float den = __builtin_sqrtf(v) / sc.c2s + sc.eps;
+  return p * sc.wdu - sc.ss * (m / den);
+}
+
 constexpr float kScaleLo = 7.888609052210118e-31f;   // 2^-100
 constexpr float kScaleHi = 1.2676506002282294e+30f;  // 2^100
 constexpr float kVGuard = 7.62939453125e-06f;        // 2^-17, in units of 16*q
@@ -503,12 +560,14 @@ __device__ __forceinline__ void setup_tables(uint2 *lds, int tid, const TableSlo
 // The step's derived scalars: the launch's arguments, or what device_step_kernel left in
 // device memory for a step whose number the host does not know (a captured graph).
 __device__ __forceinline__ StepConsts step_consts(const StepConsts &from_args, const GradOps &go) {
-  static_assert(sizeof(StepConsts) == 40, "ten floats, in the order read here and written by device_step_kernel");
+  static_assert(sizeof(StepConsts) == 48, "twelve floats; device_step_kernel writes them in the order read here, the step number between them");
   StepConsts sc = from_args;
   if (go.sc_dev) {
     const cptr<const float> f = as_constant<const float>(go.sc_dev);
     sc.b1 = f[0]; sc.b2 = f[1]; sc.r1 = f[2]; sc.r2 = f[3]; sc.wdu = f[4];
     sc.ss = f[5]; sc.c2s = f[6]; sc.eps = f[7]; sc.den_scale = f[8]; sc.den_eps = f[9];
+    sc.c2s_rcp = f[11];   // f[10] is the step number
+    sc.exact_short = as_constant<const uint32_t>(go.sc_dev)[12];
   }
   return sc;
 }

@@ -61,7 +61,7 @@ __device__ __forceinline__ void stage_columns(const RowsTile &rt, int tid) {
   }
 }
 
-template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, int SHAPE, typename Desc>
+template <int PT, int GT, bool FULL, bool EXT, bool RANK1, bool SR, int SHAPE, bool EXACT, typename Desc>
 __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane, int wave, int tid,
                                              const StepConsts &sc, uint2 *lds, const TableSlot &slot,
                                              float gscale, bool zero_g, uint32_t salt,
@@ -221,13 +221,15 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
 
   // entry numbers of the lane's codes, one per byte: even elements, odd elements
   const uint32_t three = 3u, two = 2u;
-  const uint32_t cb_bytes = cb_entry * 0x01010101u;
+  const uint32_t cb_bytes = __builtin_amdgcn_perm(cb_entry, cb_entry, 0u);   // the entry number (< 256) in all four bytes
   const uint32_t m_even = and_or(mw, 0x0F0F0F0Fu, cb_bytes), m_odd = and_or(mw >> 4, 0x0F0F0F0Fu, cb_bytes);
   const uint32_t v_even = and_or(vw, 0x0F0F0F0Fu, cb_bytes), v_odd = and_or(vw >> 4, 0x0F0F0F0Fu, cb_bytes);
 
   // dequantize, update moments and parameter (cuda_adamw_kernels.cu:334-351)
   Vals<N> mn, vn;
   float am = 0.0f, av = 0.0f;
+  float m_least = kExactHi, v_least = kExactVHi;   // EXACT: the lane's smallest |m| and v
+  float p_new[N];
 #pragma unroll
   for (int j = 0; j < N; ++j) {
     const uint32_t mo = entry_offset(j & 1 ? m_odd : m_even, j >> 1, two);
@@ -239,16 +241,36 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
     float m = m_old + sc.r1 * gj;                 // m_old, v_old: beta times the old moment
     float v = v_old + sc.r2 * (gj * gj);
     if (!FULL && j >= nv) { m = 0.0f; v = 0.0f; }
-    // parameter: only this part may use the hardware's 1-ulp square root and a reciprocal
-    // in place of the division
-    const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
-    p[j] = __builtin_fmaf(-m, __builtin_amdgcn_rcpf(den), p[j] * sc.wdu);
+    if constexpr (EXACT) {
+      // the reference's seven operations, each rounded as IEEE 754 rounds it
+      // (cuda_adamw_kernels.cu:334,351), valid inside the ranges checked below
+      const float den = div_by_reciprocal(sqrt_rn(v), sc.c2s, sc.c2s_rcp) + sc.eps;
+      p_new[j] = p[j] * sc.wdu - sc.ss * div_rn(m, den);
+      m_least = __builtin_fminf(m_least, __builtin_fabsf(m));
+      v_least = __builtin_fminf(v_least, v);
+    } else {
+      // folded form: the hardware's 1-ulp square root and a reciprocal in place of the
+      // divisions; the parameters then agree with the reference's to a tolerance only
+      const float den = __builtin_fmaf(__builtin_amdgcn_sqrtf(v), sc.den_scale, sc.den_eps);
+      p_new[j] = __builtin_fmaf(-m, __builtin_amdgcn_rcpf(den), p[j] * sc.wdu);
+    }
     mn.x[j] = m;
     vn.x[j] = v;
     am = __builtin_fmaxf(am, __builtin_fabsf(m));
     av = __builtin_fmaxf(av, v);
   }
-  if (lane_on) store_elems<PT, N, FULL>(const_cast<void *>(p_tile), e0, nv, p);
+  if constexpr (EXACT) {
+    // The short forms hold for moments inside [2^-60, 2^60] and [2^-96, 2^90] and for step
+    // constants that keep the denominator inside [2^-60, 2^60]; a NaN moment passes (the
+    // minima and maxima skip it) and comes out as the NaN the reference produces.  Any other
+    // lane -- zeros among them -- takes the general expansions for its elements.
+    const bool in_range = m_least >= kExactLo && am <= kExactHi && v_least >= kExactVLo && av <= kExactVHi;
+    if (__builtin_expect(!(sc.exact_short != 0u && in_range), 0)) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) p_new[j] = param_update_ieee(p[j], mn.x[j], vn.x[j], sc);
+    }
+  }
+  if (lane_on) store_elems<PT, N, FULL>(const_cast<void *>(p_tile), e0, nv, p_new);
 
   // block scales (exact: max is order independent)
   const float v_lane_max = av;
@@ -418,7 +440,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
   }
 }
 
-template <int PT, int GT, bool EXT, bool SR>
+template <int PT, int GT, bool EXT, bool SR, bool EXACT>
 __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs args) {
   using G = Geometry<PT, GT>;
   __shared__ uint2 lds[kLdsEntries];
@@ -446,144 +468,16 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, false, SR, kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, false, SR, kTileWide, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, false, SR, kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, false, SR, kTileWide, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // ---------------------------------------------------------------------------
-// rank-1 scaling of the second moment: statistics, update, commit
+// rank-1 scaling of the second moment: the update kernels (statistics, commit and the folds
+// for tensors of more dimensions: q4adamw_rank1.h)
 // ---------------------------------------------------------------------------
-constexpr int kStatRowsPerWave = 64;     // rows a wave walks
-constexpr int kStatRows = kStatRowsPerWave * kWaves;   // rows per workgroup of the statistics kernel
-constexpr int kStatCols = 512;           // columns per workgroup: 8 per lane
-
-// New second moments of a tile of kStatRows x kStatCols elements, reduced to row and
-// column maxima (get_variance_tensor_statistics, adamw_fourbit_triton.py:738-746).  The
-// arithmetic is the update kernel's, operation for operation, so the maxima are maxima
-// of exactly the values that kernel quantizes.  The four waves of a workgroup share the
-// columns and split the rows: every lane keeps 8 columns over its wave's rows, the waves'
-// column maxima meet in LDS, and the tile issues one atomic per column and one per row
-// (atomics on the column vector are what this kernel's time depends on most: a tile of
-// 64 rows with four times as many of them took 1.25 to 2 times as long).
-template <int GT, bool EXT>
-__global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatArgs args) {
-  constexpr int kAhead = 4;  // rows whose loads are in flight together
-  __shared__ uint32_t row_bits[4][kStatRows];       // row maxima of each 16-lane quarter of the row's wave
-  __shared__ uint32_t col_bits[kWaves][kStatCols];  // column maxima of each wave
-  const uint32_t chunk = blockIdx.x;
-  float gscale = 1.0f;
-  if (EXT && !grad_ops_begin(args.go, gscale)) return;
-  const int t = find_tensor(args, chunk);
-  const auto &T = args.desc[t];
-  const uint32_t local = chunk - args.first_chunk[t];
-  const uint32_t groups = args.col_groups[t];
-  const uint32_t rg = local / groups, cg = local - rg * groups;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int64_t col = (int64_t)cg * kStatCols + lane * 8;
-  const bool active = col < T.cols;  // cols is a multiple of 8: all 8 columns or none
-  const int64_t tile_row0 = (int64_t)rg * kStatRows;
-  const int tile_rows = (int)(tile_row0 + kStatRows < T.rows ? kStatRows : T.rows - tile_row0);
-  const int wave_row0 = wave * kStatRowsPerWave;                         // within the tile
-  int nrows = tile_rows - wave_row0;                                      // rows of this wave
-  nrows = nrows < 0 ? 0 : (nrows > kStatRowsPerWave ? kStatRowsPerWave : nrows);
-  // lanes past the last column work on zeros: code 0 under a zero scale and a zero
-  // gradient give a zero second moment, which leaves every maximum alone
-  float c_old[8], c_max[8];
-#pragma unroll
-  for (int k = 0; k < 8; ++k) {
-    c_old[k] = active ? as_global<const float>(T.cmax)[col + k] : 0.0f;
-    c_max[k] = 0.0f;
-  }
-  const uint32_t quarter = (uint32_t)lane >> 4;
-  for (int r0 = 0; r0 < nrows; r0 += kAhead) {
-    // a group past the wave's last row repeats that row: maxima do not mind
-    u32x4 gw[kAhead][GT ? 1 : 2];
-    uint32_t vw[kAhead];
-    float r_old[kAhead];
-#pragma unroll
-    for (int i = 0; i < kAhead; ++i) {
-      const int r = r0 + i < nrows ? r0 + i : nrows - 1;
-      const int64_t row = tile_row0 + wave_row0 + r;
-      r_old[i] = as_global<const float>(T.rmax)[row];
-      // row bases are uniform; the lane's column is a 32-bit offset
-      const int64_t row_first = row * T.cols + (int64_t)cg * kStatCols;
-      const uint32_t lane_elem = (uint32_t)lane * 8u;
-      const void *g_row = static_cast<const char *>(T.g) + row_first * (GT ? 2 : 4);
-      const void *v_row = T.v + (row_first >> 1);
-      vw[i] = 0u;
-#pragma unroll
-      for (int h = 0; h < (GT ? 1 : 2); ++h) gw[i][h] = u32x4{0u, 0u, 0u, 0u};
-      if (active) {
-        vw[i] = __builtin_amdgcn_raw_buffer_load_b32(tile_rsrc(v_row), lane_elem >> 1, 0, kNtReadOnly);
-        if (GT) {
-          gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 2u, 0, kNtReadOnly);
-        } else {
-          gw[i][0] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u, 0, kNtReadOnly);
-          gw[i][GT ? 0 : 1] = __builtin_amdgcn_raw_buffer_load_b128(tile_rsrc(g_row), lane_elem * 4u + 16u, 0, kNtReadOnly);
-        }
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < kAhead; ++i) {
-      float g[8];
-      if constexpr (GT != 0) {
-        widen_pair<GT>(gw[i][0].x, g[0], g[1]);
-        widen_pair<GT>(gw[i][0].y, g[2], g[3]);
-        widen_pair<GT>(gw[i][0].z, g[4], g[5]);
-        widen_pair<GT>(gw[i][0].w, g[6], g[7]);
-      } else {
-        const u32x4 lo = gw[i][0], hi = gw[i][GT ? 0 : 1];
-        g[0] = bits2f(lo.x); g[1] = bits2f(lo.y); g[2] = bits2f(lo.z); g[3] = bits2f(lo.w);
-        g[4] = bits2f(hi.x); g[5] = bits2f(hi.y); g[6] = bits2f(hi.z); g[7] = bits2f(hi.w);
-      }
-      const uint32_t even = vw[i] & 0x0F0F0F0Fu, odd = (vw[i] >> 4) & 0x0F0F0F0Fu;  // one code per byte
-      float r_max = 0.0f;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const float gk = EXT ? g[k] * gscale : g[k];
-        const uint32_t code = ((k & 1 ? odd : even) >> (8 * (k >> 1))) & 0xffu;
-        const float code_value = __builtin_fmaf((float)code, 0.0625f, 0.0625f);  // (code + 1) / 16, exact
-        const float v_old = code_value * min_nonneg(r_old[i], c_old[k]);
-        const float v = args.b2 * v_old + args.r2 * (gk * gk);
-        c_max[k] = __builtin_fmaxf(c_max[k], v);
-        r_max = __builtin_fmaxf(r_max, v);
-      }
-      uint32_t u = f2bits(r_max);
-      u = dpp_umax<0xB1>(u);
-      u = dpp_umax<0x4E>(u);
-      u = dpp_umax<0x141>(u);
-      u = dpp_umax<0x140>(u);           // maximum of each 16-lane quarter, in all its lanes
-      if ((lane & 15) == 0) row_bits[quarter][wave_row0 + r0 + i] = u;   // slots past the last row are not read
-    }
-  }
-#pragma unroll
-  for (int k = 0; k < 8; ++k) col_bits[wave][lane * 8 + k] = f2bits(c_max[k]);
-  __syncthreads();
-  // one atomic per column and per row of the tile
-#pragma unroll
-  for (int h = 0; h < kStatCols / kThreads; ++h) {
-    const int c = tid + h * kThreads;
-    uint32_t u = col_bits[0][c];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) u = u > col_bits[w][c] ? u : col_bits[w][c];
-    const int64_t cc = (int64_t)cg * kStatCols + c;
-    if (cc < T.cols && u != 0u) atomic_max_nonneg(T.cmax_next + cc, bits2f(u));
-  }
-#pragma unroll
-  for (int h = 0; h < kStatRows / kThreads; ++h) {
-    const int r = tid + h * kThreads;
-    if (r < tile_rows) {
-      uint32_t u = row_bits[0][r];
-#pragma unroll
-      for (int qi = 1; qi < 4; ++qi) u = u > row_bits[qi][r] ? u : row_bits[qi][r];
-      if (u != 0u) atomic_max_nonneg(T.rmax_next + tile_row0 + r, bits2f(u));
-    }
-  }
-}
-
-template <int PT, int GT, bool EXT, bool SR, bool NARROW>
+template <int PT, int GT, bool EXT, bool SR, bool NARROW, bool EXACT>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
   using G = Geometry<PT, GT>;
   __shared__ uint2 lds[kLdsEntries];
@@ -611,9 +505,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, true, SR, NARROW ? kTileNarrow : kTileWide>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR, NARROW ? kTileNarrow : kTileWide, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // The same for matrices whose rows are a whole number of quantization blocks and at least
@@ -621,7 +515,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
 // and tiles start at the beginning of a row, so that the last tile of a row may be a partial
 // one (whole blocks; its other lanes are idle).  T.div_magic / div_shift divide by the number
 // of tiles in a row.
-template <int PT, int GT, bool EXT, bool SR>
+template <int PT, int GT, bool EXT, bool SR, bool EXACT>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const Rank1Args args) {
   using G = Geometry<PT, GT>;
   constexpr int N = G::kEpl;
@@ -676,67 +570,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const R
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (__builtin_expect(whole, 1))
-    process_tile<PT, GT, true, EXT, true, SR, kTileRows>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
+    process_tile<PT, GT, true, EXT, true, SR, kTileRows, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
   else
-    process_tile<PT, GT, true, EXT, true, SR, kTileRowsLast>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
-}
-
-// After the update: the new statistics become the current ones and the buffers that
-// received them go back to zero for the next step's maxima.  One workgroup column per
-// tensor (blockIdx.y), grid-stride over rows + cols floats.
-__global__ __launch_bounds__(256) void rank1_commit_kernel(const Rank1Args args) {
-  float gscale;
-  if (!grad_ops_begin(args.go, gscale)) return;
-  const Rank1Desc &T = args.desc[blockIdx.y];
-  const int64_t total = T.rows + T.cols;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    const bool is_row = i < T.rows;
-    const gptr<float> cur = as_global<float>(is_row ? T.rmax : T.cmax) + (is_row ? i : i - T.rows);
-    const gptr<float> next = as_global<float>(is_row ? T.rmax_next : T.cmax_next) + (is_row ? i : i - T.rows);
-    *cur = *next;
-    *next = 0.0f;
-  }
-}
-
-// Tensors with several leading dimensions, between statistics and update: row -> its
-// index in leading dimension j (row-major).
-__device__ __forceinline__ int64_t lead_index(const FoldDesc &T, int64_t row, int j) {
-  int64_t stride = 1;
-  for (int k = T.dims - 1; k > j; --k) stride *= T.shape[k];
-  return (row / stride) % T.shape[j];
-}
-
-// mode 0: every leading dimension's new statistic = maximum over the rows that share the index
-// mode 1: every row's new scale = minimum over its leading statistics (after mode 0 is complete)
-// mode 2: after the update, new statistics become current, their buffers return to zero
-// One workgroup column per tensor (blockIdx.y), grid-stride over its rows.
-template <int MODE>
-__global__ __launch_bounds__(256) void rank1_fold_kernel(const FoldArgs args) {
-  float gscale;
-  if (!grad_ops_begin(args.go, gscale)) return;
-  const FoldDesc &T = args.desc[blockIdx.y];
-  const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x, stride = (int64_t)gridDim.x * 256;
-  if (MODE == 2) {
-    for (int j = 0; j < T.dims; ++j) {
-      for (int64_t i = first; i < T.shape[j]; i += stride) {
-        as_global<float>(T.cur[j])[i] = as_global<float>(T.next[j])[i];
-        as_global<float>(T.next[j])[i] = 0.0f;
-      }
-    }
-    return;
-  }
-  for (int64_t row = first; row < T.rows; row += stride) {
-    if (MODE == 0) {
-      const float r = as_global<const float>(T.row_next)[row];
-      if (r != 0.0f) {
-        for (int j = 0; j < T.dims; ++j) atomic_max_nonneg(T.next[j] + lead_index(T, row, j), r);
-      }
-    } else {
-      float s = as_global<const float>(T.next[0])[lead_index(T, row, 0)];
-      for (int j = 1; j < T.dims; ++j) s = min_nonneg(s, as_global<const float>(T.next[j])[lead_index(T, row, j)]);
-      as_global<float>(T.row_next)[row] = s;
-    }
-  }
+    process_tile<PT, GT, true, EXT, true, SR, kTileRowsLast, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt, &rt);
 }
 
 }  // namespace q4

@@ -75,6 +75,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         round_type: str = "real-nearest",
         seed: Optional[int] = None,
         capturable: bool = False,
+        param_update: str = "auto",
     ):
         # optim/fused_quantfour.py:38-47
         if not 0.0 < lr:
@@ -121,6 +122,16 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # for torch.optim.AdamW(capturable=True); the reference reads its step counter on the
         # host (optim/fused_quantfour.py:178, :286-290) and cannot be captured.
 
+        # how the quantized step computes the parameter: "exact" = the reference's expression
+        # (optim/cuda_adamw_kernels.cu:334,351) with each of its seven operations rounded as
+        # IEEE 754 rounds it, so the parameters come out bit-identical to it; "folded" = the
+        # short form with the hardware's square root and reciprocal (fp32 parameters within
+        # 1e-6 of max(|p|, |step|), 16-bit ones within an ulp of their type); "auto" = exact
+        # where it costs under 1 % of the step (fp32 parameters, block scales, nearest
+        # rounding: the reference's own path), folded elsewhere (5 to 10 %)
+        if param_update not in _lib.UPDATE_FORMS:
+            raise ValueError(f"Invalid param_update: {param_update=}")
+
         # tensors with numel <= threshold are not quantized
         # (FirstMoment.threshold / SecondMoment.threshold, adamw_fourbit_triton.py:118, :128)
         self.param_quant_threshold = 4096
@@ -134,6 +145,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             round_type=round_type,
             seed=seed,
             capturable=capturable,
+            param_update=param_update,
         )
         super().__init__(params, defaults)
         self._launch_cache: Dict[Any, Any] = {}
@@ -186,6 +198,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             group.setdefault("round_type", "real-nearest")
             group.setdefault("seed", None)
             group.setdefault("capturable", False)
+            group.setdefault("param_update", "auto")
         state_values = list(self.state.values())
         step_is_tensor = len(state_values) != 0 and torch.is_tensor(state_values[0]["step"])
         if not step_is_tensor:
@@ -674,7 +687,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             # pass the range check
             t_step = 1.0 if capturable else steps[b.idx[0]]
             options = _q.grad_options(b.device, host_mult, dev_mult, found_inf, zero_grad,
-                                      step_consts.get(b.device))
+                                      step_consts.get(b.device), group.get("param_update", "auto"))
             hyper = (b.device, b.p_tag, b.g_tag, beta1, beta2, lr, weight_decay, eps, t_step, options)
             if b.kind in ("sr", "rank1_sr"):
                 launch = _q.launch_rank1_table_sr if rank1 else _q.launch_table_sr

@@ -2,7 +2,7 @@
 profiles/hbm_traffic.json and read by bench.py for its `roofline.traffic` field.
 
 An entry is valid for the kernel sources it was measured on: every entry carries the hash of
-csrc/q4adamw.hip and csrc/q4adamw_*.h at that time, and `lookup` returns None for an entry
+csrc/q4adamw*.hip and csrc/q4adamw_*.h at that time, and `lookup` returns None for an entry
 whose hash differs from the sources in the tree, so a number never outlives the kernel it
 describes.
 
@@ -44,7 +44,7 @@ def source_hash():
     h = hashlib.sha256()
     csrc = os.path.join(_HERE, "csrc")
     for name in sorted(os.listdir(csrc)):
-        if name == "q4adamw.hip" or (name.startswith("q4adamw_") and name.endswith(".h")):
+        if name.startswith("q4adamw") and name.endswith((".hip", ".h")):
             h.update(name.encode())
             with open(os.path.join(csrc, name), "rb") as f:
                 h.update(f.read())

@@ -82,8 +82,14 @@ class _OnDevice:
 _on = _OnDevice
 
 
-def fused_4bit(p, g, exp, sq, exp_scale, sq_scale, beta1, beta2, lr, weight_decay, eps, step):
-    """optim/cuda_fused_interface.cc:19-39."""
+def fused_4bit(p, g, exp, sq, exp_scale, sq_scale, beta1, beta2, lr, weight_decay, eps, step,
+               update_form="auto"):
+    """optim/cuda_fused_interface.cc:19-39.  update_form ("auto", "exact", "folded"): how the
+    parameter is computed, see grad_options; anything but "auto" goes through the multi-tensor
+    entry point, which takes options."""
+    if update_form != "auto":
+        return fused_4bit_multi([p], [g], [exp], [sq], [exp_scale], [sq_scale], beta1, beta2, lr,
+                                weight_decay, eps, step, update_form=update_form)
     L = _lib.load()
     check_quantized(p, g, exp, sq, exp_scale, sq_scale)
     with torch.cuda.device(p.device):
@@ -139,14 +145,22 @@ def _device_scalar(t, device, what):
 
 
 def grad_options(device, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False,
-                 step_consts=None):
+                 step_consts=None, update_form="auto"):
     """struct q4adamw_grad_options, or None when the arguments change nothing.  The device
     scalars are referenced, not copied: keep the tensors alive until the step has run.
-    step_consts: the buffer device_step() filled, for a step whose number lives on the device."""
+    step_consts: the buffer device_step() filled, for a step whose number lives on the device.
+    update_form: "exact" = the parameter update of optim/cuda_adamw_kernels.cu:334,351 with every
+    operation rounded as IEEE 754 rounds it (parameters bit-identical to that expression),
+    "folded" = the short form with hardware square root and reciprocal (a tolerance), "auto" =
+    exact where it is nearly free (fp32 parameters, block scales, nearest rounding)."""
+    form = _lib.UPDATE_FORMS.get(update_form)
+    if form is None:
+        raise ValueError(f"Invalid update_form: {update_form=}")
     if (grad_scale == 1.0 and grad_scale_dev is None and found_inf is None and not zero_grad
-            and step_consts is None):
+            and step_consts is None and form == _lib.UPDATE_AUTO):
         return None
     o = _lib.Q4GradOptions()
+    o.update_form = form
     o.grad_scale = float(grad_scale)
     o.zero_grad = 1 if zero_grad else 0
     o.grad_scale_dev = None if grad_scale_dev is None else _device_scalar(grad_scale_dev, device, "grad_scale_dev")
@@ -221,7 +235,7 @@ def launch_small_table(arr, device, p_tag, g_tag, beta1, beta2, lr, weight_decay
 
 def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr, weight_decay,
                      eps, step, grad_scale=1.0, grad_scale_dev=None, found_inf=None, zero_grad=False,
-                     step_consts=None):
+                     step_consts=None, update_form="auto"):
     """One launch over many quantized tensors that share device, dtypes and step.  The
     gradients enter the step multiplied by grad_scale * grad_scale_dev (a device float32
     scalar); found_inf (a device float32 scalar) makes the call leave parameters and state
@@ -235,7 +249,8 @@ def fused_4bit_multi(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr,
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts,
+                           update_form)
     launch_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
 
 
@@ -275,7 +290,7 @@ def launch_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, beta2, lr
 
 def fused_4bit_multi_sr(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, lr, weight_decay, eps,
                         step, seed, salts=None, grad_scale=1.0, grad_scale_dev=None, found_inf=None,
-                        zero_grad=False):
+                        zero_grad=False, update_form="auto"):
     """fused_4bit_multi with stochastic rounding of both moments (the rule quoted at
     optim/adamw_fourbit_triton.py:1050-1075).  The noise is a function of (seed, step, the
     tensor's salt, element index): salts defaults to the tensors' positions in the list."""
@@ -286,7 +301,8 @@ def fused_4bit_multi_sr(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, 
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad,
+                           update_form=update_form)
     launch_table_sr(arr, None if salts is None else make_salts(salts), seed, ps[0].device, p_tag, g_tag,
                     beta1, beta2, lr, weight_decay, eps, step, options)
 
@@ -389,7 +405,7 @@ def launch_rank1_table_sr(arr, salts_arr, seed, device, p_tag, g_tag, beta1, bet
 def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, row_nexts, col_nexts,
                            beta1, beta2, lr, weight_decay, eps, step, grad_scale=1.0,
                            grad_scale_dev=None, found_inf=None, zero_grad=False, seed=None, salts=None,
-                           step_consts=None, leads=None):
+                           step_consts=None, leads=None, update_form="auto"):
     """The fused step over matrices whose second moment is rank-1 scaled: scale of element
     (i, j) = min(row_maxes[i], col_maxes[j]).  row_nexts / col_nexts are state-owned scratch
     that holds zeros between steps.  Gradient options as for fused_4bit_multi.  With a seed
@@ -401,7 +417,8 @@ def fused_4bit_rank1_multi(ps, gs, exps, sqs, exp_scales, row_maxes, col_maxes, 
     for p, g in zip(ps, gs):
         assert p.device == ps[0].device and _tag(p, "param") == p_tag and _tag(g, "grad") == g_tag, \
             "tensors of one launch must share device and dtypes"
-    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts)
+    options = grad_options(ps[0].device, grad_scale, grad_scale_dev, found_inf, zero_grad, step_consts,
+                           update_form)
     if seed is None:
         launch_rank1_table(arr, ps[0].device, p_tag, g_tag, beta1, beta2, lr, weight_decay, eps, step, options)
     else:

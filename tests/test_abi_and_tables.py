@@ -56,10 +56,14 @@ def test_struct_layouts_match_header():
     assert ctypes.sizeof(_lib.Q4Tensor) == 56 and ctypes.sizeof(_lib.Q4SmallTensor) == 40
     assert _lib.Q4Tensor.numel.offset == 48 and _lib.Q4SmallTensor.numel.offset == 32
     assert ctypes.sizeof(_lib.Q4Rank1Tensor) == 168 and _lib.Q4Rank1Tensor.rows.offset == 72
-    assert ctypes.sizeof(_lib.Q4GradOptions) == 32 and _lib.Q4GradOptions.grad_scale_dev.offset == 8
+    assert ctypes.sizeof(_lib.Q4GradOptions) == 40 and _lib.Q4GradOptions.grad_scale_dev.offset == 8
+    assert _lib.Q4GradOptions.update_form.offset == 32
+    assert (_lib.UPDATE_AUTO, _lib.UPDATE_EXACT, _lib.UPDATE_FOLDED) == (0, 1, 2)
     assert ctypes.sizeof(_lib.Q4Grad) == 16 and _lib.NORM_WORKSPACE_BYTES == 16384
     header = open(os.path.join(ROOT, "include", "q4adamw.h")).read()
     assert "#define Q4ADAMW_NORM_WORKSPACE_BYTES 16384" in header
+    for name, value in (("AUTO", 0), ("EXACT", 1), ("FOLDED", 2)):
+        assert f"#define Q4ADAMW_UPDATE_{name} {value}" in header
 
 
 def test_new_entry_points_validate_before_any_gpu_call(lib):

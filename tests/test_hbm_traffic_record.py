@@ -63,7 +63,7 @@ def test_a_profile_without_the_calibration_copy_is_refused(tmp_path):
 
 
 def test_source_hash_covers_the_kernel_sources_only(tmp_path, monkeypatch):
-    """the hash follows csrc/q4adamw.hip and csrc/q4adamw_*.h, and nothing else in the folder"""
+    """the hash follows csrc/q4adamw*.hip and csrc/q4adamw_*.h, and nothing else in the folder"""
     h0 = ht.source_hash()
     assert len(h0) == 16 and h0 == ht.source_hash()
     csrc = tmp_path / "pkg" / "csrc"
@@ -77,7 +77,10 @@ def test_source_hash_covers_the_kernel_sources_only(tmp_path, monkeypatch):
     (csrc / "libq4adamw.so").write_text("binary")
     assert ht.source_hash() == h1
     (csrc / "q4adamw_step.h").write_text("changed")
-    assert ht.source_hash() != h1
+    h2 = ht.source_hash()
+    assert h2 != h1
+    (csrc / "q4adamw_pick_fused.hip").write_text("a kernel's instantiations")
+    assert ht.source_hash() != h2
 
 
 def test_committed_record_is_well_formed():

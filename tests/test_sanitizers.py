@@ -1,5 +1,5 @@
 """Host code under AddressSanitizer and UndefinedBehaviorSanitizer (no GPU involved): a
-build of csrc/q4adamw.hip with sanitized host code and the C oracle, driven by tests/native/host_sanitize.c
+build of libq4adamw.so's sources with sanitized host code and the C oracle, driven by tests/native/host_sanitize.c
 through every refusal the C ABI makes before a launch and through the oracle on ragged sizes."""
 import os
 import shutil
@@ -24,10 +24,10 @@ def test_host_code_under_sanitizers(tmp_path):
     # sanitizers on the host side only (each option after -Xarch_host); the device code is
     # compiled as usual and not called by anything here
     host_san = [x for opt in SAN[:3] for x in ("-Xarch_host", opt)]
-    subprocess.check_call([hipcc, "--offload-arch=gfx950", "-O1", "-std=c++17", "-ffp-contract=off",
-                           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                           *host_san, "-shared", "-fPIC", "-o", lib, os.path.join(q4build.CSRC, "q4adamw.hip")],
-                          stderr=subprocess.DEVNULL)
+    q4build.compile_library(lib, q4build.STEP_SOURCES,
+                            flags=["--offload-arch=gfx950", "-O1", "-std=c++17", "-ffp-contract=off",
+                                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                                   *host_san, "-fPIC"], check_output=False)
     exe = str(tmp_path / "host_sanitize")
     subprocess.check_call([clang, "-std=c11", *SAN, "-I" + os.path.join(ROOT, "include"),
                            os.path.join(ROOT, "tests", "native", "host_sanitize.c"),
