@@ -432,6 +432,21 @@ int q4adamw_mtable_half_bucket(uint32_t half_index);
 int q4adamw_sr_bucket_entry(uint32_t half_index, uint32_t *out2);
 int q4adamw_sr_affine_entry(uint32_t k, float *out2);
 
+/*
+ * Self-check of the exact parameter update (Q4ADAMW_UPDATE_EXACT) on the GPU the call runs on.
+ * The exact form computes sqrtf and the two divisions of optim/cuda_adamw_kernels.cu:351 with
+ * short sequences around the hardware's square-root and reciprocal estimates; one of them rests
+ * on a property of the reciprocal estimate that arithmetic alone does not give for divisors whose
+ * mantissa is all ones.  This call walks every fp32 pattern of the sequences' domains through
+ * them on the device and adds to counts6 (six device uint64, zeroed by the caller):
+ *   [0] square roots, [1] refined reciprocals, [2] quotients that differ from the correctly
+ *   rounded result; [3] square roots and [4] quotients of the general expansions (taken by
+ *   lanes outside the domains) that differ; [5] patterns walked (2 566 914 050).
+ * [0]..[4] must come back 0; if not, pass Q4ADAMW_UPDATE_FOLDED and report the GPU.  No
+ * counterpart in the reference (its sqrtf and / are nvcc's).  About a second of GPU time.
+ */
+int q4adamw_rounding_selfcheck(uint64_t *counts6, void *stream);
+
 /* Kept for callers that pair an init with a release: the library holds no device
  * memory, so this does nothing and returns 0. */
 int q4adamw_release(void);

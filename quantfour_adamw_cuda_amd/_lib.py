@@ -112,6 +112,7 @@ EXPORTS = (
     "q4adamw_mtable_half_bucket",
     "q4adamw_sr_bucket_entry",
     "q4adamw_sr_affine_entry",
+    "q4adamw_rounding_selfcheck",
     "q4adamw_release",
     "q4adamw_last_error",
     "q4adamw_version",
@@ -186,6 +187,8 @@ def load():
     L.q4adamw_sr_bucket_entry.restype = i
     L.q4adamw_sr_affine_entry.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_float)]
     L.q4adamw_sr_affine_entry.restype = i
+    L.q4adamw_rounding_selfcheck.argtypes = [vp, vp]
+    L.q4adamw_rounding_selfcheck.restype = i
     L.q4adamw_release.argtypes = []
     L.q4adamw_release.restype = i
     L.q4adamw_last_error.argtypes = []

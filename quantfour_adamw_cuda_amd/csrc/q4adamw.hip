@@ -873,6 +873,16 @@ int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel,
   return 0;
 }
 
+int q4adamw_rounding_selfcheck(uint64_t *counts6, void *stream) {
+  if (!counts6) return fail(Q4ADAMW_ERR_ARG, "null output");
+  if (!aligned(counts6, 8)) return fail(Q4ADAMW_ERR_ALIGN, "the counters must be 8-byte aligned");
+  static_assert(sizeof(unsigned long long) == sizeof(uint64_t), "64-bit counters");
+  hipLaunchKernelGGL(rounding_selfcheck_kernel, dim3(8192), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<unsigned long long *>(counts6));
+  Q4_HIP(hipGetLastError());
+  return 0;
+}
+
 int q4adamw_release(void) { return 0; }
 
 const char *q4adamw_last_error(void) { return g_err.c_str(); }

@@ -90,6 +90,58 @@ __global__ void device_step_kernel(float *counter_, const float *table_, int64_t
 }
 
 // ---------------------------------------------------------------------------
+// self-check of the exact parameter update's short forms on the running GPU
+// ---------------------------------------------------------------------------
+// Walks every fp32 pattern of the short forms' domains through them and counts disagreements
+// with the correctly rounded results, taken in fp64 and rounded to fp32 (for a square root, a
+// reciprocal and a quotient the second rounding is harmless: 53 >= 2 * 24 + 2 bits):
+//   out[0]  sqrt_rn(x) != RN(sqrt x)                      x in [2^-96, 2^90]
+//   out[1]  estimate + one Newton step != RN(1 / d)       d in [2^-60, 2^60]
+//   out[2]  div_rn(m, d) != RN(m / d)                     every such d with three numerators:
+//           1, and two of either sign with a mantissa and exponent (2^-60 .. 2^59) hashed from d
+//   out[3]  the compiler's general sqrtf != RN(sqrt x)    (what lanes outside the domains take)
+//   out[4]  the compiler's general m / d != RN(m / d)
+//   out[5]  patterns walked
+// out[1] is a property of the hardware's reciprocal estimate: arithmetic alone promises it only
+// for divisors whose mantissa is not all ones.
+__global__ __launch_bounds__(256) void rounding_selfcheck_kernel(unsigned long long *out_) {
+  const gptr<unsigned long long> out = as_global<unsigned long long>(out_);
+  unsigned long long bad[5] = {0, 0, 0, 0, 0}, walked = 0;
+  const uint32_t first = (blockIdx.x * 256u + threadIdx.x) << 11;   // 2^21 threads x 2^11 patterns = 2^32
+  for (uint32_t k = 0; k < 2048u; ++k) {
+    const uint32_t u = first + k;
+    const float x = bits2f(u);
+    if (x >= kExactVLo && x <= kExactVHi) {
+      const float want = (float)__builtin_sqrt((double)x);
+      bad[0] += f2bits(sqrt_rn(x)) != f2bits(want);
+      bad[3] += f2bits(__builtin_sqrtf(x)) != f2bits(want);
+      ++walked;
+    }
+    if (x >= kExactLo && x <= kExactHi) {
+      const float y0 = __builtin_amdgcn_rcpf(x);
+      const float y = __builtin_fmaf(__builtin_fmaf(-x, y0, 1.0f), y0, y0);
+      bad[1] += f2bits(y) != f2bits((float)(1.0 / (double)x));
+      const uint32_t h = lowbias32(u);
+      const float m1 = bits2f((h & 0x807fffffu) | ((67u + (h >> 23) % 120u) << 23));
+      const float ms[3] = {1.0f, m1, -m1 * 0.75f};
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const float want = (float)((double)ms[j] / (double)x);
+        bad[2] += f2bits(div_rn(ms[j], x)) != f2bits(want);
+        bad[4] += f2bits(ms[j] / x) != f2bits(want);
+      }
+      ++walked;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    if (bad[j]) atomicAdd(out_ + j, bad[j]);
+  }
+  atomicAdd(out_ + 5, walked);
+  (void)out;
+}
+
+// ---------------------------------------------------------------------------
 // global gradient norm (what a caller computes before it clips)
 // ---------------------------------------------------------------------------
 // Sum over a 256-thread workgroup in a fixed order; the result is valid in thread 0.

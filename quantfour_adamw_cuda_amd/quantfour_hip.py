@@ -550,3 +550,15 @@ def dequantize_state_rank1(codes, row_max, col_max):
                                         out.data_ptr(), _stream(codes.device))
     _lib.check(rc, "dequantize_rank1")
     return out
+
+
+def rounding_selfcheck(device):
+    """q4adamw_rounding_selfcheck on `device`: dict of the six counters (sqrt, reciprocal,
+    quotient, general_sqrt, general_quotient mismatches -- all must be 0 -- and walked)."""
+    L = _lib.load()
+    counts = torch.zeros(6, dtype=torch.int64, device=device)
+    with _on(device):
+        rc = L.q4adamw_rounding_selfcheck(counts.data_ptr(), _stream(device))
+    _lib.check(rc, "rounding_selfcheck")
+    names = ("sqrt", "reciprocal", "quotient", "general_sqrt", "general_quotient", "walked")
+    return dict(zip(names, (int(x) for x in counts.cpu())))

@@ -1,7 +1,9 @@
 /*
- * Host check of the short correctly rounded division the fused kernel's exact parameter
- * update uses (div_uniform / div_rn in quantfour_adamw_cuda_amd/csrc/q4adamw_device.h):
+ * Host checks of the short correctly rounded sequences of the fused kernel's exact parameter
+ * update (sqrt_rn, div_by_reciprocal, div_rn in quantfour_adamw_cuda_amd/csrc/q4adamw_device.h),
+ * restated here in C with the same operations (fmaf is a correctly rounded fma).
  *
+ * 1. Division.
  *     y  = RN(1/c)                 (given: computed in fp64 on the host for a uniform divisor,
  *                                   or the hardware estimate plus one Newton step, which the
  *                                   GPU walk of every divisor shows to be RN(1/c))
@@ -24,7 +26,12 @@
  * It also runs a few 10^8 random pairs, and shows that the rule fails when y is off by one
  * ulp (the reason the GPU walk has to establish y == RN(1/c) for the hardware path).
  *
- * Prints "ok <cases>" and exits 0, or prints the first failures and exits 1.
+ * 2. Square root.  sqrt_rn takes an estimate s within one ulp of the root and decides between
+ * s and its two neighbours by the signs of s_dn * s - v and s_up * s - v.  Every mantissa of
+ * two neighbouring binades (which cover every parity of the exponent) is run with the estimate
+ * set to the correctly rounded root and to each of its neighbours.
+ *
+ * Prints "ok ..." and exits 0, or prints the first failures and exits 1.
  */
 #include <math.h>
 #include <stdint.h>
@@ -43,6 +50,16 @@ static inline float div3(float x, float c, float y) {
 }
 
 static inline float rn_reciprocal(float c) { return (float)(1.0 / (double)c); }
+
+static inline float b2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* sqrt_rn with the estimate passed in */
+static inline float sqrt_fix(float v, float s) {
+  const uint32_t s_dn = f2b(s) - 1u, s_up = f2b(s) + 1u;
+  const uint32_t above_dn = f2b(fmaf(b2f(s_dn), s, -v)) >> 31;
+  const uint32_t above_up = f2b(fmaf(b2f(s_up), s, -v)) >> 31;
+  return b2f(s_dn + above_dn + above_up);
+}
 
 static long g_cases, g_bad;
 
@@ -109,7 +126,19 @@ int main(int argc, char **argv) {
       ++g_bad;
     }
   }
-  if (g_bad) { printf("%ld failures in %ld cases\n", g_bad, g_cases); return 1; }
-  printf("ok %ld near-midpoint quotients, %ld random\n", worst, g_cases - worst);
+  /* square roots: every mantissa of [0.5, 2), estimates RN - 1 ulp, RN, RN + 1 ulp */
+  long roots = 0;
+  for (uint32_t u = 0x3f000000u; u < 0x40000000u; ++u) {
+    const float v = b2f(u), t = sqrtf(v);
+    for (int k = -1; k <= 1; ++k) {
+      ++roots;
+      if (f2b(sqrt_fix(v, b2f(f2b(t) + (uint32_t)k))) != f2b(t)) {
+        if (g_bad < 10) printf("FAIL sqrt v=%08x estimate %+d ulp\n", u, k);
+        ++g_bad;
+      }
+    }
+  }
+  if (g_bad) { printf("%ld failures in %ld cases\n", g_bad, g_cases + roots); return 1; }
+  printf("ok %ld near-midpoint quotients, %ld random, %ld square roots\n", worst, g_cases - worst, roots);
   return 0;
 }

@@ -158,8 +158,19 @@ def strict_atol_since(mark):
     return max((m["atol"] for _, m in STRICT_LOG[mark:]), default=0.0)
 
 
-def p_close(p_dev, p_ref, p_prev, bf16=False):
-    """Parameter tolerance for ONE step from identical inputs.
+def p_mismatches(p_dev, p_ref):
+    """Number of fp32 parameters whose bit patterns differ (a NaN on both sides counts as
+    equal, whatever its payload)."""
+    a, b = np.asarray(p_dev, np.float32).reshape(-1), np.asarray(p_ref, np.float32).reshape(-1)
+    same = (bits(a) == bits(b)) | (np.isnan(a) & np.isnan(b))
+    return int(a.size - np.count_nonzero(same))
+
+
+def p_close(p_dev, p_ref, p_prev, bf16=False, exact=False):
+    """exact=True (fp32 parameters from the exact form of the update, which the library takes
+    by itself for fp32 parameters in the block-scaled step with nearest rounding, and anywhere
+    on request): bit-identical to the oracle's; returns (ok, number of mismatches).
+    Otherwise the parameter tolerance for ONE step from identical inputs (the folded form).
     fp32: |dev - ref| <= 1e-6 * |ref| wherever the parameter is at least as large as the step it
     took (the strict bound), and 1e-6 relative to the step elsewhere (parameters that their own
     step carries towards zero, where a relative bound on the parameter alone cannot hold for
@@ -183,6 +194,9 @@ def p_close(p_dev, p_ref, p_prev, bf16=False):
         worst = float((np.abs(dev - ref) / ulp).max()) if dev.size else 0.0
         return worst <= 1.0, worst
     strict = strict_param_metrics(p_dev, p_ref, p_prev)
+    if exact:
+        bad = p_mismatches(p_dev, p_ref)
+        return bad == 0, float(bad)
     ref = p_ref.astype(np.float64)
     diff = np.abs(p_dev.astype(np.float64) - ref)
     scale = np.maximum(np.abs(ref), np.abs(ref - p_prev.astype(np.float64)))
@@ -191,9 +205,11 @@ def p_close(p_dev, p_ref, p_prev, bf16=False):
     return worst <= 1e-6 and strict["dom"] <= 1e-6, worst
 
 
-def assert_state_equal(dev, ref, p_prev, what=""):
-    """codes and scales bit-exact, parameters within tolerance; p_prev holds the
-    parameters both sides started the step from."""
+def assert_state_equal(dev, ref, p_prev, what="", exact=None):
+    """codes and scales bit-exact; parameters bit-exact where the exact form of the update ran
+    (exact=None: fp32 parameters, what the library chooses by itself in the block-scaled step
+    with nearest rounding), within tolerance otherwise; p_prev holds the parameters both sides
+    started the step from."""
     m = dev.m.cpu().numpy()
     v = dev.v.cpu().numpy()
     sm = dev.sm.cpu().numpy()
@@ -207,6 +223,12 @@ def assert_state_equal(dev, ref, p_prev, what=""):
     bad = np.flatnonzero(v != ref.v)
     assert bad.size == 0, f"{what}: second-moment codes differ at bytes {bad[:5]}: {v[bad[:5]]} vs {ref.v[bad[:5]]} ({bad.size} bytes)"
     is_bf16 = dev.p.dtype == torch.bfloat16
-    ok, worst = p_close(to_np(dev.p), ref.p, p_prev, bf16=is_bf16)
-    assert ok, f"{what}: parameters out of tolerance (worst {worst})"
-    return worst
+    if exact is None:
+        exact = dev.p.dtype == torch.float32
+    ok, worst = p_close(to_np(dev.p), ref.p, p_prev, bf16=is_bf16, exact=exact and dev.p.dtype == torch.float32)
+    if exact and dev.p.dtype != torch.float32:    # 16-bit parameters from the exact form: the stored patterns
+        bad = int(np.count_nonzero(to_np(dev.p) != ref.p))
+        assert bad == 0, f"{what}: {bad} 16-bit parameters differ from the oracle's"
+    assert ok, f"{what}: parameters differ (bit-exact expected, {worst:.0f} mismatches)" if exact else \
+        f"{what}: parameters out of tolerance (worst {worst})"
+    return 0.0 if exact else worst

@@ -19,9 +19,13 @@ def say(msg):
 
 
 def run_steps(p0, grad_fn, steps, device, hp=HP, g_dtype=torch.float32, what=""):
-    """Steps one tensor on the device and in the oracle; checks after every step."""
+    """Steps one tensor on the device and in the oracle; checks after every step.  fp32
+    parameters come from the exact form of the update and are compared bit for bit, the two
+    sides never re-based on each other: the last step's equality is the cumulative bound.
+    16-bit parameters (folded form, one ulp per step) continue from the device's values."""
     dev = DeviceTensor(p0, device)
     ref = OracleTensor(p0)
+    exact = p0.dtype == torch.float32
     worst = 0.0
     for t in range(1, steps + 1):
         g = grad_fn(t).to(g_dtype)
@@ -31,7 +35,8 @@ def run_steps(p0, grad_fn, steps, device, hp=HP, g_dtype=torch.float32, what="")
         torch.cuda.synchronize()
         prev = ref.step(g, t, hp)
         worst = max(worst, assert_state_equal(dev, ref, prev, f"{what} step {t}"))
-        ref.resync(dev.p)
+        if not exact:
+            ref.resync(dev.p)
     return worst
 
 
@@ -293,8 +298,8 @@ def test_unquantized_step_vs_oracle(cuda):
             oc.step_unquant(rp[i], g.numpy(), rm[i], rv[i], step=t, **HP)
             assert np.array_equal(bits(dm[i].cpu().numpy()), bits(rm[i]))
             assert np.array_equal(bits(dv[i].cpu().numpy()), bits(rv[i]))
-            ok, worst = p_close(dp[i].cpu().numpy(), rp[i], prev)
-            assert ok, f"unquant params worst {worst}"
+            ok, worst = p_close(dp[i].cpu().numpy(), rp[i], prev, exact=True)   # this kernel's update is the exact form
+            assert ok, f"unquant params: {worst} mismatches"
             rp[i][:] = dp[i].cpu().numpy()
 
 
@@ -431,6 +436,7 @@ def test_non_finite_gradients(cuda, p_dtype, g_dtype):
                  else (ref.p.astype(np.uint32) << 16).view(np.float32))
         finite = np.isfinite(p_ref)
         assert np.array_equal(np.isfinite(p_dev), finite), f"step {step}: finiteness of the parameters"
-        ok, worst = p_close(to_np(dev.p)[finite], ref.p[finite], prev[finite], bf16=p_dtype == torch.bfloat16)
+        ok, worst = p_close(to_np(dev.p)[finite], ref.p[finite], prev[finite], bf16=p_dtype == torch.bfloat16,
+                            exact=p_dtype == torch.float32)
         assert ok, f"step {step}: parameters out of tolerance (worst {worst})"
         ref.resync(dev.p)
