@@ -195,13 +195,14 @@ def build_inputs(torch, device, shapes, p_dtype, g_dtype, dist, grad_sets):
 
 
 def run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, steps, warmup, variance_scale="group",
-               round_type="real-nearest", clip="none", host_burst=True):
+               round_type="real-nearest", clip="none", host_burst=True, param_update="auto"):
     """W warm-up steps, then exactly K timed steps between two synchronisations, with a fresh
     optimizer over `params`.  Returns the measurements of the timed region.  host_burst=False
     leaves out the extra steps that measure the host time of step() (host_ms_per_step is then
     None): W + K steps run and no others, which a counter profile of the run relies on."""
     from quantfour_adamw_cuda_amd import AdamWFused_QuantFour
-    opt = AdamWFused_QuantFour(params, variance_scale_type=variance_scale, round_type=round_type, seed=0, **HP)
+    opt = AdamWFused_QuantFour(params, variance_scale_type=variance_scale, round_type=round_type, seed=0,
+                               param_update=param_update, **HP)
     opt.kernel_timing = []  # (kind, start event, end event) per launch
     host_s = [0.0]
 
@@ -277,11 +278,20 @@ def run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, steps, warmup, va
     return m
 
 
-def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None):
+def update_form_of(param_update, p_dtype_s, variance_scale, round_type):
+    """which form of the parameter update a run's quantized kernels compute (the library's
+    "auto" rule: exact for fp32 parameters with block scales and nearest rounding)"""
+    if param_update != "auto":
+        return param_update
+    plain = p_dtype_s == "float32" and variance_scale == "group" and round_type == "real-nearest"
+    return "exact" if plain else "folded"
+
+
+def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None, param_update="auto"):
     from quantfour_adamw_cuda_amd import hbm_traffic
     achieved = m["algo_bytes"] / m["kernel_s"] / 1e9
     n = m["launches_per_step"]
-    rec = hbm_traffic.lookup(workload, variance_scale, round_type)
+    rec = hbm_traffic.lookup(workload, variance_scale, round_type, param_update)
     r = {
         "bound": "hbm",
         "kernel": "fused_4bit_kernel" if not m["rank1"] else "rank1_stats_kernel + fused_4bit_rank1_rows_kernel",
@@ -305,14 +315,15 @@ def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None):
     return r
 
 
-def config_entry(name, desc, m, workload, variance_scale, round_type, p_dtype_s, g_dtype_s):
-    r = roofline_entry(m, workload, variance_scale, round_type)
+def config_entry(name, desc, m, workload, variance_scale, round_type, p_dtype_s, g_dtype_s, param_update="auto"):
+    r = roofline_entry(m, workload, variance_scale, round_type, param_update=param_update)
     return {
         "name": name,
         "workload": desc,
         "param_dtype": p_dtype_s,
         "grad_dtype": g_dtype_s,
         "variance_scale": variance_scale,
+        "param_update": update_form_of(param_update, p_dtype_s, variance_scale, round_type),
         "steps": m["steps"],
         "ms_per_step": m["ms_per_step"],
         "params_per_s": m["total_params"] * m["steps"] / m["elapsed"],
@@ -432,6 +443,11 @@ def main():
                          "rank-1 row/column maxima for matrices (a statistics pass precedes the update)")
     ap.add_argument("--round-type", choices=["real-nearest", "stochastic"], default="real-nearest",
                     help="rounding of the quantizer (stochastic: hash noise per element)")
+    ap.add_argument("--param-update", choices=["auto", "exact", "folded"], default="auto",
+                    help="form of the parameter update: exact = every operation of the reference's expression "
+                         "rounded as IEEE 754 rounds it (bit-identical parameters), folded = hardware square root "
+                         "and reciprocal (a tolerance), auto = exact for fp32 parameters with block scales and "
+                         "nearest rounding, folded elsewhere")
     ap.add_argument("--configs", choices=["auto", "all", "none"], default="auto",
                     help="also time the other benchmark configurations and the step's variants and report "
                          "them in `configs` (auto: only for the default workload without variant options)")
@@ -463,14 +479,15 @@ def main():
     shapes_fn, p_dtype_s, g_dtype_s, dist, desc = WORKLOADS[args.workload]
     p_dtype_s, g_dtype_s = args.param_dtype or p_dtype_s, args.grad_dtype or g_dtype_s
     plain = (args.variance_scale == "group" and args.round_type == "real-nearest" and args.clip == "none"
-             and not args.param_dtype and not args.grad_dtype)
+             and not args.param_dtype and not args.grad_dtype and args.param_update == "auto")
     all_configs = args.configs == "all" or (args.configs == "auto" and args.workload == "llama3-8b" and plain)
 
     params, grad_sets = build_inputs(torch, device, shapes_fn(), getattr(torch, p_dtype_s),
                                      getattr(torch, g_dtype_s), dist, args.grad_sets)
     phase(f"inputs of {args.workload} built")
     m = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, args.steps, args.warmup,
-                   args.variance_scale, args.round_type, args.clip, host_burst=not args.calibrate_copy)
+                   args.variance_scale, args.round_type, args.clip, host_burst=not args.calibrate_copy,
+                   param_update=args.param_update)
     phase("headline steps timed")
     if args.calibrate_copy:
         calibrate_copy(torch, device)
@@ -497,6 +514,7 @@ def main():
             "param_dtype": p_dtype_s,
             "grad_dtype": g_dtype_s,
             "grad_sets": len(grad_sets),
+            "param_update": update_form_of(args.param_update, p_dtype_s, args.variance_scale, args.round_type),
             "hyper": {"lr": HP["lr"], "betas": list(HP["betas"]), "eps": HP["eps"],
                       "weight_decay": HP["weight_decay"]},
         },
@@ -519,12 +537,13 @@ def main():
     if all_configs:
         # the step's variants on the headline workload's own tensors, then the other configurations
         k, w = 10, 3
-        for vs, rt, name in (("group", "stochastic", "stochastic rounding"),
-                             ("rank1", "real-nearest", "rank-1 scaled second moment"),
-                             ("rank1", "stochastic", "rank-1 scaled second moment + stochastic rounding")):
-            mv = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, k, w, vs, rt)
-            configs.append(config_entry(f"{args.workload}, {name}", desc + "; " + name, mv, args.workload, vs, rt,
-                                        p_dtype_s, g_dtype_s))
+        for vs, rt, pu, name in (("group", "real-nearest", "folded", "folded parameter update (a tolerance instead of bit-identical parameters)"),
+                                 ("group", "stochastic", "auto", "stochastic rounding"),
+                                 ("rank1", "real-nearest", "auto", "rank-1 scaled second moment"),
+                                 ("rank1", "stochastic", "auto", "rank-1 scaled second moment + stochastic rounding")):
+            mv = run_config(torch, params, grad_sets, p_dtype_s, g_dtype_s, k, w, vs, rt, param_update=pu)
+            configs.append(config_entry(f"{args.workload}, {name.split(' (')[0]}", desc + "; " + name, mv, args.workload, vs, rt,
+                                        p_dtype_s, g_dtype_s, pu))
             phase(f"variant timed: {name}")
     del params, grad_sets
     torch.cuda.empty_cache()
@@ -535,6 +554,13 @@ def main():
             mv = run_config(torch, pr, gr, ps, gs_, k, w)
             configs.append(config_entry(wl, desc_, mv, wl, "group", "real-nearest", ps, gs_))
             phase(f"configuration timed: {wl}")
+            if wl == "llama2-13b":      # the 16-bit kernels' variants, the ones closest to the vector ALU's limit
+                for vs, rt, pu, name in (("group", "real-nearest", "exact", "exact parameter update"),
+                                         ("group", "stochastic", "auto", "stochastic rounding"),
+                                         ("rank1", "real-nearest", "auto", "rank-1 scaled second moment")):
+                    mv = run_config(torch, pr, gr, ps, gs_, k, w, vs, rt, param_update=pu)
+                    configs.append(config_entry(f"{wl}, {name}", desc_ + "; " + name, mv, wl, vs, rt, ps, gs_, pu))
+                    phase(f"variant timed: {wl}, {name}")
             del pr, gr
             torch.cuda.empty_cache()
 
@@ -542,7 +568,7 @@ def main():
     phase("probes done")
     key = f"step_streams_{p_dtype_s}_{g_dtype_s}"
     out["roofline"] = roofline_entry(m, args.workload, args.variance_scale, args.round_type,
-                                     ceiling.get(key) if ceiling else None)
+                                     ceiling.get(key) if ceiling else None, args.param_update)
     for c in configs:
         # block-scaled variants move the bytes of the probe with their element types; rank-1
         # scaling adds a second pass and the statistics, which no probe moves

@@ -46,7 +46,7 @@ extern "C" {
 #define Q4ADAMW_ERR_ARG (-1)       /* null pointer, negative size, bad dtype tag */
 #define Q4ADAMW_ERR_ALIGN (-2)     /* pointer not aligned as its buffer requires */
 #define Q4ADAMW_ERR_HYPER (-3)     /* hyper-parameter outside its domain         */
-#define Q4ADAMW_ERR_TOO_LARGE (-4) /* launch would exceed the grid limit         */
+#define Q4ADAMW_ERR_TOO_LARGE (-4) /* a tensor beyond 2^31 - 16 chunks (2^35 elements for rank-1) */
 
 /*
  * One quantized tensor.  Field order follows the tensor arguments of
@@ -431,6 +431,25 @@ int q4adamw_mtable_half_bucket(uint32_t half_index);
  */
 int q4adamw_sr_bucket_entry(uint32_t half_index, uint32_t *out2);
 int q4adamw_sr_affine_entry(uint32_t k, float *out2);
+
+/*
+ * Host-only.  A grid of the HIP runtime holds fewer than 2^32 work-items, i.e. at most
+ * 2^24 - 8 workgroups of 256 threads (1.7e10 fp32 elements of the fused step), so the entry
+ * points run a large batch -- or one very large tensor, e.g. a flat sharded parameter -- as
+ * several grids.  q4adamw_grid_plan returns how many grids `chunks` workgroups of `threads`
+ * threads take and writes the first `capacity` of them as (first chunk, number of chunks).
+ * q4adamw_set_grid_limit lowers the number of workgroups per grid for the calling process
+ * (0 restores the runtime's limit; values are rounded down to a multiple of 8): for tests that
+ * exercise the split without 80 GB of parameters.  The reference launches one grid per tensor
+ * with a 32-bit element count (optim/cuda_adamw_kernels.cu:430-432) and stops at 2^31 elements.
+ */
+int q4adamw_grid_plan(uint64_t chunks, int threads, uint64_t *bases, uint64_t *counts, int capacity);
+/* Host-only, for tests: which of its three update kernels q4adamw_fused_4bit_rank1_multi runs on
+ * a rows x cols matrix: 0 = tiles aligned to the rows, 1 = tiles anywhere in rows of at least a
+ * tile, 2 = rows shorter than a tile.  both_16_bit: parameters and gradients are 16-bit types
+ * (tiles of 512 elements instead of 256). */
+int q4adamw_rank1_form(int64_t rows, int64_t cols, int both_16_bit);
+void q4adamw_set_grid_limit(uint64_t workgroups);
 
 /*
  * Self-check of the exact parameter update (Q4ADAMW_UPDATE_EXACT) on the GPU the call runs on.

@@ -113,6 +113,9 @@ EXPORTS = (
     "q4adamw_sr_bucket_entry",
     "q4adamw_sr_affine_entry",
     "q4adamw_rounding_selfcheck",
+    "q4adamw_grid_plan",
+    "q4adamw_rank1_form",
+    "q4adamw_set_grid_limit",
     "q4adamw_release",
     "q4adamw_last_error",
     "q4adamw_version",
@@ -188,6 +191,12 @@ def load():
     L.q4adamw_sr_affine_entry.argtypes = [ctypes.c_uint32, ctypes.POINTER(ctypes.c_float)]
     L.q4adamw_sr_affine_entry.restype = i
     L.q4adamw_rounding_selfcheck.argtypes = [vp, vp]
+    L.q4adamw_grid_plan.argtypes = [ctypes.c_uint64, i, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), i]
+    L.q4adamw_grid_plan.restype = i
+    L.q4adamw_rank1_form.argtypes = [i64, i64, i]
+    L.q4adamw_rank1_form.restype = i
+    L.q4adamw_set_grid_limit.argtypes = [ctypes.c_uint64]
+    L.q4adamw_set_grid_limit.restype = None
     L.q4adamw_rounding_selfcheck.restype = i
     L.q4adamw_release.argtypes = []
     L.q4adamw_release.restype = i

@@ -114,22 +114,58 @@ static void finish_prefix(Args &a) {
   for (int k = 0; k < Args::kPivots; ++k) a.pivot[k] = a.first_chunk[k * 8];
 }
 
+// Two limits.  A batch (one set of kernel arguments) indexes its chunks with 31 bits
+// (first_chunk's sentinel is 0x7fffffff).  A grid is smaller: HIP refuses a launch whose
+// gridDim.x * blockDim.x reaches 2^32 (hip_runtime_api.h, hipModuleLaunchKernel), i.e. more than
+// 2^24 - 1 workgroups of 256 threads, which 1.7e10 fp32 elements exceed -- a flat FSDP
+// parameter fits 288 GB several times over.  So a batch's chunks are dealt to as many grids as
+// it takes, each with the number of its first chunk in the arguments (chunk_base); a tensor
+// larger than a grid simply spans grids.  The grid size is rounded down to a multiple of 8 (the
+// fused kernels pad their grids to one).
+constexpr uint64_t kMaxChunksPerLaunch = 0x7ffffff0ull;   // per batch
+constexpr uint64_t kHipWorkItemsPerGrid = 0xffffffffull;
+constexpr int64_t kMaxInterchangeElements = 1ll << 40;     // q4adamw_quantize / q4adamw_dequantize
+static std::atomic<uint64_t> g_grid_limit_override{0};    // q4adamw_set_grid_limit (tests)
+
+static uint64_t grid_limit(unsigned threads) {
+  const uint64_t hw = (kHipWorkItemsPerGrid / threads) & ~7ull;
+  const uint64_t o = g_grid_limit_override.load(std::memory_order_relaxed) & ~7ull;
+  return o >= 8 && o < hw ? o : hw;
+}
+
+// Calls launch(base, count) for the grids of a batch of `chunks` chunks.
+template <typename F>
+static int for_each_grid(uint64_t chunks, unsigned threads, F launch) {
+  const uint64_t limit = grid_limit(threads);
+  for (uint64_t base = 0; base < chunks; base += limit) {
+    const uint64_t count = chunks - base < limit ? chunks - base : limit;
+    if (int rc = launch(base, count)) return rc;
+  }
+  return 0;
+}
+
 static int launch_fused_batch(FusedArgs &a, uint64_t chunks, void (*kernel)(const FusedArgs),
                               hipStream_t stream) {
   finish_prefix(a);
-  a.nchunks = (uint32_t)chunks;
-  a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
-  hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, stream, a);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  return for_each_grid(chunks, kThreads, [&](uint64_t base, uint64_t count) -> int {
+    a.chunk_base = (uint32_t)base;
+    a.nchunks = (uint32_t)(base + count);
+    a.chunks_per_xcd = (uint32_t)((count + 7) / 8);
+    hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, stream, a);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
 }
 
 static int launch_small_batch(SmallArgs &a, uint64_t chunks, void (*kernel)(const SmallArgs),
                               hipStream_t stream) {
   finish_prefix(a);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)chunks), dim3(256), 0, stream, a);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  return for_each_grid(chunks, 256, [&](uint64_t base, uint64_t count) -> int {
+    a.chunk_base = (uint32_t)base;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)count), dim3(256), 0, stream, a);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
 }
 
 template <bool EXT>
@@ -152,8 +188,15 @@ enum Rank1Shape { kShapeRows = 0, kShapeWide = 1, kShapeNarrow = 2 };
 static Rank1Shape rank1_shape(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
   if (t.cols < tile_elems) return kShapeNarrow;
   const int64_t padded = (t.cols + tile_elems - 1) / tile_elems * tile_elems;
-  if (t.cols % Q4ADAMW_BLOCK == 0 && t.cols >= 2 * tile_elems && t.rows >= 64 && (padded - t.cols) * 16 <= t.cols)
-    return kShapeRows;
+  if (t.cols % Q4ADAMW_BLOCK == 0 && t.cols >= 2 * tile_elems && t.rows >= 64 && (padded - t.cols) * 16 <= t.cols) {
+    // The rounding noise is keyed by an element's 64-bit index, whose high half the kernels take
+    // per tile: a tile must not straddle a multiple of 2^32.  Tiles of the other forms start at
+    // multiples of their length and never do; a tile of the rows form starts where its row
+    // does, so a matrix of more than 2^32 elements whose rows are no whole number of tiles
+    // takes the wide form.
+    const bool may_straddle = t.rows * t.cols > 0xffffffffll && t.cols % tile_elems != 0;
+    if (!may_straddle) return kShapeRows;
+  }
   return kShapeWide;
 }
 
@@ -221,7 +264,6 @@ static bool exact_update(int update_form, int p_dtype, bool sr, bool rank1) {
   return p_dtype == Q4ADAMW_FP32 && !sr && !rank1;
 }
 
-constexpr uint64_t kMaxChunksPerLaunch = 0x7ffffff0ull;  // grid.x limit, with room for padding to 8
 
 }  // namespace q4
 
@@ -357,7 +399,7 @@ static int fused_4bit_multi_impl(const q4adamw_tensor *tensors, int count, int p
         !aligned(t.exp_avg_scale, 4) || !aligned(t.exp_avg_sq_scale, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "code and scale buffers must be 4-byte aligned");
     if (((uint64_t)t.numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
-      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large: more than 2^31 - 16 chunks");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const FusedKernel kernel = pick_fused(p_dtype, g_dtype, ext, sr, exact_update(update_form, p_dtype, sr, false));
@@ -443,7 +485,7 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     const uint64_t stat_chunks = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) *
                                  (uint64_t)((t.cols + kStatCols - 1) / kStatCols);
     if (rank1_chunks(t, chunk_elems / kWaves) > kMaxChunksPerLaunch || stat_chunks > kMaxChunksPerLaunch)
-      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large: more than 2^31 - 16 chunks");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t tile_elems = chunk_elems / kWaves;
@@ -460,18 +502,28 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     sa.ntensors = a.ntensors;
     finish_prefix(sa);
     sa.nchunks = (uint32_t)stat_chunks;
-    hipLaunchKernelGGL(stat_kernel, dim3(sa.nchunks), dim3(kThreads), 0, s, sa);
-    Q4_HIP(hipGetLastError());
+    if (int rc = for_each_grid(stat_chunks, kThreads, [&](uint64_t base, uint64_t count) -> int {
+          sa.chunk_base = (uint32_t)base;
+          hipLaunchKernelGGL(stat_kernel, dim3((unsigned)count), dim3(kThreads), 0, s, sa);
+          Q4_HIP(hipGetLastError());
+          return 0;
+        }))
+      return rc;
     if (fa.ntensors > 0) {   // rows' maxima -> leading statistics -> rows' scales
       hipLaunchKernelGGL(rank1_fold_kernel<0>, dim3(64, (unsigned)fa.ntensors), dim3(256), 0, s, fa);
       hipLaunchKernelGGL(rank1_fold_kernel<1>, dim3(64, (unsigned)fa.ntensors), dim3(256), 0, s, fa);
       Q4_HIP(hipGetLastError());
     }
     finish_prefix(a);
-    a.nchunks = (uint32_t)chunks;
-    a.chunks_per_xcd = (uint32_t)((chunks + 7) / 8);
-    hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, s, a);
-    Q4_HIP(hipGetLastError());
+    if (int rc = for_each_grid(chunks, kThreads, [&](uint64_t base, uint64_t count) -> int {
+          a.chunk_base = (uint32_t)base;
+          a.nchunks = (uint32_t)(base + count);
+          a.chunks_per_xcd = (uint32_t)((count + 7) / 8);
+          hipLaunchKernelGGL(kernel, dim3(a.chunks_per_xcd * 8u), dim3(kThreads), 0, s, a);
+          Q4_HIP(hipGetLastError());
+          return 0;
+        }))
+      return rc;
     hipLaunchKernelGGL(rank1_commit_kernel, dim3(64, (unsigned)a.ntensors), dim3(256), 0, s, a);
     Q4_HIP(hipGetLastError());
     if (fa.ntensors > 0) {
@@ -601,7 +653,7 @@ static int grad_norm_impl(const q4adamw_grad *grads, int count, int g_dtype, flo
     if (!aligned(grads[i].g, g_dtype != Q4ADAMW_FP32 ? 2 : 4))
       return fail(Q4ADAMW_ERR_ALIGN, "gradients must be aligned to their element size");
     if (((uint64_t)grads[i].numel + (uint64_t)chunk_elems - 1) / (uint64_t)chunk_elems > kMaxChunksPerLaunch)
-      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large: more than 2^31 - 16 chunks");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   NormArgs a;
@@ -699,7 +751,7 @@ int q4adamw_fused_single_tensor_multi_ex(const q4adamw_small_tensor *tensors, in
     if (!aligned(t.p, pa) || !aligned(t.g, ga) || !aligned(t.exp_avg, 4) || !aligned(t.exp_avg_sq, 4))
       return fail(Q4ADAMW_ERR_ALIGN, "tensor not aligned to its element size");
     if (((uint64_t)t.numel + (uint64_t)kSmallChunk - 1) / (uint64_t)kSmallChunk > kMaxChunksPerLaunch)
-      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+      return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large: more than 2^31 - 16 chunks");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const SmallKernel kernel = pick_small(p_dtype, g_dtype, ext);
@@ -793,13 +845,15 @@ int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, f
   if (!x || !codes || !scales) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(x, 4) || !aligned(scales, 4)) return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
   const uint64_t blocks = ((uint64_t)numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
-  const uint64_t grid = (blocks + 3) / 4;
-  if (grid > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  const uint64_t groups = (blocks + 3) / 4;
+  if (numel > kMaxInterchangeElements) return fail(Q4ADAMW_ERR_TOO_LARGE, "more than 2^40 elements");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (which) hipLaunchKernelGGL(quantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, x, numel, codes, scales);
-  else hipLaunchKernelGGL(quantize_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, x, numel, codes, scales);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
+    if (which) hipLaunchKernelGGL(quantize_kernel<true>, dim3((unsigned)count), dim3(256), 0, s, x, numel, codes, scales, (int64_t)base);
+    else hipLaunchKernelGGL(quantize_kernel<false>, dim3((unsigned)count), dim3(256), 0, s, x, numel, codes, scales, (int64_t)base);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
 }
 
 static int check_rank1_shape(int64_t rows, int64_t cols) {
@@ -823,11 +877,13 @@ int q4adamw_quantize_rank1(const float *x, int64_t rows, int64_t cols, uint8_t *
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, row_max, rows);
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, col_max, cols);
   hipLaunchKernelGGL(rank1_absmax_kernel, tiles, dim3(256), 0, s, x, rows, cols, row_max, col_max);
-  const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
-  hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, rows, cols,
-                     static_cast<const float *>(row_max), static_cast<const float *>(col_max), codes);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  const uint64_t groups = ((uint64_t)rows * cols / 2 + 255) / 256;
+  return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
+    hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)count), dim3(256), 0, s, x, rows, cols,
+                       static_cast<const float *>(row_max), static_cast<const float *>(col_max), codes, (int64_t)base);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
 }
 
 int q4adamw_quantize_rank1_scaled(const float *x, int64_t rows, int64_t cols, const float *row_scale,
@@ -837,11 +893,13 @@ int q4adamw_quantize_rank1_scaled(const float *x, int64_t rows, int64_t cols, co
   if (!x || !codes || !row_scale || !col_max) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(x, 4) || !aligned(row_scale, 4) || !aligned(col_max, 4))
     return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
-  hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0, static_cast<hipStream_t>(stream), x,
-                     rows, cols, row_scale, col_max, codes);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  const uint64_t groups = ((uint64_t)rows * cols / 2 + 255) / 256;
+  return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
+    hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)count), dim3(256), 0, static_cast<hipStream_t>(stream), x,
+                       rows, cols, row_scale, col_max, codes, (int64_t)base);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
 }
 
 int q4adamw_dequantize_rank1(const uint8_t *codes, const float *row_max, const float *col_max,
@@ -851,11 +909,13 @@ int q4adamw_dequantize_rank1(const uint8_t *codes, const float *row_max, const f
   if (!codes || !row_max || !col_max || !out) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(out, 4) || !aligned(row_max, 4) || !aligned(col_max, 4))
     return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t grid = ((uint64_t)rows * cols / 2 + 255) / 256;
-  hipLaunchKernelGGL(dequantize_rank1_kernel, dim3((unsigned)grid), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), codes, row_max, col_max, rows, cols, out);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  const uint64_t groups = ((uint64_t)rows * cols / 2 + 255) / 256;
+  return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
+    hipLaunchKernelGGL(dequantize_rank1_kernel, dim3((unsigned)count), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), codes, row_max, col_max, rows, cols, out, (int64_t)base);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
 }
 
 int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel, int which,
@@ -864,13 +924,42 @@ int q4adamw_dequantize(const uint8_t *codes, const float *scales, int64_t numel,
   if (numel == 0) return 0;
   if (!out || !codes || !scales) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(out, 4) || !aligned(scales, 4)) return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t grid = (((uint64_t)numel + 1) / 2 + 255) / 256;
-  if (grid > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large for one launch");
+  const uint64_t groups = (((uint64_t)numel + 1) / 2 + 255) / 256;
+  if (numel > kMaxInterchangeElements) return fail(Q4ADAMW_ERR_TOO_LARGE, "more than 2^40 elements");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (which) hipLaunchKernelGGL(dequantize_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, codes, scales, numel, out);
-  else hipLaunchKernelGGL(dequantize_kernel<false>, dim3((unsigned)grid), dim3(256), 0, s, codes, scales, numel, out);
-  Q4_HIP(hipGetLastError());
-  return 0;
+  return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
+    if (which) hipLaunchKernelGGL(dequantize_kernel<true>, dim3((unsigned)count), dim3(256), 0, s, codes, scales, numel, out, (int64_t)base);
+    else hipLaunchKernelGGL(dequantize_kernel<false>, dim3((unsigned)count), dim3(256), 0, s, codes, scales, numel, out, (int64_t)base);
+    Q4_HIP(hipGetLastError());
+    return 0;
+  });
+}
+
+int q4adamw_rank1_form(int64_t rows, int64_t cols, int both_16_bit) {
+  if (rows <= 0 || cols <= 0 || cols > 0x40000000ll || rows > 0x7ffffffffll / cols)
+    return fail(Q4ADAMW_ERR_ARG, "bad shape");
+  q4adamw_rank1_tensor t = {};
+  t.rows = rows;
+  t.cols = cols;
+  return (int)rank1_shape(t, both_16_bit ? Geometry<1, 1>::kTile : Geometry<0, 0>::kTile);
+}
+
+void q4adamw_set_grid_limit(uint64_t workgroups) { g_grid_limit_override.store(workgroups); }
+
+int q4adamw_grid_plan(uint64_t chunks, int threads, uint64_t *bases, uint64_t *counts, int capacity) {
+  if (threads < 64 || threads > 1024 || capacity < 0 || (capacity > 0 && (!bases || !counts)))
+    return fail(Q4ADAMW_ERR_ARG, "bad workgroup size or output arrays");
+  if (chunks > kMaxChunksPerLaunch) return fail(Q4ADAMW_ERR_TOO_LARGE, "more than 2^31 - 16 chunks");
+  int n = 0;
+  for_each_grid(chunks, (unsigned)threads, [&](uint64_t base, uint64_t count) -> int {
+    if (n < capacity) {
+      bases[n] = base;
+      counts[n] = count;
+    }
+    ++n;
+    return 0;
+  });
+  return n;
 }
 
 int q4adamw_rounding_selfcheck(uint64_t *counts6, void *stream) {

@@ -70,8 +70,11 @@ struct FusedArgs {
   StepConsts sc;
   GradOps go;
   int ntensors;
-  uint32_t nchunks;        // chunks in this launch
-  uint32_t chunks_per_xcd; // ceil(nchunks / 8); the grid has 8 * chunks_per_xcd workgroups
+  // A batch's chunks run in one grid or, beyond what a grid may hold, in several: this grid
+  // takes chunks [chunk_base, nchunks), 8 * chunks_per_xcd workgroups.
+  uint32_t chunk_base;
+  uint32_t nchunks;
+  uint32_t chunks_per_xcd; // ceil((nchunks - chunk_base) / 8)
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
   TensorDesc desc[kMaxTensors];
@@ -96,6 +99,7 @@ struct SmallArgs {
   StepConsts sc;
   GradOps go;
   int ntensors;
+  uint32_t chunk_base;     // this grid's first chunk (workgroup 0)
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];
   SmallDesc desc[kMaxSmallTensors];
@@ -156,6 +160,7 @@ struct Rank1Args {
   StepConsts sc;
   GradOps go;
   int ntensors;
+  uint32_t chunk_base;     // as FusedArgs
   uint32_t nchunks;
   uint32_t chunks_per_xcd;
   uint32_t pivot[kPivots];
@@ -171,6 +176,7 @@ struct Rank1StatArgs {
   float b2, r2;
   GradOps go;
   int ntensors;
+  uint32_t chunk_base;     // this grid's first tile (workgroup 0)
   uint32_t nchunks;
   uint32_t pivot[kPivots];
   uint32_t first_chunk[kPivots * 8];

@@ -9,7 +9,7 @@ namespace q4 {
 // moments in place, same derived scalars and operation order as the fused path.
 template <int PT, int GT, bool EXT>
 __global__ __launch_bounds__(256) void single_tensor_kernel(const SmallArgs args) {
-  const uint32_t chunk = blockIdx.x;
+  const uint32_t chunk = args.chunk_base + blockIdx.x;
   float gscale = 1.0f;
   const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);
   const bool zero_g = EXT && args.go.zero != 0u;
@@ -239,10 +239,10 @@ __global__ __launch_bounds__(256) void grad_norm_finish_kernel(const double *par
 template <bool SECOND>
 __global__ __launch_bounds__(256) void quantize_kernel(const float *__restrict__ x_, int64_t numel,
                                                        uint8_t *__restrict__ codes_,
-                                                       float *__restrict__ scale_) {
+                                                       float *__restrict__ scale_, int64_t group0) {
   const gptr<const float> x = as_global<const float>(x_);
   const int lane = threadIdx.x & 63;
-  const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t blk = (group0 + blockIdx.x) * 4 + (threadIdx.x >> 6);   // group0: this grid's first workgroup
   const int64_t nblk = (numel + Q4ADAMW_BLOCK - 1) / Q4ADAMW_BLOCK;
   if (blk >= nblk) return;
   const int64_t e = blk * Q4ADAMW_BLOCK + lane * 2;
@@ -311,8 +311,8 @@ __global__ __launch_bounds__(256) void rank1_absmax_kernel(const float *x_, int6
 // 15-compare count (optim/adamw_fourbit_triton.py:834-863)
 __global__ __launch_bounds__(256) void quantize_rank1_kernel(const float *x_, int64_t rows, int64_t cols,
                                                              const float *row_max, const float *col_max,
-                                                             uint8_t *codes_) {
-  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+                                                             uint8_t *codes_, int64_t group0) {
+  const int64_t e = ((group0 + blockIdx.x) * 256 + threadIdx.x) * 2;
   if (e >= rows * cols) return;
   const int64_t i = e / cols, j = e - i * cols;  // cols is even: both elements in row i
   const float r = as_global<const float>(row_max)[i];
@@ -329,8 +329,8 @@ __global__ __launch_bounds__(256) void quantize_rank1_kernel(const float *x_, in
 // optim/adamw_fourbit_triton.py:520-527: code-book entry times min(row, column maximum)
 __global__ __launch_bounds__(256) void dequantize_rank1_kernel(const uint8_t *codes_, const float *row_max,
                                                                const float *col_max, int64_t rows,
-                                                               int64_t cols, float *out_) {
-  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+                                                               int64_t cols, float *out_, int64_t group0) {
+  const int64_t e = ((group0 + blockIdx.x) * 256 + threadIdx.x) * 2;
   if (e >= rows * cols) return;
   const int64_t i = e / cols, j = e - i * cols;
   const float r = as_global<const float>(row_max)[i];
@@ -343,8 +343,8 @@ __global__ __launch_bounds__(256) void dequantize_rank1_kernel(const uint8_t *co
 template <bool SECOND>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t *__restrict__ codes_,
                                                          const float *__restrict__ scale_,
-                                                         int64_t numel, float *__restrict__ out_) {
-  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+                                                         int64_t numel, float *__restrict__ out_, int64_t group0) {
+  const int64_t e = ((group0 + blockIdx.x) * 256 + threadIdx.x) * 2;
   if (e >= numel) return;
   const uint32_t byte = as_global<const uint8_t>(codes_)[e >> 1];
   const float s = as_global<const float>(scale_)[e / Q4ADAMW_BLOCK];

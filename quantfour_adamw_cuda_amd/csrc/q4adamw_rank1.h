@@ -23,7 +23,7 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   constexpr int kAhead = 4;  // rows whose loads are in flight together
   __shared__ uint32_t row_bits[4][kStatRows];       // row maxima of each 16-lane quarter of the row's wave
   __shared__ uint32_t col_bits[kWaves][kStatCols];  // column maxima of each wave
-  const uint32_t chunk = blockIdx.x;
+  const uint32_t chunk = args.chunk_base + blockIdx.x;
   float gscale = 1.0f;
   if (EXT && !grad_ops_begin(args.go, gscale)) return;
   const int t = find_tensor(args, chunk);

@@ -326,8 +326,9 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
   if constexpr (SR) {
     // key = low half of the element index, xor the salt, xor the mixed high half
     const uint32_t tile_salt = salt ^ ((uint32_t)((uint64_t)tb >> 32) * 0x9E3779B9u);
-    // a tile never straddles a multiple of 2^32; the lane's first element is a multiple
-    // of N, so element j's key is the first one's with j in its low bits
+    // a tile never straddles a multiple of 2^32 (the launcher sees to it: tiles start at
+    // multiples of their length, or the matrix is small enough, rank1_shape); the lane's first
+    // element is a multiple of N, so element j's key is the first one's with j in its low bits
     const uint32_t key0 = ((uint32_t)tb + e0) ^ tile_salt;
 #pragma unroll
     for (int j = 0; j < N; ++j) {
@@ -446,7 +447,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
-  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  const uint32_t chunk = args.chunk_base + (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;  // whole workgroup: the grid is padded to a multiple of 8
   float gscale = 1.0f;
   const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);  // whole grid
@@ -483,7 +484,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   __shared__ uint2 lds[kLdsEntries];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
-  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  const uint32_t chunk = args.chunk_base + (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;
   float gscale = 1.0f;
   const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);
@@ -523,7 +524,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const R
   __shared__ __attribute__((aligned(16))) float columns[2 * G::kTile];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
-  const uint32_t chunk = (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
+  const uint32_t chunk = args.chunk_base + (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
   if (chunk >= args.nchunks) return;
   float gscale = 1.0f;
   const bool cancelled = EXT && !grad_ops_begin(args.go, gscale);

@@ -51,11 +51,13 @@ def source_hash():
     return h.hexdigest()[:16]
 
 
-def key(workload, variance_scale="group", round_type="real-nearest"):
-    return f"{workload}|{variance_scale}|{round_type}"
+def key(workload, variance_scale="group", round_type="real-nearest", param_update="auto"):
+    """param_update: the optimizer's option; anything but "auto" (the library's own choice of
+    the parameter update's form) gets an entry of its own"""
+    return f"{workload}|{variance_scale}|{round_type}" + ("" if param_update == "auto" else f"|{param_update}")
 
 
-def lookup(workload, variance_scale="group", round_type="real-nearest", path=DEFAULT_PATH):
+def lookup(workload, variance_scale="group", round_type="real-nearest", param_update="auto", path=DEFAULT_PATH):
     """The recorded entry (a dict with bytes_per_step ...) if one exists for these kernel
     sources, else None."""
     try:
@@ -63,7 +65,7 @@ def lookup(workload, variance_scale="group", round_type="real-nearest", path=DEF
             entries = json.load(f)["entries"]
     except (OSError, ValueError, KeyError):
         return None
-    e = entries.get(key(workload, variance_scale, round_type))
+    e = entries.get(key(workload, variance_scale, round_type, param_update))
     if not e or e.get("source_hash") != source_hash():
         return None
     return e
@@ -84,7 +86,8 @@ def _sum_counter(csv_paths, counter):
     return out
 
 
-def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, out_path, profile=None):
+def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, out_path, profile=None,
+           param_update="auto"):
     fetch, write = _sum_counter(fetch_csv, "FETCH_SIZE"), _sum_counter(write_csv, "WRITE_SIZE")
 
     def pick(table, names):
@@ -118,7 +121,7 @@ def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, ou
             doc = json.load(f)
     except (OSError, ValueError):
         doc = {"entries": {}}
-    doc.setdefault("entries", {})[key(workload, variance_scale, round_type)] = entry
+    doc.setdefault("entries", {})[key(workload, variance_scale, round_type, param_update)] = entry
     doc["unit"] = "bytes of HBM traffic per optimizer step (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)"
     with open(out_path, "w") as f:
         json.dump(doc, f, indent=1, sort_keys=True)
@@ -131,6 +134,7 @@ def main():
     ap.add_argument("--workload", required=True)
     ap.add_argument("--variance-scale", default="group")
     ap.add_argument("--round-type", default="real-nearest")
+    ap.add_argument("--param-update", default="auto")
     ap.add_argument("--fetch-csv", nargs="+", required=True)
     ap.add_argument("--write-csv", nargs="+", required=True)
     ap.add_argument("--steps", type=int, required=True, help="optimizer steps the profiled command ran (warm-up included)")
@@ -138,7 +142,7 @@ def main():
     ap.add_argument("--profile", default=None, help="the profiles/ summary that documents the run")
     a = ap.parse_args()
     print(json.dumps(record(a.workload, a.variance_scale, a.round_type, a.fetch_csv, a.write_csv, a.steps,
-                            a.out, a.profile), indent=1))
+                            a.out, a.profile, a.param_update), indent=1))
 
 
 if __name__ == "__main__":

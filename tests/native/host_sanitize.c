@@ -27,6 +27,14 @@ void q4o_quant(const float *x, int64_t numel, int which, uint8_t *codes, float *
 void q4o_dequant(const uint8_t *codes, const float *scale, int64_t numel, int which, float *out);
 void q4o_derive_scalars(float beta1, float beta2, float lr, float weight_decay, float step, float *out6);
 
+#define TRUE_(cond)                                                        \
+  do {                                                                     \
+    if (!(cond)) {                                                         \
+      fprintf(stderr, "%s:%d %s does not hold\n", __FILE__, __LINE__, #cond); \
+      exit(1);                                                             \
+    }                                                                      \
+  } while (0)
+
 #define EXPECT(call, want)                                                                     \
   do {                                                                                         \
     int rc_ = (call);                                                                          \
@@ -102,6 +110,35 @@ static void refusals(void) {
     const float *h = bad_hyper[k];
     EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, 1000, F, F, h[0], h[1], h[2], h[3], h[4], h[5], NULL), Q4ADAMW_ERR_HYPER);
     EXPECT(q4adamw_fused_single_tensor(buf, buf + 2048, buf + 4096, buf + 6144, 1000, F, F, h[0], h[1], h[2], h[3], h[4], h[5], NULL), Q4ADAMW_ERR_HYPER);
+  }
+  /* grids: a batch beyond what one grid holds (2^32 work-items: 2^24 - 8 workgroups of 256
+     threads once rounded to a multiple of 8) is dealt to several */
+  {
+    uint64_t bases[8], counts[8];
+    const uint64_t limit = (1ull << 24) - 8;
+    TRUE_(q4adamw_grid_plan(0, 256, bases, counts, 8) == 0);
+    TRUE_(q4adamw_grid_plan(limit - 1, 256, bases, counts, 8) == 1);
+    TRUE_(q4adamw_grid_plan(limit, 256, bases, counts, 8) == 1);
+    TRUE_(bases[0] == 0 && counts[0] == limit);
+    TRUE_(q4adamw_grid_plan(limit + 1, 256, bases, counts, 8) == 2);
+    TRUE_(bases[1] == limit && counts[1] == 1);
+    TRUE_(q4adamw_grid_plan((1ull << 24) - 1, 256, bases, counts, 8) == 2);      /* what HIP itself would still take */
+    TRUE_(q4adamw_grid_plan(1ull << 24, 256, bases, counts, 8) == 2);
+    TRUE_(q4adamw_grid_plan((1ull << 24) + 1, 256, bases, counts, 8) == 2);
+    TRUE_(bases[1] + counts[1] == (1ull << 24) + 1);
+    TRUE_(q4adamw_grid_plan(0x7ffffff0ull, 256, bases, counts, 2) == 129);        /* more grids than the arrays hold */
+    EXPECT(q4adamw_grid_plan(0x7ffffff1ull, 256, bases, counts, 8), Q4ADAMW_ERR_TOO_LARGE);
+    EXPECT(q4adamw_grid_plan(10, 32, bases, counts, 8), Q4ADAMW_ERR_ARG);
+    EXPECT(q4adamw_grid_plan(10, 256, NULL, counts, 8), Q4ADAMW_ERR_ARG);
+    q4adamw_set_grid_limit(70);                 /* rounded down to 64 */
+    TRUE_(q4adamw_grid_plan(200, 256, bases, counts, 8) == 4);
+    TRUE_(bases[3] == 192 && counts[3] == 8 && counts[0] == 64);
+    q4adamw_set_grid_limit(3);                  /* below 8: ignored */
+    TRUE_(q4adamw_grid_plan(200, 256, bases, counts, 8) == 1);
+    q4adamw_set_grid_limit(0);
+    TRUE_(q4adamw_grid_plan(200, 256, bases, counts, 8) == 1);
+    /* a tensor beyond one grid is taken (the launch itself fails here: no device), one beyond a batch's 31-bit chunk index is not */
+    EXPECT(q4adamw_fused_4bit(buf, buf + 2048, codes, codes + 2048, scales, scales + 64, (int64_t)0x7ffffff0ll * 1024 + 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL), Q4ADAMW_ERR_TOO_LARGE);
   }
   /* lists */
   q4adamw_tensor t[2];

@@ -66,6 +66,49 @@ def test_struct_layouts_match_header():
         assert f"#define Q4ADAMW_UPDATE_{name} {value}" in header
 
 
+def test_grids_of_a_batch_and_the_test_hook(lib):
+    """a batch beyond one grid (HIP: gridDim.x * blockDim.x < 2^32) is dealt to several grids;
+    q4adamw_set_grid_limit lowers the grid size so that tests can cross the boundary"""
+    u64 = ctypes.c_uint64
+    bases, counts = (u64 * 8)(), (u64 * 8)()
+    limit = (1 << 24) - 8
+
+    def plan(chunks, threads=256):
+        n = lib.q4adamw_grid_plan(chunks, threads, bases, counts, 8)
+        return [(bases[k], counts[k]) for k in range(min(max(n, 0), 8))] if n >= 0 else n
+
+    assert plan(0) == [] and plan(1) == [(0, 1)] and plan(limit) == [(0, limit)]
+    assert plan(limit + 1) == [(0, limit), (limit, 1)]
+    assert plan((1 << 24) + 1) == [(0, limit), (limit, 9)]
+    assert plan(1 << 20, threads=1024) == [(0, 1 << 20)]
+    assert plan((1 << 22) - 7, threads=1024) == [(0, (1 << 22) - 8), ((1 << 22) - 8, 1)]
+    assert plan(3 * limit + 5) == [(0, limit), (limit, limit), (2 * limit, limit), (3 * limit, 5)]
+    assert plan(0x7ffffff1) == _lib.load().q4adamw_grid_plan(0x7ffffff1, 256, bases, counts, 8) == -4
+    try:
+        lib.q4adamw_set_grid_limit(1000)
+        assert plan(2500) == [(0, 1000), (1000, 1000), (2000, 500)]
+        lib.q4adamw_set_grid_limit(1001)            # rounded down to a multiple of 8
+        assert plan(2500) == [(0, 1000), (1000, 1000), (2000, 500)]
+    finally:
+        lib.q4adamw_set_grid_limit(0)
+    assert plan(2500) == [(0, 2500)]
+
+
+def test_rank1_kernel_form_by_shape(lib):
+    """rows form for the Llama shapes, wide for ragged rows, narrow below a tile; a matrix of more
+    than 2^32 elements whose rows are no whole number of tiles leaves the rows form (a tile
+    there could straddle a multiple of 2^32, where the noise key's high half changes)"""
+    form = lib.q4adamw_rank1_form
+    assert form(4096, 4096, 0) == 0 and form(128256, 4096, 1) == 0 and form(4096, 14336, 0) == 0
+    assert form(4096, 4480, 1) == 0                 # last tile 384 of 512: an 11th of the row idle... within a 16th
+    assert form(100, 520, 0) == 1 and form(32, 4096, 0) == 1 and form(4096, 11008 + 8, 1) == 1
+    assert form(1000, 248, 0) == 2 and form(1000, 504, 1) == 2 and form(1000, 504, 0) == 1
+    big_rows = (1 << 32) // 4480 + 2
+    assert form(big_rows, 4480, 1) == 1 and form(big_rows - 3, 4480, 1) == 0      # just above / below 2^32 elements
+    assert form((1 << 32) // 4096 + 4, 4096, 1) == 0                              # whole tiles: aligned anyway
+    assert form(0, 16, 0) == -1 and form(8, 1 << 31, 0) == -1
+
+
 def test_new_entry_points_validate_before_any_gpu_call(lib):
     z = ctypes.c_void_p(0)
     hp = (0.9, 0.999, 1e-3, 0.01, 1e-8, 1.0)

@@ -440,3 +440,83 @@ def test_non_finite_gradients(cuda, p_dtype, g_dtype):
                             exact=p_dtype == torch.float32)
         assert ok, f"step {step}: parameters out of tolerance (worst {worst})"
         ref.resync(dev.p)
+
+
+def test_batches_and_tensors_larger_than_a_grid(cuda):
+    """With the grid size lowered to 64 workgroups (q4adamw_set_grid_limit), a tensor of 300
+    chunks spans five grids and a list of tensors is cut in the middle of one: every entry point
+    that launches one workgroup per chunk still gives the oracle's bits -- the block-scaled step
+    (plain, with gradient options, stochastic rounding), rank-1 scaling (statistics and update),
+    the non-quantized step, and the checkpoint quantizers."""
+    from oracle import q4_oracle_torch as ot
+    from quantfour_adamw_cuda_amd import _lib
+    from quantfour_adamw_cuda_amd import quantfour_hip as qh
+    L = _lib.load()
+    hpa = (HP["beta1"], HP["beta2"], HP["lr"], HP["weight_decay"], HP["eps"])
+    gen = torch.Generator().manual_seed(99)
+    sizes = [1024 * 300 + 77, 5000, 1024 * 70, 129]
+    try:
+        L.q4adamw_set_grid_limit(64)
+        # block-scaled, one call over the list; then the same with options and with noise
+        ps = [torch.randn(n, generator=gen) * 0.02 for n in sizes]
+        for variant in ("plain", "options", "stochastic"):
+            devs = [DeviceTensor(p, cuda) for p in ps]
+            refs = [(p.clone(),) + tuple(t.cpu() for t in (d.m, d.v, d.sm, d.sv)) for p, d in zip(ps, devs)]
+            for step in (1, 2):
+                gs = [grads_config3(gen, n) for n in sizes]
+                dg = [g.to(cuda) for g in gs]
+                lists = ([d.p for d in devs], dg, [d.m for d in devs], [d.v for d in devs], [d.sm for d in devs], [d.sv for d in devs])
+                if variant == "stochastic":
+                    qh.fused_4bit_multi_sr(*lists, *hpa, step, 7, salts=[5, 6, 7, 8], update_form="exact")
+                    refs = [ot.step_quant_sr(r[0], g, *r[1:], seed=7, tensor_salt=s, step=step, **HP)
+                            for r, g, s in zip(refs, gs, (5, 6, 7, 8))]
+                else:
+                    kw = dict(grad_scale=0.5, zero_grad=True) if variant == "options" else {}
+                    qh.fused_4bit_multi(*lists, *hpa, step, **kw)
+                    refs = [ot.step_quant(r[0], g * 0.5 if kw else g, *r[1:], step=step, **HP) for r, g in zip(refs, gs)]
+                    if kw:
+                        assert all(not g.any() for g in dg), "gradients cleared in every grid"
+                for d, r, n in zip(devs, refs, sizes):
+                    assert torch.equal(d.m.cpu(), r[1]) and torch.equal(d.v.cpu(), r[2]), f"{variant} n={n} step {step}: codes"
+                    assert torch.equal(d.sm.cpu().view(torch.int32), r[3].view(torch.int32))
+                    assert torch.equal(d.p.cpu().view(torch.int32), r[0].view(torch.int32)), f"{variant} n={n} step {step}: parameters"
+        # rank-1: 300 x 1024 (rows form: 75 row groups x 4 tiles = 300 chunks; 2 statistics tiles... and a
+        # 1300 x 520 matrix in the wide form (660 chunks, 12 statistics tiles)
+        for rows, cols in ((300, 1024), (1300, 520)):
+            p0 = torch.randn(rows, cols, generator=gen) * 0.05
+            n = rows * cols
+            p = p0.clone().to(cuda)
+            m = torch.zeros((n + 1) // 2, dtype=torch.uint8, device=cuda)
+            v, sm = torch.zeros_like(m), torch.zeros((n + 127) // 128, device=cuda)
+            r, c, rn, cn = (torch.zeros(k, device=cuda) for k in (rows, cols, rows, cols))
+            ref = (p0.clone(), m.cpu(), v.cpu(), sm.cpu(), r.cpu(), c.cpu())
+            for step in (1, 2, 3):
+                g = grads_config1(gen, n).view(rows, cols)
+                ref = ot.step_quant_rank1(ref[0], g, *ref[1:], step=step, **HP)
+                qh.fused_4bit_rank1_multi([p], [g.to(cuda)], [m], [v], [sm], [r], [c], [rn], [cn], *hpa, step,
+                                          update_form="exact")
+                assert torch.equal(m.cpu(), ref[1]) and torch.equal(v.cpu(), ref[2]), f"rank-1 {rows}x{cols} step {step}"
+                assert torch.equal(r.cpu().view(torch.int32), ref[4].view(torch.int32))
+                assert torch.equal(c.cpu().view(torch.int32), ref[5].view(torch.int32))
+                assert torch.equal(p.cpu().view(torch.int32), ref[0].view(torch.int32))
+        # non-quantized step: 100 tensors of 3000 elements = 300 chunks of 1024
+        small = [torch.randn(3000, generator=gen) * 0.02 for _ in range(100)]
+        dp = [p.clone().to(cuda) for p in small]
+        dm, dv = [torch.zeros(3000, device=cuda) for _ in small], [torch.zeros(3000, device=cuda) for _ in small]
+        rp, rm, rv = [p.numpy().copy() for p in small], [np.zeros(3000, np.float32) for _ in small], [np.zeros(3000, np.float32) for _ in small]
+        gs = [torch.randn(3000, generator=gen) * 1e-3 for _ in small]
+        q4.fused_single_tensor_multi(dp, [g.to(cuda) for g in gs], dm, dv, *hpa, 1)
+        for i, g in enumerate(gs):
+            oc.step_unquant(rp[i], g.numpy(), rm[i], rv[i], step=1, **HP)
+            assert np.array_equal(bits(dp[i].cpu().numpy()), bits(rp[i])) and np.array_equal(bits(dm[i].cpu().numpy()), bits(rm[i]))
+        # checkpoint quantizers: 128 * 4 * 200 elements = 200 workgroups of four blocks
+        x = torch.randn(128 * 4 * 200 + 50, generator=gen)
+        for which in (0, 1):
+            xx = x.abs() if which else x
+            codes, scales = qh.quantize_state(xx.to(cuda), which)
+            rc, rs = oc.quant(xx.numpy(), which)
+            assert np.array_equal(codes.cpu().numpy(), rc) and np.array_equal(bits(scales.cpu().numpy()), bits(rs))
+            back = qh.dequantize_state(codes, scales, xx.numel(), which)
+            assert np.array_equal(bits(back.cpu().numpy()), bits(oc.dequant(rc, rs, xx.numel(), which)))
+    finally:
+        L.q4adamw_set_grid_limit(0)

@@ -88,8 +88,9 @@ def test_committed_record_is_well_formed():
         doc = json.load(f)
     assert doc["entries"], "profiles/hbm_traffic.json holds no entry"
     for key, e in doc["entries"].items():
-        workload, variance, rounding = key.split("|")
+        workload, variance, rounding, *form = key.split("|")
         assert variance in ("group", "rank1") and rounding in ("real-nearest", "stochastic")
+        assert form in ([], ["exact"], ["folded"])
         assert e["bytes_per_step"] == pytest.approx(e["fetch_bytes_per_step"] + e["write_bytes_per_step"])
         assert 1.9 < e["fetch_scale"] < 2.1 and 0.95 < e["write_scale"] < 1.05
         assert len(e["source_hash"]) == 16 and e["dispatches_per_step"] >= 1
