@@ -485,6 +485,9 @@ __device__ __forceinline__ float param_update_ieee(float p, float m, float v, co
 
 constexpr float kScaleLo = 7.888609052210118e-31f;   // 2^-100
 constexpr float kScaleHi = 1.2676506002282294e+30f;  // 2^100
+// 16 / scale at or above this (2^103.5) means a scale at the lower end of the range or below
+// it (16 / kScaleLo is 2^104 give or take the reciprocal's ulp)
+constexpr float kInvScaleLo16 = 1.4340386889e+31f;
 constexpr float kVGuard = 7.62939453125e-06f;        // 2^-17, in units of 16*q
 static_assert(kVGuard == 0.5f * kNoiseStep, "the fast path lets the noise's offset cancel the guard band");
 

@@ -40,7 +40,9 @@ constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2, kTileRowsLast = 3;
 // What a wave of the kTileRows form knows beyond its tile number: its row, the tile's first
 // column, and this thread's share of the workgroup's fetch of the columns' maxima (old and
 // new; kTile / 256 consecutive columns per thread), which goes to `columns` in LDS:
-// [0, kTile) old, [kTile, 2 kTile) new.
+// [0, kTile) old, [kTile, 2 kTile) 16 / max(new, kScaleLo) -- the reciprocal every element of
+// the column would otherwise take for itself -- and [2 kTile, 3 kTile) new, which only the
+// exact path reads.
 struct RowsTile {
   int64_t row;
   uint32_t col0;
@@ -52,12 +54,16 @@ struct RowsTile {
 // Writes a thread's share of the columns' maxima into LDS (before the workgroup's barrier).
 template <int N>
 __device__ __forceinline__ void stage_columns(const RowsTile &rt, int tid) {
+  const float inv_x = __builtin_amdgcn_rcpf(max_nonneg(rt.share_new.x, kScaleLo)) * 16.0f;
   if (N == 4) {
     rt.columns[tid] = rt.share_old.x;
-    rt.columns[64 * N + tid] = rt.share_new.x;
+    rt.columns[64 * N + tid] = inv_x;
+    rt.columns[128 * N + tid] = rt.share_new.x;
   } else {
+    const float inv_y = __builtin_amdgcn_rcpf(max_nonneg(rt.share_new.y, kScaleLo)) * 16.0f;
     *reinterpret_cast<float2 *>(rt.columns + 2 * tid) = rt.share_old;
-    *reinterpret_cast<float2 *>(rt.columns + 64 * N + 2 * tid) = rt.share_new;
+    *reinterpret_cast<float2 *>(rt.columns + 64 * N + 2 * tid) = make_float2(inv_x, inv_y);
+    *reinterpret_cast<float2 *>(rt.columns + 128 * N + 2 * tid) = rt.share_new;
   }
 }
 
@@ -212,6 +218,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
   if constexpr (RANK1 && kRows) {
 #pragma unroll
     for (int k = 0; k < N; k += 4) {
+      // c_new: 16 / max(new column maximum, kScaleLo) in this form, not the maximum itself
       const float4 a = *reinterpret_cast<const float4 *>(rt->columns + e0 + k);
       const float4 b = *reinterpret_cast<const float4 *>(rt->columns + 64 * N + e0 + k);
       c_old.x[k] = a.x; c_old.x[k + 1] = a.y; c_old.x[k + 2] = a.z; c_old.x[k + 3] = a.w;
@@ -306,7 +313,21 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
   // zero value under a zero scale then still gets code 0; any other value under such a
   // scale sends the lane to the exact path.
   Vals<N> s_new, inv16;
-  if constexpr (RANK1) {
+  if constexpr (RANK1 && kRows) {
+    // 16 / min(row maximum, column maximum) is the larger of the two reciprocals, the row's
+    // taken once per lane and the columns' once per workgroup (stage_columns): one
+    // instruction per element.  (Where the hardware reciprocal is not monotonic the other
+    // one is within an ulp of it, which the guard band covers all the same.)  A clamped
+    // scale shows as the reciprocal of the clamp.
+    const float row_inv16 = __builtin_amdgcn_rcpf(max_nonneg(r_new, kScaleLo)) * 16.0f;
+    float inv_max = 0.0f;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      inv16.x[j] = max_nonneg(row_inv16, c_new.x[j]);
+      inv_max = max_nonneg(inv_max, inv16.x[j]);
+    }
+    redo |= r_new > kScaleHi || (inv_max >= kInvScaleLo16 && v_lane_max != 0.0f);
+  } else if constexpr (RANK1) {
     float c_min = c_new.x[0];
 #pragma unroll
     for (int j = 0; j < N; ++j) {
@@ -396,6 +417,17 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
   if (N == 4 && !SR) mword >>= 16;   // four codes entered at the top
   redo |= vfrac < 2.0f * kVGuard;
   if (__builtin_expect(redo, 0)) {
+    if constexpr (RANK1 && kRows) {
+      // the scales themselves: the new column maxima are the third array of the staging area
+#pragma unroll
+      for (int k = 0; k < N; k += 4) {
+        const float4 c = *reinterpret_cast<const float4 *>(rt->columns + 128 * N + e0 + k);
+        s_new.x[k] = min_nonneg(r_new, c.x);                  // adamw_fourbit_triton.py:749-755
+        s_new.x[k + 1] = min_nonneg(r_new, c.y);
+        s_new.x[k + 2] = min_nonneg(r_new, c.z);
+        s_new.x[k + 3] = min_nonneg(r_new, c.w);
+      }
+    }
     if constexpr (SR) {
 #pragma unroll
       for (int j = 0; j < N; ++j) {
@@ -521,7 +553,7 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_rows_kernel(const R
   using G = Geometry<PT, GT>;
   constexpr int N = G::kEpl;
   __shared__ uint2 lds[kLdsEntries];
-  __shared__ __attribute__((aligned(16))) float columns[2 * G::kTile];
+  __shared__ __attribute__((aligned(16))) float columns[3 * G::kTile];
   const int tid = threadIdx.x;
   const TableSlot slot = request_table_slot<SR>(tid);
   const uint32_t chunk = args.chunk_base + (blockIdx.x & 7u) * args.chunks_per_xcd + (blockIdx.x >> 3);
