@@ -331,6 +331,30 @@ __host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
   return x;
 }
 
+// lowbias32 without its last step: lowbias32(x) == y ^ (y >> 16) for y = lowbias32_open(x).
+// The step kernel takes the two 16-bit halves of the hash as floats and lets the conversions
+// do that step: the high half of y ^ (y >> 16) is y's own, the low half is y's two halves
+// xor-ed, and both selections ride on the instructions' operand selectors.
+__device__ __forceinline__ uint32_t lowbias32_open(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7FEB352Du;
+  x ^= x >> 15;
+  x *= 0x846CA68Bu;
+  return x;
+}
+
+__device__ __forceinline__ float hash_high_half_as_float(uint32_t y) {
+  float r;
+  asm("v_cvt_f32_u32_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1" : "=v"(r) : "v"(y));
+  return r;
+}
+
+__device__ __forceinline__ float hash_low_half_as_float(uint32_t y) {
+  uint32_t lo;
+  asm("v_xor_b32_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1 src1_sel:WORD_0" : "=v"(lo) : "v"(y));
+  return (float)lo;
+}
+
 // noise in (0, 1) from a 16-bit number (as a float): (2 n + 1) / 2^17, exact
 constexpr float kNoiseStep = 1.52587890625e-05f;     // 2^-16
 __device__ __forceinline__ float sr_noise_value(float n16) {

@@ -353,9 +353,9 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
     const uint32_t key0 = ((uint32_t)tb + e0) ^ tile_salt;
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      const uint32_t h = lowbias32(key0 ^ (uint32_t)j);
-      um.x[j] = (float)(h >> 16);
-      uv.x[j] = (float)(h & 0xffffu);
+      const uint32_t y = lowbias32_open(key0 ^ (uint32_t)j);   // the hash is y ^ (y >> 16)
+      um.x[j] = hash_high_half_as_float(y);
+      uv.x[j] = hash_low_half_as_float(y);
     }
   }
 #pragma unroll

