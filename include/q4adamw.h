@@ -207,9 +207,11 @@ uint32_t q4adamw_sr_tensor_salt(uint64_t seed, float step, uint32_t tensor_salt)
  * keeps its per-128 block scales.  row_max/col_max (rows and cols floats) are
  * updated by the call; row_max_next/col_max_next are state-owned scratch of the same
  * sizes that must hold zeros on entry and holds zeros again afterwards.
- * rows x cols, row-major, cols a multiple of 8 and at least 16; p and g aligned to their
- * element type (see q4adamw_tensor), col_max and col_max_next 16-byte aligned, the rest
- * 4-byte aligned.
+ * rows x cols, row-major, cols >= 2; p and g aligned to their element type (see
+ * q4adamw_tensor), col_max and col_max_next 16-byte aligned, the rest 4-byte aligned.  Rows of
+ * a multiple of 8 elements (and at least 16) take the tuned kernels; any other row length is
+ * taken element by element (matrices of fewer than 2^32 elements), as the draft scales every
+ * tensor with dim() > 1 this way (optim/adamw_fourbit_triton.py:841-846).
  *
  * Tensors of three or four dimensions (lead_dims = 2 or 3): cols is the last dimension,
  * lead_shape the others, rows their product.  Every leading dimension has its own
@@ -377,7 +379,7 @@ int q4adamw_quantize_rank1_scaled(const float *x, int64_t rows, int64_t cols, co
 
 /*
  * The same pair for a second moment with rank-1 scaling: x is a rows x cols fp32
- * matrix (cols a multiple of 8); row_max[i] / col_max[j] receive the abs-maxima of
+ * matrix; row_max[i] / col_max[j] receive the abs-maxima of
  * row i / column j, every element is divided by min(row_max[i], col_max[j]) and
  * mapped to the nearest code of the second moment's map (variance_quant_scaling and
  * variance_quant, optim/adamw_fourbit_triton.py:803-863); dequantize multiplies back
@@ -446,7 +448,7 @@ int q4adamw_sr_affine_entry(uint32_t k, float *out2);
 int q4adamw_grid_plan(uint64_t chunks, int threads, uint64_t *bases, uint64_t *counts, int capacity);
 /* Host-only, for tests: which of its three update kernels q4adamw_fused_4bit_rank1_multi runs on
  * a rows x cols matrix: 0 = tiles aligned to the rows, 1 = tiles anywhere in rows of at least a
- * tile, 2 = rows shorter than a tile.  both_16_bit: parameters and gradients are 16-bit types
+ * tile, 2 = rows shorter than a tile, 3 = rows of any length (no multiple of 8, or below 16).  both_16_bit: parameters and gradients are 16-bit types
  * (tiles of 512 elements instead of 256). */
 int q4adamw_rank1_form(int64_t rows, int64_t cols, int both_16_bit);
 void q4adamw_set_grid_limit(uint64_t workgroups);

@@ -35,7 +35,7 @@ HIPCC_FLAGS = [
 # libq4adamw.so: the C ABI with its launchers and small kernels, and the step kernels'
 # instantiations in translation units of their own, compiled side by side
 STEP_SOURCES = ["q4adamw.hip", "q4adamw_pick_fused.hip", "q4adamw_pick_rank1_rows.hip",
-                "q4adamw_pick_rank1_wide.hip", "q4adamw_pick_rank1_narrow.hip"]
+                "q4adamw_pick_rank1_wide.hip", "q4adamw_pick_rank1_narrow.hip", "q4adamw_pick_rank1_any.hip"]
 PROBE_SOURCES = ["q4stream_probe.hip"]
 
 

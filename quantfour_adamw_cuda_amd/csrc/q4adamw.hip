@@ -183,9 +183,12 @@ static SmallKernel pick_small(int p_dtype, int g_dtype, bool ext) {
 // row may be a partial one as long as its idle lanes are at most a sixteenth of the row (they
 // cost issue slots, which the 16-bit kernels have none to spare of; the wide form is 5 to 8 %
 // slower than the rows form).
-enum Rank1Shape { kShapeRows = 0, kShapeWide = 1, kShapeNarrow = 2 };
+enum Rank1Shape { kShapeRows = 0, kShapeWide = 1, kShapeNarrow = 2, kShapeAny = 3 };
 
 static Rank1Shape rank1_shape(const q4adamw_rank1_tensor &t, int64_t tile_elems) {
+  // rows that are no multiple of 8 elements long, or shorter than 16: lanes no longer lie in
+  // one row, and rows start inside a byte of the packed codes; every element finds its own place
+  if (t.cols % 8 != 0 || t.cols < 16) return kShapeAny;
   if (t.cols < tile_elems) return kShapeNarrow;
   const int64_t padded = (t.cols + tile_elems - 1) / tile_elems * tile_elems;
   if (t.cols % Q4ADAMW_BLOCK == 0 && t.cols >= 2 * tile_elems && t.rows >= 64 && (padded - t.cols) * 16 <= t.cols) {
@@ -220,6 +223,26 @@ static Rank1StatKernel pick_rank1_stats_ext(int g_dtype) {
 
 static Rank1StatKernel pick_rank1_stats(int g_dtype, bool ext) {
   return ext ? pick_rank1_stats_ext<true>(g_dtype) : pick_rank1_stats_ext<false>(g_dtype);
+}
+
+template <bool EXT>
+static Rank1StatKernel pick_rank1_stats_any_ext(int g_dtype) {
+  if (g_dtype == Q4ADAMW_BF16) return rank1_stats_any_kernel<Q4ADAMW_BF16, EXT>;
+  if (g_dtype == Q4ADAMW_FP16) return rank1_stats_any_kernel<Q4ADAMW_FP16, EXT>;
+  return rank1_stats_any_kernel<Q4ADAMW_FP32, EXT>;
+}
+
+static Rank1StatKernel pick_rank1_stats_any(int g_dtype, bool ext) {
+  return ext ? pick_rank1_stats_any_ext<true>(g_dtype) : pick_rank1_stats_any_ext<false>(g_dtype);
+}
+
+// tiles of the statistics launch of a matrix, by the form its rows allow
+static uint64_t rank1_stat_chunks(const q4adamw_rank1_tensor &t, uint32_t *col_groups) {
+  const bool any = t.cols % 8 != 0 || t.cols < 16;
+  const int64_t tile_rows = any ? kAnyStatRows : kStatRows, tile_cols = any ? kAnyStatCols : kStatCols;
+  const uint64_t groups = (uint64_t)((t.cols + tile_cols - 1) / tile_cols);
+  if (col_groups) *col_groups = (uint32_t)groups;
+  return (uint64_t)((t.rows + tile_rows - 1) / tile_rows) * groups;
 }
 
 // Fills the kernels' view of the caller's gradient options; returns whether the
@@ -456,10 +479,12 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
     const q4adamw_rank1_tensor &t = tensors[i];
     if (t.rows < 0 || t.cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
     if (t.rows == 0 || t.cols == 0) continue;
-    if (t.cols % 8 != 0 || t.cols < 16)
-      return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8 and at least 16");
+    if (t.cols < 2) return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs at least 2 columns");
     if (t.cols > 0x40000000ll || t.rows > 0x7ffffffffll / t.cols)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "rank-1 scaling handles matrices of up to 2^35 - 1 elements");
+    if ((t.cols % 8 != 0 || t.cols < 16) && t.rows * t.cols > 0xffffffffll)
+      return fail(Q4ADAMW_ERR_TOO_LARGE,
+                  "rank-1 scaling of rows that are no multiple of 8 long (or shorter than 16) handles fewer than 2^32 elements");
     if (!t.p || !t.g || !t.exp_avg || !t.exp_avg_sq || !t.exp_avg_scale || !t.row_max || !t.col_max ||
         !t.row_max_next || !t.col_max_next)
       return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
@@ -482,8 +507,7 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       }
       if (prod != t.rows) return fail(Q4ADAMW_ERR_ARG, "rows must be the product of the leading dimensions");
     }
-    const uint64_t stat_chunks = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) *
-                                 (uint64_t)((t.cols + kStatCols - 1) / kStatCols);
+    const uint64_t stat_chunks = rank1_stat_chunks(t, nullptr);
     if (rank1_chunks(t, chunk_elems / kWaves) > kMaxChunksPerLaunch || stat_chunks > kMaxChunksPerLaunch)
       return fail(Q4ADAMW_ERR_TOO_LARGE, "tensor too large: more than 2^31 - 16 chunks");
   }
@@ -494,7 +518,7 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   fa.go = a.go;
   fa.ntensors = 0;
   Rank1Kernel kernel = nullptr;
-  const Rank1StatKernel stat_kernel = pick_rank1_stats(g_dtype, ext);
+  Rank1StatKernel stat_kernel = nullptr;
   a.ntensors = 0;
   uint64_t chunks = 0, stat_chunks = 0;
   // statistics of every tensor of the batch, then the update, then the commit
@@ -539,17 +563,19 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
   // three passes: matrices whose rows are whole tiles take the kernel whose workgroups share
   // the columns' maxima of four rows; other matrices with rows of at least a tile the one
   // that finds a tile's row on the scalar unit; narrower ones the one whose lanes find their own
-  for (int shape = kShapeRows; shape <= kShapeNarrow; ++shape) {
-    kernel = shape == kShapeRows   ? pick_rank1_rows(p_dtype, g_dtype, ext, sr, exact)
-             : shape == kShapeWide ? pick_rank1_wide(p_dtype, g_dtype, ext, sr, exact)
-                                   : pick_rank1_narrow(p_dtype, g_dtype, ext, sr, exact);
+  for (int shape = kShapeRows; shape <= kShapeAny; ++shape) {
+    kernel = shape == kShapeRows     ? pick_rank1_rows(p_dtype, g_dtype, ext, sr, exact)
+             : shape == kShapeWide   ? pick_rank1_wide(p_dtype, g_dtype, ext, sr, exact)
+             : shape == kShapeNarrow ? pick_rank1_narrow(p_dtype, g_dtype, ext, sr, exact)
+                                     : pick_rank1_any(p_dtype, g_dtype, ext, sr, exact);
+    stat_kernel = shape == kShapeAny ? pick_rank1_stats_any(g_dtype, ext) : pick_rank1_stats(g_dtype, ext);
     for (int i = 0; i < count; ++i) {
       const q4adamw_rank1_tensor &t = tensors[i];
       if (t.rows == 0 || t.cols == 0 || rank1_shape(t, tile_elems) != shape) continue;
       const int64_t numel = t.rows * t.cols;
       const uint64_t c = rank1_chunks(t, tile_elems);
-      const uint32_t groups = (uint32_t)((t.cols + kStatCols - 1) / kStatCols);
-      const uint64_t sc_ = (uint64_t)((t.rows + kStatRows - 1) / kStatRows) * groups;
+      uint32_t groups = 0;
+      const uint64_t sc_ = rank1_stat_chunks(t, &groups);
       if (a.ntensors == kMaxRank1Tensors || chunks + c > kMaxChunksPerLaunch ||
           stat_chunks + sc_ > kMaxChunksPerLaunch || (t.lead_dims >= 2 && fa.ntensors == kMaxFoldTensors)) {
         if (int rc = launch()) return rc;
@@ -578,8 +604,10 @@ static int fused_4bit_rank1_multi_impl(const q4adamw_rank1_tensor *tensors, int 
       d.numel = numel;
       d.rows = t.rows;
       d.cols = t.cols;
-      // the divisor the tensor's kernel needs: tiles per row, or cols / 8
-      const FastDiv fd = make_fast_div(shape == kShapeRows ? (uint32_t)rank1_tiles_per_row(t, tile_elems) : (uint32_t)(t.cols >> 3));
+      // the divisor the tensor's kernel needs: tiles per row, cols, or cols / 8
+      const FastDiv fd = make_fast_div(shape == kShapeRows  ? (uint32_t)rank1_tiles_per_row(t, tile_elems)
+                                       : shape == kShapeAny ? (uint32_t)t.cols
+                                                            : (uint32_t)(t.cols >> 3));
       d.div_magic = fd.magic;
       d.div_shift = fd.shift;
       a.sr_salt[a.ntensors] = !sr ? 0u : a.go.sc_dev ? lowbias32(salts ? salts[i] : (uint32_t)i)
@@ -858,7 +886,6 @@ int q4adamw_quantize(const float *x, int64_t numel, int which, uint8_t *codes, f
 
 static int check_rank1_shape(int64_t rows, int64_t cols) {
   if (rows < 0 || cols < 0) return fail(Q4ADAMW_ERR_ARG, "negative shape");
-  if (cols % 8 != 0) return fail(Q4ADAMW_ERR_ARG, "rank-1 scaling needs cols to be a multiple of 8");
   if (rows > 0 && cols > 0 && (cols > 0x40000000ll || rows > 0x7ffffffffll / cols))
     return fail(Q4ADAMW_ERR_TOO_LARGE, "rank-1 scaling handles matrices of up to 2^35 - 1 elements");
   return 0;
@@ -877,7 +904,7 @@ int q4adamw_quantize_rank1(const float *x, int64_t rows, int64_t cols, uint8_t *
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, row_max, rows);
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, col_max, cols);
   hipLaunchKernelGGL(rank1_absmax_kernel, tiles, dim3(256), 0, s, x, rows, cols, row_max, col_max);
-  const uint64_t groups = ((uint64_t)rows * cols / 2 + 255) / 256;
+  const uint64_t groups = (((uint64_t)rows * cols + 1) / 2 + 255) / 256;
   return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
     hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)count), dim3(256), 0, s, x, rows, cols,
                        static_cast<const float *>(row_max), static_cast<const float *>(col_max), codes, (int64_t)base);
@@ -893,7 +920,7 @@ int q4adamw_quantize_rank1_scaled(const float *x, int64_t rows, int64_t cols, co
   if (!x || !codes || !row_scale || !col_max) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(x, 4) || !aligned(row_scale, 4) || !aligned(col_max, 4))
     return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t groups = ((uint64_t)rows * cols / 2 + 255) / 256;
+  const uint64_t groups = (((uint64_t)rows * cols + 1) / 2 + 255) / 256;
   return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
     hipLaunchKernelGGL(quantize_rank1_kernel, dim3((unsigned)count), dim3(256), 0, static_cast<hipStream_t>(stream), x,
                        rows, cols, row_scale, col_max, codes, (int64_t)base);
@@ -909,7 +936,7 @@ int q4adamw_dequantize_rank1(const uint8_t *codes, const float *row_max, const f
   if (!codes || !row_max || !col_max || !out) return fail(Q4ADAMW_ERR_ARG, "null tensor pointer");
   if (!aligned(out, 4) || !aligned(row_max, 4) || !aligned(col_max, 4))
     return fail(Q4ADAMW_ERR_ALIGN, "fp32 buffers must be 4-byte aligned");
-  const uint64_t groups = ((uint64_t)rows * cols / 2 + 255) / 256;
+  const uint64_t groups = (((uint64_t)rows * cols + 1) / 2 + 255) / 256;
   return for_each_grid(groups, 256, [&](uint64_t base, uint64_t count) -> int {
     hipLaunchKernelGGL(dequantize_rank1_kernel, dim3((unsigned)count), dim3(256), 0,
                        static_cast<hipStream_t>(stream), codes, row_max, col_max, rows, cols, out, (int64_t)base);

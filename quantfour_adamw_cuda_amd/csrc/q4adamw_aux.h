@@ -308,18 +308,21 @@ __global__ __launch_bounds__(256) void rank1_absmax_kernel(const float *x_, int6
 }
 
 // one thread per packed byte: x / min(row maximum, column maximum), IEEE division, the
-// 15-compare count (optim/adamw_fourbit_triton.py:834-863)
+// 15-compare count (optim/adamw_fourbit_triton.py:834-863).  Rows may have any length, so the
+// byte's two elements find their rows and columns separately.
 __global__ __launch_bounds__(256) void quantize_rank1_kernel(const float *x_, int64_t rows, int64_t cols,
                                                              const float *row_max, const float *col_max,
                                                              uint8_t *codes_, int64_t group0) {
   const int64_t e = ((group0 + blockIdx.x) * 256 + threadIdx.x) * 2;
-  if (e >= rows * cols) return;
-  const int64_t i = e / cols, j = e - i * cols;  // cols is even: both elements in row i
-  const float r = as_global<const float>(row_max)[i];
+  const int64_t numel = rows * cols;
+  if (e >= numel) return;
   uint32_t byte = 0;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
-    const float q = as_global<const float>(x_)[e + h] / __builtin_fminf(r, as_global<const float>(col_max)[j + h]);
+    if (e + h >= numel) break;     // an odd element count: the last byte's high nibble stays 0
+    const int64_t i = (e + h) / cols, j = (e + h) - i * cols;
+    const float q = as_global<const float>(x_)[e + h] /
+                    __builtin_fminf(as_global<const float>(row_max)[i], as_global<const float>(col_max)[j]);
 #pragma unroll
     for (int k = 0; k < 15; ++k) byte += (qmid_v(k) < q) ? (1u << (4 * h)) : 0u;
   }
@@ -331,12 +334,16 @@ __global__ __launch_bounds__(256) void dequantize_rank1_kernel(const uint8_t *co
                                                                const float *col_max, int64_t rows,
                                                                int64_t cols, float *out_, int64_t group0) {
   const int64_t e = ((group0 + blockIdx.x) * 256 + threadIdx.x) * 2;
-  if (e >= rows * cols) return;
-  const int64_t i = e / cols, j = e - i * cols;
-  const float r = as_global<const float>(row_max)[i];
+  const int64_t numel = rows * cols;
+  if (e >= numel) return;
   const uint32_t byte = as_global<const uint8_t>(codes_)[e >> 1];
-  as_global<float>(out_)[e] = qmap_v((int)(byte & 15u)) * __builtin_fminf(r, as_global<const float>(col_max)[j]);
-  as_global<float>(out_)[e + 1] = qmap_v((int)(byte >> 4)) * __builtin_fminf(r, as_global<const float>(col_max)[j + 1]);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (e + h >= numel) break;
+    const int64_t i = (e + h) / cols, j = (e + h) - i * cols;
+    as_global<float>(out_)[e + h] = qmap_v((int)((byte >> (4 * h)) & 15u)) *
+                                    __builtin_fminf(as_global<const float>(row_max)[i], as_global<const float>(col_max)[j]);
+  }
 }
 
 // cuda_adamw_kernels.cu:329-343: code -> code-book entry * block scale

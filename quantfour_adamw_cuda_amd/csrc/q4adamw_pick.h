@@ -31,9 +31,10 @@ typedef void (*Rank1StatKernel)(const Rank1StatArgs);
 FusedKernel pick_fused(int p_dtype, int g_dtype, bool ext, bool sr, bool exact);
 // the rank-1 update kernels: tiles anywhere in a matrix of rows at least a tile long
 // (pick_rank1_wide), matrices narrower than a tile (pick_rank1_narrow), tiles aligned to the
-// rows of a matrix (pick_rank1_rows)
+// rows of a matrix (pick_rank1_rows), rows of any length (pick_rank1_any)
 Rank1Kernel pick_rank1_wide(int p_dtype, int g_dtype, bool ext, bool sr, bool exact);
 Rank1Kernel pick_rank1_narrow(int p_dtype, int g_dtype, bool ext, bool sr, bool exact);
 Rank1Kernel pick_rank1_rows(int p_dtype, int g_dtype, bool ext, bool sr, bool exact);
+Rank1Kernel pick_rank1_any(int p_dtype, int g_dtype, bool ext, bool sr, bool exact);
 
 }  // namespace q4

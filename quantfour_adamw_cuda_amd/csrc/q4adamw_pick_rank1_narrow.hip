@@ -1,4 +1,4 @@
-// The instantiations of fused_4bit_rank1_kernel<..., NARROW = true> (rank-1 update) and their selection.
+// The instantiations of fused_4bit_rank1_kernel<..., kTileNarrow> (rank-1 update) and their selection.
 #include <hip/hip_runtime.h>
 
 #include "q4adamw_pick.h"
@@ -8,7 +8,7 @@ namespace q4 {
 
 template <bool EXT, bool SR, bool EXACT>
 static Rank1Kernel pick_pg(int p_dtype, int g_dtype) {
-  Q4_PICK_PG(fused_4bit_rank1_kernel, EXT, SR, true, EXACT)
+  Q4_PICK_PG(fused_4bit_rank1_kernel, EXT, SR, kTileNarrow, EXACT)
 }
 
 template <bool EXT, bool SR>

@@ -135,6 +135,59 @@ __global__ __launch_bounds__(kThreads) void rank1_stats_kernel(const Rank1StatAr
   }
 }
 
+// The same statistics for rows of any length (not a multiple of 8, or shorter than 16), where a
+// row starts at any element of the packed codes: a workgroup takes kAnyStatRows rows x 256
+// columns, a thread one column, element by element; the rows' maxima meet in LDS, then one
+// atomic per row and per column.  Same arithmetic, operation for operation.
+constexpr int kAnyStatRows = 64;
+constexpr int kAnyStatCols = 256;
+
+template <int GT, bool EXT>
+__global__ __launch_bounds__(kThreads) void rank1_stats_any_kernel(const Rank1StatArgs args) {
+  __shared__ uint32_t row_bits[kAnyStatRows];
+  const uint32_t chunk = args.chunk_base + blockIdx.x;
+  float gscale = 1.0f;
+  if (EXT && !grad_ops_begin(args.go, gscale)) return;
+  const int t = find_tensor(args, chunk);
+  const auto &T = args.desc[t];
+  const uint32_t local = chunk - args.first_chunk[t];
+  const uint32_t groups = args.col_groups[t];
+  const uint32_t rg = local / groups, cg = local - rg * groups;
+  const int tid = threadIdx.x;
+  const int64_t col = (int64_t)cg * kAnyStatCols + tid;
+  const bool active = col < T.cols;
+  const int64_t row0 = (int64_t)rg * kAnyStatRows;
+  const int nrows = (int)(row0 + kAnyStatRows < T.rows ? kAnyStatRows : T.rows - row0);
+  if (tid < kAnyStatRows) row_bits[tid] = 0u;
+  __syncthreads();
+  const float c_old = active ? as_global<const float>(T.cmax)[col] : 0.0f;
+  float c_max = 0.0f;
+  for (int r = 0; r < nrows; ++r) {
+    float v = 0.0f;     // lanes past the last column leave every maximum alone
+    if (active) {
+      const int64_t e = (row0 + r) * T.cols + col;
+      float g = load_scalar<GT>(T.g, e);
+      if (EXT) g *= gscale;
+      const uint32_t code = ((uint32_t)as_global<const uint8_t>(T.v)[e >> 1] >> (4 * (int)(e & 1))) & 15u;
+      const float code_value = __builtin_fmaf((float)code, 0.0625f, 0.0625f);  // (code + 1) / 16, exact
+      const float v_old = code_value * min_nonneg(as_global<const float>(T.rmax)[row0 + r], c_old);
+      v = args.b2 * v_old + args.r2 * (g * g);
+    }
+    // fmaxf drops a NaN: a NaN never becomes a maximum, as in the update kernel's scales
+    c_max = __builtin_fmaxf(c_max, v);
+    uint32_t u = f2bits(__builtin_fmaxf(v, 0.0f));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const uint32_t o = (uint32_t)__shfl_xor((int)u, off, 64);
+      u = u > o ? u : o;
+    }
+    if ((tid & 63) == 0 && u != 0u) atomicMax(&row_bits[r], u);
+  }
+  if (active && c_max != 0.0f) atomic_max_nonneg(T.cmax_next + col, c_max);
+  __syncthreads();
+  if (tid < nrows && row_bits[tid] != 0u) atomic_max_nonneg(T.rmax_next + row0 + tid, bits2f(row_bits[tid]));
+}
+
 // After the update: the new statistics become the current ones and the buffers that
 // received them go back to zero for the next step's maxima.  One workgroup column per
 // tensor (blockIdx.y), grid-stride over rows + cols floats.

@@ -34,8 +34,10 @@ struct Geometry {
 // consecutive rows: they fetch the columns' maxima once, together, and pass them through LDS
 // (RowsTile).  kTileRowsLast is the same for the last tile of a row that is not a whole
 // number of tiles long: its first RowsTile::width elements are there (whole blocks), the
-// lanes of the others load nothing, work on zeros and store nothing.
-constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2, kTileRowsLast = 3;
+// lanes of the others load nothing, work on zeros and store nothing.  kTileAny: rows of any
+// length (not a multiple of 8, or shorter than 16): every element finds its own row and column
+// (matrices of fewer than 2^32 elements).
+constexpr int kTileWide = 0, kTileNarrow = 1, kTileRows = 2, kTileRowsLast = 3, kTileAny = 4;
 
 // What a wave of the kTileRows form knows beyond its tile number: its row, the tile's first
 // column, and this thread's share of the workgroup's fetch of the columns' maxima (old and
@@ -101,7 +103,22 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
   // rank-1: this lane's row maxima (old, new) and its N column maxima (old, new)
   float r_old = 0.0f, r_new = 0.0f;
   Vals<N> c_old, c_new;
-  if constexpr (RANK1) {
+  Vals<N> ro, rn;   // kTileAny: the row maxima of every element
+  if constexpr (RANK1 && SHAPE == kTileAny) {
+    // T.div_magic / div_shift divide by cols; indices of elements past the end are clamped
+    const uint32_t first = (uint32_t)tb + e0, cols = (uint32_t)T.cols, last = (uint32_t)T.rows - 1u;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const uint32_t e = first + (uint32_t)j;
+      uint32_t row = fast_div(e, T.div_magic, T.div_shift);
+      const uint32_t col = e - row * cols;
+      row = row < last ? row : last;
+      ro.x[j] = as_global<const float>(T.rmax)[row];
+      rn.x[j] = as_global<const float>(T.rmax_next)[row];
+      c_old.x[j] = as_global<const float>(T.cmax)[col];
+      c_new.x[j] = as_global<const float>(T.cmax_next)[col];
+    }
+  } else if constexpr (RANK1) {
     // (row, column) of the tile's first element, in units of 8 elements so that the
     // division is a 32-bit one.  A lane's N elements (N = 4 or 8, first one a multiple of N)
     // lie in one row, because rows are multiples of 8 elements long.
@@ -243,7 +260,7 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
     const uint32_t vo = entry_offset(j & 1 ? v_odd : v_even, j >> 1, two);
     const float m_old = *reinterpret_cast<const float *>(lds_bytes + mo);
     float v_old = *reinterpret_cast<const float *>(lds_bytes + vo + kLdsSecondMoment * 4u);
-    if constexpr (RANK1) v_old = sc.b2 * (v_old * min_nonneg(r_old, c_old.x[j]));  // adamw_fourbit_triton.py:520-527
+    if constexpr (RANK1) v_old = sc.b2 * (v_old * min_nonneg(SHAPE == kTileAny ? ro.x[j] : r_old, c_old.x[j]));  // adamw_fourbit_triton.py:520-527
     const float gj = g[j];
     float m = m_old + sc.r1 * gj;                 // m_old, v_old: beta times the old moment
     float v = v_old + sc.r2 * (gj * gj);
@@ -327,6 +344,17 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
       inv_max = max_nonneg(inv_max, inv16.x[j]);
     }
     redo |= r_new > kScaleHi || (inv_max >= kInvScaleLo16 && v_lane_max != 0.0f);
+  } else if constexpr (RANK1 && SHAPE == kTileAny) {
+    float s_least = rn.x[0], s_most = 0.0f;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float sj = min_nonneg(rn.x[j], c_new.x[j]);      // adamw_fourbit_triton.py:749-755
+      s_new.x[j] = sj;
+      s_least = min_nonneg(s_least, sj);
+      s_most = max_nonneg(s_most, sj);
+      inv16.x[j] = __builtin_amdgcn_rcpf(max_nonneg(sj, kScaleLo)) * 16.0f;
+    }
+    redo |= s_most > kScaleHi || (s_least < kScaleLo && v_lane_max != 0.0f);
   } else if constexpr (RANK1) {
     float c_min = c_new.x[0];
 #pragma unroll
@@ -510,7 +538,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_kernel(const FusedArgs ar
 // rank-1 scaling of the second moment: the update kernels (statistics, commit and the folds
 // for tensors of more dimensions: q4adamw_rank1.h)
 // ---------------------------------------------------------------------------
-template <int PT, int GT, bool EXT, bool SR, bool NARROW, bool EXACT>
+// FORM: how a tile lies in its matrix: kTileWide (rows of at least a tile, multiples of 8),
+// kTileNarrow (shorter rows, multiples of 8), kTileAny (rows of any length)
+template <int PT, int GT, bool EXT, bool SR, int FORM, bool EXACT>
 __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1Args args) {
   using G = Geometry<PT, GT>;
   __shared__ uint2 lds[kLdsEntries];
@@ -538,9 +568,9 @@ __global__ __launch_bounds__(kThreads) void fused_4bit_rank1_kernel(const Rank1A
   const uint32_t salt = !SR ? 0u : EXT ? step_salt(args.sr_salt[t], args.go, args.seed_lo, args.seed_hi) : args.sr_salt[t];
   const StepConsts sc = EXT ? step_consts(args.sc, args.go) : args.sc;
   if (begin + G::kTile <= T.numel)
-    process_tile<PT, GT, true, EXT, true, SR, NARROW ? kTileNarrow : kTileWide, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, true, EXT, true, SR, FORM, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
   else
-    process_tile<PT, GT, false, EXT, true, SR, NARROW ? kTileNarrow : kTileWide, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
+    process_tile<PT, GT, false, EXT, true, SR, FORM, EXACT>(T, begin, lane, wave, tid, sc, lds, slot, gscale, zero_g, salt);
 }
 
 // The same for matrices whose rows are a whole number of quantization blocks and at least

@@ -95,8 +95,9 @@ class AdamWFused_QuantFour(torch.optim.Optimizer):
         # 128 consecutive elements, what the fused CUDA path does (cuda_adamw_kernels.cu:353-383);
         # "rank1" = min(row maximum, column maximum) for matrices, the draft's SecondMoment
         # setting (adamw_fourbit_triton.py:124, :834-863), one statistic per dimension for
-        # tensors of two to four dimensions; others, and tensors whose last dimension is not
-        # a multiple of 8 or below 16, keep group scaling, as 1-D tensors do there (:841-846)
+        # tensors of two to four dimensions of any sizes; 1-D tensors keep group scaling, as
+        # there (:841-846), and so do tensors of five and more dimensions or with a last
+        # dimension of 1
         if variance_scale_type not in ("group", "rank1"):
             raise ValueError(f"Invalid variance_scale_type: {variance_scale_type=}")
         self.variance_scale_type = variance_scale_type

@@ -307,15 +307,17 @@ def fused_4bit_multi_sr(ps, gs, exps, sqs, exp_scales, sq_scales, beta1, beta2, 
                     beta1, beta2, lr, weight_decay, eps, step, options)
 
 
-RANK1_MIN_COLS = 16
-
-
 def rank1_eligible(p):
-    """Whether a parameter's second moment can take rank-1 scaling: a tensor of two to four
-    dimensions whose last dimension is a multiple of 8 and at least 16 (other tensors keep
-    per-128 block scales, as 1-D tensors do in the reference's draft,
-    optim/adamw_fourbit_triton.py:841-846)."""
-    return 2 <= p.dim() <= 4 and p.shape[-1] % 8 == 0 and p.shape[-1] >= RANK1_MIN_COLS
+    """Whether the second moment of `p` can be rank-1 scaled: every tensor of two to four
+    dimensions, as the draft scales every tensor with dim() > 1
+    (optim/adamw_fourbit_triton.py:841-846).  Left on block scales, like 1-D tensors there: a
+    last dimension of 1 (a column is a vector laid out flat), five and more dimensions, and --
+    a limit of the kernel for rows that are no multiple of 8 elements long or shorter than 16
+    -- such tensors of 2^32 elements and more."""
+    if not 2 <= p.dim() <= 4 or p.shape[-1] < 2:
+        return False
+    aligned_rows = p.shape[-1] % 8 == 0 and p.shape[-1] >= 16
+    return aligned_rows or p.numel() < (1 << 32)
 
 
 def rank1_row_scale(lead_maxes, lead_shape):
@@ -333,7 +335,7 @@ def rank1_row_scale(lead_maxes, lead_shape):
 
 def check_rank1(p, g, exp, sq, exp_scale, row_max, col_max, row_next, col_next, lead=None):
     _check_common(p, g)
-    assert rank1_eligible(p), "rank-1 scaling needs 2 to 4 dimensions, the last a multiple of 8 and at least 16"
+    assert rank1_eligible(p), "rank-1 scaling needs 2 to 4 dimensions, the last of at least 2"
     cols = p.shape[-1]
     rows = p.numel() // cols
     assert (lead is None) == (p.dim() == 2), "tensors of more than two dimensions need their leading statistics"
@@ -505,7 +507,7 @@ def quantize_state_rank1(x):
     column maxima [cols]); element (i, j) is divided by min(row_max[i], col_max[j]).  Device
     form of variance_quant with rank-1 scaling (optim/adamw_fourbit_triton.py:803-863)."""
     L = _lib.load()
-    assert x.is_cuda and x.dim() == 2 and x.shape[1] % 8 == 0, "needs a cuda matrix with cols % 8 == 0"
+    assert x.is_cuda and x.dim() == 2, "needs a cuda matrix"
     x = x.detach().to(torch.float32).contiguous()
     rows, cols = x.shape
     codes = torch.empty((rows * cols + 1) // 2, dtype=torch.uint8, device=x.device)
@@ -523,7 +525,7 @@ def quantize_state_rank1_scaled(x, row_scale, col_max):
     by min(row_scale[i], col_max[j]): the quantizer for tensors of more than two dimensions,
     whose rows' scales come from rank1_row_scale."""
     L = _lib.load()
-    assert x.is_cuda and x.dim() == 2 and x.shape[1] % 8 == 0, "needs a cuda matrix with cols % 8 == 0"
+    assert x.is_cuda and x.dim() == 2, "needs a cuda matrix"
     x = x.detach().to(torch.float32).contiguous()
     rows, cols = x.shape
     for t, n in ((row_scale, rows), (col_max, cols)):

@@ -106,6 +106,7 @@ def test_rank1_kernel_form_by_shape(lib):
     big_rows = (1 << 32) // 4480 + 2
     assert form(big_rows, 4480, 1) == 1 and form(big_rows - 3, 4480, 1) == 0      # just above / below 2^32 elements
     assert form((1 << 32) // 4096 + 4, 4096, 1) == 0                              # whole tiles: aligned anyway
+    assert form(100, 521, 0) == 3 and form(100, 12, 0) == 3 and form(5000, 2, 1) == 3 and form(64, 50257, 1) == 3
     assert form(0, 16, 0) == -1 and form(8, 1 << 31, 0) == -1
 
 
@@ -117,8 +118,12 @@ def test_new_entry_points_validate_before_any_gpu_call(lib):
     assert lib.q4adamw_fused_4bit_multi_sr(t, 1, None, 7, 0, 0, *hp, None, z) == -1      # null pointers
     assert lib.q4adamw_fused_4bit_multi_ex(t, 1, 0, 5, *hp, None, z) == -1               # dtype tag
     r = (_lib.Q4Rank1Tensor * 1)()
-    r[0].rows, r[0].cols = 4, 500
-    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -1 and b"cols" in lib.q4adamw_last_error()
+    r[0].rows, r[0].cols = 4, 1
+    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -1 and b"columns" in lib.q4adamw_last_error()
+    r[0].rows, r[0].cols = 4, 500                                                        # any row length is taken: next check
+    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -1 and b"null" in lib.q4adamw_last_error()
+    r[0].rows, r[0].cols = 1 << 20, (1 << 12) + 4                                        # ... below 2^32 elements
+    assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -4 and b"2^32" in lib.q4adamw_last_error()
     r[0].cols = 1 << 31
     assert lib.q4adamw_fused_4bit_rank1_multi(r, 1, 0, 0, *hp, None, z) == -4
     r[0].rows, r[0].cols = 0, 512                                                        # empty: nothing to do
@@ -126,7 +131,8 @@ def test_new_entry_points_validate_before_any_gpu_call(lib):
     g = (_lib.Q4Grad * 1)()
     g[0].numel = 16
     assert lib.q4adamw_grad_norm(g, 1, 0, 1.0, None, 0.0, z, 16384, z, z) == -1
-    assert lib.q4adamw_quantize_rank1(z, 4, 12, z, z, z, z) == -1 and b"multiple of 8" in lib.q4adamw_last_error()
+    assert lib.q4adamw_quantize_rank1(z, 4, 12, z, z, z, z) == -1 and b"null" in lib.q4adamw_last_error()
+    assert lib.q4adamw_quantize_rank1(z, -4, 12, z, z, z, z) == -1 and b"negative" in lib.q4adamw_last_error()
     assert lib.q4adamw_dequantize_rank1(z, z, z, 0, 512, z, z) == 0
     # hyper-parameter domain, shared by every step entry point
     t[0].numel = 0

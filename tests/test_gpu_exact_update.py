@@ -170,10 +170,10 @@ def test_exact_form_with_stochastic_rounding(cuda, p_dt, g_dt):
         assert same_params(dev.p, ref[0] if p_dt != "fp32" else ref[0].numpy()) == 0, f"step {step}"
 
 
-@pytest.mark.parametrize("shape", [(66, 1024), (257, 768), (300, 16), (70, 2560), (66, 2432)])
+@pytest.mark.parametrize("shape", [(66, 1024), (257, 768), (300, 16), (70, 2560), (66, 2432), (257, 77), (64, 2501)])
 @pytest.mark.parametrize("p_dt,g_dt,sr", [("fp32", "bf16", False), ("bf16", "bf16", False), ("fp32", "fp32", True)])
 def test_exact_form_with_rank1_scaling(cuda, shape, p_dt, g_dt, sr):
-    """the three rank-1 update kernels (row-aligned, wide, narrow), with and without stochastic rounding"""
+    """the four rank-1 update kernels (row-aligned, wide, narrow, rows of any length), with and without stochastic rounding"""
     rows, cols = shape
     gen = torch.Generator().manual_seed(rows + cols)
     p0 = (torch.randn(rows, cols, generator=gen) * 0.05).to(DT[p_dt])

@@ -62,7 +62,10 @@ SHAPES = [(66, 1024), (128, 1536), (64, 4096), (64, 512), (3, 4096), (100, 520),
           (66, 2432), (64, 4352), (65, 6272), (67, 2176),
           # narrow matrices: a tile spans several rows (fewer than 256 columns, or than 512 when
           # parameters and gradients are 16-bit types)
-          (300, 16), (77, 64), (1000, 24), (513, 248), (40, 504), (9, 256), (2000, 136)]
+          (300, 16), (77, 64), (1000, 24), (513, 248), (40, 504), (9, 256), (2000, 136),
+          # rows of any length: no multiple of 8, or shorter than 16; rows then start at any
+          # element of the packed codes and an access of 4 or 8 elements crosses rows
+          (130, 1031), (257, 77), (33, 129), (4500, 2), (700, 9), (64, 2501), (3, 4099), (1, 5001), (100, 12)]
 
 
 @pytest.mark.parametrize("p_dt,g_dt", [("fp32", "bf16"), ("bf16", "bf16"), ("fp32", "fp32"), ("bf16", "fp32"),
@@ -179,7 +182,7 @@ def test_rank1_stochastic_rounding_many_tensors_and_options(cuda):
     assert all(torch.equal(x.r, y.r) and torch.equal(x.c, y.c) for x, y in zip(a, c))   # statistics do not depend on the noise
 
 
-ND_SHAPES = [(4, 6, 64), (3, 5, 520), (2, 3, 4, 32), (8, 16, 1024), (1, 7, 16), (5, 1, 2, 264)]
+ND_SHAPES = [(4, 6, 64), (3, 5, 520), (2, 3, 4, 32), (8, 16, 1024), (1, 7, 16), (5, 1, 2, 264), (6, 7, 101), (3, 4, 5, 7)]
 
 
 @pytest.mark.parametrize("stochastic", [False, True])
@@ -305,29 +308,29 @@ def test_rank1_argument_errors(cuda):
     g = torch.zeros_like(p)
     arr = q.make_rank1_table([d.p], [g], [d.m], [d.v], [d.sm], [d.r], [d.c], [d.rn], [d.cn])
     call = lambda a: L.q4adamw_fused_4bit_rank1_multi(a, 1, 0, 0, *HPA, 1.0, None, None)
-    arr[0].cols = 500
-    assert call(arr) == -1 and b"cols" in L.q4adamw_last_error()
-    arr[0].cols = 8
-    assert call(arr) == -1 and b"cols" in L.q4adamw_last_error()
-    arr[0].cols = 512
+    arr[0].cols = 1
+    assert call(arr) == -1 and b"columns" in L.q4adamw_last_error()
+    arr[0].rows, arr[0].cols = 1 << 20, 4100           # rows of any length: fewer than 2^32 elements
+    assert call(arr) == -4 and b"2^32" in L.q4adamw_last_error()
+    arr[0].rows, arr[0].cols = 4, 512
     arr[0].col_max = d.c.data_ptr() + 4
     assert call(arr) == -2
     arr[0].col_max = None
     assert call(arr) == -1
     with pytest.raises(AssertionError, match="rank-1"):
-        q.make_rank1_table([torch.zeros(4, 100, device=cuda)], [torch.zeros(4, 100, device=cuda)], [d.m], [d.v],
+        q.make_rank1_table([torch.zeros(400, 1, device=cuda)], [torch.zeros(400, 1, device=cuda)], [d.m], [d.v],
                            [d.sm], [d.r], [d.c], [d.rn], [d.cn])
 
 
 # ---------------------------------------------------------------------------
 # interchange kernels and the optimizer class
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("shape", [(1, 8), (7, 24), (64, 512), (130, 1032), (300, 264)])
+@pytest.mark.parametrize("shape", [(1, 8), (7, 24), (64, 512), (130, 1032), (300, 264), (33, 129), (257, 77), (5, 5), (4001, 1)])
 def test_rank1_quantize_dequantize_against_oracle(cuda, shape):
     gen = torch.Generator().manual_seed(shape[0] + shape[1])
     x = torch.rand(shape, generator=gen) ** 6
     x[shape[0] // 2] = 0.0
-    x[:, 3] = 0.0
+    x[:, min(3, shape[1] - 1)] = 0.0
     codes, rmax, cmax = q.quantize_state_rank1(x.to(cuda))
     rc, rr, rcm = ot.quantize_rank1(x)
     assert torch.equal(codes.cpu(), rc) and torch.equal(rmax.cpu(), rr) and torch.equal(cmax.cpu(), rcm)

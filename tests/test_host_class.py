@@ -178,14 +178,17 @@ def test_step_counters_share_one_buffer_and_follow_replacements():
 
 
 def test_rank1_state_layout_and_round_trip():
-    """variance_scale_type="rank1": matrices with cols % 8 == 0 and cols >= 16 keep row and
-    column maxima (the draft's max_dims, keepdim shapes) instead of block scales; everything
-    else keeps block scales; a state_dict round trip keeps layout, values and dtypes"""
+    """variance_scale_type="rank1": matrices keep row and column maxima (the draft's max_dims,
+    keepdim shapes) instead of block scales, whatever their sizes; vectors and matrices of one
+    column keep block scales; a state_dict round trip keeps layout, values and dtypes"""
     wide, narrow, vec = [torch.nn.Parameter(torch.randn(s).to(torch.bfloat16))
-                         for s in ((12, 1024), (1024, 100), (8192,))]
-    opt = AdamWFused_QuantFour([wide, narrow, vec], variance_scale_type="rank1")
-    for p in (wide, narrow, vec):
+                         for s in ((12, 1024), (8192, 1), (8192,))]
+    odd = torch.nn.Parameter(torch.randn(1024, 101).to(torch.bfloat16))
+    opt = AdamWFused_QuantFour([wide, narrow, vec, odd], variance_scale_type="rank1")
+    for p in (wide, narrow, vec, odd):
         opt._init_state(p)
+    oo = opt.state[odd]["variance_qstate"]["overhead"]
+    assert oo["max1"] is None and [tuple(t.shape) for t in oo["max_dims"]] == [(1024, 1), (1, 101)]
     ov = opt.state[wide]["variance_qstate"]["overhead"]
     assert ov["max1"] is None and ov["dim"] == 2
     assert [tuple(t.shape) for t in ov["max_dims"]] == [(12, 1), (1, 1024)]
@@ -198,8 +201,8 @@ def test_rank1_state_layout_and_round_trip():
     ov["max_dims"][0].fill_(1.0 + 2.0 ** -20)            # not a bf16 value
     ov["max_dims"][1].fill_(3.0)
     ov["scratch_dims"][1].fill_(9.0)                     # scratch is not state: it restarts from zero
-    wide2, narrow2, vec2 = [torch.nn.Parameter(p.detach().clone()) for p in (wide, narrow, vec)]
-    opt2 = AdamWFused_QuantFour([wide2, narrow2, vec2])  # the layout follows the checkpoint
+    wide2, narrow2, vec2, odd2 = [torch.nn.Parameter(p.detach().clone()) for p in (wide, narrow, vec, odd)]
+    opt2 = AdamWFused_QuantFour([wide2, narrow2, vec2, odd2])  # the layout follows the checkpoint
     opt2.load_state_dict(opt.state_dict())
     o2 = opt2.state[wide2]["variance_qstate"]["overhead"]
     assert o2["max_dims"][0].dtype == torch.float32 and bool((o2["max_dims"][0] == 1.0 + 2.0 ** -20).all())
@@ -213,9 +216,12 @@ def test_rank1_state_layout_and_round_trip():
 def test_rank1_state_layout_of_tensors_with_more_than_two_dimensions():
     """one statistic per dimension in keepdim shape (the draft's max_dims), plus the derived
     scale of every flattened row; a state_dict round trip restores statistics and recomputes
-    the row scales; five dimensions, or a last dimension that is not a multiple of 8, keep
-    block scales"""
-    t3, t4, t5, odd = [torch.nn.Parameter(torch.randn(s)) for s in ((4, 6, 256), (3, 2, 5, 160), (2, 2, 2, 2, 512), (8, 8, 100))]
+    the row scales; five dimensions, or a last dimension of 1, keep block scales"""
+    t3, t4, t5, odd = [torch.nn.Parameter(torch.randn(s)) for s in ((4, 6, 256), (3, 2, 5, 160), (2, 2, 2, 2, 512), (80, 80, 1))]
+    last_odd = torch.nn.Parameter(torch.randn(8, 8, 100))
+    o_odd = AdamWFused_QuantFour([last_odd], variance_scale_type="rank1")
+    o_odd._init_state(last_odd)
+    assert [tuple(t.shape) for t in o_odd.state[last_odd]["variance_qstate"]["overhead"]["max_dims"]] == [(8, 1, 1), (1, 8, 1), (1, 1, 100)]
     opt = AdamWFused_QuantFour([t3, t4, t5, odd], variance_scale_type="rank1")
     for p in (t3, t4, t5, odd):
         opt._init_state(p)
