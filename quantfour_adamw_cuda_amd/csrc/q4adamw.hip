@@ -8,9 +8,11 @@
 //   q4adamw_rank1.h   rank-1 scaling: statistics, commit, folds
 //   q4adamw_aux.h     small-tensor step, gradient norm, quantize / dequantize
 //
-// Build: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off -shared -fPIC
-// (-ffp-contract=off matters: the moment updates must be individually rounded
-// fp32 multiplies and adds; fused multiply-adds appear only where written out).
+// Build (quantfour_adamw_cuda_amd/build.py): every q4adamw*.hip is compiled by itself with
+// hipcc --offload-arch=gfx950 -O3 -ffp-contract=off -fPIC -c, side by side, and the objects
+// are linked into one shared library (-ffp-contract=off matters: the moment updates and the
+// exact parameter update must be individually rounded fp32 operations; fused multiply-adds
+// appear only where written out).
 //
 // Work decomposition of the fused kernel (shaped by measurement: HBM on this part
 // streams best when every wave is short-lived, touches 1 KiB of the widest stream

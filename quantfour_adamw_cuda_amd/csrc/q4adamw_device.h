@@ -1,6 +1,7 @@
 // Device helpers of the 4-bit AdamW kernels: address spaces and buffer resources, wave
-// reductions, 16-bit element conversion, element loads and stores, the exact quantizers, the rounding
-// noise, the tensor search.
+// reductions, 16-bit element conversion, element loads and stores, the exact quantizers, the
+// rounding noise, the correctly rounded square root and quotients of the exact parameter
+// update, the tensor search.
 #pragma once
 #include "q4adamw_args.h"
 

@@ -1,6 +1,7 @@
 // The fused 4-bit AdamW step: one tile of one tensor (process_tile) and the kernels built on
-// it -- block-scaled, stochastic rounding, rank-1 scaled second moment (statistics, update,
-// commit).
+// it -- block-scaled, and the update kernels of the rank-1 scaled second moment -- each with
+// nearest or stochastic rounding, with or without gradient options, and with the folded or
+// the exact form of the parameter update.
 #pragma once
 #include "q4adamw_device.h"
 
@@ -27,6 +28,10 @@ struct Geometry {
 // step's new statistics (complete before this kernel starts) quantize.
 // SR: both moments are rounded stochastically between the two neighbouring code-book
 // entries; the noise of element e is a hash of e and the tensor's salt of this step.
+// EXACT: the parameter comes from the reference's expression with each of its seven
+// operations rounded as IEEE 754 rounds it (optim/cuda_adamw_kernels.cu:334,351), by short
+// sequences inside their domains and the general expansions outside them; otherwise from the
+// folded form with the hardware's square root and reciprocal (a tolerance).
 // SHAPE (with RANK1): how a tile lies in its matrix.  kTileWide: rows are at least a tile
 // long, so a tile touches one row or two.  kTileNarrow: rows may be shorter than a tile.
 // kTileRows: rows are a whole number of quantization blocks long and tiles start at the

@@ -169,10 +169,12 @@ static void refusals(void) {
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), 0);   /* 0 x 0 */
   r[0].rows = 4; r[0].cols = 520;
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* null pointers */
-  r[0].cols = 516;
-  EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* cols % 8 */
-  r[0].cols = 8;
-  EXPECT(q4adamw_fused_4bit_rank1_multi_sr(r, 1, NULL, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* cols < 16 */
+  r[0].cols = 1;
+  EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* one column */
+  r[0].rows = (int64_t)1 << 20; r[0].cols = 4100;   /* rows of any length: fewer than 2^32 elements */
+  EXPECT(q4adamw_fused_4bit_rank1_multi_sr(r, 1, NULL, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_TOO_LARGE);
+  TRUE_(q4adamw_rank1_form(100, 516, 0) == 3 && q4adamw_rank1_form(100, 8, 1) == 3 && q4adamw_rank1_form(4096, 4096, 0) == 0);
+  EXPECT(q4adamw_rank1_form(0, 16, 0), Q4ADAMW_ERR_ARG);
   r[0].rows = -1;
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);
   r[0].rows = (int64_t)1 << 40; r[0].cols = 1024;
@@ -190,7 +192,7 @@ static void refusals(void) {
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ALIGN);
   r[0].lead_max_next[1] = scales + 216; r[0].lead_shape[1] = 4;
   EXPECT(q4adamw_fused_4bit_rank1_multi(r, 1, F, F, B1, B2, LR, WD, EPS, 1.0f, NULL, NULL), Q4ADAMW_ERR_ARG);   /* 2 x 4 != 6 */
-  EXPECT(q4adamw_quantize_rank1_scaled(buf, 4, 12, scales, scales + 64, codes, NULL), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_quantize_rank1_scaled(buf, 4, -12, scales, scales + 64, codes, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_quantize_rank1_scaled(buf, 4, 16, NULL, scales + 64, codes, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_quantize_rank1_scaled(buf, 0, 16, scales, scales + 64, codes, NULL), 0);
   EXPECT(q4adamw_bias_table(0.9f, 0.999f, 1, 4, buf), 0);
@@ -198,7 +200,7 @@ static void refusals(void) {
   EXPECT(q4adamw_device_step(NULL, buf, 1, 4, NULL, B1, B2, LR, WD, EPS, NULL, buf + 64, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_device_step(buf, buf + 16, 1, 4, NULL, B1, B2, LR, WD, EPS, NULL, (char *)(buf + 64) + 4, NULL), Q4ADAMW_ERR_ALIGN);
   EXPECT(q4adamw_device_step(buf, buf + 16, 1, 0, NULL, B1, B2, LR, WD, EPS, NULL, buf + 64, NULL), Q4ADAMW_ERR_ARG);
-  EXPECT(q4adamw_quantize_rank1(buf, 4, 12, codes, scales, scales + 64, NULL), Q4ADAMW_ERR_ARG);
+  EXPECT(q4adamw_quantize_rank1(buf, -4, 12, codes, scales, scales + 64, NULL), Q4ADAMW_ERR_ARG);
   EXPECT(q4adamw_quantize_rank1(buf, 0, 16, codes, scales, scales + 64, NULL), 0);
   EXPECT(q4adamw_quantize_rank1(buf, (int64_t)1 << 23, 8, codes, scales, scales + 64, NULL), Q4ADAMW_ERR_TOO_LARGE);
   EXPECT(q4adamw_dequantize_rank1(codes, scales, scales + 64, -2, 16, buf, NULL), Q4ADAMW_ERR_ARG);
