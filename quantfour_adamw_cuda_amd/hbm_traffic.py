@@ -35,7 +35,7 @@ ROOT = os.path.dirname(_HERE)
 DEFAULT_PATH = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 COPY_KERNEL = "probe_move_kernel<0>"
 COPY_BYTES = 4 << 30
-STEP_KERNELS = ("fused_4bit_kernel", "fused_4bit_rank1", "rank1_stats_kernel", "rank1_commit_kernel",
+STEP_KERNELS = ("fused_4bit_kernel", "fused_4bit_rank1", "rank1_stats_kernel", "rank1_stats_any_kernel", "rank1_commit_kernel",
                 "rank1_fold_kernel", "single_tensor_kernel")
 
 
