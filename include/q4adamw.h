@@ -323,6 +323,9 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
  * GPU share the one array: two calls that overlap there (different streams, different
  * threads) race; calls on one stream, or otherwise ordered, do not.  The first call on a
  * device asks the runtime for the array's address (no allocation); make it outside a capture.
+ * The address is kept per device for the life of the process: the stream must belong to the
+ * current device (a stream of another device is refused with Q4ADAMW_ERR_ARG), and a process
+ * that resets a device (hipDeviceReset) must not call this entry point on it afterwards.
  */
 int q4adamw_grad_norm_static(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
                              const float *grad_scale_dev, float max_norm, float *out3, void *stream);

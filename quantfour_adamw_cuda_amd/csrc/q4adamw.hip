@@ -649,10 +649,17 @@ static __device__ __align__(256) double g_norm_scratch[kNormPartials];
 constexpr int kMaxDevices = 64;
 static std::atomic<double *> g_norm_scratch_ptr[kMaxDevices];
 
-static int norm_scratch(double **out) {
+static int norm_scratch(hipStream_t stream, double **out) {
   int dev = -1;
   Q4_HIP(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return fail(Q4ADAMW_ERR_ARG, "device ordinal beyond the scratch table");
+  // every device has its own copy of the array: a stream of another device than the current
+  // one would run the kernels there with this device's address
+  if (stream != nullptr && stream != hipStreamPerThread) {
+    hipDevice_t stream_dev = -1;
+    Q4_HIP(hipStreamGetDevice(stream, &stream_dev));
+    if (stream_dev != dev) return fail(Q4ADAMW_ERR_ARG, "the stream belongs to another device than the current one");
+  }
   double *p = g_norm_scratch_ptr[dev].load(std::memory_order_acquire);
   if (!p) {   // first call on this device (two threads racing here find the same address)
     void *sym = nullptr;
@@ -833,7 +840,7 @@ int q4adamw_grad_norm(const q4adamw_grad *grads, int count, int g_dtype, float g
 int q4adamw_grad_norm_static(const q4adamw_grad *grads, int count, int g_dtype, float grad_scale,
                              const float *grad_scale_dev, float max_norm, float *out3, void *stream) {
   double *partials = nullptr;
-  if (int rc = norm_scratch(&partials)) return rc;
+  if (int rc = norm_scratch(static_cast<hipStream_t>(stream), &partials)) return rc;
   return grad_norm_impl(grads, count, g_dtype, grad_scale, grad_scale_dev, max_norm, partials, out3, stream);
 }
 

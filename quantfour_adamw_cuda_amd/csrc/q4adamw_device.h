@@ -356,6 +356,19 @@ __device__ __forceinline__ float hash_low_half_as_float(uint32_t y) {
   return (float)lo;
 }
 
+// halves' high 16 bits if q >= thr, else its low 16 bits (a NaN on either side: the low half).
+// The select reads the halves through its operand selectors, so the choice between two small
+// numbers kept in one word costs a compare and one more instruction.
+__device__ __forceinline__ uint32_t high_half_if_ge(float q, float thr, uint32_t halves) {
+  uint32_t r;
+  asm("v_cmp_ge_f32_e32 vcc, %1, %2\n\t"
+      "v_cndmask_b32_sdwa %0, %3, %3, vcc dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
+      : "=v"(r)
+      : "v"(q), "v"(thr), "v"(halves)
+      : "vcc");
+  return r;
+}
+
 // noise in (0, 1) from a 16-bit number (as a float): (2 n + 1) / 2^17, exact
 constexpr float kNoiseStep = 1.52587890625e-05f;     // 2^-16
 __device__ __forceinline__ float sr_noise_value(float n16) {
@@ -478,7 +491,7 @@ __device__ __forceinline__ float sqrt_rn(float v) {
 // RN(x / c) given y = RN(1/c), for 2^-60 <= |x|, c <= 2^60: quotient, exact residual, one
 // correction.  The corrected value is t + r * (y - 1/c) with t the true quotient, within
 // 4.5 * 2^-24 ulp of t, so the result can differ from RN(t) only where t comes that close to
-// the midpoint of two floats; tests/native/check_division.c lists every such (x, c) -- for all
+// the midpoint of two floats; tests/native/check_exact_update.c lists every such (x, c) -- for all
 // 2^23 divisor mantissas -- and shows that the sequence rounds each of them correctly.
 __device__ __forceinline__ float div_by_reciprocal(float x, float c, float y) {
   const float q0 = x * y;
@@ -558,8 +571,8 @@ template <bool SR>
 __device__ __forceinline__ TableSlot request_table_slot(int tid) {
   TableSlot s;
   if (SR) {
-    const SrEntry e = kSrHalfTable.e[tid];
-    s.entry = make_uint2(e.thr, e.base);
+    const SrSlot e = kSrHalfTable.e[tid];
+    s.entry = make_uint2(e.thr, e.offsets);
     const SrAffine af = kSrAffine.e[tid < 17 ? tid : 0];
     s.interval = make_uint2(f2bits(af.a), f2bits(af.c));
   } else {

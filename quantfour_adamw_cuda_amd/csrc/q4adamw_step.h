@@ -411,8 +411,8 @@ __device__ __forceinline__ void process_tile(const Desc &T, int64_t tb, int lane
       const uint2 ent[2] = {ent0, ent1};
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const uint32_t k_raw = ent[h].y + (qq[h] >= bits2f(ent[h].x) ? 1u : 0u);
-        const float2 af = *reinterpret_cast<const float2 *>(lds_bytes + kLdsIntervals * 8u + k_raw * 8u);
+        const uint32_t interval = high_half_if_ge(qq[h], bits2f(ent[h].x), ent[h].y);   // byte offset into the affine table
+        const float2 af = *reinterpret_cast<const float2 *>(lds_bytes + kLdsIntervals * 8u + interval);
         const float y = __builtin_fmaf(um.x[j + h], -kNoiseStep, __builtin_fmaf(qq[h], af.x, af.y));
         vfrac = __builtin_fminf(vfrac, __builtin_amdgcn_fractf(y));
         mword = append_code<N>(mword, (uint32_t)(int)y, j + h);

@@ -189,13 +189,25 @@ Q4_HD constexpr SrEntry sr_entry(uint32_t half_index) {
   return out;
 }
 
+// The table as the kernels keep it: the interval number k_raw leads to entry [k_raw] of the
+// 8-byte affine table below, so a bucket's entry carries the two byte offsets it can lead to
+// as the halves of one word, 8 * base in the low half (q below the bucket's code-book entry,
+// or no entry in the bucket) and 8 * (base + 1) in the high half.
+struct SrSlot {
+  uint32_t thr;      // as SrEntry::thr
+  uint32_t offsets;  // 8 * base | 8 * (base + 1) << 16
+};
+
 struct SrHalfTable {
-  SrEntry e[kHalfTableEntries];
+  SrSlot e[kHalfTableEntries];
 };
 
 constexpr SrHalfTable make_sr_half_table() {
   SrHalfTable t{};
-  for (uint32_t h = 0; h < kHalfTableEntries; ++h) t.e[h] = sr_entry(h);
+  for (uint32_t h = 0; h < kHalfTableEntries; ++h) {
+    const SrEntry e = sr_entry(h);
+    t.e[h] = SrSlot{e.thr, (e.base * 8u) | ((e.base + 1u) * 8u) << 16};
+  }
   return t;
 }
 
