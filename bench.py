@@ -287,6 +287,17 @@ def update_form_of(param_update, p_dtype_s, variance_scale, round_type):
     return "exact" if plain else "folded"
 
 
+def traffic_source(rec):
+    """where roofline.traffic comes from, in words"""
+    if not rec:
+        return "no counter record for these kernel sources"
+    src = f"profiles/hbm_traffic.json, kernel sources {rec['source_hash']}"
+    if rec.get("write_source_hash", rec["source_hash"]) != rec["source_hash"]:
+        src += (f"; the written bytes are a WRITE_SIZE session on sources {rec['write_source_hash']}"
+                f" ({rec.get('write_note', 'no note')})")
+    return src
+
+
 def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None, param_update="auto"):
     from quantfour_adamw_cuda_amd import hbm_traffic
     achieved = m["algo_bytes"] / m["kernel_s"] / 1e9
@@ -302,8 +313,7 @@ def roofline_entry(m, workload, variance_scale, round_type, ceiling_gbs=None, pa
         # per launch, averaged over the step's launches (they differ in size): HBM bytes from
         # hardware counters, algorithmic bytes, duration; achieved = algorithmic bytes / duration
         "traffic": rec["bytes_per_step"] / n if rec else None,
-        "traffic_source": (f"profiles/hbm_traffic.json, kernel sources {rec['source_hash']}" if rec else
-                           "no counter record for these kernel sources"),
+        "traffic_source": traffic_source(rec),
         "algorithmic_bytes_per_launch": m["algo_bytes"] / n,
         "kernel_ms_per_launch": m["kernel_s"] * 1e3 / n,
         "kernel_launches_per_step": n,

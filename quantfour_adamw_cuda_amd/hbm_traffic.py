@@ -87,7 +87,17 @@ def _sum_counter(csv_paths, counter):
 
 
 def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, out_path, profile=None,
-           param_update="auto"):
+           param_update="auto", write_from_record=None, write_note=None):
+    """write_from_record: instead of a WRITE_SIZE session (write_csv is then ignored), take the
+    written bytes from the same key of an earlier record file -- for a session that could not
+    be taken on the present sources.  The entry then names the sources that half was measured on
+    (`write_source_hash`) and must say why it still describes the present kernels (`write_note`);
+    bench.py repeats both beside the number."""
+    if write_from_record:
+        if not write_note:
+            raise SystemExit("--write-from-record needs --write-note: why the earlier session still describes these kernels")
+        return _record_with_earlier_write(workload, variance_scale, round_type, fetch_csv, steps, out_path, profile,
+                                          param_update, write_from_record, write_note)
     fetch, write = _sum_counter(fetch_csv, "FETCH_SIZE"), _sum_counter(write_csv, "WRITE_SIZE")
 
     def pick(table, names):
@@ -129,6 +139,49 @@ def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, ou
     return entry
 
 
+def _record_with_earlier_write(workload, variance_scale, round_type, fetch_csv, steps, out_path, profile,
+                               param_update, earlier_path, note):
+    fetch = _sum_counter(fetch_csv, "FETCH_SIZE")
+    copies = {k: v for k, v in fetch.items() if COPY_KERNEL in k}
+    if not copies:
+        raise SystemExit(f"no {COPY_KERNEL} dispatch in the fetch run: profile bench.py with --calibrate-copy")
+    kib, n = map(sum, zip(*copies.values()))
+    fetch_scale = (COPY_BYTES / 1024.0) / (kib / n)
+    step_kernels = {k: v for k, v in fetch.items() if any(name in k for name in STEP_KERNELS)}
+    fetch_b = sum(v[0] for v in step_kernels.values()) * 1024.0 * fetch_scale / steps
+    k = key(workload, variance_scale, round_type, param_update)
+    with open(earlier_path) as f:
+        earlier = json.load(f)["entries"].get(k)
+    if not earlier:
+        raise SystemExit(f"{earlier_path} holds no entry {k}")
+    entry = {
+        "source_hash": source_hash(),
+        "bytes_per_step": fetch_b + earlier["write_bytes_per_step"],
+        "fetch_bytes_per_step": fetch_b,
+        "write_bytes_per_step": earlier["write_bytes_per_step"],
+        "fetch_scale": fetch_scale,
+        "write_scale": earlier["write_scale"],
+        "write_source_hash": earlier["source_hash"],
+        "write_note": note,
+        "dispatches_per_step": sum(v[1] for v in step_kernels.values()) / steps,
+        "steps_profiled": steps,
+        "kernels": sorted(step_kernels),
+    }
+    if profile:
+        entry["profile"] = profile
+    try:
+        with open(out_path) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        doc = {"entries": {}}
+    doc.setdefault("entries", {})[k] = entry
+    doc["unit"] = "bytes of HBM traffic per optimizer step (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)"
+    with open(out_path, "w") as f:
+        json.dump(doc, f, indent=1, sort_keys=True)
+        f.write("\n")
+    return entry
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--workload", required=True)
@@ -136,13 +189,19 @@ def main():
     ap.add_argument("--round-type", default="real-nearest")
     ap.add_argument("--param-update", default="auto")
     ap.add_argument("--fetch-csv", nargs="+", required=True)
-    ap.add_argument("--write-csv", nargs="+", required=True)
+    ap.add_argument("--write-csv", nargs="+", default=[])
+    ap.add_argument("--write-from-record", default=None,
+                    help="take the written bytes from this earlier record file instead of a WRITE_SIZE session")
+    ap.add_argument("--write-note", default=None,
+                    help="with --write-from-record: why that session still describes the present kernels")
     ap.add_argument("--steps", type=int, required=True, help="optimizer steps the profiled command ran (warm-up included)")
     ap.add_argument("--out", default=DEFAULT_PATH)
     ap.add_argument("--profile", default=None, help="the profiles/ summary that documents the run")
     a = ap.parse_args()
+    if not a.write_csv and not a.write_from_record:
+        ap.error("give --write-csv or --write-from-record")
     print(json.dumps(record(a.workload, a.variance_scale, a.round_type, a.fetch_csv, a.write_csv, a.steps,
-                            a.out, a.profile, a.param_update), indent=1))
+                            a.out, a.profile, a.param_update, a.write_from_record, a.write_note), indent=1))
 
 
 if __name__ == "__main__":

@@ -53,6 +53,35 @@ def test_record_scales_by_the_copy_and_lookup_follows_the_sources(tmp_path, monk
     assert ht.lookup("llama3-8b", path=out) is None
 
 
+def test_written_bytes_from_an_earlier_record_carry_their_provenance(tmp_path, monkeypatch):
+    """a WRITE_SIZE session that could not be taken on the present sources: the entry takes that
+    half from an earlier record, names the sources it was measured on and says why it still holds"""
+    four_gib_kib = float(4 << 20)
+    fetch = str(tmp_path / "f.csv")
+    write = str(tmp_path / "w.csv")
+    _write(fetch, "FETCH_SIZE", [(COPY, four_gib_kib / 2)] + [(STEP, 1000.0), (SMALL, 10.0)] * 2)
+    _write(write, "WRITE_SIZE", [(COPY, four_gib_kib)] + [(STEP, 1500.0), (SMALL, 20.0)] * 2)
+    earlier = str(tmp_path / "earlier.json")
+    monkeypatch.setattr(ht, "source_hash", lambda: "a" * 16)
+    e0 = ht.record("llama3-8b", "group", "real-nearest", [fetch], [write], 2, earlier)
+    monkeypatch.setattr(ht, "source_hash", lambda: "b" * 16)
+    out = str(tmp_path / "record.json")
+    with pytest.raises(SystemExit, match="write-note"):
+        ht.record("llama3-8b", "group", "real-nearest", [fetch], [], 2, out, write_from_record=earlier)
+    with pytest.raises(SystemExit, match="no entry"):
+        ht.record("gpt2-small", "group", "real-nearest", [fetch], [], 2, out, write_from_record=earlier, write_note="x")
+    e = ht.record("llama3-8b", "group", "real-nearest", [fetch], [], 2, out, write_from_record=earlier,
+                  write_note="same instructions")
+    assert e["source_hash"] == "b" * 16 and e["write_source_hash"] == "a" * 16 and e["write_note"] == "same instructions"
+    assert e["fetch_bytes_per_step"] == pytest.approx(e0["fetch_bytes_per_step"])
+    assert e["write_bytes_per_step"] == e0["write_bytes_per_step"]
+    assert e["bytes_per_step"] == pytest.approx(e["fetch_bytes_per_step"] + e["write_bytes_per_step"])
+    assert ht.lookup("llama3-8b", path=out)["write_source_hash"] == "a" * 16     # valid for the present sources
+    import bench
+    assert "a" * 16 in bench.traffic_source(e) and "same instructions" in bench.traffic_source(e)
+    assert "WRITE_SIZE" not in bench.traffic_source(e0)
+
+
 def test_a_profile_without_the_calibration_copy_is_refused(tmp_path):
     fetch = str(tmp_path / "f.csv")
     write = str(tmp_path / "w.csv")
@@ -94,3 +123,5 @@ def test_committed_record_is_well_formed():
         assert e["bytes_per_step"] == pytest.approx(e["fetch_bytes_per_step"] + e["write_bytes_per_step"])
         assert 1.9 < e["fetch_scale"] < 2.1 and 0.95 < e["write_scale"] < 1.05
         assert len(e["source_hash"]) == 16 and e["dispatches_per_step"] >= 1
+        if "write_source_hash" in e:      # that half was measured on other sources: it says which and why
+            assert len(e["write_source_hash"]) == 16 and len(e["write_note"]) > 20
