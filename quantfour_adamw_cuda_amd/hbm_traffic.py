@@ -4,15 +4,22 @@ profiles/hbm_traffic.json and read by bench.py for its `roofline.traffic` field.
 An entry is valid for the kernel sources it was measured on: every entry carries the hash of
 csrc/q4adamw*.hip and csrc/q4adamw_*.h at that time, and `lookup` returns None for an entry
 whose hash differs from the sources in the tree, so a number never outlives the kernel it
-describes.
+describes.  One exception is spelled out in the entry itself: when a WRITE_SIZE session could
+not be taken on the present sources, `--write-from-record` takes the written bytes from an
+earlier record file; the entry then names the sources that half was measured on
+(`write_source_hash`) and why it still describes the present kernels (`write_note`).
+
+One profiler session per job on the GPU machine, `python3 -u`, `--progress` and a hard
+`timeout -s KILL`: counter sessions of this command have stopped responding now and then, and
+that way a stalled one ends with a non-zero status and shows the phase it stopped in.
 
 Recording (rocprofv3 cannot split counters over passes, so one run per counter; on the GPU
 machine, from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd -`):
 
     rocprofv3 --pmc FETCH_SIZE --output-format csv -d out/pmc_fetch -o fetch -- \\
-        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy --progress
+        python3 -u bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy --progress
     rocprofv3 --pmc WRITE_SIZE --output-format csv -d out/pmc_write -o write -- \\
-        python3 bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy --progress
+        python3 -u bench.py --steps 3 --warmup 1 --configs none --no-ceiling --no-cpu-baseline --calibrate-copy --progress
     python3 -m quantfour_adamw_cuda_amd.hbm_traffic --workload llama3-8b --steps 4 \\
         --fetch-csv 'out/pmc_fetch/**/*counter_collection.csv' \\
         --write-csv 'out/pmc_write/**/*counter_collection.csv' \\
@@ -86,6 +93,21 @@ def _sum_counter(csv_paths, counter):
     return out
 
 
+def _store(out_path, entry_key, entry):
+    """adds or replaces one entry of the record file"""
+    try:
+        with open(out_path) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        doc = {"entries": {}}
+    doc.setdefault("entries", {})[entry_key] = entry
+    doc["unit"] = "bytes of HBM traffic per optimizer step (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)"
+    with open(out_path, "w") as f:
+        json.dump(doc, f, indent=1, sort_keys=True)
+        f.write("\n")
+    return entry
+
+
 def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, out_path, profile=None,
            param_update="auto", write_from_record=None, write_note=None):
     """write_from_record: instead of a WRITE_SIZE session (write_csv is then ignored), take the
@@ -126,17 +148,7 @@ def record(workload, variance_scale, round_type, fetch_csv, write_csv, steps, ou
     }
     if profile:
         entry["profile"] = profile
-    try:
-        with open(out_path) as f:
-            doc = json.load(f)
-    except (OSError, ValueError):
-        doc = {"entries": {}}
-    doc.setdefault("entries", {})[key(workload, variance_scale, round_type, param_update)] = entry
-    doc["unit"] = "bytes of HBM traffic per optimizer step (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)"
-    with open(out_path, "w") as f:
-        json.dump(doc, f, indent=1, sort_keys=True)
-        f.write("\n")
-    return entry
+    return _store(out_path, key(workload, variance_scale, round_type, param_update), entry)
 
 
 def _record_with_earlier_write(workload, variance_scale, round_type, fetch_csv, steps, out_path, profile,
@@ -169,17 +181,7 @@ def _record_with_earlier_write(workload, variance_scale, round_type, fetch_csv, 
     }
     if profile:
         entry["profile"] = profile
-    try:
-        with open(out_path) as f:
-            doc = json.load(f)
-    except (OSError, ValueError):
-        doc = {"entries": {}}
-    doc.setdefault("entries", {})[k] = entry
-    doc["unit"] = "bytes of HBM traffic per optimizer step (FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)"
-    with open(out_path, "w") as f:
-        json.dump(doc, f, indent=1, sort_keys=True)
-        f.write("\n")
-    return entry
+    return _store(out_path, k, entry)
 
 
 def main():
