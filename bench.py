@@ -292,9 +292,13 @@ def traffic_source(rec):
     if not rec:
         return "no counter record for these kernel sources"
     src = f"profiles/hbm_traffic.json, kernel sources {rec['source_hash']}"
-    if rec.get("write_source_hash", rec["source_hash"]) != rec["source_hash"]:
-        src += (f"; the written bytes are a WRITE_SIZE session on sources {rec['write_source_hash']}"
-                f" ({rec.get('write_note', 'no note')})")
+    for half, counter in (("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")):
+        h = rec.get(f"{half}_source_hash", rec["source_hash"])
+        if h != rec["source_hash"]:
+            src += f"; the {counter} session ran on sources {h}"
+    for k in ("write_note", "note"):
+        if rec.get(k):
+            src += f" ({rec[k]})"
     return src
 
 

@@ -358,10 +358,14 @@ __device__ __forceinline__ float hash_low_half_as_float(uint32_t y) {
 
 // halves' high 16 bits if q >= thr, else its low 16 bits (a NaN on either side: the low half).
 // The select reads the halves through its operand selectors, so the choice between two small
-// numbers kept in one word costs a compare and one more instruction.
+// numbers kept in one word costs a compare and one more instruction.  On this target a vector
+// instruction that reads VCC needs two wait states after the vector instruction that wrote it;
+// the compiler keeps that distance in its own code and does not look into this block, hence
+// the s_nop (it holds back this wave only: the other waves of the SIMD issue meanwhile).
 __device__ __forceinline__ uint32_t high_half_if_ge(float q, float thr, uint32_t halves) {
   uint32_t r;
   asm("v_cmp_ge_f32_e32 vcc, %1, %2\n\t"
+      "s_nop 1\n\t"
       "v_cndmask_b32_sdwa %0, %3, %3, vcc dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
       : "=v"(r)
       : "v"(q), "v"(thr), "v"(halves)

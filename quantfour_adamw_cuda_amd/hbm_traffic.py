@@ -4,10 +4,11 @@ profiles/hbm_traffic.json and read by bench.py for its `roofline.traffic` field.
 An entry is valid for the kernel sources it was measured on: every entry carries the hash of
 csrc/q4adamw*.hip and csrc/q4adamw_*.h at that time, and `lookup` returns None for an entry
 whose hash differs from the sources in the tree, so a number never outlives the kernel it
-describes.  One exception is spelled out in the entry itself: when a WRITE_SIZE session could
+describes.  The exceptions are spelled out in the entry itself: when a WRITE_SIZE session could
 not be taken on the present sources, `--write-from-record` takes the written bytes from an
-earlier record file; the entry then names the sources that half was measured on
-(`write_source_hash`) and why it still describes the present kernels (`write_note`).
+earlier record file, and `--restamp-from-record` carries whole entries over a change of the
+sources; such an entry names the sources each of its sessions ran on (`fetch_source_hash`,
+`write_source_hash`) and why they still describe the present kernels (`write_note`, `note`).
 
 One profiler session per job on the GPU machine, `python3 -u`, `--progress` and a hard
 `timeout -s KILL`: counter sessions of this command have stopped responding now and then, and
@@ -184,22 +185,53 @@ def _record_with_earlier_write(workload, variance_scale, round_type, fetch_csv, 
     return _store(out_path, k, entry)
 
 
+def restamp(from_path, out_path, note, keys=None):
+    """Carries entries of an earlier record over to the present sources: for a change of the
+    sources after which the sessions could not be taken again.  Every carried entry keeps the
+    hashes of the sources its two sessions ran on (`fetch_source_hash`, `write_source_hash`)
+    and says why they still describe the present kernels (`note`); `source_hash` becomes the
+    present one, which is what `lookup` compares."""
+    if not note:
+        raise SystemExit("a carried entry needs a note: why the earlier sessions still describe these kernels")
+    with open(from_path) as f:
+        earlier = json.load(f)["entries"]
+    out = []
+    for k in (keys or sorted(earlier)):
+        if k not in earlier:
+            raise SystemExit(f"{from_path} holds no entry {k}")
+        e = dict(earlier[k])
+        e["fetch_source_hash"] = e.get("fetch_source_hash", e["source_hash"])
+        e["write_source_hash"] = e.get("write_source_hash", e["source_hash"])
+        e["source_hash"] = source_hash()
+        e["note"] = note
+        out.append(_store(out_path, k, e))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--workload", required=True)
+    ap.add_argument("--workload", default=None)
     ap.add_argument("--variance-scale", default="group")
     ap.add_argument("--round-type", default="real-nearest")
     ap.add_argument("--param-update", default="auto")
-    ap.add_argument("--fetch-csv", nargs="+", required=True)
+    ap.add_argument("--fetch-csv", nargs="+", default=[])
     ap.add_argument("--write-csv", nargs="+", default=[])
     ap.add_argument("--write-from-record", default=None,
                     help="take the written bytes from this earlier record file instead of a WRITE_SIZE session")
     ap.add_argument("--write-note", default=None,
                     help="with --write-from-record: why that session still describes the present kernels")
-    ap.add_argument("--steps", type=int, required=True, help="optimizer steps the profiled command ran (warm-up included)")
+    ap.add_argument("--steps", type=int, default=None, help="optimizer steps the profiled command ran (warm-up included)")
     ap.add_argument("--out", default=DEFAULT_PATH)
     ap.add_argument("--profile", default=None, help="the profiles/ summary that documents the run")
+    ap.add_argument("--restamp-from-record", default=None,
+                    help="carry every entry of this earlier record file over to the present sources (needs --note)")
+    ap.add_argument("--note", default=None, help="with --restamp-from-record: why the earlier sessions still hold")
     a = ap.parse_args()
+    if a.restamp_from_record:
+        print(json.dumps(restamp(a.restamp_from_record, a.out, a.note), indent=1))
+        return
+    if not a.workload or not a.fetch_csv or a.steps is None:
+        ap.error("give --workload, --fetch-csv and --steps (or --restamp-from-record)")
     if not a.write_csv and not a.write_from_record:
         ap.error("give --write-csv or --write-from-record")
     print(json.dumps(record(a.workload, a.variance_scale, a.round_type, a.fetch_csv, a.write_csv, a.steps,

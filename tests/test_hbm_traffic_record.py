@@ -80,6 +80,21 @@ def test_written_bytes_from_an_earlier_record_carry_their_provenance(tmp_path, m
     import bench
     assert "a" * 16 in bench.traffic_source(e) and "same instructions" in bench.traffic_source(e)
     assert "WRITE_SIZE" not in bench.traffic_source(e0)
+    # the sources change once more and no session can be taken: the entry is carried over whole,
+    # keeps the sources of both of its sessions and gains the reason
+    monkeypatch.setattr(ht, "source_hash", lambda: "c" * 16)
+    assert ht.lookup("llama3-8b", path=out) is None
+    carried = str(tmp_path / "carried.json")
+    with pytest.raises(SystemExit, match="note"):
+        ht.restamp(out, carried, None)
+    with pytest.raises(SystemExit, match="no entry"):
+        ht.restamp(out, carried, "why", keys=["gpt2-small|group|real-nearest"])
+    (c,) = ht.restamp(out, carried, "one wait state more")
+    assert (c["source_hash"], c["fetch_source_hash"], c["write_source_hash"]) == ("c" * 16, "b" * 16, "a" * 16)
+    assert c["bytes_per_step"] == e["bytes_per_step"] and ht.lookup("llama3-8b", path=carried)["note"] == "one wait state more"
+    text = bench.traffic_source(c)
+    assert "FETCH_SIZE session ran on sources " + "b" * 16 in text and "WRITE_SIZE session ran on sources " + "a" * 16 in text
+    assert "one wait state more" in text and "same instructions" in text
 
 
 def test_a_profile_without_the_calibration_copy_is_refused(tmp_path):
@@ -123,5 +138,8 @@ def test_committed_record_is_well_formed():
         assert e["bytes_per_step"] == pytest.approx(e["fetch_bytes_per_step"] + e["write_bytes_per_step"])
         assert 1.9 < e["fetch_scale"] < 2.1 and 0.95 < e["write_scale"] < 1.05
         assert len(e["source_hash"]) == 16 and e["dispatches_per_step"] >= 1
-        if "write_source_hash" in e:      # that half was measured on other sources: it says which and why
-            assert len(e["write_source_hash"]) == 16 and len(e["write_note"]) > 20
+        for half in ("fetch", "write"):   # a half measured on other sources says which, and the entry why
+            h = e.get(half + "_source_hash", e["source_hash"])
+            assert len(h) == 16
+            if h != e["source_hash"]:
+                assert len(e.get("note", "")) > 20 or len(e.get("write_note", "")) > 20
