@@ -477,3 +477,45 @@ def test_device_code_holds_no_packed_fp32_instructions(tmp_path):
 
     assert packed(bare, "bare.s") > 0, "the probe kernel no longer provokes packed instructions: pick another"
     assert packed(flags, "flagged.s") == 0
+
+
+def test_assembly_block_keeps_the_wait_states_before_a_read_of_vcc(tmp_path):
+    """On gfx950 a vector instruction that reads VCC needs two wait states after the vector
+    instruction that wrote it.  The compiler keeps them in its own code (shown here on a plain
+    compare + select) and does not look into assembly blocks, so the one block of the kernels
+    that has such a pair (the stochastic-rounding select of the affine table's offset) must
+    keep them itself."""
+    import re
+    import subprocess
+    from quantfour_adamw_cuda_amd import build
+    csrc = os.path.join(os.path.dirname(build.__file__), "csrc")
+    src = tmp_path / "vcc.hip"
+    src.write_text('#include "q4adamw_device.h"\n'
+                   "__global__ void block(const float *q, const float *t, const uint32_t *h, uint32_t *o) {\n"
+                   "  int i = threadIdx.x; o[i] = q4::high_half_if_ge(q[i], t[i], h[i]); }\n"
+                   "__global__ void plain(const float *a, const float *b, const float *c, const float *d, float *o) {\n"
+                   "  int i = threadIdx.x; o[i] = a[i] >= b[i] ? c[i] : d[i]; }\n")
+    flags = [f for f in build.HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    out = tmp_path / "vcc.s"
+    subprocess.run([build.hipcc_path()] + flags + ["-I", csrc, "--cuda-device-only", "-S", "-o", str(out), str(src)],
+                   check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    lines = [ln.strip() for ln in out.read_text().splitlines()]
+    lines = [ln for ln in lines if ln and not ln.startswith((";", ".", "//")) and not ln.endswith(":")]
+
+    def wait_states_before_read(writer_prefix, reader_prefix):
+        found = []
+        for i, ln in enumerate(lines):
+            if ln.startswith(writer_prefix) and " vcc" in ln:
+                n = 0
+                for nxt in lines[i + 1:]:
+                    if nxt.startswith(reader_prefix) and nxt.endswith("vcc") or ", vcc " in nxt and nxt.startswith(reader_prefix):
+                        found.append(n)
+                        break
+                    m = re.match(r"s_nop (\d+)", nxt)
+                    n += int(m.group(1)) + 1 if m else 1
+        return found
+
+    own = wait_states_before_read("v_cmp_ge_f32_e32", "v_cndmask_b32_sdwa")
+    assert own and min(own) >= 2, f"the assembly block leaves {own} wait states"
+    compilers = wait_states_before_read("v_cmp_ge_f32_e32", "v_cndmask_b32_e32")
+    assert compilers and min(compilers) >= 2, f"the compiler's own pair: {compilers}"
