@@ -214,3 +214,50 @@ def test_more_than_2_to_32_elements_in_one_tensor(cuda):
     lo, hi = rep[1][:1 << 19], rep[1][1 << 31:(1 << 31) + (1 << 19)]
     assert torch.equal(rep[3][:1 << 13], rep[3][1 << 25:(1 << 25) + (1 << 13)])      # same block scales
     assert 0.01 < float((lo != hi).float().mean()) < 0.9
+
+
+@pytest.mark.parametrize("rows_half,cols,form", [(131080, 16384, 0), (130056, 16512, 1)])
+def test_more_than_2_to_32_elements_in_one_rank1_matrix(cuda, rows_half, cols, form):
+    """Rank-1 scaling couples a matrix's rows through the column maxima, so a split run is not
+    the same computation -- unless both halves hold the same data: the matrix [A; A] has A's
+    column maxima and A's row maxima twice, so its step must equal, bit for bit, the step of A
+    alone, in its upper half (elements below 2^32) and in its lower half (offsets beyond 2^32).
+    Both update forms that a matrix of this size can take: tiles aligned to the rows, and rows
+    that end in a partial tile (which such a matrix leaves to the kernel with tiles anywhere)."""
+    from quantfour_adamw_cuda_amd import _lib, quantfour_hip as q
+    half = rows_half * cols
+    assert 2 * half > 1 << 32 and half > 1 << 31
+    assert _lib.load().q4adamw_rank1_form(2 * rows_half, cols, 1) == form
+    hp = (0.9, 0.999, 1e-3, 0.01, 1e-8)
+
+    def state(rows):
+        n = rows * cols
+        g_ = torch.Generator(device=cuda).manual_seed(21)
+        p = torch.empty(half, dtype=torch.bfloat16, device=cuda).normal_(0, 0.05, generator=g_)
+        if rows != rows_half:
+            p = torch.cat([p, p])
+        return [p.view(rows, cols), torch.zeros((n + 1) // 2, dtype=torch.uint8, device=cuda),
+                torch.zeros((n + 1) // 2, dtype=torch.uint8, device=cuda), torch.zeros((n + 127) // 128, device=cuda),
+                torch.zeros(rows, device=cuda), torch.zeros(cols, device=cuda),
+                torch.zeros(rows, device=cuda), torch.zeros(cols, device=cuda)]
+
+    one, two = state(rows_half), state(2 * rows_half)
+    gen = torch.Generator(device=cuda).manual_seed(22)
+    for step in (1, 2):
+        g = torch.empty(half, dtype=torch.bfloat16, device=cuda).normal_(0, 1e-3, generator=gen)
+        g[:cols] *= 8.0                     # a loud first row and a silent column: maxima that matter
+        g.view(rows_half, cols)[:, 5] = 0
+        gg = torch.cat([g, g])
+        for st, grad in ((one, g.view(rows_half, cols)), (two, gg.view(2 * rows_half, cols))):
+            q.fused_4bit_rank1_multi([st[0]], [grad], [st[1]], [st[2]], [st[3]], [st[4]], [st[5]], [st[6]], [st[7]],
+                                     *hp, step)
+        del gg
+        names = ("p", "m codes", "v codes", "m scales", "row maxima")
+        for name, a, b in zip(names, one[:5], two[:5]):
+            a8, b8 = a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)
+            k = a8.numel()
+            assert torch.equal(b8[:k], a8), f"step {step}: {name}, upper half"
+            assert torch.equal(b8[k:], a8), f"step {step}: {name}, lower half (offsets beyond 2^32)"
+        assert torch.equal(one[5].view(torch.int32), two[5].view(torch.int32)), f"step {step}: column maxima"
+        assert not one[6].any() and not two[6].any() and not two[7].any(), "scratch maxima return to zero"
+    assert one[1].any() and one[2].any() and float(one[5][5]) == 0.0
