@@ -87,3 +87,39 @@ def test_static_scratch_refusals(cuda):
     assert call(arr, 1, _lib.FP32, out.data_ptr()) == -4 and b"too large" in L.q4adamw_last_error()
     torch.cuda.synchronize(cuda)
     assert torch.equal(out.cpu(), torch.zeros(3))
+
+
+def test_static_scratch_under_graph_capture(cuda):
+    """One of the callers the entry point is for: code under graph capture.  The call is recorded
+    once (after a first call outside the capture, which is when the library asks the runtime for
+    its array's address) and replayed with new gradient values, with the program's own eager
+    work between the replays; every replay must give the eager workspace form's bits."""
+    L = _lib.load()
+    gen = torch.Generator().manual_seed(37)
+    gs = [torch.zeros(n, dtype=torch.bfloat16, device=cuda) for n in (3_000_017, 16384 * 40, 5)]
+    arr = _table(gs)
+    out = torch.zeros(3, device=cuda)
+
+    def fill():
+        for g in gs:
+            g.copy_((torch.randn(g.numel(), generator=gen) * 2.0).to(torch.bfloat16))
+
+    fill()
+    side = torch.cuda.Stream(device=cuda)
+    with torch.cuda.stream(side):
+        rc = L.q4adamw_grad_norm_static(arr, len(gs), _lib.BF16, 0.5, None, 1.0, out.data_ptr(), side.cuda_stream)
+        assert rc == 0, L.q4adamw_last_error()
+    torch.cuda.synchronize(cuda)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        rc = L.q4adamw_grad_norm_static(arr, len(gs), _lib.BF16, 0.5, None, 1.0, out.data_ptr(),
+                                        torch.cuda.current_stream(cuda).cuda_stream)
+        assert rc == 0, L.q4adamw_last_error()
+    for replay in range(4):
+        fill()
+        _, eager = _both(L, gs, _lib.BF16, 0.5, None, 1.0, cuda, poison=True)   # eager work in between
+        out.fill_(-1.0)
+        graph.replay()
+        torch.cuda.synchronize(cuda)
+        got = out.cpu().numpy().view(np.uint32)
+        assert np.array_equal(got, eager), f"replay {replay}: {got} vs {eager}"
